@@ -1,0 +1,275 @@
+// Embedding, residual add + RMSNorm, rotary tables, rotary + cache append,
+// SiLU gate.  One workgroup per token row; 32-bit arithmetic throughout.
+//
+// Inputs that come from a matrix product may arrive as `nsplit` partial sums
+// ([nsplit][n][cols], `split_stride` elements apart); the consumer adds them
+// in a fixed order, so a split product needs no pass of its own and gives the
+// same bits on every run.
+#include "common.hpp"
+#include "kllm_kernels.h"
+
+namespace kllm {
+
+constexpr int kThreads = 256;
+
+// x[t, :] = table[ids[t], :]   (reference: backend/model.cu:89-95)
+template <typename T>
+__global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ table,
+                             const int* __restrict__ ids, int d, int vocab) {
+  const long t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // the host has checked the range
+  const T* src = table + (long)id * d;
+  float* dst = out + t * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) dst[i] = to_f32(src[i]);
+}
+
+template <typename TIN>
+__device__ __forceinline__ float sum_splits(const TIN* __restrict__ p, int nsplit, long stride) {
+  float v = to_f32(p[0]);
+  for (int s = 1; s < nsplit; ++s) v += to_f32(p[(long)s * stride]);
+  return v;
+}
+
+// v = x[src] (+ sum of delta splits); optionally x[src] = v;
+// out[r] = v * rsqrt(mean(v^2) + eps) * w   (reference: backend/model.cu:101-122, :144-165)
+template <typename TIN, typename TOUT>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const TIN* __restrict__ delta, int nsplit,
+                                   long split_stride, const float* __restrict__ w,
+                                   TOUT* __restrict__ out, const int* __restrict__ rows, int d,
+                                   float eps, int write_x) {
+  __shared__ float red[16];
+  const long r = blockIdx.x;
+  const long src = rows ? rows[r] : r;
+  float* xr = x + src * d;
+  const TIN* dr = delta ? delta + src * d : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float v = xr[i];
+    if (dr) v += sum_splits(dr + i, nsplit, split_stride);
+    if (write_x) xr[i] = v;
+    ss += v * v;
+  }
+  if (!out) return;
+  ss = block_sum(ss, red);
+  const float scale = rsqrtf(ss / (float)d + eps);
+  TOUT* orow = out + r * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float v = xr[i];  // already the sum when write_x (same thread wrote it)
+    if (dr && !write_x) v += sum_splits(dr + i, nsplit, split_stride);
+    orow[i] = from_f32<TOUT>(v * scale * w[i]);
+  }
+}
+
+// cos/sin of pos * theta^(-2j/head_dim), angle in double
+// (reference: backend/model.cu:176-178)
+__global__ void rope_tables_kernel(float* __restrict__ cos_t, float* __restrict__ sin_t,
+                                   const int* __restrict__ positions, int n, int half, int head_dim,
+                                   double theta) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)n * half) return;
+  const int t = idx / half, j = idx % half;
+  const double freq = pow(theta, -2.0 * (double)j / (double)head_dim);
+  const double ang = (double)positions[t] * freq;
+  cos_t[idx] = (float)cos(ang);
+  sin_t[idx] = (float)sin(ang);
+}
+
+// Rotate q and k (pairs (j, j + hd/2), reference: backend/model.cu:170-184),
+// store q, and put k and v into the token's page (reference: :187-201).
+// Page layout, per page and KV head: keys [slot][hd], values [hd][slot].
+template <typename TIN, typename T>
+__global__ void rope_append_kernel(const TIN* __restrict__ qkv, int nsplit, long split_stride,
+                                   T* __restrict__ q_out, const float* __restrict__ cos_t,
+                                   const float* __restrict__ sin_t, T* __restrict__ cache,
+                                   const int* __restrict__ positions,
+                                   const int* __restrict__ span_of_token,
+                                   const int* __restrict__ block_table, int max_pages,
+                                   int page_size, int H, int KV, int hd) {
+  const long t = blockIdx.x;
+  const int half = hd / 2;
+  const int qd = H * hd, kvd = cache ? KV * hd : 0;
+  const long row = qd + 2 * kvd;
+  const TIN* in = qkv + t * row;
+  const float* c = cos_t ? cos_t + t * half : nullptr;
+  const float* s = sin_t ? sin_t + t * half : nullptr;
+
+  for (int idx = threadIdx.x; idx < H * half; idx += blockDim.x) {
+    const int h = idx / half, j = idx % half;
+    const float a = sum_splits(in + h * hd + j, nsplit, split_stride);
+    const float b = sum_splits(in + h * hd + j + half, nsplit, split_stride);
+    const float cc = c ? c[j] : 1.f, sn = s ? s[j] : 0.f;
+    T* o = q_out + t * qd + h * hd;
+    o[j] = from_f32<T>(a * cc - b * sn);
+    o[j + half] = from_f32<T>(b * cc + a * sn);
+  }
+  if (!cache) return;
+
+  const int pos = positions[t];
+  const int page = block_table[(long)span_of_token[t] * max_pages + pos / page_size];
+  const int slot = pos % page_size;
+  const long block = (long)page_size * hd;  // one (page, k|v, head) block
+  T* kpage = cache + ((long)page * 2 + 0) * KV * block;
+  T* vpage = cache + ((long)page * 2 + 1) * KV * block;
+  for (int idx = threadIdx.x; idx < KV * half; idx += blockDim.x) {
+    const int h = idx / half, j = idx % half;
+    const float a = sum_splits(in + qd + h * hd + j, nsplit, split_stride);
+    const float b = sum_splits(in + qd + h * hd + j + half, nsplit, split_stride);
+    const float cc = c ? c[j] : 1.f, sn = s ? s[j] : 0.f;
+    T* o = kpage + h * block + (long)slot * hd;
+    o[j] = from_f32<T>(a * cc - b * sn);
+    o[j + half] = from_f32<T>(b * cc + a * sn);
+  }
+  for (int idx = threadIdx.x; idx < kvd; idx += blockDim.x) {
+    const int h = idx / hd, j = idx % hd;
+    const float v = sum_splits(in + qd + kvd + idx, nsplit, split_stride);
+    vpage[h * block + (long)j * page_size + slot] = from_f32<T>(v);
+  }
+}
+
+// out[t, i] = silu(gate[t, i]) * up[t, i], gate = cols [0, f), up = cols [f, 2f)
+// (reference: backend/model.cu:477-483)
+template <typename TIN, typename TOUT>
+__global__ void silu_mul_kernel(const TIN* __restrict__ gu, int nsplit, long split_stride,
+                                TOUT* __restrict__ out, long n, int f) {
+  const long total = n * f;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long t = idx / f;
+    const int i = idx % f;
+    const TIN* row = gu + t * 2 * f;
+    const float g = sum_splits(row + i, nsplit, split_stride);
+    const float u = sum_splits(row + f + i, nsplit, split_stride);
+    out[idx] = from_f32<TOUT>((g / (1.f + expf(-g))) * u);
+  }
+}
+
+}  // namespace kllm
+
+using namespace kllm;
+
+extern "C" int kllm_embed(float* out, const void* table, const int* ids, int n, int d, int vocab,
+                          int dtype, hipStream_t stream) {
+  KLLM_REQUIRE(out && table && ids, "embed: null pointer");
+  KLLM_REQUIRE(n > 0 && d > 0 && vocab > 0, "embed: bad sizes n=%d d=%d vocab=%d", n, d, vocab);
+  KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "embed: unknown dtype %d", dtype);
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(n), dim3(kThreads), 0, stream, out,
+                       (const float*)table, ids, d, vocab);
+  else
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(n), dim3(kThreads), 0, stream, out,
+                       (const bf16_t*)table, ids, d, vocab);
+  KLLM_CHECK_LAUNCH("embed");
+  return 0;
+}
+
+template <typename TIN>
+static int launch_add_rmsnorm(float* x, const void* delta, int nsplit, long split_stride,
+                              const float* w, void* out, int out_dtype, const int* rows, int n, int d,
+                              float eps, int write_x, hipStream_t stream) {
+  if (out_dtype == DT_F32)
+    hipLaunchKernelGGL((add_rmsnorm_kernel<TIN, float>), dim3(n), dim3(kThreads), 0, stream, x,
+                       (const TIN*)delta, nsplit, split_stride, w, (float*)out, rows, d, eps,
+                       write_x);
+  else
+    hipLaunchKernelGGL((add_rmsnorm_kernel<TIN, bf16_t>), dim3(n), dim3(kThreads), 0, stream, x,
+                       (const TIN*)delta, nsplit, split_stride, w, (bf16_t*)out, rows, d, eps,
+                       write_x);
+  KLLM_CHECK_LAUNCH("add_rmsnorm");
+  return 0;
+}
+
+extern "C" int kllm_add_rmsnorm(float* x, const void* delta, int delta_dtype, int nsplit,
+                                long split_stride, const float* w, void* out, int out_dtype,
+                                const int* rows, int n, int d, float eps, int write_x,
+                                hipStream_t stream) {
+  KLLM_REQUIRE(x, "add_rmsnorm: null x");
+  KLLM_REQUIRE(n > 0 && d > 0, "add_rmsnorm: bad sizes n=%d d=%d", n, d);
+  KLLM_REQUIRE(!out || w, "add_rmsnorm: a norm output needs a weight");
+  KLLM_REQUIRE(out || (delta && write_x), "add_rmsnorm: nothing to do");
+  KLLM_REQUIRE(!delta || nsplit >= 1, "add_rmsnorm: nsplit %d", nsplit);
+  KLLM_REQUIRE(!(rows && write_x), "add_rmsnorm: gathered rows cannot be written back");
+  KLLM_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "add_rmsnorm: unknown out dtype");
+  KLLM_REQUIRE(delta_dtype == DT_F32 || delta_dtype == DT_BF16, "add_rmsnorm: unknown delta dtype");
+  if (delta_dtype == DT_F32)
+    return launch_add_rmsnorm<float>(x, delta, nsplit, split_stride, w, out, out_dtype, rows, n, d,
+                                     eps, write_x, stream);
+  return launch_add_rmsnorm<bf16_t>(x, delta, nsplit, split_stride, w, out, out_dtype, rows, n, d,
+                                    eps, write_x, stream);
+}
+
+extern "C" int kllm_rope_tables(float* cos_t, float* sin_t, const int* positions, int n,
+                                int head_dim, double theta, hipStream_t stream) {
+  KLLM_REQUIRE(cos_t && sin_t && positions, "rope_tables: null pointer");
+  KLLM_REQUIRE(n > 0 && head_dim > 0 && head_dim % 2 == 0, "rope_tables: bad sizes n=%d hd=%d", n,
+               head_dim);
+  KLLM_REQUIRE(theta > 0, "rope_tables: theta must be positive");
+  const int half = head_dim / 2;
+  const long total = (long)n * half;
+  hipLaunchKernelGGL(rope_tables_kernel, dim3(ceil_div(total, kThreads)), dim3(kThreads), 0, stream,
+                     cos_t, sin_t, positions, n, half, head_dim, theta);
+  KLLM_CHECK_LAUNCH("rope_tables");
+  return 0;
+}
+
+template <typename TIN, typename T>
+static int launch_rope_append(const void* qkv, int nsplit, long split_stride, void* q_out,
+                              const float* cos_t, const float* sin_t, void* cache,
+                              const int* positions, const int* span_of_token,
+                              const int* block_table, int max_pages, int page_size, int n, int H,
+                              int KV, int hd, hipStream_t stream) {
+  hipLaunchKernelGGL((rope_append_kernel<TIN, T>), dim3(n), dim3(kThreads), 0, stream,
+                     (const TIN*)qkv, nsplit, split_stride, (T*)q_out, cos_t, sin_t, (T*)cache,
+                     positions, span_of_token, block_table, max_pages, page_size, H, KV, hd);
+  KLLM_CHECK_LAUNCH("rope_append");
+  return 0;
+}
+
+extern "C" int kllm_rope_append(const void* qkv, int in_dtype, int nsplit, long split_stride,
+                                void* q_out, const float* cos_t, const float* sin_t, void* cache,
+                                const int* positions, const int* span_of_token,
+                                const int* block_table, int max_pages, int page_size, int n, int H,
+                                int KV, int hd, int dtype, hipStream_t stream) {
+  KLLM_REQUIRE(qkv && q_out, "rope_append: null pointer");
+  KLLM_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "rope_append: cos and sin go together");
+  KLLM_REQUIRE(n > 0 && H > 0 && hd > 0 && hd % 2 == 0, "rope_append: bad sizes n=%d H=%d hd=%d", n,
+               H, hd);
+  KLLM_REQUIRE(nsplit >= 1, "rope_append: nsplit %d", nsplit);
+  if (cache) {
+    KLLM_REQUIRE(positions && span_of_token && block_table, "rope_append: null index array");
+    KLLM_REQUIRE(KV > 0 && max_pages > 0 && page_size > 0,
+                 "rope_append: bad cache sizes KV=%d max_pages=%d page_size=%d", KV, max_pages,
+                 page_size);
+  }
+  KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "rope_append: unknown dtype");
+  KLLM_REQUIRE(in_dtype == DT_F32 || in_dtype == DT_BF16, "rope_append: unknown input dtype");
+#define KLLM_RA(TIN, T)                                                                         \
+  return launch_rope_append<TIN, T>(qkv, nsplit, split_stride, q_out, cos_t, sin_t, cache,      \
+                                    positions, span_of_token, block_table, max_pages, page_size, \
+                                    n, H, KV, hd, stream)
+  if (in_dtype == DT_F32 && dtype == DT_F32) KLLM_RA(float, float);
+  if (in_dtype == DT_F32 && dtype == DT_BF16) KLLM_RA(float, bf16_t);
+  if (in_dtype == DT_BF16 && dtype == DT_BF16) KLLM_RA(bf16_t, bf16_t);
+#undef KLLM_RA
+  KLLM_FAIL(ERR_ARG, "rope_append: bfloat16 input with a float32 cache is not built");
+}
+
+extern "C" int kllm_silu_mul(const void* gu, int in_dtype, int nsplit, long split_stride, void* out,
+                             int out_dtype, int n, int f, hipStream_t stream) {
+  KLLM_REQUIRE(gu && out, "silu_mul: null pointer");
+  KLLM_REQUIRE(n > 0 && f > 0 && nsplit >= 1, "silu_mul: bad sizes n=%d f=%d nsplit=%d", n, f,
+               nsplit);
+  const long total = (long)n * f;
+  int grid = ceil_div(total, kThreads);
+  if (grid > 8192) grid = 8192;
+#define KLLM_SM(TIN, TOUT)                                                                      \
+  hipLaunchKernelGGL((silu_mul_kernel<TIN, TOUT>), dim3(grid), dim3(kThreads), 0, stream,       \
+                     (const TIN*)gu, nsplit, split_stride, (TOUT*)out, (long)n, f)
+  if (in_dtype == DT_F32 && out_dtype == DT_F32) KLLM_SM(float, float);
+  else if (in_dtype == DT_F32 && out_dtype == DT_BF16) KLLM_SM(float, bf16_t);
+  else if (in_dtype == DT_BF16 && out_dtype == DT_BF16) KLLM_SM(bf16_t, bf16_t);
+  else KLLM_FAIL(ERR_ARG, "silu_mul: dtype pair %d -> %d is not built", in_dtype, out_dtype);
+#undef KLLM_SM
+  KLLM_CHECK_LAUNCH("silu_mul");
+  return 0;
+}

@@ -1,0 +1,439 @@
+// Matrix products Y[n, m] = X[n, k] . W[m, k]^T (weights are [out, in], as the
+// reference keeps them: backend/model.cu:494-503).  Accumulation is always in
+// 32-bit.  Five kernels:
+//
+//   plain   one thread per output; any size; the yardstick the others are
+//           tested against
+//   tiled   true 32-bit FMA tiles through LDS, for the float32 engine
+//   mfma    bfloat16 MFMA 32x32x16 tiles through LDS, for prompts
+//   skinny  bfloat16 MFMA 16x16x32, weights streamed straight from memory,
+//           for up to 64 rows of X (decode batches); K may be split
+//   gemv    one wave per weight row, up to 8 rows of X; K may be split
+//
+// A split product writes `nsplit` partial results [nsplit][n][m] in float32;
+// the consumer adds them.
+#include "common.hpp"
+#include "kllm_kernels.h"
+
+namespace kllm {
+
+// ------------------------------------------------------------------ plain
+template <typename T, typename TOUT>
+__global__ void gemm_plain_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                  TOUT* __restrict__ Y, int n, int m, int k) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)n * m) return;
+  const int r = idx / m, c = idx % m;
+  const T* x = X + (long)r * k;
+  const T* w = W + (long)c * k;
+  float acc = 0.f;
+  for (int i = 0; i < k; ++i) acc = fmaf(to_f32(x[i]), to_f32(w[i]), acc);
+  Y[idx] = from_f32<TOUT>(acc);
+}
+
+// ------------------------------------------------------------------ tiled f32
+constexpr int TBM = 64, TBN = 64, TBK = 16;
+
+template <typename TOUT>
+__global__ __launch_bounds__(256) void gemm_f32_tiled_kernel(const float* __restrict__ X,
+                                                             const float* __restrict__ W,
+                                                             TOUT* __restrict__ Y, int n, int m,
+                                                             int k, int vec_ok) {
+  __shared__ float Xs[TBK][TBM + 4];
+  __shared__ float Ws[TBK][TBN + 4];
+  const int tid = threadIdx.x;
+  const int tx = tid % 16, ty = tid / 16;
+  const long row0 = (long)blockIdx.y * TBM, col0 = (long)blockIdx.x * TBN;
+  const int lr = tid / 4, lk = (tid % 4) * 4;  // this thread's part of a tile load
+
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+  for (int k0 = 0; k0 < k; k0 += TBK) {
+    float xv[4] = {0.f, 0.f, 0.f, 0.f}, wv[4] = {0.f, 0.f, 0.f, 0.f};
+    const long xr = row0 + lr, wr = col0 + lr;
+    const int kk = k0 + lk;
+    if (xr < n) {
+      const float* p = X + xr * k + kk;
+      if (vec_ok && kk + 3 < k) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) if (kk + i < k) xv[i] = p[i];
+      }
+    }
+    if (wr < m) {
+      const float* p = W + wr * k + kk;
+      if (vec_ok && kk + 3 < k) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        wv[0] = v.x; wv[1] = v.y; wv[2] = v.z; wv[3] = v.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) if (kk + i < k) wv[i] = p[i];
+      }
+    }
+    __syncthreads();  // the previous tile is no longer read
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      Xs[lk + i][lr] = xv[i];
+      Ws[lk + i][lr] = wv[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk2 = 0; kk2 < TBK; ++kk2) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = Xs[kk2][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = Ws[kk2][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const long r = row0 + ty * 4 + i;
+    if (r >= n) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const long c = col0 + tx * 4 + j;
+      if (c < m) Y[r * m + c] = from_f32<TOUT>(acc[i][j]);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ bf16 MFMA tiles
+// Workgroup tile 128 (rows of X) x 128 (rows of W), 32 of K per stage, two LDS
+// stages.  Four waves in 2 x 2, each 64 x 64 = 2 x 2 MFMA tiles of 32 x 32.
+// MFMA 32x32x16: lane l holds A[l%32][8*(l/32) .. +8], B[8*(l/32) .. +8][l%32]
+// and D[8*(i/4) + 4*(l/32) + i%4][l%32] for i = 0..15.
+constexpr int MBM = 128, MBN = 128, MBK = 32;
+constexpr int MLD = MBK + 8;  // LDS row stride in elements (80 bytes: 16-byte reads stay conflict-free)
+
+template <typename TOUT>
+__global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ X,
+                                                             const bf16_t* __restrict__ W,
+                                                             TOUT* __restrict__ Y, int n, int m,
+                                                             int k) {
+  __shared__ __attribute__((aligned(16))) bf16_t Xs[2][MBM * MLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][MBN * MLD];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wr = wave / 2, wc = wave % 2;
+  const long row0 = (long)blockIdx.y * MBM, col0 = (long)blockIdx.x * MBN;
+
+  // Loads of one stage: 128 rows x 4 chunks of 8 elements per operand; each
+  // thread takes chunk (tid % 4) of rows tid/4 and tid/4 + 64.
+  const int lrow = tid / 4, lchunk = (tid % 4) * 8;
+  bf16x8 xreg[2], wreg[2];
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  auto load_stage = [&](int k0) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const long xr = row0 + lrow + h * 64, wrow = col0 + lrow + h * 64;
+      const int kk = k0 + lchunk;
+      xreg[h] = (xr < n && kk < k) ? *reinterpret_cast<const bf16x8*>(X + xr * k + kk) : zero;
+      wreg[h] = (wrow < m && kk < k) ? *reinterpret_cast<const bf16x8*>(W + wrow * k + kk) : zero;
+    }
+  };
+  auto store_stage = [&](int buf) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      *reinterpret_cast<bf16x8*>(&Xs[buf][(lrow + h * 64) * MLD + lchunk]) = xreg[h];
+      *reinterpret_cast<bf16x8*>(&Ws[buf][(lrow + h * 64) * MLD + lchunk]) = wreg[h];
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int ktiles = (k + MBK - 1) / MBK;
+  load_stage(0);
+  store_stage(0);
+  __syncthreads();
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < ktiles) load_stage((kt + 1) * MBK);
+#pragma unroll
+    for (int ks = 0; ks < MBK; ks += 16) {
+      bf16x8 a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        a[i] = *reinterpret_cast<const bf16x8*>(
+            &Xs[cur][(wr * 64 + i * 32 + lane % 32) * MLD + ks + (lane / 32) * 8]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        b[j] = *reinterpret_cast<const bf16x8*>(
+            &Ws[cur][(wc * 64 + j * 32 + lane % 32) * MLD + ks + (lane / 32) * 8]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < ktiles) {
+      store_stage(cur ^ 1);  // the other stage was last read before the previous barrier
+      __syncthreads();
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const long c = col0 + wc * 64 + j * 32 + lane % 32;
+      if (c >= m) continue;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const long r = row0 + wr * 64 + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+        if (r < n) Y[r * m + c] = from_f32<TOUT>(acc[i][j][e]);
+      }
+    }
+}
+
+// ------------------------------------------------------------------ bf16 MFMA skinny
+// Up to 16*NT rows of X.  A wave owns 16 rows of W over one slice of K and
+// streams them from memory; MFMA 16x16x32 with A = W tile, B = X^T, so
+// D[w row][x row].  Lane l holds A[l%16][8*(l/16) .. +8], B[8*(l/16) .. +8][l%16]
+// and D[4*(l/16) + i][l%16] for i = 0..3.
+template <int NT>
+__global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ X,
+                                                               const bf16_t* __restrict__ W,
+                                                               float* __restrict__ Y, int n, int m,
+                                                               int k, int kslice) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const long tile = (long)blockIdx.x * 4 + wave;
+  const long m0 = tile * 16;
+  if (m0 >= m) return;
+  const int kbeg = blockIdx.y * kslice;
+  const int kend = min(k, kbeg + kslice);
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  const long wrow = m0 + lane % 16;
+  const bool wok = wrow < m;
+  const bf16_t* wp = W + (wok ? wrow : 0) * k + (lane / 16) * 8;
+  const bf16_t* xp[NT];
+  bool xok[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int xr = t * 16 + lane % 16;
+    xok[t] = xr < n;
+    xp[t] = X + (long)(xok[t] ? xr : 0) * k + (lane / 16) * 8;
+  }
+
+  floatx4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  constexpr int UNROLL = 4;
+  int k0 = kbeg;
+  for (; k0 + 32 * UNROLL <= kend; k0 += 32 * UNROLL) {
+    bf16x8 a[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+      a[u] = wok ? *reinterpret_cast<const bf16x8*>(wp + k0 + 32 * u) : zero;
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const bf16x8 b = xok[t] ? *reinterpret_cast<const bf16x8*>(xp[t] + k0 + 32 * u) : zero;
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b, acc[t], 0, 0, 0);
+      }
+    }
+  }
+  for (; k0 < kend; k0 += 32) {
+    const bool kin = k0 + (lane / 16) * 8 < kend;  // K is a multiple of 8
+    const bf16x8 a = (wok && kin) ? *reinterpret_cast<const bf16x8*>(wp + k0) : zero;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const bf16x8 b = (xok[t] && kin) ? *reinterpret_cast<const bf16x8*>(xp[t] + k0) : zero;
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+    }
+  }
+
+  float* out = Y + (long)blockIdx.y * n * m;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int xr = t * 16 + lane % 16;
+    if (xr >= n) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const long c = m0 + 4 * (lane / 16) + i;
+      if (c < m) out[(long)xr * m + c] = acc[t][i];
+    }
+  }
+}
+
+// ------------------------------------------------------------------ gemv
+// One wave per row of W, NT (<= 8) rows of X; lanes stride over K in chunks
+// of 8 elements.  Four rows of W per workgroup.
+template <typename T, int NT>
+__global__ __launch_bounds__(256) void gemv_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                                   float* __restrict__ Y, int n, int m, int k,
+                                                   int kslice, int vec_ok) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const long row = (long)blockIdx.x * 4 + wave;
+  if (row >= m) return;
+  const int kbeg = blockIdx.y * kslice;
+  const int kend = min(k, kbeg + kslice);
+  const T* w = W + row * k;
+  float acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = 0.f;
+
+  constexpr int V = 16 / sizeof(T);  // elements per 16-byte load
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  if (vec_ok) {
+    for (int i = kbeg + lane * V; i < kend; i += kWave * V) {
+      const vec_t wv = *reinterpret_cast<const vec_t*>(w + i);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        if (t < n) {
+          const vec_t xv = *reinterpret_cast<const vec_t*>(X + (long)t * k + i);
+#pragma unroll
+          for (int e = 0; e < V; ++e) acc[t] = fmaf(to_f32(wv[e]), to_f32(xv[e]), acc[t]);
+        }
+      }
+    }
+  } else {
+    for (int i = kbeg + lane; i < kend; i += kWave) {
+      const float wv = to_f32(w[i]);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (t < n) acc[t] = fmaf(wv, to_f32(X[(long)t * k + i]), acc[t]);
+    }
+  }
+  float* out = Y + (long)blockIdx.y * n * m;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const float s = wave_sum(acc[t]);
+    if (lane == 0 && t < n) out[(long)t * m + row] = s;
+  }
+}
+
+}  // namespace kllm
+
+using namespace kllm;
+
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, int k, int dtype,
+                         int out_dtype, int algo, int nsplit, hipStream_t stream) {
+  KLLM_REQUIRE(x && w && y, "gemm: null pointer");
+  KLLM_REQUIRE(n > 0 && m > 0 && k > 0, "gemm: bad sizes n=%d m=%d k=%d", n, m, k);
+  KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "gemm: unknown dtype %d", dtype);
+  KLLM_REQUIRE(out_dtype == DT_F32 || out_dtype == dtype, "gemm: output dtype %d with input %d",
+               out_dtype, dtype);
+  KLLM_REQUIRE(nsplit >= 1 && nsplit <= 64, "gemm: nsplit %d", nsplit);
+  KLLM_REQUIRE((long)n * m < (1L << 31) && (long)m * k < (1L << 40), "gemm: sizes overflow");
+
+  if (algo == KLLM_GEMM_PLAIN) {
+    KLLM_REQUIRE(nsplit == 1, "gemm plain: no split");
+    const long total = (long)n * m;
+    const dim3 grid(ceil_div(total, 256));
+    if (dtype == DT_F32)
+      hipLaunchKernelGGL((gemm_plain_kernel<float, float>), grid, dim3(256), 0, stream,
+                         (const float*)x, (const float*)w, (float*)y, n, m, k);
+    else if (out_dtype == DT_F32)
+      hipLaunchKernelGGL((gemm_plain_kernel<bf16_t, float>), grid, dim3(256), 0, stream,
+                         (const bf16_t*)x, (const bf16_t*)w, (float*)y, n, m, k);
+    else
+      hipLaunchKernelGGL((gemm_plain_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, stream,
+                         (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, n, m, k);
+    KLLM_CHECK_LAUNCH("gemm plain");
+    return 0;
+  }
+
+  if (algo == KLLM_GEMM_TILED_F32) {
+    KLLM_REQUIRE(dtype == DT_F32 && out_dtype == DT_F32, "gemm tiled: float32 only");
+    KLLM_REQUIRE(nsplit == 1, "gemm tiled: no split");
+    const int vec_ok = (k % 4 == 0) && aligned16(x) && aligned16(w);
+    const dim3 grid(ceil_div(m, TBN), ceil_div(n, TBM));
+    hipLaunchKernelGGL((gemm_f32_tiled_kernel<float>), grid, dim3(256), 0, stream, (const float*)x,
+                       (const float*)w, (float*)y, n, m, k, vec_ok);
+    KLLM_CHECK_LAUNCH("gemm tiled");
+    return 0;
+  }
+
+  if (algo == KLLM_GEMM_MFMA_BF16) {
+    KLLM_REQUIRE(dtype == DT_BF16, "gemm mfma: bfloat16 only");
+    KLLM_REQUIRE(nsplit == 1, "gemm mfma: no split");
+    KLLM_REQUIRE(k % 8 == 0 && aligned16(x) && aligned16(w),
+                 "gemm mfma: K=%d must be a multiple of 8 and the operands 16-byte aligned", k);
+    const dim3 grid(ceil_div(m, MBN), ceil_div(n, MBM));
+    if (out_dtype == DT_F32)
+      hipLaunchKernelGGL((gemm_bf16_mfma_kernel<float>), grid, dim3(256), 0, stream,
+                         (const bf16_t*)x, (const bf16_t*)w, (float*)y, n, m, k);
+    else
+      hipLaunchKernelGGL((gemm_bf16_mfma_kernel<bf16_t>), grid, dim3(256), 0, stream,
+                         (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, n, m, k);
+    KLLM_CHECK_LAUNCH("gemm mfma");
+    return 0;
+  }
+
+  if (algo == KLLM_GEMM_SKINNY_BF16) {
+    KLLM_REQUIRE(dtype == DT_BF16 && out_dtype == DT_F32,
+                 "gemm skinny: bfloat16 in, float32 partial sums out");
+    KLLM_REQUIRE(n <= 64, "gemm skinny: n=%d exceeds 64", n);
+    KLLM_REQUIRE(k % 8 == 0 && aligned16(x) && aligned16(w),
+                 "gemm skinny: K=%d must be a multiple of 8 and the operands 16-byte aligned", k);
+    int kslice = ceil_div(ceil_div(k, nsplit), 32) * 32;
+    KLLM_REQUIRE((long)kslice * (nsplit - 1) < k, "gemm skinny: nsplit %d leaves an empty slice of K=%d",
+                 nsplit, k);
+    const dim3 grid(ceil_div(m, 64), nsplit);
+    const bf16_t *xp = (const bf16_t*)x, *wp = (const bf16_t*)w;
+    float* yp = (float*)y;
+    const int nt = ceil_div(n, 16);
+    if (nt == 1)
+      hipLaunchKernelGGL((gemm_bf16_skinny_kernel<1>), grid, dim3(256), 0, stream, xp, wp, yp, n, m, k, kslice);
+    else if (nt == 2)
+      hipLaunchKernelGGL((gemm_bf16_skinny_kernel<2>), grid, dim3(256), 0, stream, xp, wp, yp, n, m, k, kslice);
+    else if (nt == 3)
+      hipLaunchKernelGGL((gemm_bf16_skinny_kernel<3>), grid, dim3(256), 0, stream, xp, wp, yp, n, m, k, kslice);
+    else
+      hipLaunchKernelGGL((gemm_bf16_skinny_kernel<4>), grid, dim3(256), 0, stream, xp, wp, yp, n, m, k, kslice);
+    KLLM_CHECK_LAUNCH("gemm skinny");
+    return 0;
+  }
+
+  if (algo == KLLM_GEMM_GEMV) {
+    KLLM_REQUIRE(out_dtype == DT_F32, "gemv: float32 partial sums out");
+    KLLM_REQUIRE(n <= 8, "gemv: n=%d exceeds 8", n);
+    const int vlen = dtype == DT_F32 ? 4 : 8;
+    const int vec_ok = (k % vlen == 0) && aligned16(x) && aligned16(w);
+    const int unit = kWave * vlen;
+    int kslice = ceil_div(ceil_div(k, nsplit), unit) * unit;
+    KLLM_REQUIRE((long)kslice * (nsplit - 1) < k, "gemv: nsplit %d leaves an empty slice of K=%d",
+                 nsplit, k);
+    const dim3 grid(ceil_div(m, 4), nsplit);
+#define KLLM_GEMV(T, NT)                                                                        \
+  hipLaunchKernelGGL((gemv_kernel<T, NT>), grid, dim3(256), 0, stream, (const T*)x, (const T*)w, \
+                     (float*)y, n, m, k, kslice, vec_ok)
+    if (dtype == DT_F32) {
+      if (n == 1) KLLM_GEMV(float, 1);
+      else if (n == 2) KLLM_GEMV(float, 2);
+      else if (n <= 4) KLLM_GEMV(float, 4);
+      else KLLM_GEMV(float, 8);
+    } else {
+      if (n == 1) KLLM_GEMV(bf16_t, 1);
+      else if (n == 2) KLLM_GEMV(bf16_t, 2);
+      else if (n <= 4) KLLM_GEMV(bf16_t, 4);
+      else KLLM_GEMV(bf16_t, 8);
+    }
+#undef KLLM_GEMV
+    KLLM_CHECK_LAUNCH("gemv");
+    return 0;
+  }
+  KLLM_FAIL(ERR_ARG, "gemm: unknown algorithm %d", algo);
+}

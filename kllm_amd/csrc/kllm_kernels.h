@@ -1,0 +1,79 @@
+/* C ABI of the gfx950 kernel library.
+ *
+ * Every function takes device pointers and the HIP stream to launch on, checks
+ * on the host that the sizes fit what its kernel and grid assume, and returns
+ * 0, a positive HIP error code, or a negative KLLM_ERR_* value; the text of the
+ * calling thread's last error is read with kllm_last_error.  The role is the
+ * one backend/shim.h plays in the reference (error codes :19-27), but the
+ * boundary lies lower: the host keeps the model, the cache tables and the
+ * batch, and calls one kernel at a time.
+ *
+ * dtype arguments: 0 = float32, 1 = bfloat16.
+ */
+#pragma once
+#include <hip/hip_runtime.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KLLM_ERR_STATE (-1)
+#define KLLM_ERR_ARG (-2)
+
+#define KLLM_GEMM_PLAIN 0
+#define KLLM_GEMM_TILED_F32 1
+#define KLLM_GEMM_MFMA_BF16 2
+#define KLLM_GEMM_SKINNY_BF16 3
+#define KLLM_GEMM_GEMV 4
+
+/* Copies the calling thread's last error text; returns its length. */
+int kllm_last_error(char* buf, int len);
+/* One line about the device: name, architecture, compute units, memory. */
+int kllm_device_info(int device, char* buf, int len);
+/* ABI version, bumped when a signature changes. */
+int kllm_abi_version(void);
+
+int kllm_embed(float* out, const void* table, const int* ids, int n, int d, int vocab, int dtype,
+               hipStream_t stream);
+
+/* v = x[src] + sum of the nsplit partial deltas (delta may be null);
+ * x[src] = v when write_x; out[r] = rmsnorm(v) * w when out is not null.
+ * src = rows[r] when rows is given (then write_x must be 0), else r. */
+int kllm_add_rmsnorm(float* x, const void* delta, int delta_dtype, int nsplit, long split_stride,
+                     const float* w, void* out, int out_dtype, const int* rows, int n, int d,
+                     float eps, int write_x, hipStream_t stream);
+
+/* cos and sin [n][head_dim/2] of positions[t] * theta^(-2j/head_dim), angle in double. */
+int kllm_rope_tables(float* cos_t, float* sin_t, const int* positions, int n, int head_dim,
+                     double theta, hipStream_t stream);
+
+/* qkv: [nsplit][n][H*hd + 2*KV*hd] (only [n][H*hd] when cache is null).
+ * Rotates q and k when cos/sin are given, writes q_out [n][H*hd] and puts k, v
+ * into the pages of `cache` ([pages][2][KV][page_size*hd]; keys [slot][hd],
+ * values [hd][slot]). */
+int kllm_rope_append(const void* qkv, int in_dtype, int nsplit, long split_stride, void* q_out,
+                     const float* cos_t, const float* sin_t, void* cache, const int* positions,
+                     const int* span_of_token, const int* block_table, int max_pages,
+                     int page_size, int n, int H, int KV, int hd, int dtype, hipStream_t stream);
+
+/* out[n][f] = silu(gu[:, :f]) * gu[:, f:], gu = [nsplit][n][2f]. */
+int kllm_silu_mul(const void* gu, int in_dtype, int nsplit, long split_stride, void* out,
+                  int out_dtype, int n, int f, hipStream_t stream);
+
+/* y[nsplit][n][m] = x[n][k] . w[m][k]^T, 32-bit accumulation. */
+int kllm_gemm(const void* x, const void* w, void* y, int n, int m, int k, int dtype, int out_dtype,
+              int algo, int nsplit, hipStream_t stream);
+
+/* Causal attention of n tokens over the paged cache; any head size up to 256. */
+int kllm_attn_generic(const void* q, void* out, const void* cache, const int* positions,
+                      const int* span_of_token, const int* block_table, int max_pages,
+                      int page_size, int n, int H, int KV, int hd, int window, float scale,
+                      int dtype, hipStream_t stream);
+
+/* out[r] = sampled index of logits[r][:]; temperature/uniform null: greedy. */
+int kllm_sample(int* out, const float* logits, const float* temperature, const float* uniform,
+                int rows, int vocab, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

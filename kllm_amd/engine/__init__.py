@@ -1,0 +1,6 @@
+from .engine import Engine, EngineOptions, StepEntry, StepError
+from .model import CachePlan, Model, collect_weight_specs
+from .scheduler import Request, Scheduler, SchedulerError, StepPlan
+
+__all__ = ["Engine", "EngineOptions", "StepEntry", "StepError", "CachePlan", "Model",
+           "collect_weight_specs", "Request", "Scheduler", "SchedulerError", "StepPlan"]

@@ -1,0 +1,382 @@
+"""The engine: a model on the GPU, its cache, and the one step function.
+
+``Engine.step`` takes a batch of (request, its next tokens) -- portions of
+prompts beside single decoded tokens, cut anywhere -- runs exactly those
+tokens as one batch against the cache that earlier steps left, and returns
+the logits at the wanted places.  It is the counterpart of the reference's
+``te_forward_batch`` (backend/model.cu:995-1195) together with the host
+protocol around it, reserve -> forward -> commit (engine/engine.go:160-185).
+The device side knows nothing about requests: positions and block tables are
+passed every step (backend/shim.h:106-113).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager, GroupSpec, OutOfPages
+from ..config import ModelConfig, config_from_dict, load_config, resolve_architecture
+from ..parts.base import PagedCacheView, Runtime, StateCacheView, StepContext
+from ..weights import load_weights, random_weights
+from .model import Model
+
+_DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16,
+           "bf16": torch.bfloat16}
+
+
+class StepError(ValueError):
+    """A step that cannot be run as asked (bad token id, unknown request...)."""
+
+
+@dataclass
+class EngineOptions:
+    """Sizes of the engine, apart from the model's own.  The reference's
+    Options (engine/engine.go:16-33) have one bound, MaxSeq, for both a
+    request's length and a step's tokens; here they are separate."""
+    device: int = 0
+    dtype: str = "bfloat16"               # "bfloat16" or "float32"
+    page_size: int = 16                   # tokens per page (reference default: 16)
+    max_tokens: Optional[int] = None      # cache capacity in tokens (per group)
+    num_pages: Optional[int] = None       # ... or directly in pages
+    max_requests: int = 64                # live requests (state slots)
+    max_model_len: Optional[int] = None   # longest request; default max_position_embeddings
+    gemm: str = "hip"                     # "hip" or "library" (vendor GEMM for large prompts)
+    attention: str = "auto"               # "auto" or "generic"
+    graphs: bool = True                   # replay decode steps as HIP graphs
+    poison_freed_pages: bool = False      # debugging: fill pages with NaN when they are given back
+    extra: Dict[str, object] = field(default_factory=dict)
+
+    def torch_dtype(self) -> torch.dtype:
+        try:
+            return _DTYPES[self.dtype]
+        except KeyError:
+            raise ValueError(f"dtype {self.dtype!r} is not one of {sorted(_DTYPES)}") from None
+
+
+@dataclass
+class StepEntry:
+    """One request's part of a step: its next tokens and the places among
+    them whose logits are wanted."""
+    request_id: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+class Engine:
+    def __init__(self, config: ModelConfig, raw_config: dict, weights_from, options: EngineOptions):
+        if not torch.cuda.is_available():
+            raise RuntimeError("kllm_amd runs on a GPU only; torch sees none")
+        from .. import kernels
+        kernels.library()  # fail now, and loudly, if the kernels are missing
+        self.options = options
+        self.config = config
+        self.device = torch.device("cuda", options.device)
+        torch.cuda.set_device(self.device)
+        self.dtype = options.torch_dtype()
+        rt_options = {"gemm": options.gemm, "attention": options.attention}
+        rt_options.update(options.extra)
+        self.runtime = Runtime(device=self.device, dtype=self.dtype, options=rt_options)
+        arch = resolve_architecture(raw_config)
+        self.spec = arch.build(config)
+        self.model = Model(self.spec, self.runtime)
+        self.vocab_size = self.spec.vocab_size
+        specs = self.model.weight_specs()
+        weights = weights_from(specs, self.spec)
+        self.model.bind(weights)
+        del weights
+        self.max_model_len = options.max_model_len or self.spec.max_positions
+        self._alloc_cache()
+        self._pinned: List[torch.Tensor] = []
+        self._pinned_events: List[Optional[torch.cuda.Event]] = []
+        self._pinned_next = 0
+        self._control = None
+        self.steps_run = 0
+        self.tokens_run = 0
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def from_dir(cls, model_dir: str, options: EngineOptions = None) -> "Engine":
+        """Load ``model_dir`` (config.json + safetensors); the architecture
+        named in config.json chooses the model."""
+        from ..config.base import read_config_json
+        options = options or EngineOptions()
+        raw = read_config_json(model_dir)
+        config = config_from_dict(raw, where=f"{model_dir}/config.json")
+        dtype, device = options.torch_dtype(), torch.device("cuda", options.device)
+
+        def weights_from(specs, spec):
+            return load_weights(model_dir, specs, dtype, device, optional=spec.optional_tensors)
+        return cls(config, raw, weights_from, options)
+
+    @classmethod
+    def from_random(cls, config, seed: int, options: EngineOptions = None, std=0.02,
+                    norm_std=0.02) -> "Engine":
+        """Seeded random weights for ``config`` (typed or a config.json dict),
+        made in memory; the values equal those ``write_random_model`` stores."""
+        options = options or EngineOptions()
+        raw = config.to_dict() if isinstance(config, ModelConfig) else dict(config)
+        typed = config_from_dict(raw, where="config")
+        dtype, device = options.torch_dtype(), torch.device("cuda", options.device)
+
+        def weights_from(specs, spec):
+            return random_weights(specs, seed, dtype, device, std, norm_std)
+        return cls(typed, raw, weights_from, options)
+
+    # ------------------------------------------------------------------ cache
+    def _alloc_cache(self):
+        o = self.options
+        plan = self.model.cache_plan
+        if o.num_pages is not None:
+            num_pages = int(o.num_pages)
+        else:
+            tokens = o.max_tokens
+            if tokens is None:
+                # The reference's default pool fits about four longest requests
+                # (engine/engine.go:30-32).
+                tokens = 4 * (self.max_model_len or 2048)
+            num_pages = -(-int(tokens) // o.page_size)
+        self.num_pages = num_pages
+        groups, self._paged_group_of, self.kv, self.state = [], {}, {}, {}
+        for g, gp in enumerate(plan.groups):
+            need = gp.need
+            if need.kind == "paged":
+                self._paged_group_of[g] = len(groups)
+                groups.append(GroupSpec(f"group{g}", o.page_size, num_pages, need.window))
+                self.kv[g] = torch.zeros(
+                    gp.entries, num_pages, 2, need.kv_heads, o.page_size * need.head_dim,
+                    dtype=self.dtype, device=self.device)
+            elif need.kind == "state":
+                self.state[g] = torch.zeros(gp.entries, o.max_requests, *need.state_shape,
+                                            dtype=torch.float32, device=self.device)
+            else:
+                raise ValueError(f"unknown cache kind {need.kind!r}")
+        self.cache = CacheManager(groups, o.max_requests)
+
+    def cache_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in list(self.kv.values()) + list(self.state.values()))
+
+    def _poison(self, per_group_pages):
+        for g, mg in self._paged_group_of.items():
+            ids = [p for p in per_group_pages[mg] if p >= 0]
+            if ids:
+                idx = torch.tensor(ids, dtype=torch.long, device=self.device)
+                self.kv[g][:, idx] = float("nan")
+
+    # ------------------------------------------------------------------ requests
+    def open(self, request_id: Hashable):
+        return self.cache.open(request_id)
+
+    def release(self, request_id: Hashable):
+        """The request is over; what it holds is given back."""
+        if self.options.poison_freed_pages:
+            held = [list(t) for t in self.cache.get(request_id).tables]
+            self.cache.release(request_id)
+            self._poison(held)
+        else:
+            self.cache.release(request_id)
+
+    def length(self, request_id: Hashable) -> int:
+        return self.cache.get(request_id).length
+
+    # ------------------------------------------------------------------ the step
+    def _staging(self, n_ints: int) -> torch.Tensor:
+        ring = 4
+        if len(self._pinned) < ring:
+            self._pinned.append(torch.empty(max(n_ints, 4096), dtype=torch.int32, pin_memory=True))
+            self._pinned_events.append(None)
+            i = len(self._pinned) - 1
+        else:
+            i = self._pinned_next
+            self._pinned_next = (i + 1) % ring
+            if self._pinned_events[i] is not None:
+                self._pinned_events[i].synchronize()
+            if self._pinned[i].numel() < n_ints:
+                self._pinned[i] = torch.empty(n_ints, dtype=torch.int32, pin_memory=True)
+        self._staging_index = i
+        return self._pinned[i]
+
+    def _validate(self, entries: Sequence[StepEntry]):
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        seen = set()
+        for e in entries:
+            if e.request_id in seen:
+                raise StepError(f"request {e.request_id!r} appears twice in one step")
+            seen.add(e.request_id)
+            toks = np.asarray(e.tokens, dtype=np.int64)
+            if toks.ndim != 1 or toks.size == 0:
+                raise StepError(f"request {e.request_id!r}: a step needs at least one token")
+            if toks.min() < 0 or toks.max() >= self.vocab_size:
+                bad = int(toks[(toks < 0) | (toks >= self.vocab_size)][0])
+                raise StepError(f"request {e.request_id!r}: token id {bad} is outside "
+                                f"[0, {self.vocab_size})")
+            for w in e.want:
+                if not 0 <= int(w) < toks.size:
+                    raise StepError(f"request {e.request_id!r}: wanted place {w} is outside its "
+                                    f"{toks.size} tokens")
+
+    def step(self, entries: Sequence[StepEntry], taps: Optional[list] = None):
+        """Run one batch.  Returns float32 logits [wanted, vocab] on the
+        device, in the order of the entries and of their ``want`` lists, or
+        None if nothing is wanted.  Raises OutOfPages (and changes nothing) if
+        the cache cannot hold the step's tokens."""
+        self._validate(entries)
+        opened, reserved = [], []
+        try:
+            for e in entries:
+                if e.request_id not in self.cache:
+                    self.cache.open(e.request_id)
+                    opened.append(e.request_id)
+                rc = self.cache.get(e.request_id)
+                if self.max_model_len is not None and rc.length + len(e.tokens) > self.max_model_len:
+                    raise StepError(
+                        f"request {e.request_id!r} would reach {rc.length + len(e.tokens)} tokens, "
+                        f"the longest allowed is {self.max_model_len}")
+                self.cache.reserve(e.request_id, len(e.tokens))
+                reserved.append(e.request_id)
+        except Exception:
+            for rid in reserved:
+                self.cache.cancel(rid)
+            for rid in opened:
+                self.cache.release(rid)
+            raise
+        try:
+            ctx = self._build_context(entries)
+            ctx.taps = taps
+            views = self._cache_views(ctx)
+            logits = self.model.run(ctx, views)
+        except Exception:
+            for rid in reserved:
+                self.cache.cancel(rid)
+            for rid in opened:
+                self.cache.release(rid)
+            raise
+        freed_before = None
+        if self.options.poison_freed_pages:
+            freed_before = {e.request_id: [list(t) for t in self.cache.get(e.request_id).tables]
+                            for e in entries}
+        for e in entries:
+            self.cache.commit(e.request_id, len(e.tokens))
+        if freed_before is not None:
+            for e in entries:
+                now = self.cache.get(e.request_id).tables
+                gone = [[p for p, q in zip(b, a) if p >= 0 and q < 0]
+                        for b, a in zip(freed_before[e.request_id], now)]
+                self._poison(gone)
+        self.steps_run += 1
+        self.tokens_run += ctx.n
+        return logits
+
+    def _build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+        S = len(entries)
+        lens = [len(e.tokens) for e in entries]
+        n = sum(lens)
+        rcs = [self.cache.get(e.request_id) for e in entries]
+        pos0 = [rc.length for rc in rcs]
+        starts = [0]
+        for l in lens:
+            starts.append(starts[-1] + l)
+        rows = [starts[s] + int(w) for s, e in enumerate(entries) for w in e.want]
+        R = len(rows)
+        n_groups = len(self.cache.groups)
+        maxp = [max(1, max(len(rc.tables[g]) for rc in rcs)) for g in range(n_groups)]
+
+        sizes = [n, n, n, S + 1, S, S, max(R, 1)] + [S * m for m in maxp]
+        offs = [0]
+        for s in sizes:
+            offs.append(offs[-1] + ((s + 3) // 4) * 4)   # 16-byte aligned sections
+        total = offs[-1]
+        host = self._staging(total)
+        h = host.numpy()
+        tok = h[offs[0]:offs[0] + n]
+        posv = h[offs[1]:offs[1] + n]
+        sot = h[offs[2]:offs[2] + n]
+        for s, e in enumerate(entries):
+            a, b = starts[s], starts[s + 1]
+            tok[a:b] = np.asarray(e.tokens, dtype=np.int32)
+            posv[a:b] = np.arange(pos0[s], pos0[s] + lens[s], dtype=np.int32)
+            sot[a:b] = s
+        h[offs[3]:offs[3] + S + 1] = starts
+        h[offs[4]:offs[4] + S] = pos0
+        h[offs[5]:offs[5] + S] = [rc.slot for rc in rcs]
+        if R:
+            h[offs[6]:offs[6] + R] = rows
+        for g in range(n_groups):
+            bt = h[offs[7 + g]:offs[7 + g] + S * maxp[g]].reshape(S, maxp[g])
+            bt.fill(-1)
+            for s, rc in enumerate(rcs):
+                t = rc.tables[g]
+                bt[s, :len(t)] = t
+
+        if self._control is None or self._control.numel() < total:
+            self._control = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
+        dev = self._control
+        dev[:total].copy_(host[:total], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._pinned_events[self._staging_index] = ev
+
+        def sec(i, count):
+            return dev[offs[i]:offs[i] + count]
+
+        return StepContext(
+            n=n, n_spans=S,
+            token_ids=sec(0, n), positions=sec(1, n), span_of_token=sec(2, n),
+            span_start=sec(3, S + 1), span_pos=sec(4, S), slots=sec(5, S),
+            logit_rows=sec(6, R) if R else None,
+            h_span_start=starts, h_span_pos=pos0, h_span_len=lens,
+            block_tables=[sec(7 + g, S * maxp[g]).view(S, maxp[g]) for g in range(n_groups)],
+            runtime=self.runtime, max_span_len=max(lens), all_decode=all(l == 1 for l in lens),
+        )
+
+    def _cache_views(self, ctx: StepContext):
+        views = []
+        for entry in self.model.cache_plan.runs:
+            if entry is None:
+                views.append(None)
+                continue
+            g, e, writes = entry
+            if g in self.kv:
+                views.append(PagedCacheView(self.kv[g][e], ctx.block_tables[self._paged_group_of[g]],
+                                            self.options.page_size, writes))
+            else:
+                views.append(StateCacheView(self.state[g][e], ctx.slots, writes))
+        return views
+
+    # ------------------------------------------------------------------ sampling
+    @property
+    def eos_token_ids(self):
+        return tuple(self.spec.eos_token_ids)
+
+    def sample(self, logits, temperatures, uniforms) -> List[int]:
+        """One token per row of logits (greedy where the temperature is 0)."""
+        from ..sampling import DeviceSampler
+        if getattr(self, "_sampler", None) is None:
+            self._sampler = DeviceSampler(self.device)
+        return self._sampler.sample(logits, temperatures, uniforms)
+
+    # ------------------------------------------------------------------ generation
+    def generate(self, prompts, max_new_tokens: int, temperature: float = 0.0, seed: int = 0,
+                 max_step_tokens: Optional[int] = None, max_batch: Optional[int] = None):
+        """Generate for each prompt (a list of token ids) up to
+        ``max_new_tokens`` tokens, stopping at an end-of-sequence id; all
+        prompts are scheduled together.  Returns one list of ids per prompt.
+        The reference's Generate runs one prompt, greedily
+        (engine/engine.go:192-213)."""
+        from .scheduler import Scheduler
+        single = bool(prompts) and isinstance(prompts[0], int)
+        if single:
+            prompts = [prompts]
+        sched = Scheduler(self, max_batch=max_batch, max_step_tokens=max_step_tokens)
+        ids = [sched.submit(list(p), max_new_tokens, temperature=temperature, seed=seed + i)
+               for i, p in enumerate(prompts)]
+        results = sched.run_until_done()
+        out = [results[i].tokens for i in ids]
+        for i in ids:
+            if results[i].error:
+                raise RuntimeError(f"prompt {i}: {results[i].error}")
+        return out[0] if single else out

@@ -1,0 +1,145 @@
+"""A model: parts instantiated from a ModelSpec, bound to weights, and run over
+one step's tokens.
+
+The model owns no request state.  It says what its runs need kept between
+steps (``cache_plan``), the engine allocates that and hands a view per run to
+``run``.  The order of the runs is the spec's ``schedule``; nothing here
+assumes that it is 0..L-1.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..parts.base import Runtime, make_part
+from ..parts.spec import CacheNeed, ModelSpec, PartSpec, WeightSpec
+
+
+@dataclass
+class CacheGroupPlan:
+    """Runs with the same needs: ``entries`` of them keep a cache of their own."""
+    need: CacheNeed
+    entries: int = 0
+
+
+@dataclass
+class CachePlan:
+    groups: List[CacheGroupPlan] = field(default_factory=list)
+    # per run of the schedule: (group, entry, writes) or None for a mixer without cache
+    runs: List[Optional[Tuple[int, int, bool]]] = field(default_factory=list)
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, runtime: Runtime):
+        self.spec = spec
+        self.runtime = runtime
+        self.embedding = make_part("embedding", spec.embedding, runtime)
+        self.blocks = [
+            make_part("block", PartSpec(layer.block, layer=layer, **layer.block_params), runtime)
+            for layer in spec.layers]
+        self.final_norm = make_part("norm", spec.final_norm, runtime)
+        self.head = make_part("head", spec.head, runtime)
+        self.schedule = list(spec.schedule)
+        self.cache_plan = self._plan_cache()
+
+    # ------------------------------------------------------------------ cache plan
+    def _plan_cache(self) -> CachePlan:
+        plan = CachePlan()
+        keys: Dict[tuple, int] = {}
+        for i, run in enumerate(self.schedule):
+            if not 0 <= run.layer < len(self.blocks):
+                raise ValueError(f"schedule entry {i} names layer {run.layer}, the model has "
+                                 f"{len(self.blocks)}")
+            need = self.blocks[run.layer].cache_need()
+            if need is None:
+                if run.cache_of is not None:
+                    raise ValueError(f"schedule entry {i}: its mixer keeps no cache to share")
+                plan.runs.append(None)
+                continue
+            if run.cache_of is not None:
+                j = run.cache_of
+                if not 0 <= j < i or plan.runs[j] is None or not plan.runs[j][2]:
+                    raise ValueError(
+                        f"schedule entry {i} reads the cache of entry {j}, which must be an "
+                        f"earlier entry that writes one")
+                other = self.blocks[self.schedule[j].layer].cache_need()
+                if other.group_key() != need.group_key():
+                    raise ValueError(f"schedule entry {i} cannot read the cache of entry {j}: "
+                                     f"{need} does not fit {other}")
+                g, e, _ = plan.runs[j]
+                plan.runs.append((g, e, False))
+                continue
+            key = need.group_key()
+            if key not in keys:
+                keys[key] = len(plan.groups)
+                plan.groups.append(CacheGroupPlan(need))
+            g = keys[key]
+            plan.runs.append((g, plan.groups[g].entries, True))
+            plan.groups[g].entries += 1
+        return plan
+
+    # ------------------------------------------------------------------ weights
+    def parts(self):
+        return [self.embedding, *self.blocks, self.final_norm, self.head]
+
+    def weight_specs(self) -> List[WeightSpec]:
+        return [s for p in self.parts() for s in p.weight_specs()]
+
+    def bind(self, weights: Dict[str, torch.Tensor]) -> None:
+        for p in self.parts():
+            p.bind(weights)
+
+    def weight_bytes(self) -> int:
+        """Bytes of distinct weight tensors the parts hold after bind."""
+        seen = {}
+
+        def visit(obj):
+            for v in vars(obj).values():
+                if isinstance(v, torch.Tensor):
+                    seen[v.data_ptr()] = v.numel() * v.element_size()
+                elif hasattr(v, "weight_specs") and hasattr(v, "bind"):
+                    visit(v)
+        for p in self.parts():
+            visit(p)
+        return sum(seen.values())
+
+    # ------------------------------------------------------------------ one step
+    def run(self, ctx, cache_views) -> Optional[torch.Tensor]:
+        """Run the step's tokens through every scheduled layer.  Returns
+        float32 logits [R, vocab] for ``ctx.logit_rows`` (None if no row is
+        wanted)."""
+        shared = [p for _, p in self.runtime.shared.values()]
+        for p in shared:
+            if hasattr(p, "prepare"):
+                p.prepare(ctx)
+        x = self.embedding.forward(ctx, ctx.token_ids)
+        for p in shared:
+            if hasattr(p, "on_embedding"):
+                p.on_embedding(ctx, x)
+        if ctx.taps is not None:
+            ctx.taps.append(x.clone())
+        pending = None
+        for i, run in enumerate(self.schedule):
+            x, pending = self.blocks[run.layer].forward(ctx, x, pending, cache_views[i])
+            if ctx.taps is not None:
+                if pending is not None:
+                    self.final_norm.add(ctx, x, pending)
+                    pending = None
+                ctx.taps.append(x.clone())
+        if ctx.taps is not None:
+            ctx.taps.append(self.final_norm.forward(ctx, x, delta=pending, tag="xn_tap").clone())
+            pending = None
+        if ctx.logit_rows is None or ctx.logit_rows.numel() == 0:
+            return None
+        xn = self.final_norm.forward(ctx, x, delta=pending, rows=ctx.logit_rows, tag="xn_rows")
+        return self.head.forward(ctx, xn)
+
+
+def collect_weight_specs(spec: ModelSpec) -> List[WeightSpec]:
+    """Every tensor a model of this spec wants, without touching a device."""
+    from ..weights.loader import merge_specs
+    rt = Runtime(device=torch.device("cpu"), dtype=torch.float32)
+    return merge_specs(Model(spec, rt).weight_specs())

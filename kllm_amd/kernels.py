@@ -1,0 +1,263 @@
+"""Python side of the kernel library: loads ``libkllm_hip.so`` and wraps each
+entry point so that it takes torch tensors.
+
+There is no fallback: if the library cannot be found, built or loaded, the
+first call raises.  Every wrapper checks device, dtype and contiguity of its
+tensors (the library itself checks the sizes) and launches on torch's current
+stream, so the launches order with torch's own work and are recorded by a HIP
+graph capture.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import threading
+from ctypes import c_char_p, c_double, c_float, c_int, c_long, c_void_p
+
+import torch
+
+DT_F32, DT_BF16 = 0, 1
+GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV = 0, 1, 2, 3, 4
+ABI_VERSION = 1
+
+
+class KernelError(RuntimeError):
+    """The kernel library refused a call or a launch failed."""
+
+
+_lib = None
+_lib_path = None
+_lock = threading.Lock()
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return DT_F32
+    if dtype == torch.bfloat16:
+        return DT_BF16
+    raise KernelError(f"dtype {dtype} is not a storage type of the kernels")
+
+
+def library():
+    """The loaded library; builds it on the first call if nothing is built."""
+    global _lib, _lib_path
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        from .csrc.build import ensure_built
+        path = ensure_built()
+        try:
+            lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError(f"cannot load the kernel library {path}: {e}") from None
+        lib.kllm_abi_version.restype = c_int
+        if lib.kllm_abi_version() != ABI_VERSION:
+            raise KernelError(
+                f"{path} has ABI version {lib.kllm_abi_version()}, this package needs "
+                f"{ABI_VERSION}: rebuild it (python -m kllm_amd.csrc.build)")
+        _declare(lib)
+        _lib, _lib_path = lib, path
+    return _lib
+
+
+def library_path():
+    library()
+    return _lib_path
+
+
+def _declare(lib):
+    P, I, L, F, D = c_void_p, c_int, c_long, c_float, c_double
+    sigs = {
+        "kllm_last_error": [c_char_p, I],
+        "kllm_device_info": [I, c_char_p, I],
+        "kllm_embed": [P, P, P, I, I, I, I, P],
+        "kllm_add_rmsnorm": [P, P, I, I, L, P, P, I, P, I, I, F, I, P],
+        "kllm_rope_tables": [P, P, P, I, I, D, P],
+        "kllm_rope_append": [P, I, I, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "kllm_silu_mul": [P, I, I, L, P, I, I, I, P],
+        "kllm_gemm": [P, P, P, I, I, I, I, I, I, I, P],
+        "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
+        "kllm_sample": [P, P, P, P, I, I, P],
+    }
+    for name, args in sigs.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = c_int
+    for name, args in OPTIONAL_SIGNATURES.items():
+        if hasattr(lib, name):
+            fn = getattr(lib, name)
+            fn.argtypes = args
+            fn.restype = c_int
+
+
+OPTIONAL_SIGNATURES = {}
+
+
+def _check(rc: int, what: str):
+    if rc == 0:
+        return
+    buf = ctypes.create_string_buffer(512)
+    library().kllm_last_error(buf, 512)
+    raise KernelError(f"{what}: {buf.value.decode(errors='replace')} (code {rc})")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t, name, dtype=None, allow_none=False):
+    if t is None:
+        if allow_none:
+            return None
+        raise KernelError(f"{name}: tensor is missing")
+    if not t.is_cuda:
+        raise KernelError(f"{name}: tensor is on {t.device}, the kernels run on the GPU only")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: tensor is not contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: dtype {t.dtype}, expected {dtype}")
+    return t.data_ptr()
+
+
+def device_info(device: int = 0) -> str:
+    buf = ctypes.create_string_buffer(256)
+    _check(library().kllm_device_info(device, buf, 256), "device_info")
+    return buf.value.decode()
+
+
+# ----------------------------------------------------------------------------- wrappers
+
+def embed(out, table, ids):
+    n, d = out.shape
+    if ids.numel() < n or table.shape[1] != d:
+        raise KernelError(f"embed: out {tuple(out.shape)}, table {tuple(table.shape)}, "
+                          f"{ids.numel()} ids do not fit")
+    _check(library().kllm_embed(
+        _ptr(out, "embed out", torch.float32), _ptr(table, "embed table"),
+        _ptr(ids, "embed ids", torch.int32), n, d, table.shape[0], dtype_code(table.dtype),
+        _stream()), "embed")
+
+
+def add_rmsnorm(x, delta=None, weight=None, out=None, rows=None, eps=0.0, write_x=None):
+    """x [N, d] float32 in place; delta [nsplit, N, d] or [N, d]; out [n, d]."""
+    d = x.shape[-1]
+    if rows is not None:
+        n = rows.numel()
+        write_x = False
+    else:
+        n = x.shape[0]
+        if write_x is None:
+            write_x = delta is not None
+    nsplit, stride, ddt = 1, 0, DT_F32
+    if delta is not None:
+        if delta.dim() == 3:
+            nsplit, stride = delta.shape[0], delta.shape[1] * delta.shape[2]
+        if delta.shape[-1] != d or delta.shape[-2] != x.shape[0]:
+            raise KernelError(f"add_rmsnorm: delta {tuple(delta.shape)} does not fit x {tuple(x.shape)}")
+        ddt = dtype_code(delta.dtype)
+    if out is not None:
+        if tuple(out.shape) != (n, d) or weight is None or weight.numel() != d:
+            raise KernelError("add_rmsnorm: output or weight shape does not fit")
+    _check(library().kllm_add_rmsnorm(
+        _ptr(x, "add_rmsnorm x", torch.float32), _ptr(delta, "add_rmsnorm delta", None, True), ddt,
+        nsplit, stride, _ptr(weight, "add_rmsnorm weight", torch.float32, True),
+        _ptr(out, "add_rmsnorm out", None, True),
+        dtype_code(out.dtype) if out is not None else DT_F32,
+        _ptr(rows, "add_rmsnorm rows", torch.int32, True), n, d, float(eps), int(bool(write_x)),
+        _stream()), "add_rmsnorm")
+
+
+def rope_tables(cos, sin, positions, head_dim, theta):
+    n = positions.numel()
+    if tuple(cos.shape) != (n, head_dim // 2) or tuple(sin.shape) != (n, head_dim // 2):
+        raise KernelError("rope_tables: table shapes do not fit")
+    _check(library().kllm_rope_tables(
+        _ptr(cos, "rope cos", torch.float32), _ptr(sin, "rope sin", torch.float32),
+        _ptr(positions, "rope positions", torch.int32), n, head_dim, float(theta), _stream()),
+        "rope_tables")
+
+
+def rope_append(qkv, q_out, cos, sin, cache, positions, span_of_token, block_table, page_size,
+                n_heads, n_kv_heads, head_dim):
+    """qkv [nsplit, n, cols] or [n, cols]; cache [pages, 2, KV, page_size*hd] or None."""
+    n = q_out.shape[0]
+    nsplit, stride = 1, 0
+    if qkv.dim() == 3:
+        nsplit, stride = qkv.shape[0], qkv.shape[1] * qkv.shape[2]
+    cols = n_heads * head_dim + (2 * n_kv_heads * head_dim if cache is not None else 0)
+    if qkv.shape[-1] != cols or qkv.shape[-2] != n or q_out.shape[1] != n_heads * head_dim:
+        raise KernelError(f"rope_append: qkv {tuple(qkv.shape)} does not fit {n} x {cols}")
+    max_pages = 0
+    if cache is not None:
+        if tuple(cache.shape[1:]) != (2, n_kv_heads, page_size * head_dim) or cache.dtype != q_out.dtype:
+            raise KernelError(f"rope_append: cache {tuple(cache.shape)} {cache.dtype} does not fit")
+        max_pages = block_table.shape[1]
+        if positions.numel() < n or span_of_token.numel() < n:
+            raise KernelError("rope_append: index arrays are too short")
+    if cos is not None and (tuple(cos.shape) != (n, head_dim // 2) or tuple(sin.shape) != tuple(cos.shape)):
+        raise KernelError("rope_append: cos/sin shapes do not fit")
+    _check(library().kllm_rope_append(
+        _ptr(qkv, "rope_append qkv"), dtype_code(qkv.dtype), nsplit, stride,
+        _ptr(q_out, "rope_append q_out"), _ptr(cos, "rope_append cos", torch.float32, True),
+        _ptr(sin, "rope_append sin", torch.float32, True), _ptr(cache, "rope_append cache", None, True),
+        _ptr(positions, "rope_append positions", torch.int32, True),
+        _ptr(span_of_token, "rope_append span_of_token", torch.int32, True),
+        _ptr(block_table, "rope_append block_table", torch.int32, True), max_pages, page_size, n,
+        n_heads, n_kv_heads, head_dim, dtype_code(q_out.dtype), _stream()), "rope_append")
+
+
+def silu_mul(gu, out):
+    n, f = out.shape
+    nsplit, stride = 1, 0
+    if gu.dim() == 3:
+        nsplit, stride = gu.shape[0], gu.shape[1] * gu.shape[2]
+    if gu.shape[-1] != 2 * f or gu.shape[-2] != n:
+        raise KernelError(f"silu_mul: input {tuple(gu.shape)} does not fit output {tuple(out.shape)}")
+    _check(library().kllm_silu_mul(
+        _ptr(gu, "silu_mul in"), dtype_code(gu.dtype), nsplit, stride, _ptr(out, "silu_mul out"),
+        dtype_code(out.dtype), n, f, _stream()), "silu_mul")
+
+
+def gemm(x, w, y, algo, nsplit=1):
+    """y [nsplit, n, m] (or [n, m]) = x [n, k] . w [m, k]^T."""
+    n, k = x.shape
+    m = w.shape[0]
+    if w.shape[1] != k or x.dtype != w.dtype:
+        raise KernelError(f"gemm: x {tuple(x.shape)} {x.dtype} and w {tuple(w.shape)} {w.dtype} do not fit")
+    want = (nsplit, n, m) if y.dim() == 3 else (n, m)
+    if tuple(y.shape) != want or (y.dim() == 2 and nsplit != 1):
+        raise KernelError(f"gemm: output {tuple(y.shape)} does not fit {want}")
+    _check(library().kllm_gemm(
+        _ptr(x, "gemm x"), _ptr(w, "gemm w"), _ptr(y, "gemm y"), n, m, k, dtype_code(x.dtype),
+        dtype_code(y.dtype), algo, nsplit, _stream()), "gemm")
+
+
+def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size, n_heads,
+                 n_kv_heads, head_dim, window, scale):
+    n = q.shape[0]
+    if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape)
+            or q.dtype != cache.dtype or out.dtype != q.dtype):
+        raise KernelError("attn_generic: q/out shapes or dtypes do not fit")
+    if tuple(cache.shape[1:]) != (2, n_kv_heads, page_size * head_dim):
+        raise KernelError(f"attn_generic: cache {tuple(cache.shape)} does not fit")
+    if positions.numel() < n or span_of_token.numel() < n:
+        raise KernelError("attn_generic: index arrays are too short")
+    _check(library().kllm_attn_generic(
+        _ptr(q, "attn q"), _ptr(out, "attn out"), _ptr(cache, "attn cache"),
+        _ptr(positions, "attn positions", torch.int32),
+        _ptr(span_of_token, "attn span_of_token", torch.int32),
+        _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size, n,
+        n_heads, n_kv_heads, head_dim, int(window), float(scale), dtype_code(q.dtype), _stream()),
+        "attn_generic")
+
+
+def sample(out, logits, temperature=None, uniform=None):
+    rows, vocab = logits.shape
+    if out.numel() < rows:
+        raise KernelError("sample: output is too short")
+    _check(library().kllm_sample(
+        _ptr(out, "sample out", torch.int32), _ptr(logits, "sample logits", torch.float32),
+        _ptr(temperature, "sample temperature", torch.float32, True),
+        _ptr(uniform, "sample uniform", torch.float32, True), rows, vocab, _stream()), "sample")

@@ -1,0 +1,3 @@
+from . import llama  # registers "LlamaForCausalLM"
+
+__all__ = ["llama"]

@@ -1,0 +1,88 @@
+"""Causal self-attention over a paged cache, with grouped KV heads.
+
+q, k, v projections without bias; rotary on q and k before the keys are
+cached; for the token at position p, head h reads KV head h // (H/KV) and keys
+[0, p] (or the last ``window`` of them); scores times 1/sqrt(head_dim),
+softmax in 32-bit, values, output projection
+(backend/model.cu:1090-1104, :343-408, :224-225).
+
+Parameters: ``hidden``, ``heads``, ``kv_heads``, ``head_dim``, ``window``
+(0: all keys), ``position`` (a PartSpec or None), ``own_kv`` (False: the run
+reads keys and values that another run cached and has no k/v projections).
+Tensors: ``<prefix>.{q,k,v,o}_proj.weight``.  The three input projections are
+kept as one matrix so that a step reads one weight for them.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import kernels as K
+from .base import Part, register_part
+from .linear import linear
+from .spec import CacheNeed, WeightSpec
+
+
+@register_part("mixer", "attention")
+class CausalSelfAttention(Part):
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.hidden = int(self.param("hidden"))
+        self.heads = int(self.param("heads"))
+        self.kv_heads = int(self.param("kv_heads"))
+        self.head_dim = int(self.param("head_dim"))
+        self.window = int(self.param("window", 0) or 0)
+        self.own_kv = bool(self.param("own_kv", True))
+        if self.heads % self.kv_heads:
+            raise ValueError(f"attention: {self.heads} heads are not a multiple of {self.kv_heads} KV heads")
+        if self.head_dim % 2 or self.head_dim > 256:
+            raise ValueError(f"attention: head_dim {self.head_dim} must be even and at most 256")
+        pos = self.param("position", None)
+        self.position = runtime.shared_part("position", pos) if pos is not None else None
+        self.scale = 1.0 / math.sqrt(self.head_dim)
+        self.q_dim = self.heads * self.head_dim
+        self.kv_dim = self.kv_heads * self.head_dim
+        self.w_in = None
+        self.w_o = None
+
+    def weight_specs(self):
+        specs = [WeightSpec(self.tensor_name("q_proj.weight"), (self.q_dim, self.hidden))]
+        if self.own_kv:
+            specs += [WeightSpec(self.tensor_name("k_proj.weight"), (self.kv_dim, self.hidden)),
+                      WeightSpec(self.tensor_name("v_proj.weight"), (self.kv_dim, self.hidden))]
+        specs.append(WeightSpec(self.tensor_name("o_proj.weight"), (self.hidden, self.q_dim)))
+        return specs
+
+    def bind(self, weights):
+        names = ["q_proj.weight"] + (["k_proj.weight", "v_proj.weight"] if self.own_kv else [])
+        mats = [weights[self.tensor_name(n)] for n in names]
+        self.w_in = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0]
+        self.w_o = weights[self.tensor_name("o_proj.weight")]
+
+    def cache_need(self):
+        return CacheNeed("paged", kv_heads=self.kv_heads, head_dim=self.head_dim, window=self.window)
+
+    def forward(self, ctx, xn, cache):
+        n = xn.shape[0]
+        dtype = self.runtime.dtype
+        writes = self.own_kv
+        if writes != bool(cache.write):
+            raise ValueError("attention: a run must write its cache exactly when it has k/v projections")
+        qkv = linear(ctx, xn, self.w_in, "attn.qkv")
+        q = ctx.buf("attn.q", (n, self.q_dim), dtype)
+        cos = sin = None
+        if self.position is not None and hasattr(self.position, "tables"):
+            cos, sin = self.position.tables(ctx)
+        K.rope_append(qkv, q, cos, sin, cache.pages if writes else None, ctx.positions,
+                      ctx.span_of_token, cache.block_table, cache.page_size, self.heads,
+                      self.kv_heads, self.head_dim)
+        out = ctx.buf("attn.out", (n, self.q_dim), dtype)
+        self.attend(ctx, q, out, cache)
+        return linear(ctx, out, self.w_o, "attn.proj")
+
+    def attend(self, ctx, q, out, cache):
+        K.attn_generic(q, out, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
+                       cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
+                       self.scale)

@@ -1,0 +1,209 @@
+"""What every part is: the interfaces, the registry of part kinds, and the
+step context that parts are called with.
+
+A part is built from a ``PartSpec`` (its kind, its tensor-name prefix and its
+sizes and constants), says which tensors it wants (``weight_specs``), is bound
+to them once (``bind``) and is then called once per step.  A part sees the
+step only through ``StepContext``: token positions, which span a token belongs
+to, block tables, state slots.  It does not see the model, the other layers or
+the requests.
+
+Categories and their call interface (x is the float32 residual stream
+[n, hidden]; xn a normalised activation [n, hidden] in the compute dtype;
+a *delta* is a float32 tensor [n, hidden] or [nsplit, n, hidden] of partial
+sums to be added to x):
+
+  norm          forward(ctx, x, delta=None, rows=None) -> xn
+                  adds delta into x first (fused); with ``rows`` it reads only
+                  those rows and leaves x alone
+                add(ctx, x, delta)            x += delta, nothing else
+  position      prepare(ctx)                  once per step, before any layer
+                on_embedding(ctx, x)          optional: acts on the embedded
+                                              tokens (additive encodings)
+                tables(ctx) -> (cos, sin)     optional: rotation tables
+                                              [n, head_dim/2] that a mixer
+                                              applies to queries and keys
+  mixer         cache_need() -> CacheNeed | None
+                forward(ctx, xn, cache) -> delta
+                  ``cache`` is a PagedCacheView or StateCacheView (or None)
+  feed_forward  forward(ctx, xn) -> delta
+  block         forward(ctx, x, pending, cache) -> (x, pending)
+                  ``pending`` is a delta not yet added to x (or None)
+  embedding     forward(ctx, token_ids) -> x
+  head          forward(ctx, xn_rows) -> float32 logits [rows, vocab]
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Tuple
+
+import torch
+
+from .spec import CacheNeed, PartSpec, WeightSpec
+
+CATEGORIES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head")
+_REGISTRY: Dict[Tuple[str, str], type] = {}
+
+
+def register_part(category: str, kind: str, cls: type = None):
+    """Register ``cls`` as the part ``kind`` of ``category``; usable as a decorator."""
+    if category not in CATEGORIES:
+        raise ValueError(f"unknown part category {category!r} (one of {CATEGORIES})")
+
+    def deco(c):
+        _REGISTRY[(category, kind)] = c
+        c.category = category
+        c.kind = kind
+        return c
+
+    return deco(cls) if cls is not None else deco
+
+
+def unregister_part(category: str, kind: str):
+    _REGISTRY.pop((category, kind), None)
+
+
+def registered_parts(category: str = None):
+    return sorted(k for k in _REGISTRY if category is None or k[0] == category)
+
+
+def make_part(category: str, spec: PartSpec, runtime: "Runtime"):
+    try:
+        cls = _REGISTRY[(category, spec.kind)]
+    except KeyError:
+        kinds = [k[1] for k in registered_parts(category)]
+        raise ValueError(
+            f"no {category} part of kind {spec.kind!r} is registered (registered: {kinds})") from None
+    return cls(spec, runtime)
+
+
+class Workspace:
+    """Scratch tensors that live across steps.  ``get`` returns a view of a
+    buffer kept per tag and grown when a larger one is asked for, so that a
+    step allocates nothing once sizes have been seen (a HIP graph needs that)."""
+
+    def __init__(self, device):
+        self.device = device
+        self._bufs: Dict[str, torch.Tensor] = {}
+
+    def get(self, tag: str, shape, dtype) -> torch.Tensor:
+        numel = 1
+        for s in shape:
+            numel *= int(s)
+        key = f"{tag}:{dtype}"
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < numel:
+            buf = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
+            self._bufs[key] = buf
+        return buf[:numel].view(*shape)
+
+    def bytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self._bufs.values())
+
+
+@dataclass
+class Runtime:
+    """What parts need to know about the engine they run in."""
+    device: torch.device
+    dtype: torch.dtype                      # compute/storage dtype: float32 or bfloat16
+    workspace: Workspace = None
+    options: Dict[str, Any] = field(default_factory=dict)
+    shared: Dict[int, Any] = field(default_factory=dict)   # parts used by several layers
+
+    def __post_init__(self):
+        if self.workspace is None:
+            self.workspace = Workspace(self.device)
+
+    def shared_part(self, category: str, spec: PartSpec):
+        """The one instance of a part that several layers name with the same
+        PartSpec object (a position encoding, for instance)."""
+        key = id(spec)
+        if key not in self.shared:
+            self.shared[key] = (spec, make_part(category, spec, self))
+        return self.shared[key][1]
+
+
+@dataclass
+class PagedCacheView:
+    """One run's keys and values: ``pages`` is [num_pages, 2, kv_heads,
+    page_size*head_dim] (keys [slot][hd], values [hd][slot] inside a page);
+    ``block_table`` [spans, max_pages] int32 maps a span's logical page to a
+    physical one.  ``write`` is False for a run that reads another run's cache."""
+    pages: torch.Tensor
+    block_table: torch.Tensor
+    page_size: int
+    write: bool = True
+
+
+@dataclass
+class StateCacheView:
+    """One run's per-request state: ``state`` is [num_slots, *shape] float32,
+    ``slots`` [spans] int32 gives each span's slot."""
+    state: torch.Tensor
+    slots: torch.Tensor
+    write: bool = True
+
+
+@dataclass
+class StepContext:
+    """One step's batch as the parts see it.  All index tensors are int32 on
+    the device; the ``h_`` lists are their host copies.
+
+    A *span* is one request's tokens of this step: ``span_len[s]`` tokens at
+    absolute positions ``span_pos[s] ...``; they sit at rows
+    ``span_start[s] .. span_start[s+1]`` of every [n, ...] activation."""
+    n: int
+    n_spans: int
+    token_ids: torch.Tensor
+    positions: torch.Tensor
+    span_of_token: torch.Tensor
+    span_start: torch.Tensor              # [n_spans + 1]
+    span_pos: torch.Tensor                # [n_spans]
+    slots: torch.Tensor                   # [n_spans] state slot of each span's request
+    logit_rows: Optional[torch.Tensor]    # [R] rows whose logits are wanted
+    h_span_start: List[int]
+    h_span_pos: List[int]
+    h_span_len: List[int]
+    block_tables: List[torch.Tensor]      # per cache group [n_spans, max_pages]
+    runtime: Runtime = None
+    max_span_len: int = 0
+    all_decode: bool = False              # every span is a single token
+    scratch: Dict[Any, Any] = field(default_factory=dict)   # per-step values of parts
+    taps: Optional[List[torch.Tensor]] = None               # residual-stream captures
+
+    def buf(self, tag, shape, dtype):
+        return self.runtime.workspace.get(tag, shape, dtype)
+
+
+class Part:
+    """Base of all parts."""
+    category = None
+    kind = None
+
+    def __init__(self, spec: PartSpec, runtime: Runtime):
+        self.spec = spec
+        self.runtime = runtime
+        self.prefix = spec.prefix
+
+    def param(self, key, default=...):
+        if key in self.spec.params:
+            return self.spec.params[key]
+        if default is ...:
+            raise ValueError(f"{self.category} part {self.kind!r} needs parameter {key!r}")
+        return default
+
+    def tensor_name(self, local: str) -> str:
+        names = self.spec.params.get("names") or {}
+        if local in names:
+            return names[local]
+        return f"{self.prefix}.{local}" if self.prefix else local
+
+    def weight_specs(self) -> List[WeightSpec]:
+        return []
+
+    def bind(self, weights: Dict[str, torch.Tensor]) -> None:
+        """Take the tensors named by weight_specs out of ``weights``."""
+
+    def cache_need(self) -> Optional[CacheNeed]:
+        return None

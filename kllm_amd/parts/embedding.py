@@ -1,0 +1,56 @@
+"""Token embedding and output head.
+
+Embedding: x[t, :] = E[id_t, :], no scaling (backend/model.cu:89-95,
+:1056-1060).  Head: logits = xn . W^T in float32 for the wanted rows
+(:1185-1188).  The head names its own tensor; a tied head simply names the
+embedding's table (the reference resolves tying offline by copying it:
+tools/convert_hf.py:81-82).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .. import kernels as K
+from .base import Part, register_part
+from .linear import linear
+from .spec import WeightSpec
+
+
+@register_part("embedding", "token_embedding")
+class TokenEmbedding(Part):
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.vocab = int(self.param("vocab"))
+        self.hidden = int(self.param("hidden"))
+        self.table = None
+
+    def weight_specs(self):
+        return [WeightSpec(self.tensor_name("weight"), (self.vocab, self.hidden))]
+
+    def bind(self, weights):
+        self.table = weights[self.tensor_name("weight")]
+
+    def forward(self, ctx, token_ids):
+        x = ctx.buf("x", (ctx.n, self.hidden), torch.float32)
+        K.embed(x, self.table, token_ids)
+        return x
+
+
+@register_part("head", "linear_head")
+class LinearHead(Part):
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.vocab = int(self.param("vocab"))
+        self.hidden = int(self.param("hidden"))
+        self.weight = None
+
+    def weight_specs(self):
+        return [WeightSpec(self.tensor_name("weight"), (self.vocab, self.hidden))]
+
+    def bind(self, weights):
+        self.weight = weights[self.tensor_name("weight")]
+
+    def forward(self, ctx, xn_rows):
+        logits = linear(ctx, xn_rows, self.weight, "logits", split=False)
+        return logits[0]

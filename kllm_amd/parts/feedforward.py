@@ -1,0 +1,46 @@
+"""Gated feed-forward: down(act(gate(x)) * up(x)), no biases
+(backend/model.cu:1112-1115; SiLU: :477-483).
+
+Parameters: ``hidden``, ``intermediate``, ``activation`` ("silu").  Tensors:
+``<prefix>.{gate,up,down}_proj.weight``.  Gate and up are kept as one matrix
+[2*intermediate, hidden] (gate rows first).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .. import kernels as K
+from .base import Part, register_part
+from .linear import linear
+from .spec import WeightSpec
+
+
+@register_part("feed_forward", "gated_mlp")
+class GatedFeedForward(Part):
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.hidden = int(self.param("hidden"))
+        self.intermediate = int(self.param("intermediate"))
+        act = self.param("activation", "silu")
+        if act not in ("silu", "swish"):
+            raise ValueError(f"gated_mlp: activation {act!r} is not built (silu only)")
+        self.w_gu = None
+        self.w_down = None
+
+    def weight_specs(self):
+        return [WeightSpec(self.tensor_name("gate_proj.weight"), (self.intermediate, self.hidden)),
+                WeightSpec(self.tensor_name("up_proj.weight"), (self.intermediate, self.hidden)),
+                WeightSpec(self.tensor_name("down_proj.weight"), (self.hidden, self.intermediate))]
+
+    def bind(self, weights):
+        self.w_gu = torch.cat([weights[self.tensor_name("gate_proj.weight")],
+                               weights[self.tensor_name("up_proj.weight")]], dim=0).contiguous()
+        self.w_down = weights[self.tensor_name("down_proj.weight")]
+
+    def forward(self, ctx, xn):
+        n = xn.shape[0]
+        gu = linear(ctx, xn, self.w_gu, "ffn.gu")
+        h = ctx.buf("ffn.h", (n, self.intermediate), self.runtime.dtype)
+        K.silu_mul(gu, h)
+        return linear(ctx, h, self.w_down, "ffn.down")

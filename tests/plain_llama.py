@@ -123,46 +123,60 @@ def _cfg(cfg):
     )
 
 
-def attention_sublayer(w, prefix, xn, positions, c, window=0):
+def attention_sublayer(w, prefix, xn, positions, c, window=0, kv=None):
     """q, k, v projections, rotary on q and k before they are kept, attention,
-    output projection (backend/model.cu:1090-1104)."""
+    output projection (backend/model.cu:1090-1104).  With ``kv`` given (the
+    rotated keys and the values another layer made) only q is projected.
+    Returns (output, (k, v))."""
     q = linear(xn, w[prefix + "self_attn.q_proj.weight"])
-    k = linear(xn, w[prefix + "self_attn.k_proj.weight"])
-    v = linear(xn, w[prefix + "self_attn.v_proj.weight"])
     q = rope(q, positions, c["H"], c["hd"], c["theta"])
-    k = rope(k, positions, c["KV"], c["hd"], c["theta"])
-    a = attention(q, k, v, positions, c["H"], c["KV"], c["hd"], window)
-    return linear(a, w[prefix + "self_attn.o_proj.weight"])
+    if kv is None:
+        k = linear(xn, w[prefix + "self_attn.k_proj.weight"])
+        v = linear(xn, w[prefix + "self_attn.v_proj.weight"])
+        k = rope(k, positions, c["KV"], c["hd"], c["theta"])
+    else:
+        k, v = kv
+    a = attention(q, k, v, torch.arange(len(positions)), c["H"], c["KV"], c["hd"], window)
+    return linear(a, w[prefix + "self_attn.o_proj.weight"]), (k, v)
 
 
-def decoder_layer(w, layer, x, positions, c, window=0):
+def decoder_layer(w, layer, x, positions, c, window=0, kv=None):
     """a = h + Attn(Norm_in(h)); h' = a + FFN(Norm_post(a))
     (backend/model.cu:1083-1117; the reference defers the second add into the
     next norm, which does not change the sum)."""
     p = f"model.layers.{layer}."
     xn = rmsnorm(x, w[p + "input_layernorm.weight"], c["eps"])
-    x = x + attention_sublayer(w, p, xn, positions, c, window)
+    a, kv_out = attention_sublayer(w, p, xn, positions, c, window, kv)
+    x = x + a
     xn = rmsnorm(x, w[p + "post_attention_layernorm.weight"], c["eps"])
     x = x + swiglu(xn, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                    w[p + "mlp.down_proj.weight"])
-    return x
+    return x, kv_out
 
 
-def forward(w, cfg, ids, dtype=torch.float32, return_hidden=False, schedule=None):
-    """Logits [T, vocab] at every position of one whole sequence starting at
-    position 0.  ``hidden`` follows the reference's capture order: [0] the
-    embedding, [j] the input of layer j, last the final norm's output
-    (backend/model.cu:1061, :1085, :1123-1124; engine/e2e/e2e_test.go:117-131).
-    ``schedule`` is the order in which layers run (default 0..L-1)."""
+def forward(w, cfg, ids, dtype=torch.float32, return_hidden=False, schedule=None, pos0=0,
+            windows=None, kv_from=None):
+    """Logits [T, vocab] at every position of one whole sequence whose first
+    token stands at position ``pos0`` (0 for a real sequence; another value
+    only shifts every rotary angle, which must not change anything).
+    ``hidden`` follows the reference's capture order: [0] the embedding, [j]
+    the input of layer j, last the final norm's output (backend/model.cu:1061,
+    :1085, :1123-1124; engine/e2e/e2e_test.go:117-131).  ``schedule`` is the
+    order in which layers run (default 0..L-1); ``windows`` maps a layer to
+    its attention window; ``kv_from`` maps a run of the schedule to the earlier
+    run whose keys and values it reads."""
     c = _cfg(cfg)
     w = {k: v.to(dtype) for k, v in w.items()}
     T = len(ids)
-    positions = torch.arange(T)
+    positions = torch.arange(pos0, pos0 + T)
     x = embedding(ids, w["model.embed_tokens.weight"])
     hidden = [x.clone()]
     order = list(range(c["L"])) if schedule is None else list(schedule)
-    for layer in order:
-        x = decoder_layer(w, layer, x, positions, c)
+    kept = {}
+    for run, layer in enumerate(order):
+        kv = kept[kv_from[run]] if kv_from and run in kv_from else None
+        win = (windows or {}).get(layer, 0)
+        x, kept[run] = decoder_layer(w, layer, x, positions, c, win, kv)
         hidden.append(x.clone())
     xn = rmsnorm(x, w["model.norm.weight"], c["eps"])
     hidden.append(xn.clone())

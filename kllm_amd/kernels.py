@@ -46,8 +46,11 @@ def library():
     with _lock:
         if _lib is not None:
             return _lib
-        from .csrc.build import ensure_built
-        path = ensure_built()
+        import os
+        path = os.environ.get("KLLM_AMD_LIBRARY")
+        if not path:
+            from .csrc.build import ensure_built
+            path = ensure_built()
         try:
             lib = ctypes.CDLL(path)
         except OSError as e:

@@ -1,0 +1,292 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16:
+each request alone and whole; most of it in one step and the last 32 tokens
+one by one; in portions of changing size, down to two tokens; and mixed, up to
+four live requests with so few pages that they are used again.  Then long
+decoding, the first tokens of a sequence, and generation through the entry
+points."""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+import tiny
+import traces
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DTYPES = ["float32", "bfloat16"]
+
+
+def make_requests(cfg, lengths, seed):
+    return {f"r{i}": tiny.tokens(cfg, n, seed * 100 + i) for i, n in enumerate(lengths)}
+
+
+def expected(model_dir, cfg, requests, dtype):
+    w = tiny.read_weights(model_dir, as_stored_in=dtype)
+    return {rid: P.forward(w, cfg, toks).numpy() for rid, toks in requests.items()}
+
+
+def replay(model_dir, dtype, steps, max_tokens, **opts):
+    from kllm_amd.engine import EngineOptions
+    from kllm_amd.replay import Replayer
+    options = EngineOptions(dtype=dtype, max_tokens=max_tokens, max_model_len=1 << 30,
+                            poison_freed_pages=True, **opts)
+    rep = Replayer(model_dir, dtype, max_tokens, options=options)
+    outs = [rep.step(s["entries"], s["end"]) for s in steps]
+    assert not rep.engine.cache.requests, "every request of the trace was ended"
+    rep.engine.cache.check_invariants()
+    assert all(p.free_pages == p.num_pages for p in rep.engine.cache.pools)
+    return traces.collect(steps, outs), rep
+
+
+def compare(rows, want, dtype, requests):
+    worst = 0.0
+    for rid, toks in requests.items():
+        for p in range(len(toks)):
+            got = rows[(rid, p)]
+            assert np.isfinite(got).all(), (rid, p)
+            worst = max(worst, float(np.abs(got - want[rid][p]).max()))
+            assert worst < tiny.TOL[dtype], f"{rid} position {p}: off by {worst}"
+    assert len(rows) == sum(len(t) for t in requests.values())
+    return worst
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,lengths", [("A", [5, 17, 33, 100]), ("B", [1, 9, 40, 70, 150]),
+                                          ("C", [3, 64, 65])])
+def test_alone_and_whole(model_dirs, name, lengths, dtype):
+    cfg, d = tiny.CONFIGS[name], model_dirs(name)
+    reqs = make_requests(cfg, lengths, 1)
+    steps = traces.whole(reqs)
+    rows, _ = replay(d, dtype, steps, traces.peak_tokens(steps))
+    compare(rows, expected(d, cfg, reqs, dtype), dtype, reqs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,lengths", [("A", [33, 100]), ("B", [40, 129]), ("C", [50])])
+def test_bulk_then_last_32_one_by_one(model_dirs, name, lengths, dtype):
+    cfg, d = tiny.CONFIGS[name], model_dirs(name)
+    reqs = make_requests(cfg, lengths, 2)
+    steps = traces.bulk_then_tail(reqs, 32)
+    rows, _ = replay(d, dtype, steps, traces.peak_tokens(steps))
+    compare(rows, expected(d, cfg, reqs, dtype), dtype, reqs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,lengths", [("A", [100, 37]), ("B", [150, 70]), ("C", [81])])
+def test_portions_of_changing_size(model_dirs, name, lengths, dtype):
+    cfg, d = tiny.CONFIGS[name], model_dirs(name)
+    reqs = make_requests(cfg, lengths, 3)
+    steps = traces.portions(reqs, seed=4)
+    assert min(len(s["entries"][0]["tokens"]) for s in steps if not s["end"]) == 2
+    rows, _ = replay(d, dtype, steps, traces.peak_tokens(steps))
+    compare(rows, expected(d, cfg, reqs, dtype), dtype, reqs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_mixed_with_pages_used_again(model_dirs, name, dtype):
+    cfg, d = tiny.CONFIGS[name], model_dirs(name)
+    reqs = make_requests(cfg, [70, 33, 120, 18, 64, 97, 41, 129, 5, 80], 4)
+    steps, peak = traces.mixed(reqs, seed=7)
+    assert peak == traces.peak_tokens(steps)
+    assert peak < sum(len(t) for t in reqs.values())          # the pool is smaller than the trace
+    assert max(len(s["entries"]) for s in steps) == 4
+    assert any(len(e["tokens"]) == 1 for s in steps for e in s["entries"]) and \
+        any(len(e["tokens"]) > 1 and len(s["entries"]) > 1 for s in steps for e in s["entries"])
+    rows, rep = replay(d, dtype, steps, peak)
+    pool = rep.engine.cache.pools[0]
+    assert pool.total_allocs > pool.num_pages                 # pages were handed out again
+    compare(rows, expected(d, cfg, reqs, dtype), dtype, reqs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_all_families_agree_with_each_other(model_dirs, dtype):
+    cfg, d = tiny.CONFIGS["A"], model_dirs("A")
+    reqs = make_requests(cfg, [90, 47], 5)
+    families = [traces.whole(reqs), traces.bulk_then_tail(reqs), traces.portions(reqs, 1),
+                traces.mixed(reqs, seed=2)[0]]
+    results = [replay(d, dtype, s, traces.peak_tokens(s))[0] for s in families]
+    tol = 2e-5 if dtype == "float32" else tiny.TOL[dtype]
+    for other in results[1:]:
+        for key, row in results[0].items():
+            assert float(np.abs(other[key] - row).max()) < tol, key
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(model_dirs, dtype):
+    """One token per step for 400 steps, past several pages and past the
+    model's max_position_embeddings (positions are computed, not looked up)."""
+    cfg, d = tiny.CONFIGS["B"], model_dirs("B")
+    reqs = make_requests(cfg, [400], 6)
+    steps = traces.bulk_then_tail(reqs, tail=399)
+    rows, _ = replay(d, dtype, steps, 448)
+    compare(rows, expected(d, cfg, reqs, dtype), dtype, reqs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_first_tokens_of_a_sequence(model_dirs, name, dtype):
+    """Position 0 sees only itself; 1 and 2 see little: the first rows of a
+    sequence fed one token at a time, beside another request in the batch."""
+    cfg, d = tiny.CONFIGS[name], model_dirs(name)
+    reqs = make_requests(cfg, [4, 3], 8)
+    a, b = reqs["r0"], reqs["r1"]
+    steps = [{"step": 0, "entries": [{"id": "r0", "tokens": a[:1], "want": [0]}], "end": []},
+             {"step": 1, "entries": [{"id": "r0", "tokens": a[1:2], "want": [0]},
+                                     {"id": "r1", "tokens": b[:1], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "r1", "tokens": b[1:3], "want": [0, 1]},
+                                     {"id": "r0", "tokens": a[2:4], "want": [0, 1]}], "end": ["r0", "r1"]}]
+    rows, _ = replay(d, dtype, steps, 128)
+    compare(rows, expected(d, cfg, reqs, dtype), dtype, reqs)
+
+
+def test_hidden_states_layer_by_layer(model_dirs):
+    """The residual stream after the embedding, after every layer and after the
+    final norm, as the reference's debug taps capture it
+    (backend/model.cu:1061, :1085, :1123-1124), within its own bound of 1e-4
+    (engine/e2e/e2e_test.go:21-24)."""
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry
+    for name in ("A", "B"):
+        cfg, d = tiny.CONFIGS[name], model_dirs(name)
+        eng = Engine.from_dir(d, EngineOptions(dtype="float32", max_tokens=256))
+        ids = tiny.tokens(cfg, 40, 9)
+        taps = []
+        eng.step([StepEntry("x", ids, [39])], taps=taps)
+        _, hidden = P.forward(tiny.read_weights(d), cfg, ids, return_hidden=True)
+        assert len(taps) == len(hidden) == cfg["num_hidden_layers"] + 2
+        for t, h in zip(taps, hidden):
+            assert float((t.cpu() - h).abs().max()) < 1e-4
+
+
+def test_step_refuses_bad_input_and_leaves_the_cache_alone(model_dirs):
+    from kllm_amd.cache import OutOfPages
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry, StepError
+    eng = Engine.from_dir(model_dirs("A"), EngineOptions(dtype="float32", max_tokens=64, max_model_len=100))
+    with pytest.raises(StepError, match="token id"):
+        eng.step([StepEntry("a", [1, 256], [0])])
+    with pytest.raises(StepError, match="wanted place"):
+        eng.step([StepEntry("a", [1, 2], [2])])
+    with pytest.raises(StepError, match="twice"):
+        eng.step([StepEntry("a", [1], []), StepEntry("a", [2], [])])
+    with pytest.raises(StepError, match="at least one token"):
+        eng.step([StepEntry("a", [], [])])
+    with pytest.raises(OutOfPages):
+        eng.step([StepEntry("a", [1] * 40, []), StepEntry("b", [1] * 40, [])])
+    assert not eng.cache.requests and eng.cache.pools[0].free_pages == 4
+    eng.step([StepEntry("a", [1] * 60, [])])
+    with pytest.raises(StepError, match="longest"):
+        eng.step([StepEntry("c", [1] * 101, [])])
+    assert eng.step([StepEntry("a", [5], [])]) is None        # nothing wanted, nothing returned
+    assert eng.length("a") == 61
+    eng.release("a")
+    eng.cache.check_invariants()
+
+
+def run_trace_program(model_dir, dtype, steps, max_tokens, out_dir):
+    proc = subprocess.Popen(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
+         "--out", out_dir, "--max-tokens", str(max_tokens)],
+        stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, cwd="/")
+    outs = []
+    for s in steps:
+        proc.stdin.write(json.dumps(s) + "\n")
+        proc.stdin.flush()
+        line = proc.stdout.readline().strip()
+        assert line == f"done {s['step']}", line       # the next step only after this line
+    proc.stdin.close()
+    assert proc.wait(timeout=120) == 0
+    for s in steps:
+        path = os.path.join(out_dir, f"{s['step']}.f32")
+        wanted = sum(len(e["want"]) for e in s["entries"])
+        if wanted == 0:
+            assert not os.path.exists(path)
+            outs.append(None)
+        else:
+            outs.append(np.fromfile(path, dtype="<f4").reshape(wanted, -1))
+    return outs
+
+
+@pytest.mark.parametrize("dtype,name", [("float32", "B"), ("bfloat16", "A")])
+def test_the_trace_run_program(model_dirs, tmp_path, dtype, name):
+    cfg, d = tiny.CONFIGS[name], model_dirs(name, store="bfloat16" if dtype == "bfloat16" else "float32")
+    reqs = make_requests(cfg, [50, 21, 77, 30, 64, 12], 10)
+    steps, peak = traces.mixed(reqs, seed=11)
+    steps[3]["entries"][0]["want"] = []                       # a step may want nothing of a request
+    outs = run_trace_program(d, dtype, steps, peak, str(tmp_path / "out"))
+    assert outs[0].shape[1] == cfg["vocab_size"]
+    rows = traces.collect(steps, outs)
+    want = expected(d, cfg, reqs, dtype)
+    for (rid, p), got in rows.items():
+        assert float(np.abs(got - want[rid][p]).max()) < tiny.TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "R"])
+def test_greedy_generation_through_the_entry_point(model_dirs, name, dtype):
+    """Greedy tokens through Engine.generate (scheduler, sampling kernel) equal
+    the plain implementation's, for prompts generated together."""
+    from kllm_amd.engine import Engine, EngineOptions
+    cfg, d = tiny.CONFIGS[name], model_dirs(name)
+    eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=512))
+    lengths = {"A": [5, 17, 33], "B": [1, 9, 40, 70]}.get(name)
+    prompts = tiny.REFERENCE_PROMPTS if name == "R" else [tiny.tokens(cfg, n, 20 + n) for n in lengths]
+    new = {"A": 16, "B": 24, "R": 16}[name]
+    got = eng.generate(prompts, new, max_batch=4, max_step_tokens=48)
+    w = tiny.read_weights(d, as_stored_in=dtype)
+    for p, g in zip(prompts, got):
+        want = P.generate_greedy(w, cfg, p, new, eos={cfg["eos_token_id"]} if "eos_token_id" in cfg else None)
+        if dtype == "float32":
+            assert g == want
+        else:                                            # bfloat16 may part ways at a near-tie
+            agree = next((i for i, (x, y) in enumerate(zip(g, want)) if x != y), len(want))
+            if agree < len(want):
+                logits = P.forward(w, cfg, p + want[:agree])[-1]
+                top2 = torch.topk(logits, 2).values
+                assert float(top2[0] - top2[1]) < tiny.TOL[dtype], (agree, g, want)
+    assert not eng.cache.requests
+
+
+def test_temperature_generation_matches_the_plain_sampler(model_dirs):
+    """Config B, temperature 0.8, seeded: the same tokens as the plain
+    implementation drawing with the same uniforms, alone and in a batch."""
+    from kllm_amd.engine import Engine, EngineOptions
+    from kllm_amd.sampling import uniform
+    cfg, d = tiny.CONFIGS["B"], model_dirs("B")
+    eng = Engine.from_dir(d, EngineOptions(dtype="float32", max_tokens=512))
+    prompts = [tiny.tokens(cfg, n, 30 + n) for n in (1, 9, 40, 70)]
+    got = eng.generate(prompts, 24, temperature=0.8, seed=100, max_batch=3, max_step_tokens=32)
+    alone = [eng.generate(p, 24, temperature=0.8, seed=100 + i) for i, p in enumerate(prompts)]
+    assert got == alone
+    w = tiny.read_weights(d)
+    for i, p in enumerate(prompts):
+        ids = list(p)
+        for k, tok in enumerate(got[i]):
+            row = P.forward(w, cfg, ids)[-1]
+            u = uniform(100 + i, k)
+            want = P.sample_inverse_cdf(row, 0.8, u)
+            if want != tok:                              # only at a boundary of the CDF
+                cdf = torch.cumsum(P.softmax_temperature(row, 0.8), 0)
+                assert abs(float(cdf[min(want, tok)]) - u) < 1e-4
+            ids.append(tok)
+
+
+def test_command_line_generate(model_dirs):
+    """The command line in the reference's manner (cmd/generate/main.go:15-50)."""
+    cfg, d = tiny.CONFIGS["R"], model_dirs("R")
+    out = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "generate"), "--model", d, "--ids", "1 17 42 100 7",
+         "--steps", "16", "--max-seq", "256", "--dtype", "float32"],
+        capture_output=True, text=True, timeout=120, cwd="/")
+    assert out.returncode == 0, out.stderr
+    lines = out.stdout.strip().splitlines()
+    assert lines[0] == "prompt:    [1 17 42 100 7]"
+    want = P.generate_greedy(tiny.read_weights(d), cfg, [1, 17, 42, 100, 7], 16, eos={2})
+    assert lines[1] == "generated: [" + " ".join(map(str, want)) + "]"

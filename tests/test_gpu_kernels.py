@@ -1,0 +1,405 @@
+"""Each kernel alone against its plain reference, at other sizes than the
+engine's tiny models use: widths and vocabularies that are no power of two,
+head sizes in steps of 16, odd numbers of heads and groups."""
+
+import math
+
+import pytest
+import torch
+
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def K():
+    from kllm_amd import kernels
+    return kernels
+
+
+def rnd(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def tol(dtype):
+    return 1e-5 if dtype == torch.float32 else 2e-2
+
+
+# ------------------------------------------------------------------ embedding, norm
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(dtype):
+    table = rnd(131, 72, dtype=dtype)
+    ids = torch.tensor([0, 130, 5, 5, 77], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, 72, device=DEV)
+    K().embed(out, table, ids)
+    assert torch.equal(out.cpu(), P.embedding(ids.cpu().tolist(), table.cpu().float()))
+
+
+@pytest.mark.parametrize("d", [72, 100, 2048, 4100])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm(d, out_dtype):
+    n, eps = 7, 1e-5
+    x, w = rnd(n, d, seed=1, scale=3.0), (1 + 0.2 * rnd(d, seed=2))
+    delta = rnd(3, n, d, seed=3)
+    want_x = x.cpu().double() + delta.cpu().double().sum(0)
+    want = P.rmsnorm(want_x, w.cpu().double(), eps)
+    # norm only
+    out = torch.empty(n, d, dtype=out_dtype, device=DEV)
+    x0 = x.clone()
+    K().add_rmsnorm(x0, weight=w, out=out, eps=eps)
+    assert torch.equal(x0, x)
+    ref0 = P.rmsnorm(x.cpu().double(), w.cpu().double(), eps)
+    assert (out.cpu().double() - ref0).abs().max() < tol(out_dtype) * 3
+    # add (three partial sums) + norm, x updated
+    x1 = x.clone()
+    K().add_rmsnorm(x1, delta=delta, weight=w, out=out, eps=eps)
+    assert (x1.cpu().double() - want_x).abs().max() < 1e-5
+    assert (out.cpu().double() - want).abs().max() < tol(out_dtype) * 3
+    # add only
+    x2 = x.clone()
+    K().add_rmsnorm(x2, delta=delta[0], write_x=True)
+    assert torch.allclose(x2, x + delta[0])
+    # gathered rows: x untouched
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    x3 = x.clone()
+    out3 = torch.empty(3, d, dtype=out_dtype, device=DEV)
+    K().add_rmsnorm(x3, delta=delta, weight=w, out=out3, rows=rows, eps=eps)
+    assert torch.equal(x3, x)
+    assert (out3.cpu().double() - want[[6, 0, 3]]).abs().max() < tol(out_dtype) * 3
+
+
+def test_rmsnorm_zero_row_and_eps_inside_the_root():
+    x = torch.zeros(2, 64, device=DEV)
+    x[1] = 2.0
+    out = torch.empty(2, 64, device=DEV)
+    K().add_rmsnorm(x, weight=torch.ones(64, device=DEV), out=out, eps=5.0)
+    assert torch.equal(out[0].cpu(), torch.zeros(64))
+    assert torch.allclose(out[1].cpu(), torch.full((64,), 2.0 / 3.0), atol=1e-6)
+
+
+# ------------------------------------------------------------------ rotary, append
+
+@pytest.mark.parametrize("hd,theta", [(16, 10000.0), (48, 1000.0), (128, 500000.0)])
+def test_rope_tables_large_positions(hd, theta):
+    pos = torch.tensor([0, 1, 17, 4095, 100000], dtype=torch.int32, device=DEV)
+    cos = torch.empty(5, hd // 2, device=DEV)
+    sin = torch.empty(5, hd // 2, device=DEV)
+    K().rope_tables(cos, sin, pos, hd, theta)
+    ang = P.rope_angles(pos.cpu().tolist(), hd, theta)
+    assert (cos.cpu().double() - torch.cos(ang)).abs().max() < 1e-6
+    assert (sin.cpu().double() - torch.sin(ang)).abs().max() < 1e-6
+
+
+def read_cache(cache, table, length, KV, hd, ps):
+    """Keys and values [length, KV*hd] of one request out of the paged layout."""
+    c = cache.cpu().float()
+    k = torch.zeros(length, KV, hd)
+    v = torch.zeros(length, KV, hd)
+    for p in range(length):
+        page, slot = table[p // ps], p % ps
+        for h in range(KV):
+            k[p, h] = c[page, 0, h].reshape(ps, hd)[slot]
+            v[p, h] = c[page, 1, h].reshape(hd, ps)[:, slot]
+    return k.reshape(length, KV * hd), v.reshape(length, KV * hd)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,KV,hd,ps", [(4, 2, 16, 16), (3, 1, 32, 16), (5, 5, 48, 32), (6, 3, 80, 16)])
+def test_rope_append(dtype, H, KV, hd, ps):
+    theta, nsplit = 10000.0, 2
+    # two spans: positions 30..36 of request 0 and 0..4 of request 1, scattered pages
+    spans = [(30, 7), (0, 5)]
+    n = sum(l for _, l in spans)
+    pos = torch.tensor([p0 + i for p0, l in spans for i in range(l)], dtype=torch.int32, device=DEV)
+    sot = torch.tensor([s for s, (_, l) in enumerate(spans) for _ in range(l)], dtype=torch.int32, device=DEV)
+    tables = [[9, 4, 11], [2, -1, -1]]
+    bt = torch.tensor(tables, dtype=torch.int32, device=DEV)
+    qd, kvd = H * hd, KV * hd
+    qkv = rnd(nsplit, n, qd + 2 * kvd, seed=5)
+    cos = torch.empty(n, hd // 2, device=DEV)
+    sin = torch.empty(n, hd // 2, device=DEV)
+    K().rope_tables(cos, sin, pos, hd, theta)
+    cache = torch.full((12, 2, KV, ps * hd), float("nan"), dtype=dtype, device=DEV)
+    q_out = torch.empty(n, qd, dtype=dtype, device=DEV)
+    K().rope_append(qkv, q_out, cos, sin, cache, pos, sot, bt, ps, H, KV, hd)
+    full = qkv.cpu().double().sum(0)
+    want_q = P.rope(full[:, :qd], pos.cpu().tolist(), H, hd, theta)
+    want_k = P.rope(full[:, qd:qd + kvd], pos.cpu().tolist(), KV, hd, theta)
+    want_v = full[:, qd + kvd:]
+    assert (q_out.cpu().double() - want_q).abs().max() < tol(dtype) * 4
+    off = 0
+    for s, (p0, l) in enumerate(spans):
+        k, v = read_cache(cache, tables[s], p0 + l, KV, hd, ps)
+        assert (k[p0:].double() - want_k[off:off + l]).abs().max() < tol(dtype) * 4
+        assert (v[p0:].double() - want_v[off:off + l]).abs().max() < tol(dtype) * 4
+        assert torch.isnan(k[:p0]).all()          # nothing else was written
+        off += l
+    # without tables: no rotation; without cache: q only
+    q2 = torch.empty(n, qd, dtype=dtype, device=DEV)
+    K().rope_append(qkv[0, :, :qd].contiguous(), q2, None, None, None, None, None, None, ps, H, KV, hd)
+    assert (q2.cpu().double() - qkv[0, :, :qd].cpu().double()).abs().max() < tol(dtype) * 4
+
+
+# ------------------------------------------------------------------ silu gate
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_silu_mul(out_dtype):
+    n, f = 5, 176
+    gu = rnd(2, n, 2 * f, seed=4, scale=3.0)
+    gu[0, 0, 0], gu[1, 0, 0] = -60.0, -60.0       # far negative gate: 0, not NaN
+    out = torch.empty(n, f, dtype=out_dtype, device=DEV)
+    K().silu_mul(gu, out)
+    s = gu.cpu().double().sum(0)
+    want = P.silu(s[:, :f]) * s[:, f:]
+    assert torch.isfinite(out).all()
+    assert (out.cpu().double() - want).abs().max() < tol(out_dtype) * 10
+
+
+# ------------------------------------------------------------------ matrix products
+
+GEMM_SIZES = [(1, 64, 64), (2, 131, 88), (5, 100, 72), (8, 515, 2048), (17, 96, 176),
+              (33, 320, 96), (64, 200, 264), (65, 130, 40), (130, 515, 1032), (300, 257, 520)]
+
+
+@pytest.mark.parametrize("n,m,k", GEMM_SIZES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gemm_kernels_against_plain(n, m, k, dtype):
+    k_ = K()
+    x, w = rnd(n, k, seed=1, dtype=dtype), rnd(m, k, seed=2, dtype=dtype)
+    want = P.linear(x.cpu().double(), w.cpu().double())
+    bound = 1e-5 * k ** 0.5 * 8
+    algos = [(k_.GEMM_PLAIN, 1)]
+    if dtype == torch.float32:
+        algos.append((k_.GEMM_TILED_F32, 1))
+    elif k % 8 == 0:
+        algos.append((k_.GEMM_MFMA_BF16, 1))
+        if n <= 64:
+            algos += [(k_.GEMM_SKINNY_BF16, 1)] + ([(k_.GEMM_SKINNY_BF16, 3)] if k >= 256 else [])
+    if n <= 8:
+        algos += [(k_.GEMM_GEMV, 1)] + ([(k_.GEMM_GEMV, 2)] if k >= 2048 else [])
+    for algo, ns in algos:
+        y = torch.full((ns, n, m), float("nan"), device=DEV)
+        k_.gemm(x, w, y, algo, ns)
+        err = (y.cpu().double().sum(0) - want).abs().max()
+        assert err < bound, (algo, ns, float(err))
+    if dtype == torch.bfloat16 and k % 8 == 0:      # rounded output
+        y = torch.empty(n, m, dtype=dtype, device=DEV)
+        k_.gemm(x, w, y, k_.GEMM_MFMA_BF16)
+        assert (y.cpu().double() - want).abs().max() < 0.01 * want.abs().max()
+
+
+def test_gemm_refuses_what_it_does_not_take():
+    k_ = K()
+    x, w = rnd(70, 72, dtype=torch.bfloat16), rnd(16, 72, dtype=torch.bfloat16)
+    y = torch.empty(1, 70, 16, device=DEV)
+    with pytest.raises(k_.KernelError, match="exceeds 64"):
+        k_.gemm(x, w, y, k_.GEMM_SKINNY_BF16)
+    x2, w2 = rnd(4, 12, dtype=torch.bfloat16), rnd(16, 12, dtype=torch.bfloat16)
+    with pytest.raises(k_.KernelError, match="multiple of 8"):
+        k_.gemm(x2, w2, torch.empty(1, 4, 16, device=DEV), k_.GEMM_MFMA_BF16)
+    with pytest.raises(k_.KernelError, match="GPU only"):
+        k_.gemm(x2.cpu(), w2, torch.empty(1, 4, 16, device=DEV), k_.GEMM_PLAIN)
+
+
+def test_linear_chooses_a_kernel_for_every_size():
+    from kllm_amd.parts.linear import choose
+    k_ = K()
+    assert choose(torch.float32, 1, 64, 64)[0] == k_.GEMM_GEMV
+    assert choose(torch.float32, 100, 64, 64)[0] == k_.GEMM_TILED_F32
+    assert choose(torch.bfloat16, 40, 64, 64)[0] == k_.GEMM_SKINNY_BF16
+    assert choose(torch.bfloat16, 40, 64, 60)[0] == k_.GEMM_PLAIN          # K not a multiple of 8
+    assert choose(torch.bfloat16, 400, 64, 64)[0] == k_.GEMM_MFMA_BF16
+    assert choose(torch.bfloat16, 400, 64, 64, {"gemm": "library"})[0] == "library"
+    a, ns = choose(torch.bfloat16, 1, 2048, 5632)
+    assert a == k_.GEMM_GEMV and 1 <= ns <= 16
+
+
+# ------------------------------------------------------------------ attention
+
+def build_paged(k, v, tables, lens, KV, hd, ps, num_pages, dtype, poison=True):
+    """Put [len, KV*hd] keys/values of several requests into a paged cache."""
+    cache = torch.full((num_pages, 2, KV, ps * hd), float("nan") if poison else 0.0)
+    for s, L in enumerate(lens):
+        for p in range(L):
+            page, slot = tables[s][p // ps], p % ps
+            for h in range(KV):
+                cache[page, 0, h].view(ps, hd)[slot] = k[s][p, h * hd:(h + 1) * hd]
+                cache[page, 1, h].view(hd, ps)[:, slot] = v[s][p, h * hd:(h + 1) * hd]
+    return cache.to(dtype).to(DEV)
+
+
+def attention_case(H, KV, hd, ps, dtype, window, spans, seed=0):
+    """spans: list of (cached_len, new_len).  Returns (engine output, reference)."""
+    lens = [a + b for a, b in spans]
+    maxp = max(-(-L // ps) for L in lens)
+    num_pages = sum(-(-L // ps) for L in lens) + 3
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    tables, used = [], 0
+    for L in lens:
+        cnt = -(-L // ps)
+        tables.append(perm[used:used + cnt] + [-1] * (maxp - cnt))
+        used += cnt
+    ks = [torch.randn(L, KV * hd, generator=g).to(dtype).float() for L in lens]
+    vs = [torch.randn(L, KV * hd, generator=g).to(dtype).float() for L in lens]
+    qs = [torch.randn(b, H * hd, generator=g).to(dtype).float() * 2 for _, b in spans]
+    cache = build_paged(ks, vs, tables, lens, KV, hd, ps, num_pages, dtype)
+    q = torch.cat(qs).to(dtype).to(DEV)
+    pos = torch.tensor([a + i for a, b in spans for i in range(b)], dtype=torch.int32, device=DEV)
+    sot = torch.tensor([s for s, (_, b) in enumerate(spans) for _ in range(b)], dtype=torch.int32, device=DEV)
+    bt = torch.tensor(tables, dtype=torch.int32, device=DEV)
+    want = torch.cat([
+        P.attention(qs[s].double(), ks[s].double(), vs[s].double(), range(a, a + b), H, KV, hd, window)
+        for s, (a, b) in enumerate(spans)])
+    return dict(q=q, cache=cache, pos=pos, sot=sot, bt=bt, want=want, ps=ps, H=H, KV=KV, hd=hd,
+                window=window, scale=1.0 / math.sqrt(hd), tables=tables, lens=lens)
+
+
+ATTN_SHAPES = [(4, 2, 16, 16), (3, 1, 32, 16), (5, 5, 48, 16), (8, 2, 64, 16), (6, 3, 80, 32),
+               (2, 1, 128, 16), (2, 2, 256, 16), (32, 4, 64, 64)]
+
+
+@pytest.mark.parametrize("H,KV,hd,ps", ATTN_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_generic(H, KV, hd, ps, dtype, window):
+    # a whole prompt, a portion behind 300 cached keys, a decode token at a
+    # page's first slot, one at its last, and a sequence's very first token
+    c = attention_case(H, KV, hd, ps, dtype, window, [(0, 45), (300, 9), (ps * 3, 1), (ps * 2 - 1, 1), (0, 1)])
+    out = torch.empty_like(c["q"])
+    K().attn_generic(c["q"], out, c["cache"], c["pos"], c["sot"], c["bt"], ps, H, KV, hd, window, c["scale"])
+    err = (out.cpu().double() - c["want"]).abs().max()
+    assert torch.isfinite(out).all()
+    assert err < (2e-5 if dtype == torch.float32 else 2e-2), float(err)
+
+
+def standout_case(H, KV, hd, key_pos, ctx_len):
+    """One decode token whose query matches exactly one key, far stronger than
+    all others (score 40 against about 0): the output must be that key's
+    value.  A kernel that skips the key (a page's edge, the first or last key)
+    or reads beyond the context (the slot after the last key holds a still
+    stronger key, score 120) shows at once."""
+    g = torch.Generator().manual_seed(1000 + key_pos)
+    L, G = ctx_len, H // KV
+    k = torch.randn(L + 1, KV * hd, generator=g) * 0.1
+    v = torch.randn(L + 1, KV * hd, generator=g)
+    u = torch.randn(KV, hd, generator=g)
+    u = u / u.norm(dim=1, keepdim=True)
+    a = math.sqrt(40.0 * math.sqrt(hd))
+    k[key_pos] = (a * u).reshape(-1)
+    k[L] = (3.0 * a * u).reshape(-1)
+    q = (a * u).repeat_interleave(G, dim=0).reshape(1, H * hd)
+    return q, k, v, L
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("key_pos,ctx", [(0, 500), (15, 500), (16, 500), (255, 500), (256, 500),
+                                         (499, 500), (311, 312), (0, 1), (16, 17)])
+def test_attention_finds_one_key_among_hundreds(dtype, key_pos, ctx):
+    H, KV, hd, ps = 4, 2, 32, 16
+    q, k, v, L = standout_case(H, KV, hd, key_pos, ctx)
+    pages = -(-(L + 1) // ps)
+    table = list(range(pages - 1, -1, -1))
+    cache = build_paged([k], [v], [table], [L + 1], KV, hd, ps, pages, dtype, poison=False)
+    qd = q.to(dtype).to(DEV)
+    out = torch.empty_like(qd)
+    pos = torch.tensor([L - 1], dtype=torch.int32, device=DEV)
+    sot = torch.zeros(1, dtype=torch.int32, device=DEV)
+    bt = torch.tensor([table], dtype=torch.int32, device=DEV)
+    K().attn_generic(qd, out, cache, pos, sot, bt, ps, H, KV, hd, 0, 1.0 / math.sqrt(hd))
+    want = v[key_pos].to(dtype).float().reshape(KV, hd).repeat_interleave(H // KV, 0).reshape(-1)
+    assert (out.cpu().float()[0] - want).abs().max() < (1e-3 if dtype == torch.float32 else 3e-2)
+
+
+@pytest.mark.parametrize("window", [1, 16, 17, 33])
+def test_attention_window_edge(window):
+    H, KV, hd, ps, L = 2, 1, 32, 16, 100
+    dtype = torch.float32
+    # the key just outside the window is overwhelming; it must not be seen
+    g = torch.Generator().manual_seed(window)
+    k = torch.randn(L, hd, generator=g) * 0.1
+    v = torch.randn(L, hd, generator=g)
+    q = torch.randn(1, H * hd, generator=g)
+    q[0, hd:] = q[0, :hd]
+    outside, inside = L - 1 - window, L - window
+    k[outside] = 50.0 * q[0, :hd]
+    table = list(range(-(-L // ps)))
+    cache = build_paged([k], [v], [table], [L], KV, hd, ps, len(table), dtype, poison=False)
+    qd = q.to(DEV)
+    out = torch.empty_like(qd)
+    pos = torch.tensor([L - 1], dtype=torch.int32, device=DEV)
+    sot = torch.zeros(1, dtype=torch.int32, device=DEV)
+    bt = torch.tensor([table], dtype=torch.int32, device=DEV)
+    K().attn_generic(qd, out, cache, pos, sot, bt, ps, H, KV, hd, window, 1.0 / math.sqrt(hd))
+    want = P.attention(q.double(), k.double(), v.double(), [L - 1], H, KV, hd, window)
+    assert (out.cpu().double() - want).abs().max() < 1e-4
+    assert (out.cpu().float()[0, :hd] - v[outside]).abs().max() > 0.1
+    # pages wholly before the window may be gone (-1 in the table)
+    gone = inside // ps
+    bt2 = bt.clone()
+    bt2[0, :gone] = -1
+    out2 = torch.empty_like(qd)
+    K().attn_generic(qd, out2, cache, pos, sot, bt2, ps, H, KV, hd, window, 1.0 / math.sqrt(hd))
+    assert torch.equal(out2, out)
+
+
+def test_attention_refuses_sizes_it_does_not_take():
+    k_ = K()
+    q = torch.zeros(1, 2 * 272, device=DEV)
+    cache = torch.zeros(1, 2, 1, 16 * 272, device=DEV)
+    i32 = torch.zeros(1, dtype=torch.int32, device=DEV)
+    with pytest.raises(k_.KernelError, match="head_dim"):
+        k_.attn_generic(q, torch.empty_like(q), cache, i32, i32, i32.view(1, 1), 16, 2, 1, 272, 0, 1.0)
+
+
+# ------------------------------------------------------------------ sampling
+
+def test_sample_greedy_first_maximum():
+    logits = rnd(6, 1031, seed=9)
+    logits[2, 77] = logits[2, 900] = 50.0
+    logits[3, 1030] = 60.0
+    logits[4, 0] = 60.0
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    K().sample(out, logits)
+    want = [P.argmax_first(r) for r in logits.cpu()]
+    assert out.tolist() == want and want[2] == 77 and want[3] == 1030 and want[4] == 0
+
+
+@pytest.mark.parametrize("temperature", [0.3, 1.0, 2.0])
+def test_sample_temperature_inverts_the_cdf(temperature):
+    from kllm_amd.sampling import uniform
+    rows, vocab = 64, 517
+    logits = rnd(rows, vocab, seed=3, scale=2.0)
+    us = [uniform(5, i) for i in range(rows)]
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    t = torch.full((rows,), temperature, device=DEV)
+    K().sample(out, logits, t, torch.tensor(us, device=DEV))
+    got = out.tolist()
+    for r in range(rows):
+        p = P.softmax_temperature(logits[r].cpu(), temperature)
+        cdf = torch.cumsum(p, 0)
+        lo = float(cdf[got[r] - 1]) if got[r] > 0 else 0.0
+        hi = float(cdf[got[r]])
+        assert lo - 1e-5 <= us[r] < hi + 1e-5, (r, got[r], lo, us[r], hi)
+    # mixed rows: temperature 0 is greedy
+    t[::2] = 0.0
+    K().sample(out, logits, t, torch.tensor(us, device=DEV))
+    assert out.tolist()[::2] == [P.argmax_first(r) for r in logits.cpu()[::2]]
+
+
+def test_sample_frequencies_follow_softmax():
+    from kllm_amd.sampling import uniform
+    n = 4096
+    row = torch.tensor([0.0, math.log(2.0), math.log(5.0), -40.0])
+    logits = row.repeat(n, 1).to(DEV)
+    us = torch.tensor([uniform(2, i) for i in range(n)], device=DEV)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    K().sample(out, logits, torch.ones(n, device=DEV), us)
+    counts = torch.bincount(out.cpu().long(), minlength=4).tolist()
+    want = [1 / 8, 2 / 8, 5 / 8]
+    chi2 = sum((counts[k] - n * want[k]) ** 2 / (n * want[k]) for k in range(3))
+    assert chi2 < 13.8 and counts[3] == 0

@@ -1,0 +1,321 @@
+"""That the engine takes parts and architectures it has never seen, without a
+change to its files: a toy mixer with state of its own, a toy feed-forward
+with routing, another position encoding, a running order that names a layer
+twice and lets a layer read another layer's cache, and layers with a window
+beside layers without (two cache groups).  The toy parts are written with
+ordinary torch operations here in the test; they are no model of anyone's."""
+
+import math
+
+import pytest
+import torch
+
+import plain_llama as P
+import tiny
+import traces
+from kllm_amd.config import LlamaConfig, register_architecture, unregister_architecture
+from kllm_amd.parts import (CacheNeed, LayerSpec, ModelSpec, Part, PartSpec, Run, WeightSpec,
+                            register_part, unregister_part)
+
+pytestmark = pytest.mark.gpu
+
+
+# ----------------------------------------------------------------------------- toy parts
+
+class ToyDecayMixer(Part):
+    """s_t = decay * s_{t-1} + W_in x_t ;  out_t = W_out s_t.  The state s is
+    one vector per request, kept in a slot between steps."""
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.hidden, self.width, self.decay = self.param("hidden"), self.param("width"), self.param("decay")
+
+    def weight_specs(self):
+        return [WeightSpec(self.tensor_name("in.weight"), (self.width, self.hidden)),
+                WeightSpec(self.tensor_name("out.weight"), (self.hidden, self.width))]
+
+    def bind(self, weights):
+        self.w_in = weights[self.tensor_name("in.weight")].float()
+        self.w_out = weights[self.tensor_name("out.weight")].float()
+
+    def cache_need(self):
+        return CacheNeed("state", state_shape=(self.width,))
+
+    def forward(self, ctx, xn, cache):
+        u = xn.float() @ self.w_in.t()
+        out = torch.empty(ctx.n, self.hidden, dtype=torch.float32, device=xn.device)
+        slots = cache.slots.tolist()
+        for s in range(ctx.n_spans):
+            a, b = ctx.h_span_start[s], ctx.h_span_start[s + 1]
+            state = cache.state[slots[s]]
+            if ctx.h_span_pos[s] == 0:
+                state.zero_()                       # a new request starts from nothing
+            for t in range(a, b):
+                state.mul_(self.decay).add_(u[t])
+                out[t] = self.w_out @ state
+        return out
+
+
+class ToyRoutedFeedForward(Part):
+    """Two tiny experts; each token goes to the one its router prefers."""
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.hidden, self.width = self.param("hidden"), self.param("width")
+
+    def weight_specs(self):
+        specs = [WeightSpec(self.tensor_name("router.weight"), (2, self.hidden))]
+        for e in range(2):
+            specs += [WeightSpec(self.tensor_name(f"experts.{e}.up.weight"), (self.width, self.hidden)),
+                      WeightSpec(self.tensor_name(f"experts.{e}.down.weight"), (self.hidden, self.width))]
+        return specs
+
+    def bind(self, weights):
+        self.router = weights[self.tensor_name("router.weight")].float()
+        self.up = [weights[self.tensor_name(f"experts.{e}.up.weight")].float() for e in range(2)]
+        self.down = [weights[self.tensor_name(f"experts.{e}.down.weight")].float() for e in range(2)]
+
+    def forward(self, ctx, xn):
+        x = xn.float()
+        choice = (x @ self.router.t()).argmax(-1)
+        out = torch.zeros_like(x)
+        for e in range(2):
+            m = choice == e
+            out[m] = torch.relu(x[m] @ self.up[e].t()) @ self.down[e].t()
+        return out
+
+
+class ToyAdditivePositions(Part):
+    """Adds sin(position * rate) to every channel of the embedded tokens."""
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.rate = self.param("rate")
+
+    def prepare(self, ctx):
+        pass
+
+    def on_embedding(self, ctx, x):
+        x.add_(torch.sin(ctx.positions[:ctx.n].float() * self.rate)[:, None])
+
+
+def toy_reference(w, cfg, ids, dtype_round):
+    """The toy architecture written plainly, whole sequence, on the CPU.
+    Returns (logits, margins): margins[t] is the gap between the router's two
+    scores at position t; where it is tiny, rounding may send the token to the
+    other expert, and everything after it in the sequence differs."""
+    d, eps = cfg["hidden_size"], cfg["rms_norm_eps"]
+    r = (lambda t: t.to(torch.bfloat16).float()) if dtype_round else (lambda t: t)
+    T = len(ids)
+    pos = torch.arange(T)
+    x = P.embedding(ids, w["model.embed_tokens.weight"]) + torch.sin(pos.float() * 0.37)[:, None]
+    c = P._cfg(cfg)
+    # layer 0: attention (no rotary here: positions come from the embedding) + routed feed-forward
+    xn = r(P.rmsnorm(x, w["model.layers.0.input_layernorm.weight"], eps))
+    q = P.linear(xn, w["model.layers.0.self_attn.q_proj.weight"])
+    k = P.linear(xn, w["model.layers.0.self_attn.k_proj.weight"])
+    v = P.linear(xn, w["model.layers.0.self_attn.v_proj.weight"])
+    a = P.attention(r(q), r(k), r(v), pos, c["H"], c["KV"], c["hd"])
+    x = x + P.linear(r(a), w["model.layers.0.self_attn.o_proj.weight"])
+    xn = r(P.rmsnorm(x, w["model.layers.0.post_attention_layernorm.weight"], eps))
+    scores = xn @ w["model.layers.0.moe.router.weight"].t()
+    choice = scores.argmax(-1)
+    margins = (scores[:, 0] - scores[:, 1]).abs()
+    ff = torch.zeros_like(x)
+    for e in range(2):
+        m = choice == e
+        ff[m] = torch.relu(xn[m] @ w[f"model.layers.0.moe.experts.{e}.up.weight"].t()) @ \
+            w[f"model.layers.0.moe.experts.{e}.down.weight"].t()
+    x = x + ff
+    # layer 1: decay mixer + gated feed-forward
+    xn = r(P.rmsnorm(x, w["model.layers.1.input_layernorm.weight"], eps))
+    u = xn @ w["model.layers.1.mix.in.weight"].t()
+    s = torch.zeros(u.shape[1])
+    mix = torch.zeros_like(x)
+    for t in range(T):
+        s = 0.9 * s + u[t]
+        mix[t] = w["model.layers.1.mix.out.weight"] @ s
+    x = x + mix
+    xn = r(P.rmsnorm(x, w["model.layers.1.post_attention_layernorm.weight"], eps))
+    x = x + P.swiglu(xn, w["model.layers.1.mlp.gate_proj.weight"], w["model.layers.1.mlp.up_proj.weight"],
+                     w["model.layers.1.mlp.down_proj.weight"]) if not dtype_round else x + P.linear(
+        r(P.silu(P.linear(xn, w["model.layers.1.mlp.gate_proj.weight"])) * P.linear(xn, w["model.layers.1.mlp.up_proj.weight"])),
+        w["model.layers.1.mlp.down_proj.weight"])
+    xn = r(P.rmsnorm(x, w["model.norm.weight"], eps))
+    return P.linear(xn, w["lm_head.weight"]), margins
+
+
+def build_toy(cfg: LlamaConfig) -> ModelSpec:
+    d = cfg.hidden_size
+    positions = PartSpec("toy_additive", rate=0.37)
+    norm = lambda name: PartSpec("rmsnorm", name, size=d, eps=cfg.rms_norm_eps)
+    layers = [
+        LayerSpec(norm_mixer=norm("model.layers.0.input_layernorm"),
+                  mixer=PartSpec("attention", "model.layers.0.self_attn", hidden=d, heads=cfg.num_attention_heads,
+                                 kv_heads=cfg.num_key_value_heads, head_dim=cfg.head_dim, position=positions),
+                  norm_feed_forward=norm("model.layers.0.post_attention_layernorm"),
+                  feed_forward=PartSpec("toy_routed", "model.layers.0.moe", hidden=d, width=24)),
+        LayerSpec(norm_mixer=norm("model.layers.1.input_layernorm"),
+                  mixer=PartSpec("toy_decay", "model.layers.1.mix", hidden=d, width=40, decay=0.9),
+                  norm_feed_forward=norm("model.layers.1.post_attention_layernorm"),
+                  feed_forward=PartSpec("gated_mlp", "model.layers.1.mlp", hidden=d,
+                                        intermediate=cfg.intermediate_size)),
+    ]
+    return ModelSpec(
+        embedding=PartSpec("token_embedding", "model.embed_tokens", vocab=cfg.vocab_size, hidden=d),
+        layers=layers, schedule=[Run(0), Run(1)], final_norm=norm("model.norm"),
+        head=PartSpec("linear_head", "lm_head", vocab=cfg.vocab_size, hidden=d),
+        vocab_size=cfg.vocab_size, hidden_size=d)
+
+
+@pytest.fixture
+def toy_registered():
+    register_part("mixer", "toy_decay", ToyDecayMixer)
+    register_part("feed_forward", "toy_routed", ToyRoutedFeedForward)
+    register_part("position", "toy_additive", ToyAdditivePositions)
+    register_architecture("ToyForCausalLM", LlamaConfig, build_toy)
+    yield dict(tiny.CONFIGS["A"], architectures=["ToyForCausalLM"])
+    unregister_architecture("ToyForCausalLM")
+    for cat, kind in (("mixer", "toy_decay"), ("feed_forward", "toy_routed"), ("position", "toy_additive")):
+        unregister_part(cat, kind)
+
+
+def engine_weights(eng):
+    """name -> float32 CPU tensor of what the engine's parts were given."""
+    from kllm_amd.weights import random_weights
+    return {k: v.float().cpu() for k, v in random_weights(eng.model.weight_specs(), 5, eng.dtype, "cpu", 0.08, 0.2).items()}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_is_registered_built_and_stepped(toy_registered, dtype):
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry
+    cfg = toy_registered
+    eng = Engine.from_random(cfg, 5, EngineOptions(dtype=dtype, max_tokens=256, max_requests=3), std=0.08, norm_std=0.2)
+    plan = eng.model.cache_plan
+    assert [g.need.kind for g in plan.groups] == ["paged", "state"] and plan.runs == [(0, 0, True), (1, 0, True)]
+    assert tuple(eng.state[1].shape) == (1, 3, 40)
+    w = engine_weights(eng)
+    reqs = {"a": tiny.tokens(cfg, 45, 1), "b": tiny.tokens(cfg, 30, 2), "c": tiny.tokens(cfg, 22, 3),
+            "d": tiny.tokens(cfg, 37, 4)}
+    want = {rid: toy_reference(w, cfg, toks, dtype == "bfloat16") for rid, toks in reqs.items()}
+    steps, peak = traces.mixed(reqs, seed=3, max_live=3, tail=6, max_portion=9)
+    outs = []
+    for s in steps:
+        out = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        outs.append(out.cpu().numpy())
+        for rid in s["end"]:
+            eng.release(rid)                      # the slot goes back and is taken again by "d"
+    rows = traces.collect(steps, outs)
+    compared = 0
+    for rid, toks in reqs.items():
+        logits, margins = want[rid]
+        close = (margins < (1e-4 if dtype == "float32" else 8e-3)).nonzero()
+        upto = int(close[0]) if len(close) else len(toks)     # a near-tie of the router ends the comparison
+        for p in range(upto):
+            err = float((torch.from_numpy(rows[(rid, p)]) - logits[p]).abs().max())
+            assert err < (2e-4 if dtype == "float32" else 8e-2), (rid, p, err)
+        compared += upto
+    assert compared >= 60, compared
+    assert eng.cache.slots.free_slots == 3 and not eng.cache.requests
+
+
+# ----------------------------------------------------------------------------- running order
+
+def build_repeat_and_share(cfg: LlamaConfig) -> ModelSpec:
+    """Three layers; layer 1 runs twice (a cache for each run); layer 2 has no
+    k/v projections and reads the cache of layer 1's first run."""
+    from kllm_amd.models.llama import build_llama
+    spec = build_llama(cfg)
+    spec.layers[2].mixer.params["own_kv"] = False
+    spec.schedule = [Run(0), Run(1), Run(1), Run(2, cache_of=1)]
+    return spec
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_twice_and_a_layer_reading_anothers_cache(dtype, tmp_path):
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry
+    register_architecture("ToyScheduleForCausalLM", LlamaConfig, build_repeat_and_share)
+    try:
+        cfg = dict(tiny.CONFIGS["B"], architectures=["ToyScheduleForCausalLM"])
+        w = P.random_weights(cfg, 4, std=0.05, norm_std=0.1)
+        del w["model.layers.2.self_attn.k_proj.weight"], w["model.layers.2.self_attn.v_proj.weight"]
+        d = tiny.write_model(str(tmp_path), cfg, 0, weights=w)
+        eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=192))
+        plan = eng.model.cache_plan
+        assert plan.groups[0].entries == 3 and plan.runs == [(0, 0, True), (0, 1, True), (0, 2, True), (0, 1, False)]
+        ids = tiny.tokens(cfg, 60, 1)
+        ws = tiny.read_weights(d, as_stored_in=dtype)
+        want = P.forward(ws, cfg, ids, schedule=[0, 1, 1, 2], kv_from={3: 1})
+        got = torch.cat([eng.step([StepEntry("r", ids[a:b], list(range(b - a)))]).cpu()
+                         for a, b in [(0, 23), (23, 25), (25, 59), (59, 60)]])
+        assert float((got - want).abs().max()) < tiny.TOL[dtype]
+        assert float((want - P.forward(ws | {"model.layers.2.self_attn.k_proj.weight": ws["model.layers.1.self_attn.k_proj.weight"],
+                                             "model.layers.2.self_attn.v_proj.weight": ws["model.layers.1.self_attn.v_proj.weight"]},
+                                       cfg, ids, schedule=[0, 1, 1, 2])).abs().max()) > 1e-3
+    finally:
+        unregister_architecture("ToyScheduleForCausalLM")
+
+
+def test_a_bad_running_order_is_refused():
+    from kllm_amd.engine.model import Model
+    from kllm_amd.models.llama import build_llama
+    from kllm_amd.config import config_from_dict
+    from kllm_amd.parts import Runtime
+    cfg = config_from_dict(tiny.CONFIGS["B"])
+    rt = lambda: Runtime(device=torch.device("cpu"), dtype=torch.float32)
+    spec = build_llama(cfg)
+    spec.schedule = [Run(0), Run(5)]
+    with pytest.raises(ValueError, match="names layer 5"):
+        Model(spec, rt())
+    spec.schedule = [Run(0, cache_of=0)]
+    with pytest.raises(ValueError, match="earlier entry"):
+        Model(spec, rt())
+
+
+# ----------------------------------------------------------------------------- windows
+
+WINDOW = 20
+
+
+def build_windowed(cfg: LlamaConfig) -> ModelSpec:
+    from kllm_amd.models.llama import build_llama
+    spec = build_llama(cfg)
+    for i in (0, 2):
+        spec.layers[i].mixer.params["window"] = WINDOW
+    return spec
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_with_a_window_have_pages_of_their_own(dtype, model_dirs, tmp_path):
+    import json
+    import os
+    import shutil
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry
+    register_architecture("ToyWindowForCausalLM", LlamaConfig, build_windowed)
+    try:
+        cfg = dict(tiny.CONFIGS["B"], architectures=["ToyWindowForCausalLM"])
+        d = str(tmp_path / "m")
+        shutil.copytree(model_dirs("B"), d)
+        with open(os.path.join(d, "config.json"), "w") as f:
+            json.dump(cfg, f)
+        eng = Engine.from_dir(d, EngineOptions(dtype=dtype, num_pages=14, max_model_len=1 << 20,
+                                               poison_freed_pages=True))
+        plan = eng.model.cache_plan
+        assert [(g.need.window, g.entries) for g in plan.groups] == [(WINDOW, 2), (0, 1)]
+        ids = tiny.tokens(cfg, 200, 1)
+        want = P.forward(tiny.read_weights(d, as_stored_in=dtype), cfg, ids, windows={0: WINDOW, 2: WINDOW})
+        cuts = [0, 37, 39, 70, 71, 72, 130, 133] + list(range(134, 201))
+        got = []
+        for a, b in zip(cuts, cuts[1:]):
+            got.append(eng.step([StepEntry("r", ids[a:b], list(range(b - a)))]).cpu())
+            win, full = eng.cache.pools
+            assert win.used_pages <= -(-(WINDOW + (b - a)) // 16) + 1     # the window's pages only
+            assert full.used_pages == -(-b // 16)
+        got = torch.cat(got)
+        assert torch.isfinite(got).all()
+        assert float((got - want).abs().max()) < tiny.TOL[dtype]
+        assert eng.cache.pools[0].total_allocs == 13 and eng.cache.pools[0].used_pages <= 3
+        eng.release("r")
+        eng.cache.check_invariants()
+    finally:
+        unregister_architecture("ToyWindowForCausalLM")

@@ -22,6 +22,7 @@ from ..cache import CacheManager, GroupSpec, OutOfPages
 from ..config import ModelConfig, config_from_dict, load_config, resolve_architecture
 from ..parts.base import PagedCacheView, Runtime, StateCacheView, StepContext
 from ..weights import load_weights, random_weights
+from . import control
 from .model import Model
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16,
@@ -47,6 +48,7 @@ class EngineOptions:
     gemm: str = "hip"                     # "hip" or "library" (vendor GEMM for large prompts)
     attention: str = "auto"               # "auto" or "generic"
     graphs: bool = True                   # replay decode steps as HIP graphs
+    max_graph_batch: int = 256            # largest decode batch that is recorded as a graph
     poison_freed_pages: bool = False      # debugging: fill pages with NaN when they are given back
     extra: Dict[str, object] = field(default_factory=dict)
 
@@ -96,6 +98,8 @@ class Engine:
         self._control = None
         self.steps_run = 0
         self.tokens_run = 0
+        from .graph import DecodeGraphs
+        self._graphs = DecodeGraphs(self)
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -184,6 +188,8 @@ class Engine:
 
     # ------------------------------------------------------------------ the step
     def _staging(self, n_ints: int) -> torch.Tensor:
+        """A pinned host buffer; a small ring, so that filling the next step
+        does not wait for the copy of the last one."""
         ring = 4
         if len(self._pinned) < ring:
             self._pinned.append(torch.empty(max(n_ints, 4096), dtype=torch.int32, pin_memory=True))
@@ -198,6 +204,12 @@ class Engine:
                 self._pinned[i] = torch.empty(n_ints, dtype=torch.int32, pin_memory=True)
         self._staging_index = i
         return self._pinned[i]
+
+    def _send(self, host: torch.Tensor, dev: torch.Tensor, total: int):
+        dev[:total].copy_(host[:total], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._pinned_events[self._staging_index] = ev
 
     def _validate(self, entries: Sequence[StepEntry]):
         if not entries:
@@ -219,12 +231,9 @@ class Engine:
                     raise StepError(f"request {e.request_id!r}: wanted place {w} is outside its "
                                     f"{toks.size} tokens")
 
-    def step(self, entries: Sequence[StepEntry], taps: Optional[list] = None):
-        """Run one batch.  Returns float32 logits [wanted, vocab] on the
-        device, in the order of the entries and of their ``want`` lists, or
-        None if nothing is wanted.  Raises OutOfPages (and changes nothing) if
-        the cache cannot hold the step's tokens."""
-        self._validate(entries)
+    def _reserve(self, entries: Sequence[StepEntry]):
+        """Room for every entry's tokens, or nothing taken.  Returns what to
+        undo if the step fails."""
         opened, reserved = [], []
         try:
             for e in entries:
@@ -239,99 +248,82 @@ class Engine:
                 self.cache.reserve(e.request_id, len(e.tokens))
                 reserved.append(e.request_id)
         except Exception:
-            for rid in reserved:
-                self.cache.cancel(rid)
-            for rid in opened:
-                self.cache.release(rid)
+            self._undo(opened, reserved)
             raise
-        try:
-            ctx = self._build_context(entries)
-            ctx.taps = taps
-            views = self._cache_views(ctx)
-            logits = self.model.run(ctx, views)
-        except Exception:
-            for rid in reserved:
-                self.cache.cancel(rid)
-            for rid in opened:
-                self.cache.release(rid)
-            raise
-        freed_before = None
+        return opened, reserved
+
+    def _undo(self, opened, reserved):
+        for rid in reserved:
+            self.cache.cancel(rid)
+        for rid in opened:
+            self.cache.release(rid)
+
+    def _commit(self, entries: Sequence[StepEntry]):
+        before = None
         if self.options.poison_freed_pages:
-            freed_before = {e.request_id: [list(t) for t in self.cache.get(e.request_id).tables]
-                            for e in entries}
+            before = {e.request_id: [list(t) for t in self.cache.get(e.request_id).tables]
+                      for e in entries}
         for e in entries:
             self.cache.commit(e.request_id, len(e.tokens))
-        if freed_before is not None:
+        if before is not None:
             for e in entries:
                 now = self.cache.get(e.request_id).tables
-                gone = [[p for p, q in zip(b, a) if p >= 0 and q < 0]
-                        for b, a in zip(freed_before[e.request_id], now)]
-                self._poison(gone)
+                self._poison([[p for p, q in zip(b, a) if p >= 0 and q < 0]
+                              for b, a in zip(before[e.request_id], now)])
         self.steps_run += 1
-        self.tokens_run += ctx.n
-        return logits
+        self.tokens_run += sum(len(e.tokens) for e in entries)
 
-    def _build_context(self, entries: Sequence[StepEntry]) -> StepContext:
-        S = len(entries)
-        lens = [len(e.tokens) for e in entries]
-        n = sum(lens)
+    def _describe(self, entries: Sequence[StepEntry]):
         rcs = [self.cache.get(e.request_id) for e in entries]
-        pos0 = [rc.length for rc in rcs]
+        lens = [len(e.tokens) for e in entries]
         starts = [0]
         for l in lens:
             starts.append(starts[-1] + l)
         rows = [starts[s] + int(w) for s, e in enumerate(entries) for w in e.want]
-        R = len(rows)
         n_groups = len(self.cache.groups)
-        maxp = [max(1, max(len(rc.tables[g]) for rc in rcs)) for g in range(n_groups)]
+        tables = [[rc.tables[g] for rc in rcs] for g in range(n_groups)]
+        return rcs, lens, rows, tables
 
-        sizes = [n, n, n, S + 1, S, S, max(R, 1)] + [S * m for m in maxp]
-        offs = [0]
-        for s in sizes:
-            offs.append(offs[-1] + ((s + 3) // 4) * 4)   # 16-byte aligned sections
-        total = offs[-1]
-        host = self._staging(total)
-        h = host.numpy()
-        tok = h[offs[0]:offs[0] + n]
-        posv = h[offs[1]:offs[1] + n]
-        sot = h[offs[2]:offs[2] + n]
-        for s, e in enumerate(entries):
-            a, b = starts[s], starts[s + 1]
-            tok[a:b] = np.asarray(e.tokens, dtype=np.int32)
-            posv[a:b] = np.arange(pos0[s], pos0[s] + lens[s], dtype=np.int32)
-            sot[a:b] = s
-        h[offs[3]:offs[3] + S + 1] = starts
-        h[offs[4]:offs[4] + S] = pos0
-        h[offs[5]:offs[5] + S] = [rc.slot for rc in rcs]
-        if R:
-            h[offs[6]:offs[6] + R] = rows
-        for g in range(n_groups):
-            bt = h[offs[7 + g]:offs[7 + g] + S * maxp[g]].reshape(S, maxp[g])
-            bt.fill(-1)
-            for s, rc in enumerate(rcs):
-                t = rc.tables[g]
-                bt[s, :len(t)] = t
+    def step(self, entries: Sequence[StepEntry], taps: Optional[list] = None):
+        """Run one batch.  Returns float32 logits [wanted, vocab] on the
+        device, in the order of the entries and of their ``want`` lists, or
+        None if nothing is wanted.  Raises OutOfPages (and changes nothing) if
+        the cache cannot hold the step's tokens."""
+        self._validate(entries)
+        opened, reserved = self._reserve(entries)
+        try:
+            rcs, lens, rows, tables = self._describe(entries)
+            pages = tuple(max(1, max(len(t) for t in tg)) for tg in tables)
+            layout = control.ControlLayout(sum(lens), len(entries), len(rows), pages)
+            total = layout.total
+            host = self._staging(total)
+            pos0 = [rc.length for rc in rcs]
+            starts = control.fill(host.numpy(), layout, [e.tokens for e in entries], pos0,
+                                  [rc.slot for rc in rcs], rows, tables)
+            if self._control is None or self._control.numel() < total:
+                self._control = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
+            self._send(host, self._control, total)
+            ctx = control.context(self._control, layout, self.runtime, starts, pos0, lens)
+            ctx.taps = taps
+            logits = self.model.run(ctx, self._cache_views(ctx))
+        except Exception:
+            self._undo(opened, reserved)
+            raise
+        self._commit(entries)
+        return logits
 
-        if self._control is None or self._control.numel() < total:
-            self._control = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
-        dev = self._control
-        dev[:total].copy_(host[:total], non_blocking=True)
-        ev = torch.cuda.Event()
-        ev.record()
-        self._pinned_events[self._staging_index] = ev
-
-        def sec(i, count):
-            return dev[offs[i]:offs[i] + count]
-
-        return StepContext(
-            n=n, n_spans=S,
-            token_ids=sec(0, n), positions=sec(1, n), span_of_token=sec(2, n),
-            span_start=sec(3, S + 1), span_pos=sec(4, S), slots=sec(5, S),
-            logit_rows=sec(6, R) if R else None,
-            h_span_start=starts, h_span_pos=pos0, h_span_len=lens,
-            block_tables=[sec(7 + g, S * maxp[g]).view(S, maxp[g]) for g in range(n_groups)],
-            runtime=self.runtime, max_span_len=max(lens), all_decode=all(l == 1 for l in lens),
-        )
+    def step_sample(self, entries: Sequence[StepEntry], temperatures, uniforms) -> List[int]:
+        """A step whose wanted places are sampled on the device: one token per
+        wanted place, as host ints.  Batches of single decode tokens are
+        replayed as a HIP graph (forward pass and sampling in one launch)."""
+        if (self.options.graphs and self.model.graph_safe
+                and len(entries) <= self.options.max_graph_batch
+                and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)):
+            return self._graphs.decode(entries, temperatures, uniforms)
+        logits = self.step(entries)
+        if logits is None:
+            return []
+        return self.sample(logits, temperatures, uniforms)
 
     def _cache_views(self, ctx: StepContext):
         views = []

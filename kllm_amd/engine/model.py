@@ -92,6 +92,12 @@ class Model:
         for p in self.parts():
             p.bind(weights)
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a step of this model can be recorded in a HIP graph."""
+        shared = [p for _, p in self.runtime.shared.values()]
+        return all(p.graph_safe for p in self.parts() + shared)
+
     def weight_bytes(self) -> int:
         """Bytes of distinct weight tensors the parts hold after bind."""
         seen = {}

@@ -247,8 +247,15 @@ class Scheduler:
             toks = pe.request.all_tokens()[pe.start:pe.start + pe.count]
             entries.append(StepEntry(self._key(pe.request), toks,
                                      [pe.count - 1] if pe.wants_logits else []))
+        wanting = [pe for pe in plan.entries if pe.wants_logits]
+        temps = [pe.request.temperature for pe in wanting]
+        us = [uniform(pe.request.seed, len(pe.request.generated)) for pe in wanting]
         try:
-            logits = self.engine.step(entries)
+            if hasattr(self.engine, "step_sample"):
+                toks = self.engine.step_sample(entries, temps, us)
+            else:
+                logits = self.engine.step(entries)
+                toks = self.engine.sample(logits, temps, us) if wanting else []
         except Exception as exc:  # a failed forward fails every request of the step
             for pe in plan.entries:  # (engine/scheduler.go:197-203)
                 r = pe.request
@@ -261,16 +268,12 @@ class Scheduler:
         self.stats["steps"] += 1
         self.stats["tokens"] += plan.tokens
         self.stats["max_batch_seen"] = max(self.stats["max_batch_seen"], len(entries))
-        wanting = [pe for pe in plan.entries if pe.wants_logits]
         for pe in plan.entries:
             pe.request.cursor += pe.count
             key = "decode_tokens" if (pe.count == 1 and pe.request.generated) else "prefill_tokens"
             self.stats[key] += pe.count
         produced = []
         if wanting:
-            temps = [pe.request.temperature for pe in wanting]
-            us = [uniform(pe.request.seed, len(pe.request.generated)) for pe in wanting]
-            toks = self.engine.sample(logits, temps, us)
             eos = set(getattr(self.engine, "eos_token_ids", ()) or ())
             for pe, tok in zip(wanting, toks):
                 r = pe.request

@@ -27,6 +27,8 @@ from .spec import CacheNeed, WeightSpec
 
 @register_part("mixer", "attention")
 class CausalSelfAttention(Part):
+    graph_safe = True
+
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)
         self.hidden = int(self.param("hidden"))

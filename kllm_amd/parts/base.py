@@ -171,15 +171,21 @@ class StepContext:
     all_decode: bool = False              # every span is a single token
     scratch: Dict[Any, Any] = field(default_factory=dict)   # per-step values of parts
     taps: Optional[List[torch.Tensor]] = None               # residual-stream captures
+    workspace: Optional["Workspace"] = None                 # scratch of this step (default: the runtime's)
 
     def buf(self, tag, shape, dtype):
-        return self.runtime.workspace.get(tag, shape, dtype)
+        return (self.workspace or self.runtime.workspace).get(tag, shape, dtype)
 
 
 class Part:
     """Base of all parts."""
     category = None
     kind = None
+    # True if the part's forward only launches kernels on the current stream with
+    # addresses and sizes that depend on nothing but the batch's shape: such a
+    # part can be recorded in a HIP graph.  A part that reads device values on
+    # the host, or loops over host-side span data, leaves this False.
+    graph_safe = False
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
         self.spec = spec

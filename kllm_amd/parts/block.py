@@ -25,6 +25,10 @@ class PreNormBlock(Part):
     def parts(self):
         return [self.norm_mixer, self.mixer, self.norm_ff, self.feed_forward]
 
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self.parts())
+
     def weight_specs(self):
         return [s for p in self.parts() for s in p.weight_specs()]
 

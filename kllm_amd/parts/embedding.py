@@ -19,6 +19,8 @@ from .spec import WeightSpec
 
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)
         self.vocab = int(self.param("vocab"))
@@ -39,6 +41,8 @@ class TokenEmbedding(Part):
 
 @register_part("head", "linear_head")
 class LinearHead(Part):
+    graph_safe = True
+
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)
         self.vocab = int(self.param("vocab"))

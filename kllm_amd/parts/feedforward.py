@@ -18,6 +18,8 @@ from .spec import WeightSpec
 
 @register_part("feed_forward", "gated_mlp")
 class GatedFeedForward(Part):
+    graph_safe = True
+
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)
         self.hidden = int(self.param("hidden"))

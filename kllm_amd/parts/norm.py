@@ -18,6 +18,8 @@ from .spec import WeightSpec
 
 @register_part("norm", "rmsnorm")
 class RMSNorm(Part):
+    graph_safe = True
+
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)
         self.size = int(self.param("size"))

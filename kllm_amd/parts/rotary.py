@@ -19,6 +19,8 @@ from .base import Part, register_part
 
 @register_part("position", "rotary")
 class RotaryEncoding(Part):
+    graph_safe = True
+
 
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)

@@ -28,6 +28,7 @@ def main(argv=None):
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--gemm", default="hip", choices=["hip", "library"])
+    ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill only (for profiles)")
     args = ap.parse_args(argv)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not built")
@@ -45,6 +46,10 @@ def main(argv=None):
     eng = B.make_engine(cfg, args.dtype, max_tokens=max_batch * args.context + 4096,
                         max_model_len=args.context + 64, gemm=args.gemm)
 
+    if args.prefill_only:
+        pms = B.measure_prefill(eng, 2048, reps=max(1, args.steps), warmup=args.warmup)
+        print(json.dumps({"prefill_ms": round(pms, 3), "tok_s": round(2048e3 / pms, 1)}))
+        return 0
     ms, ctx = B.measure_decode(eng, args.batch, args.context, args.steps, args.warmup)
     value = args.batch * 1e3 / ms
     need = B.decode_step_bytes(cfg, args.batch, int(ctx), elem)

@@ -1,0 +1,267 @@
+// Decode attention over the paged cache on the matrix cores (bfloat16).
+//
+// One wave takes one token, one KV head with up to 16 of its query heads, and
+// one slice of the token's keys; it streams that slice's pages from memory
+// once, for all heads of the group, and leaves a partial result (running
+// maximum, sum, unnormalised output).  A second kernel merges the slices.  The
+// launch does not depend on any context length, so a recorded step can be
+// replayed as contexts grow.
+//
+// Formulas as in the generic kernel (reference: backend/model.cu:343-408):
+// score = (q.k)/sqrt(hd) over keys [max(0, p-window+1), p], softmax with the
+// maximum subtracted, all in 32-bit; probabilities are rounded to bfloat16 for
+// the product with the values and their sum is taken over the rounded numbers.
+//
+// MFMA 16x16x32 (lane l: g = l/16, c = l%16): A[c][8g..8g+7], B[8g..8g+7][c],
+// D[4g+i][c].  Scores: A = 16 keys x 32 of hd (one key row per lane, straight
+// from its page), B = q of 16 heads, D[key 4g+i][head c].  Values: the 32 k
+// slots of one MFMA are keys (4g+j) of page-tile 0 for j < 4 and of page-tile 1
+// for j >= 4, which is exactly how a lane holds its probabilities; A = values
+// [hd row c][those keys], two 8-byte reads from the [hd][slot] value layout.
+#include <math.h>
+
+#include "common.hpp"
+#include "kllm_kernels.h"
+
+namespace kllm {
+
+constexpr int kDecodeWaves = 4;
+
+__device__ __forceinline__ float group4_max(float v) {   // over lanes c, c+16, c+32, c+48
+  v = fmaxf(v, __shfl_xor(v, 16, kWave));
+  return fmaxf(v, __shfl_xor(v, 32, kWave));
+}
+__device__ __forceinline__ float group4_sum(float v) {
+  v += __shfl_xor(v, 16, kWave);
+  return v + __shfl_xor(v, 32, kWave);
+}
+
+template <int HDT>  // head_dim = 16 * HDT
+__global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
+    const bf16_t* __restrict__ q, float* __restrict__ part, const bf16_t* __restrict__ cache,
+    const int* __restrict__ positions, const int* __restrict__ span_of_token,
+    const int* __restrict__ block_table, int max_pages, int page_size, int H, int KV, int window,
+    float scale, int head_tiles) {
+  constexpr int hd = 16 * HDT;
+  constexpr int KS = (hd + 31) / 32;           // MFMA steps over head_dim for the scores
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int g = lane / 16, c = lane % 16;
+  const int t = blockIdx.x;
+  const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y % head_tiles;
+  const int G = H / KV;
+  const int nslices = gridDim.z * kDecodeWaves;
+  const int slice = blockIdx.z * kDecodeWaves + wave;
+
+  const int len = positions[t] + 1;
+  const int start = (window > 0 && len > window) ? len - window : 0;
+  const int first = start / 32 * 32;                       // tiles of 32 keys from here
+  const int tiles = (len - first + 31) / 32;
+  const int per = (tiles + nslices - 1) / nslices;
+  const int tile0 = slice * per, tile1 = min(tile0 + per, tiles);
+  const int* table = block_table + (long)span_of_token[t] * max_pages;
+  const long block = (long)page_size * hd;
+
+  const int head_in_group = ht * 16 + c;                   // this lane's column
+  const bool head_ok = head_in_group < G;
+  const int head = kvh * G + (head_ok ? head_in_group : 0);
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  bf16x8 qb[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d0 = 32 * ks + 8 * g;
+    qb[ks] = (head_ok && d0 < hd)
+                 ? *reinterpret_cast<const bf16x8*>(q + ((long)t * H + head) * hd + d0)
+                 : zero8;
+  }
+
+  float m = -INFINITY, l = 0.f;
+  floatx4 acc[HDT];
+#pragma unroll
+  for (int i = 0; i < HDT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  for (int tile = tile0; tile < tile1; ++tile) {
+    const int kb = first + tile * 32;
+    const bool edge = kb < start || kb + 32 > len;
+    const bf16_t* kpage[2];
+    const bf16_t* vpage[2];
+    bool live[2];
+    floatx4 s[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int k0 = kb + 16 * u;
+      live[u] = k0 < len && k0 + 16 > start;               // some key of these 16 is read
+      int page = 0;
+      if (live[u]) page = table[k0 / page_size];
+      const long base = ((long)page * 2 * KV + kvh) * block;
+      kpage[u] = cache + base + (long)(k0 % page_size) * hd;                 // [slot][hd]
+      vpage[u] = cache + base + (long)KV * block + (k0 % page_size);          // [hd][slot]
+      s[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+      if (live[u]) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const int d0 = 32 * ks + 8 * g;
+          const bf16x8 a = (d0 < hd) ? *reinterpret_cast<const bf16x8*>(kpage[u] + (long)c * hd + d0)
+                                     : zero8;
+          s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ks], s[u], 0, 0, 0);
+        }
+      }
+    }
+    // ---- online softmax for this lane's head over its 8 keys, then the 4 lanes of the column
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kb + 16 * u + 4 * g + i;
+        const bool ok = live[u] && key >= start && key < len;
+        s[u][i] = ok ? s[u][i] * scale : -INFINITY;
+        tmax = fmaxf(tmax, s[u][i]);
+      }
+    tmax = group4_max(tmax);
+    const float m_new = fmaxf(m, tmax);                    // finite: every tile holds a readable key
+    const float alpha = expf(m - m_new);
+    bf16x8 pb;
+    float psum = 0.f;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = (s[u][i] == -INFINITY) ? 0.f : expf(s[u][i] - m_new);
+        const bf16_t pr = (bf16_t)p;
+        pb[4 * u + i] = pr;
+        psum += (float)pr;
+      }
+    l = l * alpha + psum;
+    m = m_new;
+    // ---- values
+#pragma unroll
+    for (int r = 0; r < HDT; ++r) {
+      acc[r] *= alpha;
+      bf16x8 a = zero8;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        if (!live[u]) continue;
+        const bf16x4 v = *reinterpret_cast<const bf16x4*>(vpage[u] + (long)(16 * r + c) * page_size + 4 * g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb + 16 * u + 4 * g + i;
+          const bool ok = !edge || (key >= start && key < len);   // stale slots may hold anything
+          a[4 * u + i] = ok ? v[i] : (bf16_t)0.f;
+        }
+      }
+      acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[r], 0, 0, 0);
+    }
+  }
+
+  l = group4_sum(l);
+  if (!head_ok) return;
+  float* out = part + (((long)t * H + head) * nslices + slice) * (hd + 2);
+#pragma unroll
+  for (int r = 0; r < HDT; ++r)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[16 * r + 4 * g + i] = acc[r][i];
+  if (g == 0) {
+    out[hd] = m;
+    out[hd + 1] = l;
+  }
+}
+
+// out[t, h, :] = sum_s w_s o_s / sum_s w_s l_s with w_s = exp(m_s - max m).
+// One wave per (token, head); eight slices are read at a time.
+template <typename T>
+__global__ __launch_bounds__(64) void attn_merge_kernel(T* __restrict__ out,
+                                                        const float* __restrict__ part, int H, int hd,
+                                                        int nslices) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int stride = hd + 2;
+  const float* p = part + ((long)t * H + h) * nslices * stride;
+  float M = -INFINITY;
+  for (int s = lane; s < nslices; s += kWave) M = fmaxf(M, p[(long)s * stride + hd]);
+  M = wave_max(M);
+  float denom = 0.f;
+  for (int s = lane; s < nslices; s += kWave) {
+    const float ms = p[(long)s * stride + hd];
+    if (ms != -INFINITY) denom += expf(ms - M) * p[(long)s * stride + hd + 1];
+  }
+  denom = wave_sum(denom);
+  for (int d = lane; d < hd; d += kWave) {
+    float o = 0.f;
+    for (int s0 = 0; s0 < nslices; s0 += 8) {
+      float ms[8], os[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const bool ok = s0 + j < nslices;
+        ms[j] = ok ? p[(long)(s0 + j) * stride + hd] : -INFINITY;
+        os[j] = ok ? p[(long)(s0 + j) * stride + d] : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (ms[j] != -INFINITY) o += expf(ms[j] - M) * os[j];
+    }
+    out[((long)t * H + h) * hd + d] = from_f32<T>(o / denom);
+  }
+}
+
+template <int HDT>
+static void launch_decode(dim3 grid, hipStream_t stream, const void* q, float* part, const void* cache,
+                          const int* positions, const int* span_of_token, const int* block_table,
+                          int max_pages, int page_size, int H, int KV, int window, float scale,
+                          int head_tiles) {
+  hipLaunchKernelGGL(attn_decode_mfma_kernel<HDT>, grid, dim3(64 * kDecodeWaves), 0, stream,
+                     (const bf16_t*)q, part, (const bf16_t*)cache, positions, span_of_token,
+                     block_table, max_pages, page_size, H, KV, window, scale, head_tiles);
+}
+
+}  // namespace kllm
+
+using namespace kllm;
+
+extern "C" int kllm_attn_decode_slices(int n, int KV, int H) {
+  // Waves wanted across the chip, shared out over tokens x KV heads x head tiles.
+  const int head_tiles = (H / KV + 15) / 16;
+  long groups = (long)n * KV * head_tiles;
+  long want = 1024 / (groups > 0 ? groups : 1);
+  int wg = (int)((want + kDecodeWaves - 1) / kDecodeWaves);
+  if (wg < 1) wg = 1;
+  if (wg > 16) wg = 16;
+  return wg * kDecodeWaves;
+}
+
+extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part_floats,
+                                const void* cache, const int* positions, const int* span_of_token,
+                                const int* block_table, int max_pages, int page_size, int n, int H,
+                                int KV, int hd, int window, float scale, int nslices, int dtype,
+                                hipStream_t stream) {
+  KLLM_REQUIRE(q && out && part && cache && positions && span_of_token && block_table,
+               "attn_decode: null pointer");
+  KLLM_REQUIRE(dtype == DT_BF16, "attn_decode: bfloat16 only (float32 uses the generic kernel)");
+  KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && H % KV == 0, "attn_decode: bad heads n=%d H=%d KV=%d", n, H, KV);
+  KLLM_REQUIRE(hd % 16 == 0 && hd >= 16 && hd <= 256 && (hd <= 128 || hd == 192 || hd == 256),
+               "attn_decode: head_dim %d is not built (16..128 in steps of 16, 192, 256)", hd);
+  KLLM_REQUIRE(page_size % 16 == 0 && page_size > 0 && max_pages > 0,
+               "attn_decode: page_size %d must be a multiple of 16", page_size);
+  KLLM_REQUIRE(nslices >= kDecodeWaves && nslices % kDecodeWaves == 0 && nslices <= 1024,
+               "attn_decode: nslices %d must be a multiple of %d", nslices, kDecodeWaves);
+  KLLM_REQUIRE(window >= 0, "attn_decode: negative window");
+  KLLM_REQUIRE(part_floats >= (long)n * H * nslices * (hd + 2), "attn_decode: workspace too small");
+  const int head_tiles = (H / KV + 15) / 16;
+  KLLM_REQUIRE((long)KV * head_tiles <= 65535 && H <= 65535, "attn_decode: too many heads for the grid");
+  const dim3 grid(n, KV * head_tiles, nslices / kDecodeWaves);
+#define KLLM_DEC(HDT)                                                                             \
+  case HDT:                                                                                       \
+    launch_decode<HDT>(grid, stream, q, part, cache, positions, span_of_token, block_table,       \
+                       max_pages, page_size, H, KV, window, scale, head_tiles);                   \
+    break
+  switch (hd / 16) {
+    KLLM_DEC(1); KLLM_DEC(2); KLLM_DEC(3); KLLM_DEC(4); KLLM_DEC(5); KLLM_DEC(6); KLLM_DEC(7);
+    KLLM_DEC(8); KLLM_DEC(12); KLLM_DEC(16);
+    default: KLLM_FAIL(ERR_ARG, "attn_decode: head_dim %d is not built", hd);
+  }
+#undef KLLM_DEC
+  KLLM_CHECK_LAUNCH("attn_decode");
+  hipLaunchKernelGGL(attn_merge_kernel<bf16_t>, dim3(n, H), dim3(64), 0, stream, (bf16_t*)out, part, H,
+                     hd, nslices);
+  KLLM_CHECK_LAUNCH("attn_merge");
+  return 0;
+}

@@ -24,10 +24,26 @@ __global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ tabl
   for (int i = threadIdx.x; i < d; i += blockDim.x) dst[i] = to_f32(src[i]);
 }
 
+// Sum of the nsplit partial values p[0], p[stride], ...: eight loads are in
+// flight at a time and the order of additions is fixed.
 template <typename TIN>
 __device__ __forceinline__ float sum_splits(const TIN* __restrict__ p, int nsplit, long stride) {
-  float v = to_f32(p[0]);
-  for (int s = 1; s < nsplit; ++s) v += to_f32(p[(long)s * stride]);
+  float v = 0.f;
+  int s = 0;
+  for (; s + 8 <= nsplit; s += 8) {
+    float t[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t[j] = to_f32(p[(long)(s + j) * stride]);
+    v += ((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]));
+  }
+  if (s + 4 <= nsplit) {
+    float t[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t[j] = to_f32(p[(long)(s + j) * stride]);
+    v += (t[0] + t[1]) + (t[2] + t[3]);
+    s += 4;
+  }
+  for (; s < nsplit; ++s) v += to_f32(p[(long)s * stride]);
   return v;
 }
 
@@ -39,24 +55,34 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TIN* __restrict_
                                    TOUT* __restrict__ out, const int* __restrict__ rows, int d,
                                    float eps, int write_x) {
   __shared__ float red[16];
+  constexpr int KEEP = 8;  // elements of the row a thread keeps in registers
   const long r = blockIdx.x;
   const long src = rows ? rows[r] : r;
   float* xr = x + src * d;
   const TIN* dr = delta ? delta + src * d : nullptr;
+  float keep[KEEP];
   float ss = 0.f;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+  int it = 0;
+  for (int i = threadIdx.x; i < d; i += blockDim.x, ++it) {
     float v = xr[i];
     if (dr) v += sum_splits(dr + i, nsplit, split_stride);
     if (write_x) xr[i] = v;
+    if (it < KEEP) keep[it] = v;
     ss += v * v;
   }
   if (!out) return;
   ss = block_sum(ss, red);
   const float scale = rsqrtf(ss / (float)d + eps);
   TOUT* orow = out + r * d;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    float v = xr[i];  // already the sum when write_x (same thread wrote it)
-    if (dr && !write_x) v += sum_splits(dr + i, nsplit, split_stride);
+  it = 0;
+  for (int i = threadIdx.x; i < d; i += blockDim.x, ++it) {
+    float v;
+    if (it < KEEP) {
+      v = keep[it];
+    } else {
+      v = xr[i];  // already the sum when write_x (same thread wrote it)
+      if (dr && !write_x) v += sum_splits(dr + i, nsplit, split_stride);
+    }
     orow[i] = from_f32<TOUT>(v * scale * w[i]);
   }
 }
@@ -93,37 +119,35 @@ __global__ void rope_append_kernel(const TIN* __restrict__ qkv, int nsplit, long
   const TIN* in = qkv + t * row;
   const float* c = cos_t ? cos_t + t * half : nullptr;
   const float* s = sin_t ? sin_t + t * half : nullptr;
-
-  for (int idx = threadIdx.x; idx < H * half; idx += blockDim.x) {
-    const int h = idx / half, j = idx % half;
-    const float a = sum_splits(in + h * hd + j, nsplit, split_stride);
-    const float b = sum_splits(in + h * hd + j + half, nsplit, split_stride);
-    const float cc = c ? c[j] : 1.f, sn = s ? s[j] : 0.f;
-    T* o = q_out + t * qd + h * hd;
-    o[j] = from_f32<T>(a * cc - b * sn);
-    o[j + half] = from_f32<T>(b * cc + a * sn);
-  }
-  if (!cache) return;
-
-  const int pos = positions[t];
-  const int page = block_table[(long)span_of_token[t] * max_pages + pos / page_size];
-  const int slot = pos % page_size;
+  // Items of a token: H*half query pairs, KV*half key pairs, KV*hd values.
+  const int q_items = H * half, k_items = cache ? KV * half : 0;
+  const int items = q_items + k_items + kvd;
   const long block = (long)page_size * hd;  // one (page, k|v, head) block
-  T* kpage = cache + ((long)page * 2 + 0) * KV * block;
-  T* vpage = cache + ((long)page * 2 + 1) * KV * block;
-  for (int idx = threadIdx.x; idx < KV * half; idx += blockDim.x) {
-    const int h = idx / half, j = idx % half;
-    const float a = sum_splits(in + qd + h * hd + j, nsplit, split_stride);
-    const float b = sum_splits(in + qd + h * hd + j + half, nsplit, split_stride);
-    const float cc = c ? c[j] : 1.f, sn = s ? s[j] : 0.f;
-    T* o = kpage + h * block + (long)slot * hd;
-    o[j] = from_f32<T>(a * cc - b * sn);
-    o[j + half] = from_f32<T>(b * cc + a * sn);
+  int page = 0, slot = 0;
+  if (cache) {
+    const int pos = positions[t];
+    page = block_table[(long)span_of_token[t] * max_pages + pos / page_size];
+    slot = pos % page_size;
   }
-  for (int idx = threadIdx.x; idx < kvd; idx += blockDim.x) {
-    const int h = idx / hd, j = idx % hd;
-    const float v = sum_splits(in + qd + kvd + idx, nsplit, split_stride);
-    vpage[h * block + (long)j * page_size + slot] = from_f32<T>(v);
+  for (int item = blockIdx.y * blockDim.x + threadIdx.x; item < items; item += gridDim.y * blockDim.x) {
+    if (item < q_items + k_items) {
+      const bool is_q = item < q_items;
+      const int idx = is_q ? item : item - q_items;
+      const int h = idx / half, j = idx % half;
+      const TIN* src = in + (is_q ? 0 : qd) + h * hd + j;
+      const float a = sum_splits(src, nsplit, split_stride);
+      const float b = sum_splits(src + half, nsplit, split_stride);
+      const float cc = c ? c[j] : 1.f, sn = s ? s[j] : 0.f;
+      T* o = is_q ? q_out + t * qd + h * hd
+                  : cache + (((long)page * 2 + 0) * KV + h) * block + (long)slot * hd;
+      o[j] = from_f32<T>(a * cc - b * sn);
+      o[j + half] = from_f32<T>(b * cc + a * sn);
+    } else {
+      const int idx = item - q_items - k_items;
+      const int h = idx / hd, j = idx % hd;
+      const float v = sum_splits(in + qd + kvd + idx, nsplit, split_stride);
+      cache[(((long)page * 2 + 1) * KV + h) * block + (long)j * page_size + slot] = from_f32<T>(v);
+    }
   }
 }
 
@@ -144,9 +168,34 @@ __global__ void silu_mul_kernel(const TIN* __restrict__ gu, int nsplit, long spl
   }
 }
 
+// out[i] = sum over splits of in[s][i]
+template <typename TOUT>
+__global__ void sum_splits_kernel(const float* __restrict__ in, int nsplit, long count,
+                                  TOUT* __restrict__ out) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < count;
+       i += (long)gridDim.x * blockDim.x)
+    out[i] = from_f32<TOUT>(sum_splits(in + i, nsplit, count));
+}
+
 }  // namespace kllm
 
 using namespace kllm;
+
+extern "C" int kllm_sum_splits(const float* in, int nsplit, long count, void* out, int out_dtype,
+                               hipStream_t stream) {
+  KLLM_REQUIRE(in && out && nsplit >= 1 && count > 0, "sum_splits: bad arguments");
+  KLLM_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "sum_splits: unknown dtype");
+  int grid = ceil_div(count, kThreads);
+  if (grid > 8192) grid = 8192;
+  if (out_dtype == DT_F32)
+    hipLaunchKernelGGL(sum_splits_kernel<float>, dim3(grid), dim3(kThreads), 0, stream, in, nsplit, count,
+                       (float*)out);
+  else
+    hipLaunchKernelGGL(sum_splits_kernel<bf16_t>, dim3(grid), dim3(kThreads), 0, stream, in, nsplit, count,
+                       (bf16_t*)out);
+  KLLM_CHECK_LAUNCH("sum_splits");
+  return 0;
+}
 
 extern "C" int kllm_embed(float* out, const void* table, const int* ids, int n, int d, int vocab,
                           int dtype, hipStream_t stream) {
@@ -167,12 +216,14 @@ template <typename TIN>
 static int launch_add_rmsnorm(float* x, const void* delta, int nsplit, long split_stride,
                               const float* w, void* out, int out_dtype, const int* rows, int n, int d,
                               float eps, int write_x, hipStream_t stream) {
+  // Few rows: more threads per row, so that a row's loads are all in flight.
+  const int threads = (n <= 256 && d > 1024) ? 1024 : kThreads;
   if (out_dtype == DT_F32)
-    hipLaunchKernelGGL((add_rmsnorm_kernel<TIN, float>), dim3(n), dim3(kThreads), 0, stream, x,
+    hipLaunchKernelGGL((add_rmsnorm_kernel<TIN, float>), dim3(n), dim3(threads), 0, stream, x,
                        (const TIN*)delta, nsplit, split_stride, w, (float*)out, rows, d, eps,
                        write_x);
   else
-    hipLaunchKernelGGL((add_rmsnorm_kernel<TIN, bf16_t>), dim3(n), dim3(kThreads), 0, stream, x,
+    hipLaunchKernelGGL((add_rmsnorm_kernel<TIN, bf16_t>), dim3(n), dim3(threads), 0, stream, x,
                        (const TIN*)delta, nsplit, split_stride, w, (bf16_t*)out, rows, d, eps,
                        write_x);
   KLLM_CHECK_LAUNCH("add_rmsnorm");
@@ -218,7 +269,10 @@ static int launch_rope_append(const void* qkv, int nsplit, long split_stride, vo
                               const int* positions, const int* span_of_token,
                               const int* block_table, int max_pages, int page_size, int n, int H,
                               int KV, int hd, hipStream_t stream) {
-  hipLaunchKernelGGL((rope_append_kernel<TIN, T>), dim3(n), dim3(kThreads), 0, stream,
+  const int items = H * (hd / 2) + (cache ? KV * (hd / 2) + KV * hd : 0);
+  int chunks = ceil_div(items, kThreads);
+  if ((long)n * chunks > 16384) chunks = ceil_div(16384, n);   // many tokens: fewer, longer workgroups
+  hipLaunchKernelGGL((rope_append_kernel<TIN, T>), dim3(n, chunks), dim3(kThreads), 0, stream,
                      (const TIN*)qkv, nsplit, split_stride, (T*)q_out, cos_t, sin_t, (T*)cache,
                      positions, span_of_token, block_table, max_pages, page_size, H, KV, hd);
   KLLM_CHECK_LAUNCH("rope_append");

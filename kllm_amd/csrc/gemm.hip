@@ -203,74 +203,84 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
 }
 
 // ------------------------------------------------------------------ bf16 MFMA skinny
-// Up to 16*NT rows of X.  A wave owns 16 rows of W over one slice of K and
-// streams them from memory; MFMA 16x16x32 with A = W tile, B = X^T, so
-// D[w row][x row].  Lane l holds A[l%16][8*(l/16) .. +8], B[8*(l/16) .. +8][l%16]
-// and D[4*(l/16) + i][l%16] for i = 0..3.
+// Up to 16*NT rows of X (decode batches).  A workgroup takes 64 rows of W and
+// one slice of K: it first puts its slice of X into LDS, then each of its four
+// waves streams 16 rows of W straight from memory, eight 16-byte loads ahead,
+// and multiplies them with X from LDS.  MFMA 16x16x32 with A = W tile,
+// B = X^T, so D[w row][x row]: lane l (g = l/16, c = l%16) holds
+// A[c][8g..8g+7], B[8g..8g+7][c], D[4g+i][c].
+constexpr int SK_SLICE_MAX = 512;             // K per workgroup at most
+constexpr int SK_LD = SK_SLICE_MAX + 8;       // LDS row stride (elements): 16-byte reads conflict-free
+constexpr int SK_AHEAD = 8;                   // W loads in flight per lane
+
 template <int NT>
 __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ X,
                                                                const bf16_t* __restrict__ W,
                                                                float* __restrict__ Y, int n, int m,
                                                                int k, int kslice) {
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const long tile = (long)blockIdx.x * 4 + wave;
-  const long m0 = tile * 16;
-  if (m0 >= m) return;
+  extern __shared__ __attribute__((aligned(16))) bf16_t xs[];   // [NT*16][SK_LD]
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int g = lane / 16, c = lane % 16;
   const int kbeg = blockIdx.y * kslice;
   const int kend = min(k, kbeg + kslice);
+  const int klen = kend - kbeg;                                  // a multiple of 8
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  const long wrow = m0 + lane % 16;
-  const bool wok = wrow < m;
-  const bf16_t* wp = W + (wok ? wrow : 0) * k + (lane / 16) * 8;
-  const bf16_t* xp[NT];
-  bool xok[NT];
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int xr = t * 16 + lane % 16;
-    xok[t] = xr < n;
-    xp[t] = X + (long)(xok[t] ? xr : 0) * k + (lane / 16) * 8;
+  const int chunks = (klen + 7) / 8;
+  for (int idx = tid; idx < NT * 16 * chunks; idx += 256) {
+    const int r = idx / chunks, ch = idx % chunks;
+    const bf16x8 v = (r < n) ? *reinterpret_cast<const bf16x8*>(X + (long)r * k + kbeg + ch * 8) : zero;
+    *reinterpret_cast<bf16x8*>(&xs[r * SK_LD + ch * 8]) = v;
   }
+  __syncthreads();
+
+  const long m0 = ((long)blockIdx.x * 4 + wave) * 16;
+  if (m0 >= m) return;
+  const long wrow = m0 + c;
+  const bool wok = wrow < m;
+  const bf16_t* wp = W + (wok ? wrow : 0) * k + kbeg + 8 * g;
+  const int steps = (klen + 31) / 32;
 
   floatx4 acc[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  constexpr int UNROLL = 4;
-  int k0 = kbeg;
-  for (; k0 + 32 * UNROLL <= kend; k0 += 32 * UNROLL) {
-    bf16x8 a[UNROLL];
+  auto load_a = [&](int s) -> bf16x8 {
+    return (wok && s < steps && 32 * s + 8 * g < klen) ? *reinterpret_cast<const bf16x8*>(wp + 32 * s)
+                                                        : zero;
+  };
+  bf16x8 cur[SK_AHEAD], nxt[SK_AHEAD];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
-      a[u] = wok ? *reinterpret_cast<const bf16x8*>(wp + k0 + 32 * u) : zero;
+  for (int u = 0; u < SK_AHEAD; ++u) cur[u] = load_a(u);
+  for (int s0 = 0; s0 < steps; s0 += SK_AHEAD) {
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
+    for (int u = 0; u < SK_AHEAD; ++u) nxt[u] = load_a(s0 + SK_AHEAD + u);
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        const bf16x8 b = xok[t] ? *reinterpret_cast<const bf16x8*>(xp[t] + k0 + 32 * u) : zero;
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b, acc[t], 0, 0, 0);
+    for (int u = 0; u < SK_AHEAD; ++u) {
+      const int s1 = s0 + u;
+      if (s1 < steps) {
+        const bool kin = 32 * s1 + 8 * g < klen;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          const bf16x8 b = kin ? *reinterpret_cast<const bf16x8*>(&xs[(t * 16 + c) * SK_LD + 32 * s1 + 8 * g])
+                               : zero;
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u], b, acc[t], 0, 0, 0);
+        }
       }
     }
-  }
-  for (; k0 < kend; k0 += 32) {
-    const bool kin = k0 + (lane / 16) * 8 < kend;  // K is a multiple of 8
-    const bf16x8 a = (wok && kin) ? *reinterpret_cast<const bf16x8*>(wp + k0) : zero;
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const bf16x8 b = (xok[t] && kin) ? *reinterpret_cast<const bf16x8*>(xp[t] + k0) : zero;
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
-    }
+    for (int u = 0; u < SK_AHEAD; ++u) cur[u] = nxt[u];
   }
 
   float* out = Y + (long)blockIdx.y * n * m;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const int xr = t * 16 + lane % 16;
+    const int xr = t * 16 + c;
     if (xr >= n) continue;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const long c = m0 + 4 * (lane / 16) + i;
-      if (c < m) out[(long)xr * m + c] = acc[t][i];
+      const long col = m0 + 4 * g + i;
+      if (col < m) out[(long)xr * m + col] = acc[t][i];
     }
   }
 }
@@ -322,11 +332,84 @@ __global__ __launch_bounds__(256) void gemv_kernel(const T* __restrict__ X, cons
   }
 }
 
+// ------------------------------------------------------------------ streaming gemv
+// Up to 4 rows of X.  A wave takes R rows of W and one slice of K and has all
+// of a slice's loads in flight at once: U steps of 64 lanes x 16 bytes per row.
+template <typename T, int NT, int R, int U>
+__global__ __launch_bounds__(256) void gemv_stream_kernel(const T* __restrict__ X,
+                                                          const T* __restrict__ W,
+                                                          float* __restrict__ Y, int n, int m, int k,
+                                                          int kslice) {
+  constexpr int V = 16 / sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const long row0 = ((long)blockIdx.x * 4 + wave) * R;
+  if (row0 >= m) return;
+  const int kbeg = blockIdx.y * kslice;
+  const int kend = min(k, kbeg + kslice);
+  float acc[R][NT];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[r][t] = 0.f;
+
+  for (int k0 = kbeg + lane * V; k0 < kend; k0 += U * kWave * V) {
+    vec_t wv[U][R], xv[U][NT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kk = k0 + u * kWave * V;
+      const bool kin = kk < kend;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const bool ok = kin && row0 + r < m;
+        wv[u][r] = ok ? *reinterpret_cast<const vec_t*>(W + (row0 + r) * k + kk) : vec_t{};
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const bool ok = kin && t < n;
+        xv[u][t] = ok ? *reinterpret_cast<const vec_t*>(X + (long)t * k + kk) : vec_t{};
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int e = 0; e < V; ++e)
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const float wf = to_f32(wv[u][r][e]);
+#pragma unroll
+          for (int t = 0; t < NT; ++t) acc[r][t] = fmaf(wf, to_f32(xv[u][t][e]), acc[r][t]);
+        }
+  }
+  float* out = Y + (long)blockIdx.y * n * m;
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const float sum = wave_sum(acc[r][t]);
+      if (lane == 0 && t < n && row0 + r < m) out[(long)t * m + row0 + r] = sum;
+    }
+}
+
 }  // namespace kllm
 
 using namespace kllm;
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// The 64-row variant of the skinny kernel stages 66,560 bytes of LDS, above the
+// default limit of a launch; raise it once per kernel.
+template <int NT>
+static int allow_skinny_lds() {
+  static int done = 0;
+  if (done) return 0;
+  hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_skinny_kernel<NT>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     NT * 16 * SK_LD * (int)sizeof(bf16_t));
+  if (e != hipSuccess) KLLM_FAIL((int)e, "gemm skinny: cannot raise the LDS limit: %s", hipGetErrorString(e));
+  done = 1;
+  return 0;
+}
 
 extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, int k, int dtype,
                          int out_dtype, int algo, int nsplit, hipStream_t stream) {
@@ -388,21 +471,26 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
     KLLM_REQUIRE(n <= 64, "gemm skinny: n=%d exceeds 64", n);
     KLLM_REQUIRE(k % 8 == 0 && aligned16(x) && aligned16(w),
                  "gemm skinny: K=%d must be a multiple of 8 and the operands 16-byte aligned", k);
-    int kslice = ceil_div(ceil_div(k, nsplit), 32) * 32;
+    const int kslice = ceil_div(ceil_div(k, nsplit), 32) * 32;
+    KLLM_REQUIRE(kslice <= SK_SLICE_MAX, "gemm skinny: K=%d in %d slices exceeds %d per slice", k,
+                 nsplit, SK_SLICE_MAX);
     KLLM_REQUIRE((long)kslice * (nsplit - 1) < k, "gemm skinny: nsplit %d leaves an empty slice of K=%d",
                  nsplit, k);
     const dim3 grid(ceil_div(m, 64), nsplit);
     const bf16_t *xp = (const bf16_t*)x, *wp = (const bf16_t*)w;
     float* yp = (float*)y;
     const int nt = ceil_div(n, 16);
-    if (nt == 1)
-      hipLaunchKernelGGL((gemm_bf16_skinny_kernel<1>), grid, dim3(256), 0, stream, xp, wp, yp, n, m, k, kslice);
-    else if (nt == 2)
-      hipLaunchKernelGGL((gemm_bf16_skinny_kernel<2>), grid, dim3(256), 0, stream, xp, wp, yp, n, m, k, kslice);
-    else if (nt == 3)
-      hipLaunchKernelGGL((gemm_bf16_skinny_kernel<3>), grid, dim3(256), 0, stream, xp, wp, yp, n, m, k, kslice);
-    else
-      hipLaunchKernelGGL((gemm_bf16_skinny_kernel<4>), grid, dim3(256), 0, stream, xp, wp, yp, n, m, k, kslice);
+    const size_t lds = (size_t)nt * 16 * SK_LD * sizeof(bf16_t);
+#define KLLM_SK(NT)                                                                              \
+  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<NT>), grid, dim3(256), lds, stream, xp, wp, yp, n, m, k, kslice)
+    int rc = nt == 1 ? allow_skinny_lds<1>() : nt == 2 ? allow_skinny_lds<2>()
+             : nt == 3 ? allow_skinny_lds<3>() : allow_skinny_lds<4>();
+    if (rc) return rc;
+    if (nt == 1) KLLM_SK(1);
+    else if (nt == 2) KLLM_SK(2);
+    else if (nt == 3) KLLM_SK(3);
+    else KLLM_SK(4);
+#undef KLLM_SK
     KLLM_CHECK_LAUNCH("gemm skinny");
     return 0;
   }
@@ -413,6 +501,27 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
     const int vlen = dtype == DT_F32 ? 4 : 8;
     const int vec_ok = (k % vlen == 0) && aligned16(x) && aligned16(w);
     const int unit = kWave * vlen;
+    if (vec_ok && n <= 4) {
+      constexpr int R = 2, U = 4;
+      const int ks = ceil_div(ceil_div(k, nsplit), unit) * unit;
+      KLLM_REQUIRE((long)ks * (nsplit - 1) < k, "gemv: nsplit %d leaves an empty slice of K=%d", nsplit, k);
+      const dim3 sgrid(ceil_div(m, 4 * R), nsplit);
+#define KLLM_GS(T, NT)                                                                           \
+  hipLaunchKernelGGL((gemv_stream_kernel<T, NT, R, U>), sgrid, dim3(256), 0, stream, (const T*)x, \
+                     (const T*)w, (float*)y, n, m, k, ks)
+      if (dtype == DT_F32) {
+        if (n == 1) KLLM_GS(float, 1);
+        else if (n == 2) KLLM_GS(float, 2);
+        else KLLM_GS(float, 4);
+      } else {
+        if (n == 1) KLLM_GS(bf16_t, 1);
+        else if (n == 2) KLLM_GS(bf16_t, 2);
+        else KLLM_GS(bf16_t, 4);
+      }
+#undef KLLM_GS
+      KLLM_CHECK_LAUNCH("gemv stream");
+      return 0;
+    }
     int kslice = ceil_div(ceil_div(k, nsplit), unit) * unit;
     KLLM_REQUIRE((long)kslice * (nsplit - 1) < k, "gemv: nsplit %d leaves an empty slice of K=%d",
                  nsplit, k);

@@ -60,6 +60,10 @@ int kllm_rope_append(const void* qkv, int in_dtype, int nsplit, long split_strid
 int kllm_silu_mul(const void* gu, int in_dtype, int nsplit, long split_stride, void* out,
                   int out_dtype, int n, int f, hipStream_t stream);
 
+/* out[count] = sum over s of in[s][count], rounded to out_dtype. */
+int kllm_sum_splits(const float* in, int nsplit, long count, void* out, int out_dtype,
+                    hipStream_t stream);
+
 /* y[nsplit][n][m] = x[n][k] . w[m][k]^T, 32-bit accumulation. */
 int kllm_gemm(const void* x, const void* w, void* y, int n, int m, int k, int dtype, int out_dtype,
               int algo, int nsplit, hipStream_t stream);
@@ -69,6 +73,16 @@ int kllm_attn_generic(const void* q, void* out, const void* cache, const int* po
                       const int* span_of_token, const int* block_table, int max_pages,
                       int page_size, int n, int H, int KV, int hd, int window, float scale,
                       int dtype, hipStream_t stream);
+
+/* Decode attention on the matrix cores (bfloat16): every token's keys are cut
+ * into `nslices` slices (a multiple of 4) that run side by side; `part` is
+ * float32 scratch of n*H*nslices*(hd+2) elements.  kllm_attn_decode_slices
+ * proposes nslices for a batch. */
+int kllm_attn_decode_slices(int n, int KV, int H);
+int kllm_attn_decode(const void* q, void* out, float* part, long part_floats, const void* cache,
+                     const int* positions, const int* span_of_token, const int* block_table,
+                     int max_pages, int page_size, int n, int H, int KV, int hd, int window,
+                     float scale, int nslices, int dtype, hipStream_t stream);
 
 /* out[r] = sampled index of logits[r][:]; temperature/uniform null: greedy. */
 int kllm_sample(int* out, const float* logits, const float* temperature, const float* uniform,

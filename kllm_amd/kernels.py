@@ -81,8 +81,11 @@ def _declare(lib):
         "kllm_rope_append": [P, I, I, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "kllm_silu_mul": [P, I, I, L, P, I, I, I, P],
         "kllm_gemm": [P, P, P, I, I, I, I, I, I, I, P],
+        "kllm_sum_splits": [P, I, L, P, I, P],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
+        "kllm_attn_decode_slices": [I, I, I],
+        "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -237,6 +240,16 @@ def gemm(x, w, y, algo, nsplit=1):
         dtype_code(y.dtype), algo, nsplit, _stream()), "gemm")
 
 
+def sum_splits(parts, out):
+    """out [n, m] = parts [nsplit, n, m] summed over the first axis."""
+    nsplit = parts.shape[0]
+    if tuple(parts.shape[1:]) != tuple(out.shape):
+        raise KernelError("sum_splits: shapes do not fit")
+    _check(library().kllm_sum_splits(_ptr(parts, "sum_splits in", torch.float32), nsplit, out.numel(),
+                                     _ptr(out, "sum_splits out"), dtype_code(out.dtype), _stream()),
+           "sum_splits")
+
+
 def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size, n_heads,
                  n_kv_heads, head_dim, window, scale):
     n = q.shape[0]
@@ -254,6 +267,32 @@ def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size, n,
         n_heads, n_kv_heads, head_dim, int(window), float(scale), dtype_code(q.dtype), _stream()),
         "attn_generic")
+
+
+DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
+
+
+def attn_decode_slices(n, n_kv_heads, n_heads) -> int:
+    return library().kllm_attn_decode_slices(n, n_kv_heads, n_heads)
+
+
+def attn_decode(q, out, part, cache, positions, span_of_token, block_table, page_size, n_heads,
+                n_kv_heads, head_dim, window, scale, nslices):
+    n = q.shape[0]
+    if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape)
+            or q.dtype != cache.dtype or out.dtype != q.dtype):
+        raise KernelError("attn_decode: q/out shapes or dtypes do not fit")
+    if tuple(cache.shape[1:]) != (2, n_kv_heads, page_size * head_dim):
+        raise KernelError(f"attn_decode: cache {tuple(cache.shape)} does not fit")
+    if positions.numel() < n or span_of_token.numel() < n:
+        raise KernelError("attn_decode: index arrays are too short")
+    _check(library().kllm_attn_decode(
+        _ptr(q, "attn q"), _ptr(out, "attn out"), _ptr(part, "attn part", torch.float32),
+        part.numel(), _ptr(cache, "attn cache"), _ptr(positions, "attn positions", torch.int32),
+        _ptr(span_of_token, "attn span_of_token", torch.int32),
+        _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size, n,
+        n_heads, n_kv_heads, head_dim, int(window), float(scale), int(nslices), dtype_code(q.dtype),
+        _stream()), "attn_decode")
 
 
 def sample(out, logits, temperature=None, uniform=None):

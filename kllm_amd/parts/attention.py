@@ -85,6 +85,18 @@ class CausalSelfAttention(Part):
         return linear(ctx, out, self.w_o, "attn.proj")
 
     def attend(self, ctx, q, out, cache):
+        """Choose the attention kernel by dtype and by the spans' lengths."""
+        mode = self.runtime.options.get("attention", "auto")
+        fast = (mode != "generic" and q.dtype == torch.bfloat16 and cache.page_size % 16 == 0
+                and self.head_dim in K.DECODE_HEAD_DIMS)
+        if fast and ctx.max_span_len <= 4:
+            n = q.shape[0]
+            nslices = K.attn_decode_slices(n, self.kv_heads, self.heads)
+            part = ctx.buf("attn.part", (n * self.heads * nslices * (self.head_dim + 2),), torch.float32)
+            K.attn_decode(q, out, part, cache.pages, ctx.positions, ctx.span_of_token,
+                          cache.block_table, cache.page_size, self.heads, self.kv_heads,
+                          self.head_dim, self.window, self.scale, nslices)
+            return
         K.attn_generic(q, out, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                        cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
                        self.scale)

@@ -56,5 +56,4 @@ class LinearHead(Part):
         self.weight = weights[self.tensor_name("weight")]
 
     def forward(self, ctx, xn_rows):
-        logits = linear(ctx, xn_rows, self.weight, "logits", split=False)
-        return logits[0]
+        return linear(ctx, xn_rows, self.weight, "logits", split=False)

@@ -6,7 +6,7 @@ rotary + append, SiLU gate); with the compute dtype as result it returns
 [n, m].  Which kernel runs depends only on the dtype and on n:
 
   float32   n <= 8: gemv      else: tiled FMA (true 32-bit)
-  bfloat16  n <= 8: gemv      n <= 64: MFMA skinny      else: MFMA tiles,
+  bfloat16  n <= 4: gemv      n <= 64: MFMA skinny      else: MFMA tiles,
             or the vendor library (torch.matmul) when the engine option
             ``gemm`` is "library" -- the reference uses its vendor library for
             every product (backend/model.cu:494-503)
@@ -21,17 +21,28 @@ import torch
 
 from .. import kernels as K
 
-TARGET_WAVES = 2048
+def _gemv_split(dtype, n, m, k):
+    """Slices of K for the streaming gemv: a wave covers two rows and up to
+    2048 (bfloat16) or 1024 (float32) of K with all loads in flight; K is cut
+    unless the rows alone already give the chip enough waves."""
+    per = 2048 if dtype == torch.bfloat16 else 1024
+    if m // 2 >= 4096:
+        return 1
+    return int(max(1, min(16, -(-k // per))))
 
 
-def _split_for(n, m, k, rows_per_wave, min_slice):
-    """How many slices of K: enough waves to fill the chip, but partial sums
-    must stay small beside the weights they come from."""
-    tiles = -(-m // rows_per_wave)
-    by_fill = max(1, TARGET_WAVES // max(tiles, 1))
-    by_traffic = max(1, k // (16 * n))
-    by_slice = max(1, k // min_slice)
-    return int(max(1, min(by_fill, by_traffic, by_slice, 16)))
+def _skinny_split(n, m, k):
+    """Slices of K for the skinny MFMA kernel: at most 512 of K per workgroup
+    (its LDS stage); more slices while the chip is not full, as long as a slice
+    keeps 128 of K and the partial sums stay small beside the weights."""
+    nsplit = -(-k // 512)
+    wgs = -(-m // 64)
+    most = max(nsplit, k // (16 * n))
+    while wgs * nsplit < 512 and nsplit * 2 <= most and k // (nsplit * 2) >= 128:
+        nsplit *= 2
+    while (-(-(-(-k // nsplit)) // 32) * 32) * (nsplit - 1) >= k:   # no empty slice
+        nsplit -= 1
+    return int(nsplit)
 
 
 def choose(dtype, n, m, k, options=None):
@@ -40,46 +51,50 @@ def choose(dtype, n, m, k, options=None):
     forced = options.get("gemm_algo")
     if forced is not None:
         return forced, 1
-    if n <= 8:
-        return K.GEMM_GEMV, _split_for(n, m, k, 1, 1024)
+    if n <= 4 or (n <= 8 and dtype == torch.float32):
+        return K.GEMM_GEMV, _gemv_split(dtype, n, m, k)
     if dtype == torch.float32:
         return K.GEMM_TILED_F32, 1
     if k % 8 != 0:
-        return K.GEMM_PLAIN, 1
+        return (K.GEMM_GEMV, 1) if n <= 8 else (K.GEMM_PLAIN, 1)
     if n <= 64:
-        return K.GEMM_SKINNY_BF16, _split_for(n, m, k, 16, 128)
+        return K.GEMM_SKINNY_BF16, _skinny_split(n, m, k)
     if options.get("gemm") == "library":
         return "library", 1
     return K.GEMM_MFMA_BF16, 1
 
 
 def linear(ctx, x, w, tag, out_dtype=torch.float32, split=True):
-    """x [n, k] . w [m, k]^T.  float32 result: [nsplit, n, m]; else [n, m]."""
+    """x [n, k] . w [m, k]^T.  With a float32 result and ``split``: partial
+    sums [nsplit, n, m] for a consumer that adds them; otherwise one [n, m]
+    tensor of ``out_dtype``."""
     n, k = x.shape
     m = w.shape[0]
     rt = ctx.runtime
     algo, nsplit = choose(x.dtype, n, m, k, rt.options)
-    if not split or out_dtype != torch.float32:
-        nsplit = 1
+    whole = not split or out_dtype != torch.float32
     if algo == "library":
         y = ctx.buf(tag, (n, m), x.dtype)
         torch.matmul(x, w.t(), out=y)
         if out_dtype == torch.float32:
             y32 = ctx.buf(tag + ".f32", (1, n, m), torch.float32)
             y32[0].copy_(y)
-            return y32
+            return y32[0] if whole else y32
         return y
-    if out_dtype == torch.float32:
-        y = ctx.buf(tag, (nsplit, n, m), torch.float32)
-        K.gemm(x, w, y, algo, nsplit)
+    if algo == K.GEMM_MFMA_BF16 or algo == K.GEMM_PLAIN:      # write either dtype themselves
+        if whole:
+            y = ctx.buf(tag, (n, m), out_dtype)
+            K.gemm(x, w, y, algo, 1)
+            return y
+        y = ctx.buf(tag, (1, n, m), torch.float32)
+        K.gemm(x, w, y, algo, 1)
         return y
-    if algo in (K.GEMM_GEMV, K.GEMM_SKINNY_BF16) or (algo == K.GEMM_TILED_F32):
-        # These write float32 only; round once afterwards.
-        y32 = ctx.buf(tag + ".f32", (1, n, m), torch.float32)
-        K.gemm(x, w, y32, algo, 1)
-        y = ctx.buf(tag, (n, m), out_dtype)
-        y.copy_(y32[0])
-        return y
-    y = ctx.buf(tag, (n, m), out_dtype)
-    K.gemm(x, w, y, algo, 1)
+    parts = ctx.buf(tag, (nsplit, n, m), torch.float32)       # float32 partial sums only
+    K.gemm(x, w, parts, algo, nsplit)
+    if not whole:
+        return parts
+    if nsplit == 1 and out_dtype == torch.float32:
+        return parts[0]
+    y = ctx.buf(tag + ".sum", (n, m), out_dtype)
+    K.sum_splits(parts, y)
     return y

@@ -178,7 +178,8 @@ def test_gemm_kernels_against_plain(n, m, k, dtype):
     elif k % 8 == 0:
         algos.append((k_.GEMM_MFMA_BF16, 1))
         if n <= 64:
-            algos += [(k_.GEMM_SKINNY_BF16, 1)] + ([(k_.GEMM_SKINNY_BF16, 3)] if k >= 256 else [])
+            base = -(-k // 512)
+            algos += [(k_.GEMM_SKINNY_BF16, base)] + ([(k_.GEMM_SKINNY_BF16, base + 2)] if k >= 256 else [])
     if n <= 8:
         algos += [(k_.GEMM_GEMV, 1)] + ([(k_.GEMM_GEMV, 2)] if k >= 2048 else [])
     for algo, ns in algos:
@@ -212,6 +213,13 @@ def test_linear_chooses_a_kernel_for_every_size():
     assert choose(torch.float32, 100, 64, 64)[0] == k_.GEMM_TILED_F32
     assert choose(torch.bfloat16, 40, 64, 64)[0] == k_.GEMM_SKINNY_BF16
     assert choose(torch.bfloat16, 40, 64, 60)[0] == k_.GEMM_PLAIN          # K not a multiple of 8
+    assert choose(torch.bfloat16, 8, 2560, 2048) == (k_.GEMM_SKINNY_BF16, 16)
+    assert choose(torch.bfloat16, 64, 2048, 5632) == (k_.GEMM_SKINNY_BF16, 11)
+    assert choose(torch.bfloat16, 3, 32000, 2048) == (k_.GEMM_GEMV, 1)
+    for n, m, k in [(5, 100, 72), (64, 2048, 5632), (33, 96, 176), (9, 320, 520), (20, 64, 4104)]:
+        ns = choose(torch.bfloat16, n, m, k)[1]
+        kslice = -(-(-(-k // ns)) // 32) * 32
+        assert kslice <= 512 and kslice * (ns - 1) < k, (n, m, k, ns)
     assert choose(torch.bfloat16, 400, 64, 64)[0] == k_.GEMM_MFMA_BF16
     assert choose(torch.bfloat16, 400, 64, 64, {"gemm": "library"})[0] == "library"
     a, ns = choose(torch.bfloat16, 1, 2048, 5632)
@@ -259,6 +267,22 @@ def attention_case(H, KV, hd, ps, dtype, window, spans, seed=0):
                 window=window, scale=1.0 / math.sqrt(hd), tables=tables, lens=lens)
 
 
+def run_attention(kernel, q, cache, pos, sot, bt, ps, H, KV, hd, window, scale, nslices=None):
+    out = torch.full_like(q, float("nan"))
+    if kernel == "generic":
+        K().attn_generic(q, out, cache, pos, sot, bt, ps, H, KV, hd, window, scale)
+    else:
+        n = q.shape[0]
+        ns = nslices or K().attn_decode_slices(n, KV, H)
+        part = torch.full((n * H * ns * (hd + 2),), float("nan"), device=DEV)
+        K().attn_decode(q, out, part, cache, pos, sot, bt, ps, H, KV, hd, window, scale, ns)
+    return out
+
+
+def kernels_for(dtype):
+    return ["generic", "decode"] if dtype == torch.bfloat16 else ["generic"]
+
+
 ATTN_SHAPES = [(4, 2, 16, 16), (3, 1, 32, 16), (5, 5, 48, 16), (8, 2, 64, 16), (6, 3, 80, 32),
                (2, 1, 128, 16), (2, 2, 256, 16), (32, 4, 64, 64)]
 
@@ -270,11 +294,22 @@ def test_attention_generic(H, KV, hd, ps, dtype, window):
     # a whole prompt, a portion behind 300 cached keys, a decode token at a
     # page's first slot, one at its last, and a sequence's very first token
     c = attention_case(H, KV, hd, ps, dtype, window, [(0, 45), (300, 9), (ps * 3, 1), (ps * 2 - 1, 1), (0, 1)])
-    out = torch.empty_like(c["q"])
-    K().attn_generic(c["q"], out, c["cache"], c["pos"], c["sot"], c["bt"], ps, H, KV, hd, window, c["scale"])
-    err = (out.cpu().double() - c["want"]).abs().max()
+    for kernel in kernels_for(dtype):
+        out = run_attention(kernel, c["q"], c["cache"], c["pos"], c["sot"], c["bt"], ps, H, KV, hd, window, c["scale"])
+        err = (out.cpu().double() - c["want"]).abs().max()
+        assert torch.isfinite(out).all(), kernel
+        assert err < (2e-5 if dtype == torch.float32 else 2e-2), (kernel, float(err))
+
+
+@pytest.mark.parametrize("H,KV,hd,ps", [(40, 2, 32, 16), (17, 1, 64, 16), (12, 4, 192, 16), (8, 8, 112, 48)])
+@pytest.mark.parametrize("nslices", [4, 8, 64])
+def test_attention_decode_many_heads_and_slices(H, KV, hd, ps, nslices):
+    """More than 16 query heads per KV head (several head tiles), odd groups,
+    more slices than there are keys."""
+    c = attention_case(H, KV, hd, ps, torch.bfloat16, 0, [(700, 1), (ps - 1, 1), (0, 1), (33, 2)], seed=3)
+    out = run_attention("decode", c["q"], c["cache"], c["pos"], c["sot"], c["bt"], ps, H, KV, hd, 0, c["scale"], nslices)
     assert torch.isfinite(out).all()
-    assert err < (2e-5 if dtype == torch.float32 else 2e-2), float(err)
+    assert (out.cpu().double() - c["want"]).abs().max() < 2e-2
 
 
 def standout_case(H, KV, hd, key_pos, ctx_len):
@@ -306,19 +341,19 @@ def test_attention_finds_one_key_among_hundreds(dtype, key_pos, ctx):
     table = list(range(pages - 1, -1, -1))
     cache = build_paged([k], [v], [table], [L + 1], KV, hd, ps, pages, dtype, poison=False)
     qd = q.to(dtype).to(DEV)
-    out = torch.empty_like(qd)
     pos = torch.tensor([L - 1], dtype=torch.int32, device=DEV)
     sot = torch.zeros(1, dtype=torch.int32, device=DEV)
     bt = torch.tensor([table], dtype=torch.int32, device=DEV)
-    K().attn_generic(qd, out, cache, pos, sot, bt, ps, H, KV, hd, 0, 1.0 / math.sqrt(hd))
     want = v[key_pos].to(dtype).float().reshape(KV, hd).repeat_interleave(H // KV, 0).reshape(-1)
-    assert (out.cpu().float()[0] - want).abs().max() < (1e-3 if dtype == torch.float32 else 3e-2)
+    for kernel in kernels_for(dtype):
+        out = run_attention(kernel, qd, cache, pos, sot, bt, ps, H, KV, hd, 0, 1.0 / math.sqrt(hd))
+        assert (out.cpu().float()[0] - want).abs().max() < (1e-3 if dtype == torch.float32 else 3e-2), kernel
 
 
 @pytest.mark.parametrize("window", [1, 16, 17, 33])
-def test_attention_window_edge(window):
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_window_edge(window, dtype):
     H, KV, hd, ps, L = 2, 1, 32, 16, 100
-    dtype = torch.float32
     # the key just outside the window is overwhelming; it must not be seen
     g = torch.Generator().manual_seed(window)
     k = torch.randn(L, hd, generator=g) * 0.1
@@ -329,22 +364,22 @@ def test_attention_window_edge(window):
     k[outside] = 50.0 * q[0, :hd]
     table = list(range(-(-L // ps)))
     cache = build_paged([k], [v], [table], [L], KV, hd, ps, len(table), dtype, poison=False)
-    qd = q.to(DEV)
-    out = torch.empty_like(qd)
+    q, k, v = (t.to(dtype).float() for t in (q, k, v))
+    qd = q.to(dtype).to(DEV)
     pos = torch.tensor([L - 1], dtype=torch.int32, device=DEV)
     sot = torch.zeros(1, dtype=torch.int32, device=DEV)
     bt = torch.tensor([table], dtype=torch.int32, device=DEV)
-    K().attn_generic(qd, out, cache, pos, sot, bt, ps, H, KV, hd, window, 1.0 / math.sqrt(hd))
     want = P.attention(q.double(), k.double(), v.double(), [L - 1], H, KV, hd, window)
-    assert (out.cpu().double() - want).abs().max() < 1e-4
-    assert (out.cpu().float()[0, :hd] - v[outside]).abs().max() > 0.1
-    # pages wholly before the window may be gone (-1 in the table)
-    gone = inside // ps
-    bt2 = bt.clone()
-    bt2[0, :gone] = -1
-    out2 = torch.empty_like(qd)
-    K().attn_generic(qd, out2, cache, pos, sot, bt2, ps, H, KV, hd, window, 1.0 / math.sqrt(hd))
-    assert torch.equal(out2, out)
+    for kernel in kernels_for(dtype):
+        out = run_attention(kernel, qd, cache, pos, sot, bt, ps, H, KV, hd, window, 1.0 / math.sqrt(hd))
+        assert (out.cpu().double() - want).abs().max() < (1e-4 if dtype == torch.float32 else 2e-2), kernel
+        assert (out.cpu().float()[0, :hd] - v[outside]).abs().max() > 0.1
+        # pages wholly before the window may be gone (-1 in the table)
+        gone = inside // ps
+        bt2 = bt.clone()
+        bt2[0, :gone] = -1
+        out2 = run_attention(kernel, qd, cache, pos, sot, bt2, ps, H, KV, hd, window, 1.0 / math.sqrt(hd))
+        assert torch.equal(out2, out), kernel
 
 
 def test_attention_refuses_sizes_it_does_not_take():

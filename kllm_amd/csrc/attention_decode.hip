@@ -41,12 +41,12 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, float* __restrict__ part, const bf16_t* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token,
     const int* __restrict__ block_table, int max_pages, int page_size, int H, int KV, int window,
-    float scale, int head_tiles) {
+    float scale, int head_tiles, const int* __restrict__ token_list) {
   constexpr int hd = 16 * HDT;
   constexpr int KS = (hd + 31) / 32;           // MFMA steps over head_dim for the scores
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int g = lane / 16, c = lane % 16;
-  const int t = blockIdx.x;
+  const int t = token_list ? token_list[blockIdx.x] : blockIdx.x;
   const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y % head_tiles;
   const int G = H / KV;
   const int nslices = gridDim.z * kDecodeWaves;
@@ -172,8 +172,9 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
 template <typename T>
 __global__ __launch_bounds__(64) void attn_merge_kernel(T* __restrict__ out,
                                                         const float* __restrict__ part, int H, int hd,
-                                                        int nslices) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+                                                        int nslices, const int* __restrict__ token_list) {
+  const int t = token_list ? token_list[blockIdx.x] : blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
   const int stride = hd + 2;
   const float* p = part + ((long)t * H + h) * nslices * stride;
   float M = -INFINITY;
@@ -207,10 +208,10 @@ template <int HDT>
 static void launch_decode(dim3 grid, hipStream_t stream, const void* q, float* part, const void* cache,
                           const int* positions, const int* span_of_token, const int* block_table,
                           int max_pages, int page_size, int H, int KV, int window, float scale,
-                          int head_tiles) {
+                          int head_tiles, const int* token_list) {
   hipLaunchKernelGGL(attn_decode_mfma_kernel<HDT>, grid, dim3(64 * kDecodeWaves), 0, stream,
                      (const bf16_t*)q, part, (const bf16_t*)cache, positions, span_of_token,
-                     block_table, max_pages, page_size, H, KV, window, scale, head_tiles);
+                     block_table, max_pages, page_size, H, KV, window, scale, head_tiles, token_list);
 }
 
 }  // namespace kllm
@@ -232,7 +233,7 @@ extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part
                                 const void* cache, const int* positions, const int* span_of_token,
                                 const int* block_table, int max_pages, int page_size, int n, int H,
                                 int KV, int hd, int window, float scale, int nslices, int dtype,
-                                hipStream_t stream) {
+                                const int* token_list, int n_listed, hipStream_t stream) {
   KLLM_REQUIRE(q && out && part && cache && positions && span_of_token && block_table,
                "attn_decode: null pointer");
   KLLM_REQUIRE(dtype == DT_BF16, "attn_decode: bfloat16 only (float32 uses the generic kernel)");
@@ -247,11 +248,13 @@ extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part
   KLLM_REQUIRE(part_floats >= (long)n * H * nslices * (hd + 2), "attn_decode: workspace too small");
   const int head_tiles = (H / KV + 15) / 16;
   KLLM_REQUIRE((long)KV * head_tiles <= 65535 && H <= 65535, "attn_decode: too many heads for the grid");
-  const dim3 grid(n, KV * head_tiles, nslices / kDecodeWaves);
+  KLLM_REQUIRE(!token_list || (n_listed > 0 && n_listed <= n), "attn_decode: bad token list");
+  const int count = token_list ? n_listed : n;     // part and out are indexed by token, not by list place
+  const dim3 grid(count, KV * head_tiles, nslices / kDecodeWaves);
 #define KLLM_DEC(HDT)                                                                             \
   case HDT:                                                                                       \
     launch_decode<HDT>(grid, stream, q, part, cache, positions, span_of_token, block_table,       \
-                       max_pages, page_size, H, KV, window, scale, head_tiles);                   \
+                       max_pages, page_size, H, KV, window, scale, head_tiles, token_list);       \
     break
   switch (hd / 16) {
     KLLM_DEC(1); KLLM_DEC(2); KLLM_DEC(3); KLLM_DEC(4); KLLM_DEC(5); KLLM_DEC(6); KLLM_DEC(7);
@@ -260,8 +263,8 @@ extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part
   }
 #undef KLLM_DEC
   KLLM_CHECK_LAUNCH("attn_decode");
-  hipLaunchKernelGGL(attn_merge_kernel<bf16_t>, dim3(n, H), dim3(64), 0, stream, (bf16_t*)out, part, H,
-                     hd, nslices);
+  hipLaunchKernelGGL(attn_merge_kernel<bf16_t>, dim3(count, H), dim3(64), 0, stream, (bf16_t*)out, part,
+                     H, hd, nslices, token_list);
   KLLM_CHECK_LAUNCH("attn_merge");
   return 0;
 }

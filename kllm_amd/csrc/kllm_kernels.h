@@ -77,12 +77,21 @@ int kllm_attn_generic(const void* q, void* out, const void* cache, const int* po
 /* Decode attention on the matrix cores (bfloat16): every token's keys are cut
  * into `nslices` slices (a multiple of 4) that run side by side; `part` is
  * float32 scratch of n*H*nslices*(hd+2) elements.  kllm_attn_decode_slices
- * proposes nslices for a batch. */
+ * proposes nslices for a batch.  With token_list only the n_listed tokens it
+ * names are computed (q, out and part stay indexed by token row). */
 int kllm_attn_decode_slices(int n, int KV, int H);
 int kllm_attn_decode(const void* q, void* out, float* part, long part_floats, const void* cache,
                      const int* positions, const int* span_of_token, const int* block_table,
                      int max_pages, int page_size, int n, int H, int KV, int hd, int window,
-                     float scale, int nslices, int dtype, hipStream_t stream);
+                     float scale, int nslices, int dtype, const int* token_list, int n_listed,
+                     hipStream_t stream);
+
+/* Prompt attention on the matrix cores (bfloat16).  query_tiles holds
+ * (first token row, span) pairs: up to 32 consecutive tokens of one span. */
+int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
+                      int n_tiles, const int* span_start, const int* span_pos,
+                      const int* block_table, int max_pages, int page_size, int H, int KV, int hd,
+                      int window, float scale, int dtype, hipStream_t stream);
 
 /* out[r] = sampled index of logits[r][:]; temperature/uniform null: greedy. */
 int kllm_sample(int* out, const float* logits, const float* temperature, const float* uniform,

@@ -17,7 +17,7 @@ from typing import List, Sequence
 import numpy as np
 import torch
 
-from ..parts.base import StepContext
+from ..parts.base import StepContext, span_lists
 
 
 def _pad4(n: int) -> int:
@@ -31,6 +31,8 @@ class ControlLayout:
     rows: int              # wanted logit rows
     pages: tuple           # table width per cache group
     samples: int = 0       # rows of sampling parameters (temperature, uniform)
+    short: int = 0         # tokens of short spans, listed for the decode attention kernel
+    tiles: int = 0         # query tiles of longer spans, for the prompt attention kernel
 
     def sections(self):
         s = [("token_ids", self.n), ("positions", self.n), ("span_of_token", self.n),
@@ -38,6 +40,7 @@ class ControlLayout:
              ("logit_rows", max(self.rows, 1))]
         s += [(f"table{g}", self.spans * m) for g, m in enumerate(self.pages)]
         s += [("temperature", self.samples), ("uniform", self.samples)]
+        s += [("short_tokens", self.short), ("query_tiles", 2 * self.tiles)]
         return s
 
     def offsets(self):
@@ -50,6 +53,14 @@ class ControlLayout:
     @property
     def total(self) -> int:
         return self.offsets()[1]
+
+
+def layout_for(lens: Sequence[int], rows: int, pages: tuple, samples: int = 0) -> ControlLayout:
+    starts = [0]
+    for l in lens:
+        starts.append(starts[-1] + l)
+    short, tiles = span_lists(starts, lens)
+    return ControlLayout(sum(lens), len(lens), rows, tuple(pages), samples, len(short), len(tiles))
 
 
 def fill(host: np.ndarray, layout: ControlLayout, tokens: Sequence[Sequence[int]],
@@ -81,6 +92,13 @@ def fill(host: np.ndarray, layout: ControlLayout, tokens: Sequence[Sequence[int]
         bt.fill(-1)
         for s, t in enumerate(tables[g]):
             bt[s, :len(t)] = t
+    short, tiles = span_lists(starts, [len(t) for t in tokens])
+    if len(short) != layout.short or len(tiles) != layout.tiles:
+        raise ValueError("control layout does not fit the step's spans")
+    if layout.short:
+        sec("short_tokens")[:] = short
+    if layout.tiles:
+        sec("query_tiles")[:] = np.asarray(tiles, dtype=np.int32).reshape(-1)
     if layout.samples:
         sec("temperature").view(np.float32)[:] = np.asarray(temperatures, dtype=np.float32)
         sec("uniform").view(np.float32)[:] = np.asarray(uniforms, dtype=np.float32)
@@ -101,7 +119,10 @@ def context(dev: torch.Tensor, layout: ControlLayout, runtime, starts, pos0, len
         logit_rows=sec("logit_rows") if layout.rows else None,
         h_span_start=list(starts), h_span_pos=list(pos0), h_span_len=list(lens),
         block_tables=[sec(f"table{g}").view(layout.spans, m) for g, m in enumerate(layout.pages)],
-        runtime=runtime, max_span_len=max(lens), all_decode=all(l == 1 for l in lens))
+        runtime=runtime, max_span_len=max(lens), all_decode=all(l == 1 for l in lens),
+        short_tokens=sec("short_tokens") if layout.short else None, n_short=layout.short,
+        query_tiles=sec("query_tiles").view(layout.tiles, 2) if layout.tiles else None,
+        n_tiles=layout.tiles)
 
 
 def sampling_views(dev: torch.Tensor, layout: ControlLayout):

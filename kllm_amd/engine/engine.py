@@ -294,7 +294,7 @@ class Engine:
         try:
             rcs, lens, rows, tables = self._describe(entries)
             pages = tuple(max(1, max(len(t) for t in tg)) for tg in tables)
-            layout = control.ControlLayout(sum(lens), len(entries), len(rows), pages)
+            layout = control.layout_for(lens, len(rows), pages)
             total = layout.total
             host = self._staging(total)
             pos0 = [rc.length for rc in rcs]

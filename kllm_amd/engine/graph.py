@@ -37,7 +37,7 @@ def _bucket(pages: int) -> int:
 
 class _Recording:
     def __init__(self, engine, batch: int, caps: tuple):
-        self.layout = control.ControlLayout(batch, batch, batch, caps, samples=batch)
+        self.layout = control.layout_for([1] * batch, batch, caps, samples=batch)
         self.control = torch.zeros(self.layout.total, dtype=torch.int32, device=engine.device)
         self.tokens = torch.zeros(batch, dtype=torch.int32, device=engine.device)
         self.workspace = Workspace(engine.device)

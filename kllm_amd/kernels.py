@@ -85,7 +85,8 @@ def _declare(lib):
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
         "kllm_attn_decode_slices": [I, I, I],
-        "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
+        "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, P],
+        "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -276,8 +277,31 @@ def attn_decode_slices(n, n_kv_heads, n_heads) -> int:
     return library().kllm_attn_decode_slices(n, n_kv_heads, n_heads)
 
 
+PREFILL_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
+
+
+def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, block_table, page_size,
+                 n_heads, n_kv_heads, head_dim, window, scale):
+    """query_tiles [n_tiles, 2] int32: (first token row, span) of each tile of 32 tokens."""
+    n = q.shape[0]
+    if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape)
+            or q.dtype != cache.dtype or out.dtype != q.dtype):
+        raise KernelError("attn_prefill: q/out shapes or dtypes do not fit")
+    if tuple(cache.shape[1:]) != (2, n_kv_heads, page_size * head_dim):
+        raise KernelError(f"attn_prefill: cache {tuple(cache.shape)} does not fit")
+    if query_tiles.numel() < 2 * n_tiles:
+        raise KernelError("attn_prefill: tile list is too short")
+    _check(library().kllm_attn_prefill(
+        _ptr(q, "attn q"), _ptr(out, "attn out"), _ptr(cache, "attn cache"),
+        _ptr(query_tiles, "attn query_tiles", torch.int32), n_tiles,
+        _ptr(span_start, "attn span_start", torch.int32), _ptr(span_pos, "attn span_pos", torch.int32),
+        _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size,
+        n_heads, n_kv_heads, head_dim, int(window), float(scale), dtype_code(q.dtype), _stream()),
+        "attn_prefill")
+
+
 def attn_decode(q, out, part, cache, positions, span_of_token, block_table, page_size, n_heads,
-                n_kv_heads, head_dim, window, scale, nslices):
+                n_kv_heads, head_dim, window, scale, nslices, token_list=None, n_listed=0):
     n = q.shape[0]
     if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape)
             or q.dtype != cache.dtype or out.dtype != q.dtype):
@@ -292,7 +316,8 @@ def attn_decode(q, out, part, cache, positions, span_of_token, block_table, page
         _ptr(span_of_token, "attn span_of_token", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size, n,
         n_heads, n_kv_heads, head_dim, int(window), float(scale), int(nslices), dtype_code(q.dtype),
-        _stream()), "attn_decode")
+        _ptr(token_list, "attn token_list", torch.int32, True), int(n_listed), _stream()),
+        "attn_decode")
 
 
 def sample(out, logits, temperature=None, uniform=None):

@@ -85,18 +85,35 @@ class CausalSelfAttention(Part):
         return linear(ctx, out, self.w_o, "attn.proj")
 
     def attend(self, ctx, q, out, cache):
-        """Choose the attention kernel by dtype and by the spans' lengths."""
+        """Choose the attention kernels by dtype and by the spans' lengths:
+        in bfloat16, tokens of short spans (decode tokens) go to the kernel
+        that splits a token's keys over many waves, longer spans to the prompt
+        kernel in tiles of 32 queries; float32, and sizes those kernels do not
+        take, go to the kernel that takes every size."""
         mode = self.runtime.options.get("attention", "auto")
         fast = (mode != "generic" and q.dtype == torch.bfloat16 and cache.page_size % 16 == 0
                 and self.head_dim in K.DECODE_HEAD_DIMS)
-        if fast and ctx.max_span_len <= 4:
-            n = q.shape[0]
-            nslices = K.attn_decode_slices(n, self.kv_heads, self.heads)
-            part = ctx.buf("attn.part", (n * self.heads * nslices * (self.head_dim + 2),), torch.float32)
-            K.attn_decode(q, out, part, cache.pages, ctx.positions, ctx.span_of_token,
-                          cache.block_table, cache.page_size, self.heads, self.kv_heads,
-                          self.head_dim, self.window, self.scale, nslices)
+        if not fast:
+            K.attn_generic(q, out, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
+                           cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
+                           self.scale)
             return
-        K.attn_generic(q, out, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
-                       cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
-                       self.scale)
+        n = q.shape[0]
+        listed = ctx.n_short + ctx.n_tiles > 0          # a context built by hand may carry no lists
+        if not listed or (ctx.n_tiles and self.head_dim not in K.PREFILL_HEAD_DIMS):
+            self._decode(ctx, q, out, cache, None, n)   # token by token
+            return
+        if ctx.n_short:
+            self._decode(ctx, q, out, cache, None if ctx.n_short == n else ctx.short_tokens, ctx.n_short)
+        if ctx.n_tiles:
+            K.attn_prefill(q, out, cache.pages, ctx.query_tiles, ctx.n_tiles, ctx.span_start,
+                           ctx.span_pos, cache.block_table, cache.page_size, self.heads,
+                           self.kv_heads, self.head_dim, self.window, self.scale)
+
+    def _decode(self, ctx, q, out, cache, token_list, count):
+        n = q.shape[0]
+        nslices = K.attn_decode_slices(count, self.kv_heads, self.heads)
+        part = ctx.buf("attn.part", (n * self.heads * nslices * (self.head_dim + 2),), torch.float32)
+        K.attn_decode(q, out, part, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
+                      cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
+                      self.scale, nslices, token_list, count)

@@ -145,6 +145,24 @@ class StateCacheView:
     write: bool = True
 
 
+# How a step's spans are listed for the attention kernels: tokens of spans of at
+# most SHORT_SPAN tokens one by one, longer spans in tiles of QUERY_TILE tokens.
+SHORT_SPAN = 4
+QUERY_TILE = 32
+
+
+def span_lists(starts, lens):
+    """(token rows of short spans, (first row, span) of the long spans' tiles)."""
+    short, tiles = [], []
+    for s, n in enumerate(lens):
+        a = starts[s]
+        if n <= SHORT_SPAN:
+            short.extend(range(a, a + n))
+        else:
+            tiles.extend((t, s) for t in range(a, a + n, QUERY_TILE))
+    return short, tiles
+
+
 @dataclass
 class StepContext:
     """One step's batch as the parts see it.  All index tensors are int32 on
@@ -172,6 +190,10 @@ class StepContext:
     scratch: Dict[Any, Any] = field(default_factory=dict)   # per-step values of parts
     taps: Optional[List[torch.Tensor]] = None               # residual-stream captures
     workspace: Optional["Workspace"] = None                 # scratch of this step (default: the runtime's)
+    short_tokens: Optional[torch.Tensor] = None             # token rows of spans of <= SHORT_SPAN tokens
+    n_short: int = 0
+    query_tiles: Optional[torch.Tensor] = None              # [n_tiles, 2]: (first row, span), longer spans
+    n_tiles: int = 0
 
     def buf(self, tag, shape, dtype):
         return (self.workspace or self.runtime.workspace).get(tag, shape, dtype)

@@ -263,8 +263,30 @@ def attention_case(H, KV, hd, ps, dtype, window, spans, seed=0):
     want = torch.cat([
         P.attention(qs[s].double(), ks[s].double(), vs[s].double(), range(a, a + b), H, KV, hd, window)
         for s, (a, b) in enumerate(spans)])
+    starts = [0]
+    for _, b in spans:
+        starts.append(starts[-1] + b)
     return dict(q=q, cache=cache, pos=pos, sot=sot, bt=bt, want=want, ps=ps, H=H, KV=KV, hd=hd,
-                window=window, scale=1.0 / math.sqrt(hd), tables=tables, lens=lens)
+                window=window, scale=1.0 / math.sqrt(hd), tables=tables, lens=lens, spans=spans,
+                span_start=torch.tensor(starts, dtype=torch.int32, device=DEV),
+                span_pos=torch.tensor([a for a, _ in spans], dtype=torch.int32, device=DEV))
+
+
+def run_prefill(c, min_len=1):
+    """The prompt kernel over the spans of at least min_len tokens; returns
+    (output, mask of the rows it computed)."""
+    tiles, rows = [], torch.zeros(c["q"].shape[0], dtype=torch.bool)
+    start = 0
+    for s, (_, b) in enumerate(c["spans"]):
+        if b >= min_len:
+            tiles += [(t, s) for t in range(start, start + b, 32)]
+            rows[start:start + b] = True
+        start += b
+    qt = torch.tensor(tiles, dtype=torch.int32, device=DEV)
+    out = torch.full_like(c["q"], float("nan"))
+    K().attn_prefill(c["q"], out, c["cache"], qt, len(tiles), c["span_start"], c["span_pos"], c["bt"],
+                     c["ps"], c["H"], c["KV"], c["hd"], c["window"], c["scale"])
+    return out, rows
 
 
 def run_attention(kernel, q, cache, pos, sot, bt, ps, H, KV, hd, window, scale, nslices=None):
@@ -299,6 +321,30 @@ def test_attention_generic(H, KV, hd, ps, dtype, window):
         err = (out.cpu().double() - c["want"]).abs().max()
         assert torch.isfinite(out).all(), kernel
         assert err < (2e-5 if dtype == torch.float32 else 2e-2), (kernel, float(err))
+
+
+@pytest.mark.parametrize("H,KV,hd,ps", [(4, 2, 32, 16), (3, 1, 64, 16), (8, 2, 64, 32), (5, 5, 96, 16),
+                                        (2, 1, 128, 16), (2, 2, 192, 16), (2, 1, 256, 16), (32, 4, 64, 16)])
+@pytest.mark.parametrize("window", [0, 37, 200])
+def test_attention_prefill(H, KV, hd, ps, window):
+    """Whole prompts of ragged lengths, portions behind cached keys that start
+    and end inside pages and query tiles, and a one-token span, in one launch."""
+    c = attention_case(H, KV, hd, ps, torch.bfloat16, window,
+                       [(0, 45), (300, 9), (0, 100), (37, 70), (5, 1), (16, 32), (31, 33)], seed=5)
+    out, rows = run_prefill(c)
+    assert rows.all() and torch.isfinite(out).all()
+    err = (out.cpu().double() - c["want"]).abs().max()
+    assert err < 2e-2, float(err)
+    # only the listed spans are touched
+    out2, rows2 = run_prefill(c, min_len=33)
+    assert torch.isnan(out2.cpu()[~rows2]).all() and torch.equal(out2.cpu()[rows2], out.cpu()[rows2])
+
+
+def test_attention_prefill_refuses_what_it_does_not_take():
+    k_ = K()
+    c = attention_case(2, 1, 48, 16, torch.bfloat16, 0, [(0, 40)])
+    with pytest.raises(k_.KernelError, match="head_dim 48"):
+        run_prefill(c)
 
 
 @pytest.mark.parametrize("H,KV,hd,ps", [(40, 2, 32, 16), (17, 1, 64, 16), (12, 4, 192, 16), (8, 8, 112, 48)])

@@ -80,32 +80,58 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
 #pragma unroll
   for (int i = 0; i < HDT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+  // One tile's operands: the loads of tile i+1 are issued before tile i is
+  // computed, and its page ids were read one tile earlier still.
+  struct Tile {
+    bf16x8 k[2][KS];
+    bf16x4 v[2][HDT];
+    bool live[2];
+  };
+  auto page_of = [&](int tile, int u) -> int {
+    const int k0 = first + tile * 32 + 16 * u;
+    return (tile < tile1 && k0 < len && k0 + 16 > start) ? table[k0 / page_size] : -1;
+  };
+  auto fetch = [&](int tile, int page0, int page1) -> Tile {
+    Tile T;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int page = u ? page1 : page0;
+      const int k0 = first + tile * 32 + 16 * u;
+      T.live[u] = page >= 0;
+      const long base = ((long)(T.live[u] ? page : 0) * 2 * KV + kvh) * block;
+      const bf16_t* kp = cache + base + (long)(k0 % page_size + c) * hd;        // keys [slot][hd]
+      const bf16_t* vp = cache + base + (long)KV * block + (k0 % page_size);     // values [hd][slot]
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d0 = 32 * ks + 8 * g;
+        T.k[u][ks] = (T.live[u] && d0 < hd) ? *reinterpret_cast<const bf16x8*>(kp + d0) : zero8;
+      }
+#pragma unroll
+      for (int r = 0; r < HDT; ++r)
+        T.v[u][r] = T.live[u] ? *reinterpret_cast<const bf16x4*>(vp + (long)(16 * r + c) * page_size + 4 * g)
+                              : bf16x4{0, 0, 0, 0};
+    }
+    return T;
+  };
+
+  int pg0 = page_of(tile0, 0), pg1 = page_of(tile0, 1);
+  Tile nxt = fetch(tile0, pg0, pg1);
+  pg0 = page_of(tile0 + 1, 0);
+  pg1 = page_of(tile0 + 1, 1);
   for (int tile = tile0; tile < tile1; ++tile) {
+    const Tile cur = nxt;
+    nxt = fetch(tile + 1, pg0, pg1);
+    pg0 = page_of(tile + 2, 0);
+    pg1 = page_of(tile + 2, 1);
     const int kb = first + tile * 32;
     const bool edge = kb < start || kb + 32 > len;
-    const bf16_t* kpage[2];
-    const bf16_t* vpage[2];
-    bool live[2];
     floatx4 s[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int k0 = kb + 16 * u;
-      live[u] = k0 < len && k0 + 16 > start;               // some key of these 16 is read
-      int page = 0;
-      if (live[u]) page = table[k0 / page_size];
-      const long base = ((long)page * 2 * KV + kvh) * block;
-      kpage[u] = cache + base + (long)(k0 % page_size) * hd;                 // [slot][hd]
-      vpage[u] = cache + base + (long)KV * block + (k0 % page_size);          // [hd][slot]
       s[u] = floatx4{0.f, 0.f, 0.f, 0.f};
-      if (live[u]) {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const int d0 = 32 * ks + 8 * g;
-          const bf16x8 a = (d0 < hd) ? *reinterpret_cast<const bf16x8*>(kpage[u] + (long)c * hd + d0)
-                                     : zero8;
-          s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ks], s[u], 0, 0, 0);
-        }
-      }
+      for (int ks = 0; ks < KS; ++ks)
+        s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[u][ks], qb[ks], s[u], 0, 0, 0);
     }
     // ---- online softmax for this lane's head over its 8 keys, then the 4 lanes of the column
     float tmax = -INFINITY;
@@ -114,7 +140,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = kb + 16 * u + 4 * g + i;
-        const bool ok = live[u] && key >= start && key < len;
+        const bool ok = cur.live[u] && key >= start && key < len;
         s[u][i] = ok ? s[u][i] * scale : -INFINITY;
         tmax = fmaxf(tmax, s[u][i]);
       }
@@ -138,18 +164,15 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
 #pragma unroll
     for (int r = 0; r < HDT; ++r) {
       acc[r] *= alpha;
-      bf16x8 a = zero8;
+      bf16x8 a;
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        if (!live[u]) continue;
-        const bf16x4 v = *reinterpret_cast<const bf16x4*>(vpage[u] + (long)(16 * r + c) * page_size + 4 * g);
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = kb + 16 * u + 4 * g + i;
-          const bool ok = !edge || (key >= start && key < len);   // stale slots may hold anything
-          a[4 * u + i] = ok ? v[i] : (bf16_t)0.f;
+          const bool ok = cur.live[u] && (!edge || (key >= start && key < len));   // stale slots may hold anything
+          a[4 * u + i] = ok ? cur.v[u][r][i] : (bf16_t)0.f;
         }
-      }
       acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[r], 0, 0, 0);
     }
   }
@@ -222,10 +245,10 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H) {
   // Waves wanted across the chip, shared out over tokens x KV heads x head tiles.
   const int head_tiles = (H / KV + 15) / 16;
   long groups = (long)n * KV * head_tiles;
-  long want = 1024 / (groups > 0 ? groups : 1);
+  long want = 2048 / (groups > 0 ? groups : 1);
   int wg = (int)((want + kDecodeWaves - 1) / kDecodeWaves);
   if (wg < 1) wg = 1;
-  if (wg > 16) wg = 16;
+  if (wg > 4) wg = 4;
   return wg * kDecodeWaves;
 }
 

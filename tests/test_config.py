@@ -25,13 +25,13 @@ def test_defaults_are_the_references():
     assert c.q_dim == 64 and c.kv_dim == 64
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C", "R"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "R"])
 def test_every_size_comes_from_config_json(name, tmp_path):
     raw = tiny.CONFIGS[name]
     (tmp_path / "config.json").write_text(json.dumps(raw))
     c = load_config(str(tmp_path))
     assert c.hidden_size == raw["hidden_size"] and c.head_dim == raw["head_dim"]
-    assert c.num_key_value_heads == raw["num_key_value_heads"]
+    assert c.num_key_value_heads == raw.get("num_key_value_heads", raw["num_attention_heads"])
     assert c.rope_theta == raw["rope_theta"] and c.rms_norm_eps == raw["rms_norm_eps"]
     assert c.tie_word_embeddings == raw["tie_word_embeddings"]
     assert c.max_position_embeddings == raw["max_position_embeddings"]

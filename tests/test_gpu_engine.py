@@ -60,7 +60,7 @@ def compare(rows, want, dtype, requests):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name,lengths", [("A", [5, 17, 33, 100]), ("B", [1, 9, 40, 70, 150]),
-                                          ("C", [3, 64, 65])])
+                                          ("C", [3, 64, 65]), ("D", [2, 90])])
 def test_alone_and_whole(model_dirs, name, lengths, dtype):
     cfg, d = tiny.CONFIGS[name], model_dirs(name)
     reqs = make_requests(cfg, lengths, 1)
@@ -70,7 +70,7 @@ def test_alone_and_whole(model_dirs, name, lengths, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,lengths", [("A", [33, 100]), ("B", [40, 129]), ("C", [50])])
+@pytest.mark.parametrize("name,lengths", [("A", [33, 100]), ("B", [40, 129]), ("C", [50]), ("D", [45])])
 def test_bulk_then_last_32_one_by_one(model_dirs, name, lengths, dtype):
     cfg, d = tiny.CONFIGS[name], model_dirs(name)
     reqs = make_requests(cfg, lengths, 2)
@@ -80,7 +80,7 @@ def test_bulk_then_last_32_one_by_one(model_dirs, name, lengths, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,lengths", [("A", [100, 37]), ("B", [150, 70]), ("C", [81])])
+@pytest.mark.parametrize("name,lengths", [("A", [100, 37]), ("B", [150, 70]), ("C", [81]), ("D", [77])])
 def test_portions_of_changing_size(model_dirs, name, lengths, dtype):
     cfg, d = tiny.CONFIGS[name], model_dirs(name)
     reqs = make_requests(cfg, lengths, 3)
@@ -91,7 +91,7 @@ def test_portions_of_changing_size(model_dirs, name, lengths, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "D"])
 def test_mixed_with_pages_used_again(model_dirs, name, dtype):
     cfg, d = tiny.CONFIGS[name], model_dirs(name)
     reqs = make_requests(cfg, [70, 33, 120, 18, 64, 97, 41, 129, 5, 80], 4)

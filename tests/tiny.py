@@ -4,7 +4,8 @@ A and B are the two tiny Llama configurations that differ in every size and
 option: layers, width, heads and groups (GQA / MQA), head size, feed-forward
 width, vocabulary, rotary base, context, eps, tying.  C is multi-head
 (KV = H) with a head size that is not hidden/heads, a width and a vocabulary
-that are not powers of two.  R is the reference's own tiny model
+that are not powers of two.  D has sizes the fast kernels refuse (they must
+fall back, never give a wrong result).  R is the reference's own tiny model
 (tools/make_test_model.py:47-100).
 """
 
@@ -32,6 +33,11 @@ CONFIGS = {
     "C": _cfg(num_hidden_layers=1, hidden_size=88, num_attention_heads=5, num_key_value_heads=5,
               head_dim=48, intermediate_size=120, vocab_size=131, rope_theta=1000.0,
               max_position_embeddings=512, rms_norm_eps=1e-4, tie_word_embeddings=False),
+    # sizes the fast kernels do not take: a width that is no multiple of 8, a head size
+    # with no prompt kernel, an odd vocabulary, no num_key_value_heads key (defaults to heads)
+    "D": _cfg(num_hidden_layers=2, hidden_size=100, num_attention_heads=5, head_dim=80,
+              intermediate_size=172, vocab_size=257, rope_theta=20000.0,
+              max_position_embeddings=64, rms_norm_eps=1e-3, tie_word_embeddings=True),
     "R": _cfg(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2,
               head_dim=16, intermediate_size=128, vocab_size=512, rope_theta=10000.0,
               max_position_embeddings=256, rms_norm_eps=1e-6, tie_word_embeddings=False,

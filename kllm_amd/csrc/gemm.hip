@@ -226,25 +226,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
   const int klen = kend - kbeg;                                  // a multiple of 8
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  const int chunks = (klen + 7) / 8;
-  for (int idx = tid; idx < NT * 16 * chunks; idx += 256) {
-    const int r = idx / chunks, ch = idx % chunks;
-    const bf16x8 v = (r < n) ? *reinterpret_cast<const bf16x8*>(X + (long)r * k + kbeg + ch * 8) : zero;
-    *reinterpret_cast<bf16x8*>(&xs[r * SK_LD + ch * 8]) = v;
-  }
-  __syncthreads();
-
+  // This wave's rows of W; their first loads go out before X is staged.
   const long m0 = ((long)blockIdx.x * 4 + wave) * 16;
-  if (m0 >= m) return;
   const long wrow = m0 + c;
   const bool wok = wrow < m;
   const bf16_t* wp = W + (wok ? wrow : 0) * k + kbeg + 8 * g;
   const int steps = (klen + 31) / 32;
-
-  floatx4 acc[NT];
-#pragma unroll
-  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-
   auto load_a = [&](int s) -> bf16x8 {
     return (wok && s < steps && 32 * s + 8 * g < klen) ? *reinterpret_cast<const bf16x8*>(wp + 32 * s)
                                                         : zero;
@@ -252,6 +239,34 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
   bf16x8 cur[SK_AHEAD], nxt[SK_AHEAD];
 #pragma unroll
   for (int u = 0; u < SK_AHEAD; ++u) cur[u] = load_a(u);
+
+  // Stage X[0..16*NT)[kbeg..kend) in LDS, eight 16-byte loads in flight per thread.
+  const int chunks = (klen + 7) / 8;
+  const int total = NT * 16 * chunks;
+  for (int base = tid; base < total; base += 256 * 8) {
+    bf16x8 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int idx = base + j * 256;
+      const int r = idx / chunks, ch = idx % chunks;
+      v[j] = (idx < total && r < n) ? *reinterpret_cast<const bf16x8*>(X + (long)r * k + kbeg + ch * 8) : zero;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int idx = base + j * 256;
+      if (idx < total) {
+        const int r = idx / chunks, ch = idx % chunks;
+        *reinterpret_cast<bf16x8*>(&xs[r * SK_LD + ch * 8]) = v[j];
+      }
+    }
+  }
+  __syncthreads();
+  if (m0 >= m) return;
+
+  floatx4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
   for (int s0 = 0; s0 < steps; s0 += SK_AHEAD) {
 #pragma unroll
     for (int u = 0; u < SK_AHEAD; ++u) nxt[u] = load_a(s0 + SK_AHEAD + u);
@@ -418,7 +433,7 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "gemm: unknown dtype %d", dtype);
   KLLM_REQUIRE(out_dtype == DT_F32 || out_dtype == dtype, "gemm: output dtype %d with input %d",
                out_dtype, dtype);
-  KLLM_REQUIRE(nsplit >= 1 && nsplit <= 64, "gemm: nsplit %d", nsplit);
+  KLLM_REQUIRE(nsplit >= 1 && nsplit <= 256, "gemm: nsplit %d is outside [1, 256]", nsplit);
   KLLM_REQUIRE((long)n * m < (1L << 31) && (long)m * k < (1L << 40), "gemm: sizes overflow");
 
   if (algo == KLLM_GEMM_PLAIN) {

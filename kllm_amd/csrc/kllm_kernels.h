@@ -25,6 +25,7 @@ extern "C" {
 #define KLLM_GEMM_MFMA_BF16 2
 #define KLLM_GEMM_SKINNY_BF16 3
 #define KLLM_GEMM_GEMV 4
+#define KLLM_GEMM_GEMV_LDS 5 /* kllm_gemv_plain, reached through the Python wrapper */
 
 /* Copies the calling thread's last error text; returns its length. */
 int kllm_last_error(char* buf, int len);
@@ -67,6 +68,24 @@ int kllm_sum_splits(const float* in, int nsplit, long count, void* out, int out_
 /* y[nsplit][n][m] = x[n][k] . w[m][k]^T, 32-bit accumulation. */
 int kllm_gemm(const void* x, const void* w, void* y, int n, int m, int k, int dtype, int out_dtype,
               int algo, int nsplit, hipStream_t stream);
+
+/* Products for up to 8 rows of x with the whole of K in one wave (no partial
+ * sums) and the next elementwise step in the epilogue.  m even, K a multiple
+ * of 8 (bfloat16) or 4 (float32).
+ *   plain:       y[n][m] float32 = x . w^T
+ *   swiglu:      h[n][f] = silu(x . w[0:f]^T) * (x . w[f:2f]^T), h in dtype
+ *   rope_append: w = [q; k; v] rows (only q when cache is null); rotates q and k
+ *                with cos/sin [n][hd/2] (if given), writes q_out [n][H*hd] and
+ *                puts k, v into the pages of `cache` */
+int kllm_gemv_plain(const void* x, const void* w, float* y, int n, int m, int k, int dtype,
+                    hipStream_t stream);
+int kllm_gemv_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f, int k, int dtype,
+                     hipStream_t stream);
+int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_out, const float* cos_t,
+                          const float* sin_t, void* cache, const int* positions,
+                          const int* span_of_token, const int* block_table, int max_pages,
+                          int page_size, int n, int H, int KV, int hd, int k, int dtype,
+                          hipStream_t stream);
 
 /* Causal attention of n tokens over the paged cache; any head size up to 256. */
 int kllm_attn_generic(const void* q, void* out, const void* cache, const int* positions,

@@ -17,7 +17,9 @@ from ctypes import c_char_p, c_double, c_float, c_int, c_long, c_void_p
 import torch
 
 DT_F32, DT_BF16 = 0, 1
-GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV = 0, 1, 2, 3, 4
+GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS = 0, 1, 2, 3, 4, 5
+GEMV_MAX_ROWS = 8          # what the fused kernels take
+GEMV_BEST_ROWS = 4         # up to here they beat the MFMA kernel with split K
 ABI_VERSION = 1
 
 
@@ -82,6 +84,9 @@ def _declare(lib):
         "kllm_silu_mul": [P, I, I, L, P, I, I, I, P],
         "kllm_gemm": [P, P, P, I, I, I, I, I, I, I, P],
         "kllm_sum_splits": [P, I, L, P, I, P],
+        "kllm_gemv_plain": [P, P, P, I, I, I, I, P],
+        "kllm_gemv_swiglu": [P, P, P, I, I, I, I, P],
+        "kllm_gemv_rope_append": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
         "kllm_attn_decode_slices": [I, I, I],
@@ -236,9 +241,61 @@ def gemm(x, w, y, algo, nsplit=1):
     want = (nsplit, n, m) if y.dim() == 3 else (n, m)
     if tuple(y.shape) != want or (y.dim() == 2 and nsplit != 1):
         raise KernelError(f"gemm: output {tuple(y.shape)} does not fit {want}")
+    if algo == GEMM_GEMV_LDS:
+        if nsplit != 1:
+            raise KernelError("gemm: the LDS gemv does not split K")
+        _check(library().kllm_gemv_plain(
+            _ptr(x, "gemv x"), _ptr(w, "gemv w"), _ptr(y, "gemv y", torch.float32), n, m, k,
+            dtype_code(x.dtype), _stream()), "gemv_plain")
+        return
     _check(library().kllm_gemm(
         _ptr(x, "gemm x"), _ptr(w, "gemm w"), _ptr(y, "gemm y"), n, m, k, dtype_code(x.dtype),
         dtype_code(y.dtype), algo, nsplit, _stream()), "gemm")
+
+
+def gemv_fits(n, m, k, dtype) -> bool:
+    """Whether the fused small-batch products take these sizes and are the
+    faster choice: always in float32 (which has no MFMA kernel), up to
+    GEMV_BEST_ROWS rows in bfloat16."""
+    v = 4 if dtype == torch.float32 else 8
+    most = GEMV_MAX_ROWS if dtype == torch.float32 else GEMV_BEST_ROWS
+    return n <= most and m % 2 == 0 and k % v == 0
+
+
+def gemv_swiglu(x, w_gate_up, h):
+    """h [n, f] = silu(x . gate^T) * (x . up^T); w_gate_up is [2f, k], gate rows first."""
+    n, k = x.shape
+    f = h.shape[1]
+    if tuple(w_gate_up.shape) != (2 * f, k) or h.shape[0] != n or x.dtype != w_gate_up.dtype or h.dtype != x.dtype:
+        raise KernelError("gemv_swiglu: shapes or dtypes do not fit")
+    _check(library().kllm_gemv_swiglu(_ptr(x, "gemv x"), _ptr(w_gate_up, "gemv w"), _ptr(h, "gemv h"), n, f, k,
+                                      dtype_code(x.dtype), _stream()), "gemv_swiglu")
+
+
+def gemv_rope_append(x, w_qkv, q_out, cos, sin, cache, positions, span_of_token, block_table, page_size,
+                     n_heads, n_kv_heads, head_dim):
+    """q, k, v projections of up to 8 rows, rotation, q_out and the cache append in one launch."""
+    n, k = x.shape
+    rows = n_heads * head_dim + (2 * n_kv_heads * head_dim if cache is not None else 0)
+    if (tuple(w_qkv.shape) != (rows, k) or tuple(q_out.shape) != (n, n_heads * head_dim)
+            or x.dtype != w_qkv.dtype or q_out.dtype != x.dtype):
+        raise KernelError("gemv_rope_append: shapes or dtypes do not fit")
+    max_pages = 0
+    if cache is not None:
+        if tuple(cache.shape[1:]) != (2, n_kv_heads, page_size * head_dim) or cache.dtype != x.dtype:
+            raise KernelError(f"gemv_rope_append: cache {tuple(cache.shape)} {cache.dtype} does not fit")
+        max_pages = block_table.shape[1]
+        if positions.numel() < n or span_of_token.numel() < n:
+            raise KernelError("gemv_rope_append: index arrays are too short")
+    if cos is not None and (tuple(cos.shape) != (n, head_dim // 2) or tuple(sin.shape) != tuple(cos.shape)):
+        raise KernelError("gemv_rope_append: cos/sin shapes do not fit")
+    _check(library().kllm_gemv_rope_append(
+        _ptr(x, "gemv x"), _ptr(w_qkv, "gemv w"), _ptr(q_out, "gemv q_out"),
+        _ptr(cos, "gemv cos", torch.float32, True), _ptr(sin, "gemv sin", torch.float32, True),
+        _ptr(cache, "gemv cache", None, True), _ptr(positions, "gemv positions", torch.int32, True),
+        _ptr(span_of_token, "gemv span_of_token", torch.int32, True),
+        _ptr(block_table, "gemv block_table", torch.int32, True), max_pages, page_size, n, n_heads,
+        n_kv_heads, head_dim, k, dtype_code(x.dtype), _stream()), "gemv_rope_append")
 
 
 def sum_splits(parts, out):

@@ -72,14 +72,22 @@ class CausalSelfAttention(Part):
         writes = self.own_kv
         if writes != bool(cache.write):
             raise ValueError("attention: a run must write its cache exactly when it has k/v projections")
-        qkv = linear(ctx, xn, self.w_in, "attn.qkv")
         q = ctx.buf("attn.q", (n, self.q_dim), dtype)
         cos = sin = None
         if self.position is not None and hasattr(self.position, "tables"):
             cos, sin = self.position.tables(ctx)
-        K.rope_append(qkv, q, cos, sin, cache.pages if writes else None, ctx.positions,
-                      ctx.span_of_token, cache.block_table, cache.page_size, self.heads,
-                      self.kv_heads, self.head_dim)
+        pages = cache.pages if writes else None
+        if (K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype)
+                and not self.runtime.options.get("no_fused_gemv")):
+            # few tokens: projections, rotation and append in one launch
+            K.gemv_rope_append(xn, self.w_in, q, cos, sin, pages, ctx.positions, ctx.span_of_token,
+                               cache.block_table, cache.page_size, self.heads, self.kv_heads,
+                               self.head_dim)
+        else:
+            qkv = linear(ctx, xn, self.w_in, "attn.qkv")
+            K.rope_append(qkv, q, cos, sin, pages, ctx.positions, ctx.span_of_token,
+                          cache.block_table, cache.page_size, self.heads, self.kv_heads,
+                          self.head_dim)
         out = ctx.buf("attn.out", (n, self.q_dim), dtype)
         self.attend(ctx, q, out, cache)
         return linear(ctx, out, self.w_o, "attn.proj")

@@ -42,7 +42,11 @@ class GatedFeedForward(Part):
 
     def forward(self, ctx, xn):
         n = xn.shape[0]
-        gu = linear(ctx, xn, self.w_gu, "ffn.gu")
         h = ctx.buf("ffn.h", (n, self.intermediate), self.runtime.dtype)
-        K.silu_mul(gu, h)
+        if (K.gemv_fits(n, 2 * self.intermediate, self.hidden, xn.dtype)
+                and not self.runtime.options.get("no_fused_gemv")):
+            K.gemv_swiglu(xn, self.w_gu, h)          # few tokens: both products and the gate in one launch
+        else:
+            gu = linear(ctx, xn, self.w_gu, "ffn.gu")
+            K.silu_mul(gu, h)
         return linear(ctx, h, self.w_down, "ffn.down")

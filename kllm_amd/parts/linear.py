@@ -5,8 +5,10 @@ it returns partial sums [nsplit, n, m] that the consuming kernel adds (norm,
 rotary + append, SiLU gate); with the compute dtype as result it returns
 [n, m].  Which kernel runs depends only on the dtype and on n:
 
-  float32   n <= 8: gemv      else: tiled FMA (true 32-bit)
-  bfloat16  n <= 4: gemv      n <= 64: MFMA skinny      else: MFMA tiles,
+  n <= 8    gemv with X in LDS and the whole of K in one wave (no partial
+            sums), if the sizes fit; else the streaming or the general gemv
+  float32   else: tiled FMA (true 32-bit)
+  bfloat16  n <= 64: MFMA skinny      else: MFMA tiles,
             or the vendor library (torch.matmul) when the engine option
             ``gemm`` is "library" -- the reference uses its vendor library for
             every product (backend/model.cu:494-503)
@@ -51,6 +53,8 @@ def choose(dtype, n, m, k, options=None):
     forced = options.get("gemm_algo")
     if forced is not None:
         return forced, 1
+    if K.gemv_fits(n, m, k, dtype) and not options.get("no_fused_gemv"):
+        return K.GEMM_GEMV_LDS, 1
     if n <= 4 or (n <= 8 and dtype == torch.float32):
         return K.GEMM_GEMV, _gemv_split(dtype, n, m, k)
     if dtype == torch.float32:

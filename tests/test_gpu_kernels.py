@@ -161,7 +161,8 @@ def test_silu_mul(out_dtype):
 
 # ------------------------------------------------------------------ matrix products
 
-GEMM_SIZES = [(1, 64, 64), (2, 131, 88), (5, 100, 72), (8, 515, 2048), (17, 96, 176),
+GEMM_SIZES = [(1, 64, 64), (2, 131, 88), (5, 100, 72), (8, 515, 2048), (3, 130, 5632), (8, 64, 20480),
+              (7, 258, 4100), (17, 96, 176),
               (33, 320, 96), (64, 200, 264), (65, 130, 40), (130, 515, 1032), (300, 257, 520)]
 
 
@@ -179,9 +180,11 @@ def test_gemm_kernels_against_plain(n, m, k, dtype):
         algos.append((k_.GEMM_MFMA_BF16, 1))
         if n <= 64:
             base = -(-k // 512)
-            algos += [(k_.GEMM_SKINNY_BF16, base)] + ([(k_.GEMM_SKINNY_BF16, base + 2)] if k >= 256 else [])
+            algos += [(k_.GEMM_SKINNY_BF16, base)] + ([(k_.GEMM_SKINNY_BF16, base * 2)] if k >= 256 else [])
     if n <= 8:
         algos += [(k_.GEMM_GEMV, 1)] + ([(k_.GEMM_GEMV, 2)] if k >= 2048 else [])
+        if m % 2 == 0 and k % (4 if dtype == torch.float32 else 8) == 0:
+            algos.append((k_.GEMM_GEMV_LDS, 1))
     for algo, ns in algos:
         y = torch.full((ns, n, m), float("nan"), device=DEV)
         k_.gemm(x, w, y, algo, ns)
@@ -191,6 +194,69 @@ def test_gemm_kernels_against_plain(n, m, k, dtype):
         y = torch.empty(n, m, dtype=dtype, device=DEV)
         k_.gemm(x, w, y, k_.GEMM_MFMA_BF16)
         assert (y.cpu().double() - want).abs().max() < 0.01 * want.abs().max()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,f,k", [(1, 176, 64), (3, 120, 88), (8, 5632, 2048), (5, 33, 4104)])
+def test_gemv_swiglu(dtype, n, f, k):
+    x, w = rnd(n, k, seed=1, dtype=dtype, scale=0.5), rnd(2 * f, k, seed=2, dtype=dtype, scale=0.1)
+    h = torch.full((n, f), float("nan"), dtype=dtype, device=DEV)
+    K().gemv_swiglu(x, w, h)
+    xd, wd = x.cpu().double(), w.cpu().double()
+    want = P.silu(P.linear(xd, wd[:f])) * P.linear(xd, wd[f:])
+    assert (h.cpu().double() - want).abs().max() < (1e-4 if dtype == torch.float32 else 0.01 * want.abs().max() + 1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,KV,hd,ps,d", [(4, 2, 16, 16, 64), (3, 1, 32, 16, 96), (5, 5, 48, 32, 88), (32, 4, 64, 16, 2048)])
+def test_gemv_rope_append(dtype, H, KV, hd, ps, d):
+    """Projections, rotation and append in one launch, against the plain functions."""
+    theta = 10000.0
+    spans = [(37, 3), (0, 2), (ps - 1, 1)]                # six tokens of three requests
+    n = sum(l for _, l in spans)
+    pos = torch.tensor([p0 + i for p0, l in spans for i in range(l)], dtype=torch.int32, device=DEV)
+    sot = torch.tensor([s for s, (_, l) in enumerate(spans) for _ in range(l)], dtype=torch.int32, device=DEV)
+    tables = [[9, 4, 11], [2, -1, -1], [7, -1, -1]]
+    bt = torch.tensor(tables, dtype=torch.int32, device=DEV)
+    qd, kvd = H * hd, KV * hd
+    x = rnd(n, d, seed=3, dtype=dtype, scale=0.5)
+    w = rnd(qd + 2 * kvd, d, seed=4, dtype=dtype, scale=0.1)
+    cos = torch.empty(n, hd // 2, device=DEV)
+    sin = torch.empty(n, hd // 2, device=DEV)
+    K().rope_tables(cos, sin, pos, hd, theta)
+    cache = torch.full((12, 2, KV, ps * hd), float("nan"), dtype=dtype, device=DEV)
+    q_out = torch.full((n, qd), float("nan"), dtype=dtype, device=DEV)
+    K().gemv_rope_append(x, w, q_out, cos, sin, cache, pos, sot, bt, ps, H, KV, hd)
+    full = P.linear(x.cpu().double(), w.cpu().double())
+    want_q = P.rope(full[:, :qd], pos.cpu().tolist(), H, hd, theta)
+    want_k = P.rope(full[:, qd:qd + kvd], pos.cpu().tolist(), KV, hd, theta)
+    want_v = full[:, qd + kvd:]
+    t = 1e-4 if dtype == torch.float32 else 3e-2
+    assert (q_out.cpu().double() - want_q).abs().max() < t
+    off = 0
+    for s, (p0, l) in enumerate(spans):
+        k, v = read_cache(cache, tables[s], p0 + l, KV, hd, ps)
+        assert (k[p0:].double() - want_k[off:off + l]).abs().max() < t
+        assert (v[p0:].double() - want_v[off:off + l]).abs().max() < t
+        assert torch.isnan(k[:p0]).all() and torch.isnan(v[:p0]).all()
+        off += l
+    # query only (a run that reads another run's cache), without rotation
+    q2 = torch.full((n, qd), float("nan"), dtype=dtype, device=DEV)
+    K().gemv_rope_append(x, w[:qd].contiguous(), q2, None, None, None, None, None, None, ps, H, KV, hd)
+    assert (q2.cpu().double() - full[:, :qd]).abs().max() < t
+
+
+def test_fused_gemv_refuses_what_it_does_not_take():
+    k_ = K()
+    x = rnd(9, 64, dtype=torch.bfloat16)
+    with pytest.raises(k_.KernelError, match="outside"):
+        k_.gemv_swiglu(x, rnd(32, 64, dtype=torch.bfloat16), torch.empty(9, 16, dtype=torch.bfloat16, device=DEV))
+    x = rnd(2, 60, dtype=torch.bfloat16)
+    with pytest.raises(k_.KernelError, match="multiple of 8"):
+        k_.gemv_swiglu(x, rnd(32, 60, dtype=torch.bfloat16), torch.empty(2, 16, dtype=torch.bfloat16, device=DEV))
+    assert not k_.gemv_fits(2, 131, 64, torch.bfloat16) and not k_.gemv_fits(9, 64, 64, torch.float32)
+    assert k_.gemv_fits(8, 64, 100, torch.float32) and not k_.gemv_fits(4, 64, 100, torch.bfloat16)
+    assert k_.gemv_fits(4, 64, 64, torch.bfloat16) and not k_.gemv_fits(5, 64, 64, torch.bfloat16)
 
 
 def test_gemm_refuses_what_it_does_not_take():
@@ -209,20 +275,23 @@ def test_gemm_refuses_what_it_does_not_take():
 def test_linear_chooses_a_kernel_for_every_size():
     from kllm_amd.parts.linear import choose
     k_ = K()
-    assert choose(torch.float32, 1, 64, 64)[0] == k_.GEMM_GEMV
+    assert choose(torch.float32, 1, 64, 64)[0] == k_.GEMM_GEMV_LDS
+    assert choose(torch.float32, 1, 65, 64)[0] == k_.GEMM_GEMV          # odd number of rows of W
+    assert choose(torch.bfloat16, 4, 2560, 2048) == (k_.GEMM_GEMV_LDS, 1)
+    assert choose(torch.float32, 8, 2560, 2048) == (k_.GEMM_GEMV_LDS, 1)
+    assert choose(torch.bfloat16, 8, 2560, 2048) == (k_.GEMM_SKINNY_BF16, 16)
     assert choose(torch.float32, 100, 64, 64)[0] == k_.GEMM_TILED_F32
     assert choose(torch.bfloat16, 40, 64, 64)[0] == k_.GEMM_SKINNY_BF16
     assert choose(torch.bfloat16, 40, 64, 60)[0] == k_.GEMM_PLAIN          # K not a multiple of 8
-    assert choose(torch.bfloat16, 8, 2560, 2048) == (k_.GEMM_SKINNY_BF16, 16)
     assert choose(torch.bfloat16, 64, 2048, 5632) == (k_.GEMM_SKINNY_BF16, 11)
-    assert choose(torch.bfloat16, 3, 32000, 2048) == (k_.GEMM_GEMV, 1)
+    assert choose(torch.bfloat16, 3, 32001, 2048) == (k_.GEMM_GEMV, 1)
     for n, m, k in [(5, 100, 72), (64, 2048, 5632), (33, 96, 176), (9, 320, 520), (20, 64, 4104)]:
         ns = choose(torch.bfloat16, n, m, k)[1]
         kslice = -(-(-(-k // ns)) // 32) * 32
         assert kslice <= 512 and kslice * (ns - 1) < k, (n, m, k, ns)
     assert choose(torch.bfloat16, 400, 64, 64)[0] == k_.GEMM_MFMA_BF16
     assert choose(torch.bfloat16, 400, 64, 64, {"gemm": "library"})[0] == "library"
-    a, ns = choose(torch.bfloat16, 1, 2048, 5632)
+    a, ns = choose(torch.bfloat16, 1, 2049, 5632)
     assert a == k_.GEMM_GEMV and 1 <= ns <= 16
 
 

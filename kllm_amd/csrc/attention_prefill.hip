@@ -6,7 +6,8 @@
 // this step has just written alike, so a prompt's portion at a position > 0
 // needs no other path.  Running maximum and sum per query (online softmax), no
 // score matrix in memory, context bounded by pages only.  Formulas as in the
-// generic kernel (reference: backend/model.cu:343-408, window :224-225).
+// generic kernel (reference: backend/model.cu:343-408, window :224-225), in
+// 32-bit; probabilities are rounded to bfloat16 for the product with the values.
 //
 // The scores are computed transposed, S^T = K Q^T, so that a query is a
 // column: MFMA 32x32x16, lane l (g = l/32, c = l%32) holds A[c][8g..8g+7],
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void attn_prefill_mfma_kernel(
   const int g = lane / 32, c = lane % 32;
   const long item = (long)blockIdx.x * kPrefillWaves + wave;   // (tile, head), head fastest
   if (item >= (long)n_tiles * H) return;
-  const int tile = item / H, h = item % H;
+  const int tile = n_tiles - 1 - (int)(item / H), h = item % H;   // later tiles read more keys: start them first
   const int kvh = h / (H / KV);
   const int t0 = query_tiles[2 * tile], span = query_tiles[2 * tile + 1];
   const int s_begin = span_start[span], s_end = span_start[span + 1];
@@ -54,6 +55,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void attn_prefill_mfma_kernel(
   const int* table = block_table + (long)span * max_pages;
   const long block = (long)page_size * hd;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const float c2 = scale * 1.4426950408889634f;             // scale * log2(e)
 
   bf16x8 qb[KS];
 #pragma unroll
@@ -67,73 +69,126 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void attn_prefill_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[r][i] = 0.f;
 
-  for (int kb = lowest / 32 * 32; kb <= qpos_max; kb += 32) {
-    // ---- scores: this lane's key row is kb + c
+  // One tile's operands.  The loads of tile i+1 go out before tile i is
+  // computed; its page ids were read one tile earlier still.
+  struct Tile {
+    bf16x8 k[KS];
+    bf16x4 vlo[HDT][2], vhi[HDT][2];
+    bool row_ok, live[2];
+  };
+  const int kb0 = lowest / 32 * 32;
+  const int first_page_key = lowest / page_size * page_size;   // pages before this may be gone
+  auto pages_of = [&](int kb, int& prow, int& p0, int& p1) {
     const int key_row = kb + c;
-    const bool row_live = key_row < kv_len && key_row >= lowest / page_size * page_size;
-    int page = 0;
-    if (row_live) page = table[key_row / page_size];
-    const bool row_ok = row_live && page >= 0;
-    const bf16_t* krow = cache + (((long)page * 2 + 0) * KV + kvh) * block + (long)(key_row % page_size) * hd;
+    const bool in = kb <= qpos_max;
+    prow = (in && key_row < kv_len && key_row >= first_page_key) ? table[key_row / page_size] : -1;
+    p0 = (in && kb < kv_len && kb + 16 > lowest) ? table[kb / page_size] : -1;
+    p1 = (in && kb + 16 < kv_len && kb + 32 > lowest) ? table[(kb + 16) / page_size] : -1;
+  };
+  auto fetch = [&](int kb, int prow, int p0, int p1) -> Tile {
+    Tile T;
+    const int key_row = kb + c;
+    T.row_ok = prow >= 0;
+    const bf16_t* krow = cache + (((long)(T.row_ok ? prow : 0) * 2 + 0) * KV + kvh) * block +
+                         (long)(key_row % page_size) * hd;
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk)
+      T.k[kk] = T.row_ok ? *reinterpret_cast<const bf16x8*>(krow + 16 * kk + 8 * g) : zero8;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int vp = u ? p1 : p0;
+      const int k0 = kb + 16 * u;
+      T.live[u] = vp >= 0;
+      const bf16_t* vbase = cache + (((long)(T.live[u] ? vp : 0) * 2 + 1) * KV + kvh) * block + (k0 % page_size);
+#pragma unroll
+      for (int r = 0; r < HDT; ++r) {
+        const bf16_t* vrow = vbase + (long)(32 * r + c) * page_size;
+        T.vlo[r][u] = T.live[u] ? *reinterpret_cast<const bf16x4*>(vrow + 4 * g) : bf16x4{0, 0, 0, 0};
+        T.vhi[r][u] = T.live[u] ? *reinterpret_cast<const bf16x4*>(vrow + 8 + 4 * g) : bf16x4{0, 0, 0, 0};
+      }
+    }
+    return T;
+  };
+
+  int prow, pg0, pg1;
+  pages_of(kb0, prow, pg0, pg1);
+  Tile nxt = fetch(kb0, prow, pg0, pg1);
+  pages_of(kb0 + 32, prow, pg0, pg1);
+  for (int kb = kb0; kb <= qpos_max; kb += 32) {
+    const Tile cur = nxt;
+    nxt = fetch(kb + 32, prow, pg0, pg1);
+    pages_of(kb + 64, prow, pg0, pg1);
+    // ---- scores: this lane's key row is kb + c
     floatx16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
 #pragma unroll
-    for (int kk = 0; kk < KS; ++kk) {
-      const bf16x8 a = row_ok ? *reinterpret_cast<const bf16x8*>(krow + 16 * kk + 8 * g) : zero8;
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qb[kk], s, 0, 0, 0);
-    }
-    // ---- mask, maximum, probabilities
+    for (int kk = 0; kk < KS; ++kk)
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur.k[kk], qb[kk], s, 0, 0, 0);
+    // ---- mask (only where a tile touches an edge), maximum, probabilities.
+    // exp(x) is taken as exp2(x * log2 e) with the hardware's exp2.
     const bool inner = kb >= my_start && kb + 31 <= qpos && kb + 32 <= kv_len;   // no mask needed
-    float tmax = -INFINITY;
+    if (__any(!inner)) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int key = kb + 8 * (i / 4) + 4 * g + i % 4;
-      const bool ok = inner || (key <= qpos && key >= my_start);
-      s[i] = ok ? s[i] * scale : -INFINITY;
-      tmax = fmaxf(tmax, s[i]);
+      for (int i = 0; i < 16; ++i) {
+        const int key = kb + 8 * (i / 4) + 4 * g + i % 4;
+        const bool ok = inner || (key <= qpos && key >= my_start);
+        s[i] = ok ? s[i] : -INFINITY;
+      }
     }
+    float tmax = s[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) tmax = fmaxf(tmax, s[i]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-    const float m_new = fmaxf(m, tmax);
-    const float alpha = (m_new == -INFINITY) ? 1.f : expf(m - m_new);
+    const float m_new = fmaxf(m, tmax);                       // in units of raw scores
+    const float mc = (m_new == -INFINITY) ? 0.f : m_new * c2;
+    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m * c2 - mc);
     bf16x8 pb[2];
     float psum = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const float p = (s[i] == -INFINITY) ? 0.f : expf(s[i] - m_new);
-      const bf16_t pr = (bf16_t)p;
-      pb[i / 8][i % 8] = pr;
-      psum += (float)pr;
+      const float p = __builtin_amdgcn_exp2f(fmaf(s[i], c2, -mc));   // exp2(-inf) = 0
+      pb[i / 8][i % 8] = (bf16_t)p;
+      psum += p;
     }
     l = l * alpha + psum;
     m = m_new;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int r = 0; r < HDT; ++r)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[r][i] *= alpha;
+    }
     // ---- values: page u of this tile holds keys kb + 16u .. kb + 16u + 15
     const bool v_edge = kb < lowest || kb + 32 > kv_len;     // slots that may hold anything
+    if (!v_edge) {
 #pragma unroll
-    for (int r = 0; r < HDT; ++r) {
+      for (int r = 0; r < HDT; ++r)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[r][i] *= alpha;
+        for (int u = 0; u < 2; ++u) {
+          bf16x8 a;
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int k0 = kb + 16 * u;
-        const bool live = k0 < kv_len && k0 + 16 > lowest;
-        int vp = 0;
-        if (live) vp = table[k0 / page_size];
-        bf16x8 a = zero8;
-        if (live && vp >= 0) {
-          const bf16_t* vrow = cache + (((long)vp * 2 + 1) * KV + kvh) * block +
-                               (long)(32 * r + c) * page_size + (k0 % page_size);
-          const bf16x4 lo = *reinterpret_cast<const bf16x4*>(vrow + 4 * g);
-          const bf16x4 hi = *reinterpret_cast<const bf16x4*>(vrow + 8 + 4 * g);
+          for (int j = 0; j < 4; ++j) {
+            a[j] = cur.vlo[r][u][j];
+            a[4 + j] = cur.vhi[r][u][j];
+          }
+          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[u], acc[r], 0, 0, 0);
+        }
+    } else {
+#pragma unroll
+      for (int r = 0; r < HDT; ++r)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int k0 = kb + 16 * u;
+          bf16x8 a;
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const int key_lo = k0 + 4 * g + j, key_hi = k0 + 8 + 4 * g + j;
-            a[j] = (!v_edge || (key_lo >= lowest && key_lo < kv_len)) ? lo[j] : (bf16_t)0.f;
-            a[4 + j] = (!v_edge || (key_hi >= lowest && key_hi < kv_len)) ? hi[j] : (bf16_t)0.f;
+            a[j] = (cur.live[u] && key_lo >= lowest && key_lo < kv_len) ? cur.vlo[r][u][j] : (bf16_t)0.f;
+            a[4 + j] = (cur.live[u] && key_hi >= lowest && key_hi < kv_len) ? cur.vhi[r][u][j] : (bf16_t)0.f;
           }
+          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[u], acc[r], 0, 0, 0);
         }
-        acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[u], acc[r], 0, 0, 0);
-      }
     }
   }
 

@@ -60,29 +60,49 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TIN* __restrict_
   const long src = rows ? rows[r] : r;
   float* xr = x + src * d;
   const TIN* dr = delta ? delta + src * d : nullptr;
-  float keep[KEEP];
+  const int tid = threadIdx.x, T = blockDim.x;
+  // The first KEEP*T elements: every load of the thread goes out before any sum.
+  float keep[KEEP], wkeep[KEEP];
+#pragma unroll
+  for (int it = 0; it < KEEP; ++it) {
+    const int i = tid + it * T;
+    keep[it] = i < d ? xr[i] : 0.f;
+    wkeep[it] = (out && i < d) ? w[i] : 0.f;
+  }
+  if (dr) {
+#pragma unroll
+    for (int it = 0; it < KEEP; ++it) {
+      const int i = tid + it * T;
+      if (i < d) keep[it] += sum_splits(dr + i, nsplit, split_stride);
+    }
+  }
   float ss = 0.f;
-  int it = 0;
-  for (int i = threadIdx.x; i < d; i += blockDim.x, ++it) {
+#pragma unroll
+  for (int it = 0; it < KEEP; ++it) {
+    const int i = tid + it * T;
+    if (i < d) {
+      if (write_x) xr[i] = keep[it];
+      ss += keep[it] * keep[it];
+    }
+  }
+  for (int i = tid + KEEP * T; i < d; i += T) {   // rows longer than KEEP*T
     float v = xr[i];
     if (dr) v += sum_splits(dr + i, nsplit, split_stride);
     if (write_x) xr[i] = v;
-    if (it < KEEP) keep[it] = v;
     ss += v * v;
   }
   if (!out) return;
   ss = block_sum(ss, red);
   const float scale = rsqrtf(ss / (float)d + eps);
   TOUT* orow = out + r * d;
-  it = 0;
-  for (int i = threadIdx.x; i < d; i += blockDim.x, ++it) {
-    float v;
-    if (it < KEEP) {
-      v = keep[it];
-    } else {
-      v = xr[i];  // already the sum when write_x (same thread wrote it)
-      if (dr && !write_x) v += sum_splits(dr + i, nsplit, split_stride);
-    }
+#pragma unroll
+  for (int it = 0; it < KEEP; ++it) {
+    const int i = tid + it * T;
+    if (i < d) orow[i] = from_f32<TOUT>(keep[it] * scale * wkeep[it]);
+  }
+  for (int i = tid + KEEP * T; i < d; i += T) {
+    float v = xr[i];  // already the sum when write_x (same thread wrote it)
+    if (dr && !write_x) v += sum_splits(dr + i, nsplit, split_stride);
     orow[i] = from_f32<TOUT>(v * scale * w[i]);
   }
 }

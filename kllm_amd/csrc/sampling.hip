@@ -12,75 +12,92 @@
 
 namespace kllm {
 
-constexpr int kSampleThreads = 256;
+constexpr int kSampleThreads = 1024;
+constexpr int kSampleWaves = kSampleThreads / kWave;
+
+// (value, index) with the larger value, the smaller index on equal values
+__device__ __forceinline__ void better(float& v, int& i, float ov, int oi) {
+  if (ov > v || (ov == v && oi < i)) {
+    v = ov;
+    i = oi;
+  }
+}
 
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     int* __restrict__ out, const float* __restrict__ logits, const float* __restrict__ temperature,
     const float* __restrict__ uniform, int vocab) {
-  __shared__ float red[16];
-  __shared__ float best_val[kSampleThreads];
-  __shared__ int best_idx[kSampleThreads];
-  __shared__ float partial[kSampleThreads];
+  __shared__ float wave_val[kSampleWaves];
+  __shared__ int wave_idx[kSampleWaves];
+  __shared__ float wave_tot[kSampleWaves];
   __shared__ int chosen;
 
-  const int r = blockIdx.x, tid = threadIdx.x;
+  const int r = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const float* row = logits + (long)r * vocab;
   // Each thread owns one contiguous segment, so thread order is index order.
   const int seg = (vocab + kSampleThreads - 1) / kSampleThreads;
   const int lo = min(tid * seg, vocab), hi = min(lo + seg, vocab);
 
   float bv = -INFINITY;
-  int bi = vocab;  // "none"
+  int bi = vocab;  // "none": loses against every index
   for (int i = lo; i < hi; ++i) {
     const float v = row[i];
-    if (bi == vocab || v > bv) { bv = v; bi = i; }  // strict: the first maximum stays
+    if (bi == vocab || v > bv) { bv = v; bi = i; }   // strict: the first maximum stays
   }
-  best_val[tid] = bv;
-  best_idx[tid] = bi;
-  __syncthreads();
-  if (tid == 0) {
-    float v = best_val[0];
-    int idx = best_idx[0];
-    for (int i = 1; i < kSampleThreads; ++i)
-      if (best_idx[i] < vocab && (idx == vocab || best_val[i] > v)) { v = best_val[i]; idx = best_idx[i]; }
-    best_val[0] = v;
-    chosen = idx;
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, kWave);
+    const int oi = __shfl_xor(bi, off, kWave);
+    if (oi < vocab && (bi == vocab || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
   }
+  if (lane == 0) {
+    wave_val[wave] = bv;
+    wave_idx[wave] = bi;
+  }
+  if (tid == 0) chosen = vocab - 1;
   __syncthreads();
+  float mx = wave_val[0];
+  int arg = wave_idx[0];
+  for (int w = 1; w < kSampleWaves; ++w)
+    if (wave_idx[w] < vocab && (arg == vocab || wave_val[w] > mx)) { mx = wave_val[w]; arg = wave_idx[w]; }
   const float temp = temperature ? temperature[r] : 0.f;
   if (!(temp > 0.f)) {
-    if (tid == 0) out[r] = chosen;
+    if (tid == 0) out[r] = arg;
     return;
   }
-  const float mx = best_val[0];
   const float inv_t = 1.f / temp;
   float sum = 0.f;
   for (int i = lo; i < hi; ++i) sum += expf((row[i] - mx) * inv_t);
-  partial[tid] = sum;
-  __syncthreads();
-  if (tid == 0) {
-    float total = 0.f;
-    for (int i = 0; i < kSampleThreads; ++i) total += partial[i];
-    const float target = uniform[r] * total;
-    // Segment that holds the target, then the element inside it.
-    float before = 0.f;
-    int owner = -1;
-    for (int i = 0; i < kSampleThreads; ++i) {
-      if (target < before + partial[i]) { owner = i; break; }
-      before += partial[i];
-    }
-    int idx = vocab - 1;
-    if (owner >= 0) {
-      const int olo = min(owner * seg, vocab), ohi = min(olo + seg, vocab);
-      float c = before;
-      idx = ohi - 1;
-      for (int i = olo; i < ohi; ++i) {
-        c += expf((row[i] - mx) * inv_t);
-        if (target < c) { idx = i; break; }
-      }
-    }
-    out[r] = idx;
+  // inclusive scan over the wave, then over the waves: thread t's probability
+  // mass lies in [incl - sum, incl)
+  float incl = sum;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const float up = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += up;
   }
+  if (lane == kWave - 1) wave_tot[wave] = incl;
+  __syncthreads();
+  float before = 0.f, total = 0.f;
+  for (int w = 0; w < kSampleWaves; ++w) {
+    if (w < wave) before += wave_tot[w];
+    total += wave_tot[w];
+  }
+  // excl is the previous thread's incl, bit for bit: the ranges leave no gap
+  const float prev = __shfl_up(incl, 1, kWave);
+  const float excl = before + (lane == 0 ? 0.f : prev);
+  incl += before;
+  const float target = uniform[r] * total;
+  if (sum > 0.f && target >= excl && target < incl) {
+    float c = excl;
+    int idx = hi - 1;
+    for (int i = lo; i < hi; ++i) {
+      c += expf((row[i] - mx) * inv_t);
+      if (target < c) { idx = i; break; }
+    }
+    chosen = idx;
+  }
+  __syncthreads();
+  if (tid == 0) out[r] = chosen;
 }
 
 }  // namespace kllm

@@ -116,7 +116,11 @@ __global__ __launch_bounds__(256) void gemm_f32_tiled_kernel(const float* __rest
 constexpr int MBM = 128, MBN = 128, MBK = 32;
 constexpr int MLD = MBK + 8;  // LDS row stride in elements (80 bytes: 16-byte reads stay conflict-free)
 
-template <typename TOUT>
+// DUAL: W is [gate rows; up rows] = [2m, k]; a workgroup takes 64 gate rows and
+// the 64 up rows that belong to them, and writes silu(gate) * up for m columns
+// (reference: backend/model.cu:477-483, :1112-1114) -- the gated activation
+// never exists in 32-bit in memory.
+template <typename TOUT, bool DUAL>
 __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ X,
                                                              const bf16_t* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
@@ -125,10 +129,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
   __shared__ __attribute__((aligned(16))) bf16_t Ws[2][MBN * MLD];
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int wr = wave / 2, wc = wave % 2;
-  const long row0 = (long)blockIdx.y * MBM, col0 = (long)blockIdx.x * MBN;
+  const long row0 = (long)blockIdx.y * MBM, col0 = (long)blockIdx.x * (DUAL ? MBN / 2 : MBN);
 
   // Loads of one stage: 128 rows x 4 chunks of 8 elements per operand; each
-  // thread takes chunk (tid % 4) of rows tid/4 and tid/4 + 64.
+  // thread takes chunk (tid % 4) of rows tid/4 and tid/4 + 64.  DUAL: LDS rows
+  // 0..63 of W are gate rows, 64..127 the up rows of the same columns.
   const int lrow = tid / 4, lchunk = (tid % 4) * 8;
   bf16x8 xreg[2], wreg[2];
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -136,10 +141,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
   auto load_stage = [&](int k0) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const long xr = row0 + lrow + h * 64, wrow = col0 + lrow + h * 64;
+      const long xr = row0 + lrow + h * 64;
+      const long wcol = DUAL ? col0 + lrow : col0 + lrow + h * 64;   // output column
+      const long wrow = DUAL ? wcol + (long)h * m : wcol;
       const int kk = k0 + lchunk;
       xreg[h] = (xr < n && kk < k) ? *reinterpret_cast<const bf16x8*>(X + xr * k + kk) : zero;
-      wreg[h] = (wrow < m && kk < k) ? *reinterpret_cast<const bf16x8*>(W + wrow * k + kk) : zero;
+      wreg[h] = (wcol < m && kk < k) ? *reinterpret_cast<const bf16x8*>(W + wrow * k + kk) : zero;
     }
   };
   auto store_stage = [&](int buf) {
@@ -175,7 +182,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
 #pragma unroll
       for (int j = 0; j < 2; ++j)
         b[j] = *reinterpret_cast<const bf16x8*>(
-            &Ws[cur][(wc * 64 + j * 32 + lane % 32) * MLD + ks + (lane / 32) * 8]);
+            &Ws[cur][((DUAL ? j * 64 + wc * 32 : wc * 64 + j * 32) + lane % 32) * MLD + ks + (lane / 32) * 8]);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -188,6 +195,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
     }
   }
 
+  if (DUAL) {
+    const long c = col0 + wc * 32 + lane % 32;
+    if (c >= m) return;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const long r = row0 + wr * 64 + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+        const float gate = acc[i][0][e], up = acc[i][1][e];
+        if (r < n) Y[r * m + c] = from_f32<TOUT>((gate / (1.f + expf(-gate))) * up);
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -471,10 +491,10 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
                  "gemm mfma: K=%d must be a multiple of 8 and the operands 16-byte aligned", k);
     const dim3 grid(ceil_div(m, MBN), ceil_div(n, MBM));
     if (out_dtype == DT_F32)
-      hipLaunchKernelGGL((gemm_bf16_mfma_kernel<float>), grid, dim3(256), 0, stream,
+      hipLaunchKernelGGL((gemm_bf16_mfma_kernel<float, false>), grid, dim3(256), 0, stream,
                          (const bf16_t*)x, (const bf16_t*)w, (float*)y, n, m, k);
     else
-      hipLaunchKernelGGL((gemm_bf16_mfma_kernel<bf16_t>), grid, dim3(256), 0, stream,
+      hipLaunchKernelGGL((gemm_bf16_mfma_kernel<bf16_t, false>), grid, dim3(256), 0, stream,
                          (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, n, m, k);
     KLLM_CHECK_LAUNCH("gemm mfma");
     return 0;
@@ -560,4 +580,19 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
     return 0;
   }
   KLLM_FAIL(ERR_ARG, "gemm: unknown algorithm %d", algo);
+}
+
+extern "C" int kllm_gemm_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f, int k,
+                                int dtype, hipStream_t stream) {
+  KLLM_REQUIRE(x && w_gate_up && h, "gemm_swiglu: null pointer");
+  KLLM_REQUIRE(n > 0 && f > 0 && k > 0, "gemm_swiglu: bad sizes n=%d f=%d k=%d", n, f, k);
+  KLLM_REQUIRE(dtype == DT_BF16, "gemm_swiglu: bfloat16 only");
+  KLLM_REQUIRE(k % 8 == 0 && aligned16(x) && aligned16(w_gate_up),
+               "gemm_swiglu: K=%d must be a multiple of 8 and the operands 16-byte aligned", k);
+  KLLM_REQUIRE((long)n * f < (1L << 31), "gemm_swiglu: sizes overflow");
+  const dim3 grid(ceil_div(f, MBN / 2), ceil_div(n, MBM));
+  hipLaunchKernelGGL((gemm_bf16_mfma_kernel<bf16_t, true>), grid, dim3(256), 0, stream,
+                     (const bf16_t*)x, (const bf16_t*)w_gate_up, (bf16_t*)h, n, f, k);
+  KLLM_CHECK_LAUNCH("gemm_swiglu");
+  return 0;
 }

@@ -69,6 +69,10 @@ int kllm_sum_splits(const float* in, int nsplit, long count, void* out, int out_
 int kllm_gemm(const void* x, const void* w, void* y, int n, int m, int k, int dtype, int out_dtype,
               int algo, int nsplit, hipStream_t stream);
 
+/* h[n][f] = silu(x . w[0:f]^T) * (x . w[f:2f]^T) on the MFMA tiles, bfloat16. */
+int kllm_gemm_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f, int k, int dtype,
+                     hipStream_t stream);
+
 /* Products for up to 8 rows of x with the whole of K in one wave (no partial
  * sums) and the next elementwise step in the epilogue.  m even, K a multiple
  * of 8 (bfloat16) or 4 (float32).

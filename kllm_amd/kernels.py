@@ -84,6 +84,7 @@ def _declare(lib):
         "kllm_silu_mul": [P, I, I, L, P, I, I, I, P],
         "kllm_gemm": [P, P, P, I, I, I, I, I, I, I, P],
         "kllm_sum_splits": [P, I, L, P, I, P],
+        "kllm_gemm_swiglu": [P, P, P, I, I, I, I, P],
         "kllm_gemv_plain": [P, P, P, I, I, I, I, P],
         "kllm_gemv_swiglu": [P, P, P, I, I, I, I, P],
         "kllm_gemv_rope_append": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
@@ -260,6 +261,16 @@ def gemv_fits(n, m, k, dtype) -> bool:
     v = 4 if dtype == torch.float32 else 8
     most = GEMV_MAX_ROWS if dtype == torch.float32 else GEMV_BEST_ROWS
     return n <= most and m % 2 == 0 and k % v == 0
+
+
+def gemm_swiglu(x, w_gate_up, h):
+    """h [n, f] = silu(x . gate^T) * (x . up^T) on the MFMA tiles (bfloat16, any n)."""
+    n, k = x.shape
+    f = h.shape[1]
+    if tuple(w_gate_up.shape) != (2 * f, k) or h.shape[0] != n or x.dtype != w_gate_up.dtype or h.dtype != x.dtype:
+        raise KernelError("gemm_swiglu: shapes or dtypes do not fit")
+    _check(library().kllm_gemm_swiglu(_ptr(x, "gemm x"), _ptr(w_gate_up, "gemm w"), _ptr(h, "gemm h"), n, f, k,
+                                      dtype_code(x.dtype), _stream()), "gemm_swiglu")
 
 
 def gemv_swiglu(x, w_gate_up, h):

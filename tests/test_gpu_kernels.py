@@ -207,6 +207,17 @@ def test_gemv_swiglu(dtype, n, f, k):
     assert (h.cpu().double() - want).abs().max() < (1e-4 if dtype == torch.float32 else 0.01 * want.abs().max() + 1e-3)
 
 
+@pytest.mark.parametrize("n,f,k", [(65, 176, 64), (130, 120, 88), (300, 515, 264), (128, 5632, 2048)])
+def test_gemm_swiglu(n, f, k):
+    dtype = torch.bfloat16
+    x, w = rnd(n, k, seed=1, dtype=dtype, scale=0.5), rnd(2 * f, k, seed=2, dtype=dtype, scale=0.1)
+    h = torch.full((n, f), float("nan"), dtype=dtype, device=DEV)
+    K().gemm_swiglu(x, w, h)
+    xd, wd = x.cpu().double(), w.cpu().double()
+    want = P.silu(P.linear(xd, wd[:f])) * P.linear(xd, wd[f:])
+    assert (h.cpu().double() - want).abs().max() < 0.01 * want.abs().max() + 1e-3
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,KV,hd,ps,d", [(4, 2, 16, 16, 64), (3, 1, 32, 16, 96), (5, 5, 48, 32, 88), (32, 4, 64, 16, 2048)])
 def test_gemv_rope_append(dtype, H, KV, hd, ps, d):

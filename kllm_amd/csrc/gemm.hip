@@ -113,113 +113,179 @@ __global__ __launch_bounds__(256) void gemm_f32_tiled_kernel(const float* __rest
 // stages.  Four waves in 2 x 2, each 64 x 64 = 2 x 2 MFMA tiles of 32 x 32.
 // MFMA 32x32x16: lane l holds A[l%32][8*(l/32) .. +8], B[8*(l/32) .. +8][l%32]
 // and D[8*(i/4) + 4*(l/32) + i%4][l%32] for i = 0..15.
-constexpr int MBM = 128, MBN = 128, MBK = 32;
+constexpr int MBN = 128, MBK = 32;
 constexpr int MLD = MBK + 8;  // LDS row stride in elements (80 bytes: 16-byte reads stay conflict-free)
 
 // DUAL: W is [gate rows; up rows] = [2m, k]; a workgroup takes 64 gate rows and
 // the 64 up rows that belong to them, and writes silu(gate) * up for m columns
 // (reference: backend/model.cu:477-483, :1112-1114) -- the gated activation
 // never exists in 32-bit in memory.
+//
+// Global loads run three stages ahead of the MFMAs (three register sets in
+// rotation, two LDS stages), so that a stage's loads have two stages of
+// compute to arrive.  Workgroups are numbered so that the eight XCDs (which
+// take workgroups round-robin, each with an L2 of its own) each get a
+// contiguous run of tiles that share rows of X.
 template <typename TOUT, bool DUAL>
 __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ X,
                                                              const bf16_t* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
-                                                             int k) {
-  __shared__ __attribute__((aligned(16))) bf16_t Xs[2][MBM * MLD];
-  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][MBN * MLD];
+                                                             int k, int tiles_x, int tiles_y) {
+  // 32-row MFMA tiles per wave.  4 (a 256-row workgroup tile) halves the traffic per flop
+  // but needs 268 registers, one wave per SIMD, and measured 15% slower than 2.
+  constexpr int WTM = 2;
+  constexpr int BM = 64 * WTM;                  // rows of X per workgroup
+  constexpr int XPASS = BM / 64;                // loads of X per thread and stage
+  extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
+  bf16_t* Xs = lds;                             // [2][BM * MLD]
+  bf16_t* Ws = lds + 2 * BM * MLD;              // [2][MBN * MLD]
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int wr = wave / 2, wc = wave % 2;
-  const long row0 = (long)blockIdx.y * MBM, col0 = (long)blockIdx.x * (DUAL ? MBN / 2 : MBN);
+  const long total = (long)tiles_x * tiles_y;
+  const long per_xcd = (total + 7) / 8;
+  const long id = (long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (id >= total) return;
+  // An XCD's run of tiles walks the shorter side fastest: it then reads only its share
+  // of the larger operand and shares the smaller one.
+  const bool x_major = tiles_x >= tiles_y;
+  const long trow = x_major ? id % tiles_y : id / tiles_x;
+  const long tcol = x_major ? id / tiles_y : id % tiles_x;
+  const long row0 = trow * BM, col0 = tcol * (DUAL ? MBN / 2 : MBN);
 
-  // Loads of one stage: 128 rows x 4 chunks of 8 elements per operand; each
-  // thread takes chunk (tid % 4) of rows tid/4 and tid/4 + 64.  DUAL: LDS rows
-  // 0..63 of W are gate rows, 64..127 the up rows of the same columns.
+  // Loads of one stage: rows x 4 chunks of 8 elements per operand; each thread takes
+  // chunk (tid % 4) of rows tid/4 + 64h.  DUAL: LDS rows 0..63 of W are gate rows,
+  // 64..127 the up rows of the same columns.
   const int lrow = tid / 4, lchunk = (tid % 4) * 8;
-  bf16x8 xreg[2], wreg[2];
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-
-  auto load_stage = [&](int k0) {
+  const bf16_t* xptr[XPASS];
+  const bf16_t* wptr[2];
+  bool xok[XPASS], wok[2];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const long xr = row0 + lrow + h * 64;
-      const long wcol = DUAL ? col0 + lrow : col0 + lrow + h * 64;   // output column
-      const long wrow = DUAL ? wcol + (long)h * m : wcol;
-      const int kk = k0 + lchunk;
-      xreg[h] = (xr < n && kk < k) ? *reinterpret_cast<const bf16x8*>(X + xr * k + kk) : zero;
-      wreg[h] = (wcol < m && kk < k) ? *reinterpret_cast<const bf16x8*>(W + wrow * k + kk) : zero;
-    }
+  for (int h = 0; h < XPASS; ++h) {
+    const long xr = row0 + lrow + h * 64;
+    xok[h] = xr < n;
+    xptr[h] = X + (xok[h] ? xr : 0) * k + lchunk;
+  }
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const long wcol = DUAL ? col0 + lrow : col0 + lrow + h * 64;   // output column
+    const long wrow = DUAL ? wcol + (long)h * m : wcol;
+    wok[h] = wcol < m;
+    wptr[h] = W + (wok[h] ? wrow : 0) * k + lchunk;
+  }
+  // Loads carry no branch and no select: rows and K offsets outside the matrices are
+  // clamped to valid addresses here and replaced by zeros when the stage is stored, so
+  // that the loop is straight-line code and a store waits only for its own, oldest loads.
+  struct Stage {
+    bf16x8 x[XPASS], w[2];
   };
-  auto store_stage = [&](int buf) {
+  auto load_stage = [&](int kt) -> Stage {
+    Stage st;
+    const int kk = kt * MBK;
+    const int koff = (kk + lchunk < k) ? kk : 0;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      *reinterpret_cast<bf16x8*>(&Xs[buf][(lrow + h * 64) * MLD + lchunk]) = xreg[h];
-      *reinterpret_cast<bf16x8*>(&Ws[buf][(lrow + h * 64) * MLD + lchunk]) = wreg[h];
-    }
+    for (int h = 0; h < XPASS; ++h) st.x[h] = *reinterpret_cast<const bf16x8*>(xptr[h] + koff);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) st.w[h] = *reinterpret_cast<const bf16x8*>(wptr[h] + koff);
+    return st;
+  };
+  auto store_stage = [&](const Stage& st, int kt, int buf) {
+    const bool kin = kt * MBK + lchunk < k;
+#pragma unroll
+    for (int h = 0; h < XPASS; ++h)
+      *reinterpret_cast<bf16x8*>(&Xs[buf * BM * MLD + (lrow + h * 64) * MLD + lchunk]) =
+          (xok[h] && kin) ? st.x[h] : zero;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      *reinterpret_cast<bf16x8*>(&Ws[buf * MBN * MLD + (lrow + h * 64) * MLD + lchunk]) =
+          (wok[h] && kin) ? st.w[h] : zero;
   };
 
-  floatx16 acc[2][2];
+  floatx16 acc[WTM][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WTM; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int ktiles = (k + MBK - 1) / MBK;
-  load_stage(0);
-  store_stage(0);
-  __syncthreads();
-  for (int kt = 0; kt < ktiles; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < ktiles) load_stage((kt + 1) * MBK);
+  auto compute = [&](int cur) {
 #pragma unroll
     for (int ks = 0; ks < MBK; ks += 16) {
-      bf16x8 a[2], b[2];
+      bf16x8 a[WTM], b[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < WTM; ++i)
         a[i] = *reinterpret_cast<const bf16x8*>(
-            &Xs[cur][(wr * 64 + i * 32 + lane % 32) * MLD + ks + (lane / 32) * 8]);
+            &Xs[cur * BM * MLD + (wr * 32 * WTM + i * 32 + lane % 32) * MLD + ks + (lane / 32) * 8]);
 #pragma unroll
       for (int j = 0; j < 2; ++j)
         b[j] = *reinterpret_cast<const bf16x8*>(
-            &Ws[cur][((DUAL ? j * 64 + wc * 32 : wc * 64 + j * 32) + lane % 32) * MLD + ks + (lane / 32) * 8]);
+            &Ws[cur * MBN * MLD + ((DUAL ? j * 64 + wc * 32 : wc * 64 + j * 32) + lane % 32) * MLD + ks +
+                (lane / 32) * 8]);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < WTM; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
     }
-    if (kt + 1 < ktiles) {
-      store_stage(cur ^ 1);  // the other stage was last read before the previous barrier
-      __syncthreads();
-    }
+  };
+
+  const int ktiles = (k + MBK - 1) / MBK;
+  Stage r0 = load_stage(0), r1 = load_stage(1), r2 = load_stage(2);
+  store_stage(r0, 0, 0);
+  __syncthreads();
+  // Stage kt: tile kt is in LDS[kt & 1]; SA holds tile kt+1, SL is free for tile kt+3.
+#define KLLM_GEMM_STAGE(kt_, SA, SL)                                                    \
+  if ((kt_) < ktiles) {                                                                 \
+    SL = load_stage((kt_) + 3);                                                         \
+    compute((kt_) & 1);                                                                 \
+    if ((kt_) + 1 < ktiles) {                                                           \
+      store_stage(SA, (kt_) + 1, ((kt_) + 1) & 1); /* read before the last barrier */   \
+      __syncthreads();                                                                  \
+    }                                                                                   \
   }
+  for (int kt = 0; kt < ktiles; kt += 3) {
+    KLLM_GEMM_STAGE(kt, r1, r0)
+    KLLM_GEMM_STAGE(kt + 1, r2, r1)
+    KLLM_GEMM_STAGE(kt + 2, r0, r2)
+  }
+#undef KLLM_GEMM_STAGE
 
   if (DUAL) {
     const long c = col0 + wc * 32 + lane % 32;
     if (c >= m) return;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WTM; ++i)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const long r = row0 + wr * 64 + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+        const long r = row0 + wr * 32 * WTM + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
         const float gate = acc[i][0][e], up = acc[i][1][e];
         if (r < n) Y[r * m + c] = from_f32<TOUT>((gate / (1.f + expf(-gate))) * up);
       }
     return;
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WTM; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const long c = col0 + wc * 64 + j * 32 + lane % 32;
       if (c >= m) continue;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const long r = row0 + wr * 64 + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+        const long r = row0 + wr * 32 * WTM + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
         if (r < n) Y[r * m + c] = from_f32<TOUT>(acc[i][j][e]);
       }
     }
+}
+
+template <typename TOUT, bool DUAL>
+static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, hipStream_t stream) {
+  const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN), ty = ceil_div(n, 128);
+  const dim3 grid(ceil_div((long)tx * ty, 8) * 8);   // padded so that every XCD gets as many
+  const size_t lds = (size_t)2 * (128 + MBN) * MLD * sizeof(bf16_t);
+  hipLaunchKernelGGL((gemm_bf16_mfma_kernel<TOUT, DUAL>), grid, dim3(256), lds, stream,
+                     (const bf16_t*)x, (const bf16_t*)w, (TOUT*)y, n, m, k, tx, ty);
+  return 0;
 }
 
 // ------------------------------------------------------------------ bf16 MFMA skinny
@@ -489,13 +555,9 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
     KLLM_REQUIRE(nsplit == 1, "gemm mfma: no split");
     KLLM_REQUIRE(k % 8 == 0 && aligned16(x) && aligned16(w),
                  "gemm mfma: K=%d must be a multiple of 8 and the operands 16-byte aligned", k);
-    const dim3 grid(ceil_div(m, MBN), ceil_div(n, MBM));
-    if (out_dtype == DT_F32)
-      hipLaunchKernelGGL((gemm_bf16_mfma_kernel<float, false>), grid, dim3(256), 0, stream,
-                         (const bf16_t*)x, (const bf16_t*)w, (float*)y, n, m, k);
-    else
-      hipLaunchKernelGGL((gemm_bf16_mfma_kernel<bf16_t, false>), grid, dim3(256), 0, stream,
-                         (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, n, m, k);
+    int rc = out_dtype == DT_F32 ? launch_mfma<float, false>(x, w, y, n, m, k, stream)
+                                 : launch_mfma<bf16_t, false>(x, w, y, n, m, k, stream);
+    if (rc) return rc;
     KLLM_CHECK_LAUNCH("gemm mfma");
     return 0;
   }
@@ -590,9 +652,7 @@ extern "C" int kllm_gemm_swiglu(const void* x, const void* w_gate_up, void* h, i
   KLLM_REQUIRE(k % 8 == 0 && aligned16(x) && aligned16(w_gate_up),
                "gemm_swiglu: K=%d must be a multiple of 8 and the operands 16-byte aligned", k);
   KLLM_REQUIRE((long)n * f < (1L << 31), "gemm_swiglu: sizes overflow");
-  const dim3 grid(ceil_div(f, MBN / 2), ceil_div(n, MBM));
-  hipLaunchKernelGGL((gemm_bf16_mfma_kernel<bf16_t, true>), grid, dim3(256), 0, stream,
-                     (const bf16_t*)x, (const bf16_t*)w_gate_up, (bf16_t*)h, n, f, k);
+  if (int rc = launch_mfma<bf16_t, true>(x, w_gate_up, h, n, f, k, stream)) return rc;
   KLLM_CHECK_LAUNCH("gemm_swiglu");
   return 0;
 }

@@ -2,8 +2,9 @@
 //
 // One wave takes one token, one KV head with up to 16 of its query heads, and
 // one slice of the token's keys; it streams that slice's pages from memory
-// once, for all heads of the group, and leaves a partial result (running
-// maximum, sum, unnormalised output).  A second kernel merges the slices.  The
+// once, for all heads of the group.  The four waves of a workgroup merge their
+// results in LDS and leave one partial result (running maximum, sum,
+// unnormalised output); a second kernel merges the workgroups' partials.  The
 // launch does not depend on any context length, so a recorded step can be
 // replayed as contexts grow.
 //
@@ -26,6 +27,8 @@
 namespace kllm {
 
 constexpr int kDecodeWaves = 4;
+// Tiles of 32 keys in a group; two groups are in registers.
+constexpr int decode_ahead(int hdt) { return 1; }
 
 __device__ __forceinline__ float group4_max(float v) {   // over lanes c, c+16, c+32, c+48
   v = fmaxf(v, __shfl_xor(v, 16, kWave));
@@ -44,6 +47,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
     float scale, int head_tiles, const int* __restrict__ token_list) {
   constexpr int hd = 16 * HDT;
   constexpr int KS = (hd + 31) / 32;           // MFMA steps over head_dim for the scores
+  constexpr int kDecodeAhead = decode_ahead(HDT);
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int g = lane / 16, c = lane % 16;
   const int t = token_list ? token_list[blockIdx.x] : blockIdx.x;
@@ -80,16 +84,20 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
 #pragma unroll
   for (int i = 0; i < HDT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  // One tile's operands: the loads of tile i+1 are issued before tile i is
-  // computed, and its page ids were read one tile earlier still.
+  // One tile's operands.
   struct Tile {
     bf16x8 k[2][KS];
     bf16x4 v[2][HDT];
     bool live[2];
   };
+  // Loads carry no branch: a tile or a page that does not exist reads a valid address
+  // (table entry 0, page 0) and is marked dead, so that the compiler can count the loads in
+  // flight and a tile's arithmetic waits for its own operands only.
   auto page_of = [&](int tile, int u) -> int {
     const int k0 = first + tile * 32 + 16 * u;
-    return (tile < tile1 && k0 < len && k0 + 16 > start) ? table[k0 / page_size] : -1;
+    const bool ok = tile < tile1 && k0 < len && k0 + 16 > start;
+    const int page = table[ok ? k0 / page_size : 0];
+    return ok ? page : -1;
   };
   auto fetch = [&](int tile, int page0, int page1) -> Tile {
     Tile T;
@@ -104,25 +112,31 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const int d0 = 32 * ks + 8 * g;
-        T.k[u][ks] = (T.live[u] && d0 < hd) ? *reinterpret_cast<const bf16x8*>(kp + d0) : zero8;
+        T.k[u][ks] = *reinterpret_cast<const bf16x8*>(kp + (d0 < hd ? d0 : 0));
       }
 #pragma unroll
       for (int r = 0; r < HDT; ++r)
-        T.v[u][r] = T.live[u] ? *reinterpret_cast<const bf16x4*>(vp + (long)(16 * r + c) * page_size + 4 * g)
-                              : bf16x4{0, 0, 0, 0};
+        T.v[u][r] = *reinterpret_cast<const bf16x4*>(vp + (long)(16 * r + c) * page_size + 4 * g);
     }
     return T;
   };
 
-  int pg0 = page_of(tile0, 0), pg1 = page_of(tile0, 1);
-  Tile nxt = fetch(tile0, pg0, pg1);
-  pg0 = page_of(tile0 + 1, 0);
-  pg1 = page_of(tile0 + 1, 1);
-  for (int tile = tile0; tile < tile1; ++tile) {
-    const Tile cur = nxt;
-    nxt = fetch(tile + 1, pg0, pg1);
-    pg0 = page_of(tile + 2, 0);
-    pg1 = page_of(tile + 2, 1);
+  // Tiles go in groups of kDecodeAhead: while one group is multiplied the next group's
+  // operands are on their way, and the page ids of the group after that.
+  int pg[kDecodeAhead][2];
+  Tile cur[kDecodeAhead];
+#pragma unroll
+  for (int j = 0; j < kDecodeAhead; ++j) {
+    pg[j][0] = page_of(tile0 + j, 0);
+    pg[j][1] = page_of(tile0 + j, 1);
+  }
+#pragma unroll
+  for (int j = 0; j < kDecodeAhead; ++j) {
+    cur[j] = fetch(tile0 + j, pg[j][0], pg[j][1]);
+    pg[j][0] = page_of(tile0 + kDecodeAhead + j, 0);
+    pg[j][1] = page_of(tile0 + kDecodeAhead + j, 1);
+  }
+  auto compute = [&](const Tile& cur, int tile) {
     const int kb = first + tile * 32;
     const bool edge = kb < start || kb + 32 > len;
     floatx4 s[2];
@@ -130,8 +144,10 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
     for (int u = 0; u < 2; ++u) {
       s[u] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[u][ks], qb[ks], s[u], 0, 0, 0);
+      for (int ks = 0; ks < KS; ++ks) {
+        const bool kin = cur.live[u] && 32 * ks + 8 * g < hd;   // a dead page may hold anything
+        s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kin ? cur.k[u][ks] : zero8, qb[ks], s[u], 0, 0, 0);
+      }
     }
     // ---- online softmax for this lane's head over its 8 keys, then the 4 lanes of the column
     float tmax = -INFINITY;
@@ -175,17 +191,67 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
         }
       acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[r], 0, 0, 0);
     }
+  };
+  for (int tile = tile0; tile < tile1; tile += kDecodeAhead) {
+    Tile nxt[kDecodeAhead];
+#pragma unroll
+    for (int j = 0; j < kDecodeAhead; ++j) {
+      nxt[j] = fetch(tile + kDecodeAhead + j, pg[j][0], pg[j][1]);
+      pg[j][0] = page_of(tile + 2 * kDecodeAhead + j, 0);
+      pg[j][1] = page_of(tile + 2 * kDecodeAhead + j, 1);
+    }
+#pragma unroll
+    for (int j = 0; j < kDecodeAhead; ++j)
+      if (tile + j < tile1) compute(cur[j], tile + j);
+#pragma unroll
+    for (int j = 0; j < kDecodeAhead; ++j) cur[j] = nxt[j];
   }
 
   l = group4_sum(l);
-  if (!head_ok) return;
-  float* out = part + (((long)t * H + head) * nslices + slice) * (hd + 2);
+
+  // ---- the four waves' results meet in LDS; wave 0 merges them in a fixed order and
+  // writes the workgroup's partial result
+  __shared__ float red[(kDecodeWaves - 1) * 16 * (hd + 2)];
+  if (wave > 0) {
+    float* mine = red + ((wave - 1) * 16 + c) * (hd + 2);
+#pragma unroll
+    for (int r = 0; r < HDT; ++r)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mine[16 * r + 4 * g + i] = acc[r][i];
+    if (g == 0) {
+      mine[hd] = m;
+      mine[hd + 1] = l;
+    }
+  }
+  __syncthreads();
+  if (wave > 0 || !head_ok) return;
+  float mj[kDecodeWaves - 1], M = m;
+#pragma unroll
+  for (int j = 0; j < kDecodeWaves - 1; ++j) {
+    mj[j] = red[(j * 16 + c) * (hd + 2) + hd];
+    M = fmaxf(M, mj[j]);
+  }
+  const bool any = M != -INFINITY;                          // a workgroup beyond the last key has nothing
+  const float w0 = any ? expf(m - M) : 0.f;
+  float wj[kDecodeWaves - 1];
+  l *= w0;
+#pragma unroll
+  for (int j = 0; j < kDecodeWaves - 1; ++j) {
+    wj[j] = any ? expf(mj[j] - M) : 0.f;
+    l += wj[j] * red[(j * 16 + c) * (hd + 2) + hd + 1];
+  }
+  float* out = part + (((long)t * H + head) * gridDim.z + blockIdx.z) * (hd + 2);
 #pragma unroll
   for (int r = 0; r < HDT; ++r)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) out[16 * r + 4 * g + i] = acc[r][i];
+    for (int i = 0; i < 4; ++i) {
+      float v = acc[r][i] * w0;
+#pragma unroll
+      for (int j = 0; j < kDecodeWaves - 1; ++j) v += wj[j] * red[(j * 16 + c) * (hd + 2) + 16 * r + 4 * g + i];
+      out[16 * r + 4 * g + i] = v;
+    }
   if (g == 0) {
-    out[hd] = m;
+    out[hd] = M;
     out[hd + 1] = l;
   }
 }
@@ -242,14 +308,15 @@ static void launch_decode(dim3 grid, hipStream_t stream, const void* q, float* p
 using namespace kllm;
 
 extern "C" int kllm_attn_decode_slices(int n, int KV, int H) {
-  // Waves wanted across the chip, shared out over tokens x KV heads x head tiles.
+  // About 2048 waves across the chip, shared out over tokens x KV heads x head tiles; a
+  // workgroup is four waves and leaves one partial result.
   const int head_tiles = (H / KV + 15) / 16;
   long groups = (long)n * KV * head_tiles;
   long want = 2048 / (groups > 0 ? groups : 1);
   int wg = (int)((want + kDecodeWaves - 1) / kDecodeWaves);
   if (wg < 1) wg = 1;
-  if (wg > 4) wg = 4;
-  return wg * kDecodeWaves;
+  if (wg > 16) wg = 16;
+  return wg;
 }
 
 extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part_floats,
@@ -265,15 +332,14 @@ extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part
                "attn_decode: head_dim %d is not built (16..128 in steps of 16, 192, 256)", hd);
   KLLM_REQUIRE(page_size % 16 == 0 && page_size > 0 && max_pages > 0,
                "attn_decode: page_size %d must be a multiple of 16", page_size);
-  KLLM_REQUIRE(nslices >= kDecodeWaves && nslices % kDecodeWaves == 0 && nslices <= 1024,
-               "attn_decode: nslices %d must be a multiple of %d", nslices, kDecodeWaves);
+  KLLM_REQUIRE(nslices >= 1 && nslices <= 256, "attn_decode: nslices %d is outside [1, 256]", nslices);
   KLLM_REQUIRE(window >= 0, "attn_decode: negative window");
   KLLM_REQUIRE(part_floats >= (long)n * H * nslices * (hd + 2), "attn_decode: workspace too small");
   const int head_tiles = (H / KV + 15) / 16;
   KLLM_REQUIRE((long)KV * head_tiles <= 65535 && H <= 65535, "attn_decode: too many heads for the grid");
   KLLM_REQUIRE(!token_list || (n_listed > 0 && n_listed <= n), "attn_decode: bad token list");
   const int count = token_list ? n_listed : n;     // part and out are indexed by token, not by list place
-  const dim3 grid(count, KV * head_tiles, nslices / kDecodeWaves);
+  const dim3 grid(count, KV * head_tiles, nslices);
 #define KLLM_DEC(HDT)                                                                             \
   case HDT:                                                                                       \
     launch_decode<HDT>(grid, stream, q, part, cache, positions, span_of_token, block_table,       \

@@ -49,13 +49,12 @@ __device__ __forceinline__ float sum_splits(const TIN* __restrict__ p, int nspli
 
 // v = x[src] (+ sum of delta splits); optionally x[src] = v;
 // out[r] = v * rsqrt(mean(v^2) + eps) * w   (reference: backend/model.cu:101-122, :144-165)
-template <typename TIN, typename TOUT>
+template <typename TIN, typename TOUT, int KEEP>   // KEEP: elements of the row a thread keeps in registers
 __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TIN* __restrict__ delta, int nsplit,
                                    long split_stride, const float* __restrict__ w,
                                    TOUT* __restrict__ out, const int* __restrict__ rows, int d,
                                    float eps, int write_x) {
   __shared__ float red[16];
-  constexpr int KEEP = 8;  // elements of the row a thread keeps in registers
   const long r = blockIdx.x;
   const long src = rows ? rows[r] : r;
   float* xr = x + src * d;
@@ -69,11 +68,52 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TIN* __restrict_
     keep[it] = i < d ? xr[i] : 0.f;
     wkeep[it] = (out && i < d) ? w[i] : 0.f;
   }
-  if (dr) {
+  if (dr && KEEP > 4) {                                 // long rows: element by element
 #pragma unroll
     for (int it = 0; it < KEEP; ++it) {
       const int i = tid + it * T;
       if (i < d) keep[it] += sum_splits(dr + i, nsplit, split_stride);
+    }
+  } else if (dr) {
+    // Eight partial sums of every kept element are loaded before any is added, so that a
+    // thread's loads wait for each other once per eight splits, not once per element; the
+    // order of additions is that of sum_splits.
+    int s = 0;
+    for (; s + 8 <= nsplit; s += 8) {
+      float t[KEEP][8];
+#pragma unroll
+      for (int it = 0; it < KEEP; ++it) {
+        const int i = tid + it * T;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t[it][j] = i < d ? to_f32(dr[i + (long)(s + j) * split_stride]) : 0.f;
+      }
+#pragma unroll
+      for (int it = 0; it < KEEP; ++it)
+        keep[it] += ((t[it][0] + t[it][1]) + (t[it][2] + t[it][3])) + ((t[it][4] + t[it][5]) + (t[it][6] + t[it][7]));
+    }
+    if (s < nsplit) {                                   // up to seven more, again all loaded first
+      float t[KEEP][7];
+#pragma unroll
+      for (int it = 0; it < KEEP; ++it) {
+        const int i = tid + it * T;
+#pragma unroll
+        for (int j = 0; j < 7; ++j)
+          t[it][j] = (i < d && s + j < nsplit) ? to_f32(dr[i + (long)(s + j) * split_stride]) : 0.f;
+      }
+      const int rest = nsplit - s;
+#pragma unroll
+      for (int it = 0; it < KEEP; ++it) {
+        float v = keep[it];
+        if (rest >= 4) {
+          v += (t[it][0] + t[it][1]) + (t[it][2] + t[it][3]);
+#pragma unroll
+          for (int j = 4; j < 7; ++j) v += t[it][j];    // zeros beyond the last split
+        } else {
+#pragma unroll
+          for (int j = 0; j < 3; ++j) v += t[it][j];
+        }
+        keep[it] = v;
+      }
     }
   }
   float ss = 0.f;
@@ -238,14 +278,20 @@ static int launch_add_rmsnorm(float* x, const void* delta, int nsplit, long spli
                               float eps, int write_x, hipStream_t stream) {
   // Few rows: more threads per row, so that a row's loads are all in flight.
   const int threads = (n <= 256 && d > 1024) ? 1024 : kThreads;
-  if (out_dtype == DT_F32)
-    hipLaunchKernelGGL((add_rmsnorm_kernel<TIN, float>), dim3(n), dim3(threads), 0, stream, x,
-                       (const TIN*)delta, nsplit, split_stride, w, (float*)out, rows, d, eps,
-                       write_x);
-  else
-    hipLaunchKernelGGL((add_rmsnorm_kernel<TIN, bf16_t>), dim3(n), dim3(threads), 0, stream, x,
-                       (const TIN*)delta, nsplit, split_stride, w, (bf16_t*)out, rows, d, eps,
-                       write_x);
+  const int per_thread = ceil_div(d, threads);
+#define KLLM_NORM(TOUT, KEEP)                                                                       \
+  hipLaunchKernelGGL((add_rmsnorm_kernel<TIN, TOUT, KEEP>), dim3(n), dim3(threads), 0, stream, x,    \
+                     (const TIN*)delta, nsplit, split_stride, w, (TOUT*)out, rows, d, eps, write_x)
+  if (out_dtype == DT_F32) {
+    if (per_thread <= 2) KLLM_NORM(float, 2);
+    else if (per_thread <= 4) KLLM_NORM(float, 4);
+    else KLLM_NORM(float, 8);
+  } else {
+    if (per_thread <= 2) KLLM_NORM(bf16_t, 2);
+    else if (per_thread <= 4) KLLM_NORM(bf16_t, 4);
+    else KLLM_NORM(bf16_t, 8);
+  }
+#undef KLLM_NORM
   KLLM_CHECK_LAUNCH("add_rmsnorm");
   return 0;
 }

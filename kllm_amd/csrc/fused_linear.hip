@@ -1,0 +1,502 @@
+// Matrix products of a decode batch (up to 32 rows of X, bfloat16) on MFMA,
+// with the step before and the step after done in the same launch:
+//
+//   input    activations in bfloat16 [n, k], or the float32 residual rows, to
+//            which partial sums are added first and which are normalised on
+//            the way (RMSNorm: reference backend/model.cu:101-122, with the
+//            add: :144-165)
+//   output   float32 sums [nsplit, n, m]; or the sums added into float32 rows
+//            in place (the residual add); or silu(gate) * up in bfloat16
+//            (reference backend/model.cu:477-483); or rotated queries and
+//            keys, and values, written to q_out and to the tokens' pages
+//            (reference backend/model.cu:170-201).
+//
+// A workgroup owns tiles of 16 rows of W and one slice of K (all of K unless
+// the caller splits).  It puts its slice of X, all rows, into LDS once.  Each
+// of its four waves takes a quarter of the slice: it streams its part of the 16
+// rows of W straight from memory, sixteen 16-byte loads per lane in flight,
+// the first of them before X is staged, and multiplies with X from LDS (MFMA
+// 16x16x32: A = W tile, B = X^T, D[w row][x row]).  The four partial tiles meet
+// in LDS, are added in a fixed order, and the epilogue runs on the sums; no
+// partial sum crosses memory unless the caller splits K.
+//
+// Normalisation commutes with the product: LDS holds bfloat16(x * weight) and
+// the epilogue multiplies row t's sums with rsqrt(mean(x_t^2) + eps) in
+// float32, so that one pass over x serves every size of K.
+//
+// What the 16 MFMA rows of a tile are depends on the epilogue: 16 consecutive
+// rows of W, or 8 pairs (gate row p and up row p; rows j and j + hd/2 of one
+// head; two neighbouring value rows) with the first members in MFMA rows 0-7
+// and the second in rows 8-15.
+#include <math.h>
+
+#include "common.hpp"
+#include "kllm_kernels.h"
+
+namespace kllm {
+
+constexpr int FL_AHEAD = 8;        // W loads per lane and round; two rounds are in flight
+constexpr int FL_PAD = 8;          // LDS row padding (elements): 16-byte reads without conflicts
+constexpr int FL_LDS_MAX = 160 * 1024;
+
+enum : int { FL_X_BF16 = 0, FL_X_RESIDUAL = 1 };
+enum : int { FL_PARTS = 0, FL_ADD = 1, FL_SWIGLU = 2, FL_ROPE = 3 };
+
+struct FlIn {
+  const void* x;
+  const float* delta;
+  float* x_out;
+  const float* norm_weight;
+  const int* rows;
+  int delta_splits;
+  float eps;
+};
+
+struct FlOut {
+  void* y;
+  const float* cos_t;
+  const float* sin_t;
+  void* cache;
+  const int* positions;
+  const int* span_of_token;
+  const int* block_table;
+  int max_pages, page_size, H, KV, hd;
+};
+
+// Row of W behind MFMA row c of a tile, or -1.  Pair epilogues: unit = pair.
+template <int EP>
+__device__ __forceinline__ long fl_row(int tile, int c, int m, const FlOut& o) {
+  if (EP == FL_PARTS || EP == FL_ADD) {
+    const long r = (long)tile * 16 + c;
+    return r < m ? r : -1;
+  }
+  const int pair = tile * 8 + (c & 7);          // m < 2^31, so pairs and tiles fit an int
+  const int pairs = m / 2;
+  if (pair >= pairs) return -1;
+  const bool second = c >= 8;
+  if (EP == FL_SWIGLU) return second ? pairs + pair : pair;
+  const int half = o.hd / 2;
+  const int rot_pairs = (o.H + (o.cache ? o.KV : 0)) * half;
+  if (pair < rot_pairs) {
+    const long a = (long)(pair / half) * o.hd + pair % half;   // q and k rows follow each other in W
+    return second ? a + half : a;
+  }
+  const long e = 2 * (long)(pair - rot_pairs);
+  return (long)(o.H + o.KV) * o.hd + e + (second ? 1 : 0);
+}
+
+template <int NT, int XKIND, int EP>
+__global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
+                                                           const bf16_t* __restrict__ W, int n, int m,
+                                                           int k, int kslice, int tiles, int tiles_per_wg,
+                                                           int x_stride) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int ld = kslice + FL_PAD;
+  bf16_t* xs = reinterpret_cast<bf16_t*>(lds_raw);                            // [n][ld]
+  float* part = reinterpret_cast<float*>(lds_raw + (size_t)n * ld * sizeof(bf16_t));   // [2][4][NT][16][16]
+  float* inv = part + 2 * 4 * NT * 256;                                       // [NT * 16]
+
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int g = lane / 16, c = lane % 16;
+  const int kbeg = blockIdx.y * kslice;
+  const int klen = min(k, kbeg + kslice) - kbeg;            // a multiple of 8
+  const int kw = ((klen + 3) / 4 + 31) / 32 * 32;           // K of one wave
+  const int wk0 = wave * kw;                                // this wave's offset in the slice
+  const int wlen = max(0, min(klen, wk0 + kw) - wk0);
+  const int steps = kw / 32;
+  const int tile0 = blockIdx.x * tiles_per_wg;
+  const int my_tiles = min(tiles_per_wg, tiles - tile0);
+  const int rsteps = (steps + FL_AHEAD - 1) / FL_AHEAD * FL_AHEAD;   // a tile's steps in whole rounds
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  // ---- rotate-and-append epilogue: thread (pair tid / 16, token tid % 16) needs the token's
+  // page and slot, and cos and sin of its pair.  Loads return in order, so the position and
+  // the span are asked for before the weights, and what depends on them after X is on its
+  // way: none of it then holds up the weights or X, and all of it is there at the epilogue.
+  int ep_pos[NT], ep_span[NT];
+  if (EP == FL_ROPE) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int xr = t * 16 + tid % 16;
+      const bool ok = out.cache && xr < n && tid < 128;
+      ep_pos[t] = ok ? out.positions[xr] : 0;
+      ep_span[t] = ok ? out.span_of_token[xr] : 0;
+    }
+  }
+
+  // ---- W loads.  A tile's steps are padded to whole rounds of FL_AHEAD, so that a round
+  // belongs to one tile; three rounds are in registers (being multiplied, next, far).
+  auto tile_ptr = [&](int t) -> const bf16_t* {
+    if (t >= my_tiles) return nullptr;
+    const long r = fl_row<EP>((int)tile0 + t, c, m, out);
+    return r >= 0 ? W + r * k + kbeg + wk0 + 8 * g : nullptr;
+  };
+  auto load_a = [&](const bf16_t* ptr, int s) -> bf16x8 {
+    return (ptr && s < steps && 32 * s + 8 * g < wlen) ? *reinterpret_cast<const bf16x8*>(ptr + 32 * s) : zero;
+  };
+  int far_tile = 0, far_s0 = 0;                             // the round that is loaded next
+  const bf16_t* far_ptr = tile_ptr(0);
+  auto advance = [&]() {
+    far_s0 += FL_AHEAD;
+    if (far_s0 == rsteps) {
+      far_s0 = 0;
+      far_ptr = tile_ptr(++far_tile);
+    }
+  };
+  bf16x8 cur[FL_AHEAD], nxt[FL_AHEAD];
+#pragma unroll
+  for (int u = 0; u < FL_AHEAD; ++u) cur[u] = load_a(far_ptr, far_s0 + u);
+  advance();
+#pragma unroll
+  for (int u = 0; u < FL_AHEAD; ++u) nxt[u] = load_a(far_ptr, far_s0 + u);
+  advance();
+
+  // ---- X into LDS: wave w takes rows w, w + 4, ...; eight loads in flight per lane
+  constexpr int RPW = NT * 4;                               // rows per wave at most
+  if (XKIND == FL_X_BF16) {
+    const bf16_t* X = reinterpret_cast<const bf16_t*>(in.x);
+    const int chunks = klen / 8;
+    const int mine = (n - wave + 3) / 4;                    // rows of this wave
+    const int items = mine * chunks;
+    for (int base = lane; base < items; base += kWave * 8) {
+      bf16x8 v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int idx = base + j * kWave;
+        const int ri = idx / chunks, ch = idx - ri * chunks;
+        v[j] = idx < items ? *reinterpret_cast<const bf16x8*>(X + (long)(wave + 4 * ri) * x_stride + kbeg + ch * 8)
+                           : zero;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int idx = base + j * kWave;
+        if (idx < items) {
+          const int ri = idx / chunks, ch = idx - ri * chunks;
+          *reinterpret_cast<bf16x8*>(&xs[(wave + 4 * ri) * ld + ch * 8]) = v[j];
+        }
+      }
+    }
+  } else {
+    // float32 residual rows (+ partial sums) -> x_out, sum of squares, bfloat16(x * weight)
+    const float* X = reinterpret_cast<const float*>(in.x);
+    const int chunks = klen / 4;                            // klen == k here
+    const int mine = (n - wave + 3) / 4;
+    const int items = mine * chunks;
+    const bool write_x = in.x_out != nullptr && blockIdx.x == 0;
+    float ss[RPW];
+#pragma unroll
+    for (int j = 0; j < RPW; ++j) ss[j] = 0.f;
+    for (int base = lane; base < items; base += kWave * 4) {
+      floatx4 v[4], wv[4];
+      int ri[4], ch[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int idx = base + j * kWave;
+        ri[j] = idx / chunks;
+        ch[j] = idx - ri[j] * chunks;
+        const bool ok = idx < items;
+        const int r = wave + 4 * ri[j];
+        const long src = (ok && in.rows) ? in.rows[r] : r;
+        v[j] = ok ? *reinterpret_cast<const floatx4*>(X + src * (long)x_stride + ch[j] * 4) : floatx4{0, 0, 0, 0};
+        wv[j] = ok ? *reinterpret_cast<const floatx4*>(in.norm_weight + ch[j] * 4) : floatx4{0, 0, 0, 0};
+      }
+      for (int s = 0; s < in.delta_splits; ++s) {
+        floatx4 d[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int idx = base + j * kWave;
+          d[j] = idx < items ? *reinterpret_cast<const floatx4*>(
+                                   in.delta + ((long)s * n + wave + 4 * ri[j]) * k + ch[j] * 4)
+                             : floatx4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] += d[j];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int idx = base + j * kWave;
+        if (idx < items) {
+          const int r = wave + 4 * ri[j];
+          if (write_x) *reinterpret_cast<floatx4*>(in.x_out + (long)r * k + ch[j] * 4) = v[j];
+          const float sq = v[j][0] * v[j][0] + v[j][1] * v[j][1] + v[j][2] * v[j][2] + v[j][3] * v[j][3];
+#pragma unroll
+          for (int q = 0; q < RPW; ++q) ss[q] += (ri[j] == q) ? sq : 0.f;
+          bf16x4 b;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) b[e] = from_f32<bf16_t>(v[j][e] * wv[j][e]);
+          *reinterpret_cast<bf16x4*>(&xs[r * ld + ch[j] * 4]) = b;
+        }
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < RPW; ++q) {
+      const float s = wave_sum(ss[q]);
+      const int r = wave + 4 * q;
+      if (lane == 0 && r < n) inv[r] = rsqrtf(s / (float)k + in.eps);
+    }
+  }
+  int ep_page[NT], ep_slot[NT];
+  float ep_cos[NT], ep_sin[NT];
+  auto rope_angles = [&](int tile_index) {
+    if (EP != FL_ROPE || tid >= 128) return;
+    const int half = out.hd / 2;
+    const int pair = (tile0 + tile_index) * 8 + tid / 16;
+    const int rot_pairs = (out.H + (out.cache ? out.KV : 0)) * half;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int xr = t * 16 + tid % 16;
+      const bool ok = out.cos_t && xr < n && pair < rot_pairs && tile_index < my_tiles;
+      ep_cos[t] = ok ? out.cos_t[(long)xr * half + pair % half] : 1.f;
+      ep_sin[t] = ok ? out.sin_t[(long)xr * half + pair % half] : 0.f;
+    }
+  };
+  if (EP == FL_ROPE) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int xr = t * 16 + tid % 16;
+      ep_page[t] = ep_slot[t] = 0;
+      if (out.cache && xr < n && tid < 128) {
+        ep_page[t] = out.block_table[(long)ep_span[t] * out.max_pages + ep_pos[t] / out.page_size];
+        ep_slot[t] = ep_pos[t] % out.page_size;
+      }
+    }
+    rope_angles(0);
+  }
+  __syncthreads();
+
+  floatx4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  for (int tile = 0; tile < my_tiles; ++tile) {
+    for (int s0 = 0; s0 < rsteps; s0 += FL_AHEAD) {
+      bf16x8 far[FL_AHEAD];
+#pragma unroll
+      for (int u = 0; u < FL_AHEAD; ++u) far[u] = load_a(far_ptr, far_s0 + u);
+      advance();
+#pragma unroll
+      for (int u = 0; u < FL_AHEAD; ++u) {
+        const int s = s0 + u;
+        if (s < steps) {
+          const bool kin = 32 * s + 8 * g < wlen;
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const int xr = t * 16 + c;
+            const bf16x8 b = (kin && xr < n)
+                                 ? *reinterpret_cast<const bf16x8*>(&xs[xr * ld + wk0 + 32 * s + 8 * g])
+                                 : zero;
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u], b, acc[t], 0, 0, 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < FL_AHEAD; ++u) {
+        cur[u] = nxt[u];
+        nxt[u] = far[u];
+      }
+    }
+    // ---- the tile is complete in this wave: meet the other waves in LDS
+    float* pb = part + (tile & 1) * 4 * NT * 256;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pb[((wave * NT + t) * 16 + 4 * g + i) * 16 + c] = acc[t][i];
+      acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    __syncthreads();
+    const int tl = tile0 + tile;
+    const int xc = tid % 16;
+    if (EP == FL_PARTS || EP == FL_ADD) {
+      const int r16 = tid / 16;
+      const long row = (long)tl * 16 + r16;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const int xr = t * 16 + xc;
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) v += pb[((w * NT + t) * 16 + r16) * 16 + xc];
+        if (XKIND == FL_X_RESIDUAL && xr < n) v *= inv[xr];
+        if (row < m && xr < n) {
+          float* y = reinterpret_cast<float*>(out.y);
+          if (EP == FL_ADD) y[(long)xr * m + row] += v;
+          else y[((long)blockIdx.y * n + xr) * m + row] = v;
+        }
+      }
+    } else if (tid < 128) {
+      const int p8 = tid / 16;
+      const int pair = tl * 8 + p8, pairs = m / 2;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const int xr = t * 16 + xc;
+        float a = 0.f, b = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          a += pb[((w * NT + t) * 16 + p8) * 16 + xc];
+          b += pb[((w * NT + t) * 16 + p8 + 8) * 16 + xc];
+        }
+        if (pair >= pairs || xr >= n) continue;
+        if (XKIND == FL_X_RESIDUAL) {
+          a *= inv[xr];
+          b *= inv[xr];
+        }
+        if (EP == FL_SWIGLU) {
+          bf16_t* h = reinterpret_cast<bf16_t*>(out.y);
+          h[(long)xr * pairs + pair] = from_f32<bf16_t>((a / (1.f + expf(-a))) * b);
+        } else {
+          const int half = out.hd / 2;
+          const int q_pairs = out.H * half, k_pairs = out.cache ? out.KV * half : 0;
+          const int region = pair < q_pairs ? 0 : pair < q_pairs + k_pairs ? 1 : 2;
+          const int page = ep_page[t], slot = ep_slot[t];
+          const long block = (long)out.page_size * out.hd;
+          if (region < 2) {
+            const int p = region ? pair - q_pairs : pair;
+            const int head = p / half, j = p % half;
+            const float cc = ep_cos[t], sn = ep_sin[t];
+            const float ra = a * cc - b * sn, rb = b * cc + a * sn;
+            bf16_t* o = region == 0
+                            ? reinterpret_cast<bf16_t*>(out.y) + ((long)xr * out.H + head) * out.hd
+                            : reinterpret_cast<bf16_t*>(out.cache) +
+                                  (((long)page * 2 + 0) * out.KV + head) * block + (long)slot * out.hd;
+            o[j] = from_f32<bf16_t>(ra);
+            o[j + half] = from_f32<bf16_t>(rb);
+          } else {
+            const int e = 2 * (pair - q_pairs - k_pairs);
+            const int head = e / out.hd, j = e % out.hd;
+            bf16_t* v = reinterpret_cast<bf16_t*>(out.cache) + (((long)page * 2 + 1) * out.KV + head) * block;
+            v[(long)j * out.page_size + slot] = from_f32<bf16_t>(a);
+            v[(long)(j + 1) * out.page_size + slot] = from_f32<bf16_t>(b);
+          }
+        }
+      }
+    }
+    rope_angles(tile + 1);
+  }
+}
+
+static size_t fl_lds_bytes(int n, int nt, int kslice) {
+  return (size_t)n * (kslice + FL_PAD) * sizeof(bf16_t) + (size_t)(2 * 4 * nt * 256 + nt * 16) * sizeof(float);
+}
+
+template <int NT, int XKIND, int EP>
+static int fl_launch(const FlIn& in, const FlOut& out, const void* w, int n, int m, int k, int kslice,
+                     int nsplit, int tiles, int tiles_per_wg, int x_stride, hipStream_t stream) {
+  const size_t lds = fl_lds_bytes(n, NT, kslice);
+  static size_t allowed = 64 * 1024;
+  if (lds > allowed) {
+    hipError_t e = hipFuncSetAttribute((const void*)fused_linear_kernel<NT, XKIND, EP>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, FL_LDS_MAX);
+    if (e != hipSuccess) KLLM_FAIL((int)e, "fused_linear: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    allowed = FL_LDS_MAX;
+  }
+  const dim3 grid(ceil_div(tiles, tiles_per_wg), nsplit);
+  hipLaunchKernelGGL((fused_linear_kernel<NT, XKIND, EP>), grid, dim3(256), lds, stream, in, out,
+                     (const bf16_t*)w, n, m, k, kslice, tiles, tiles_per_wg, x_stride);
+  return 0;
+}
+
+template <int NT, int XKIND>
+static int fl_launch_ep(int ep, const FlIn& in, const FlOut& out, const void* w, int n, int m, int k,
+                        int kslice, int nsplit, int tiles, int tpw, int xs, hipStream_t st) {
+  switch (ep) {
+    case FL_PARTS: return fl_launch<NT, XKIND, FL_PARTS>(in, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+    case FL_ADD: return fl_launch<NT, XKIND, FL_ADD>(in, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+    case FL_SWIGLU: return fl_launch<NT, XKIND, FL_SWIGLU>(in, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+    default: return fl_launch<NT, XKIND, FL_ROPE>(in, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+  }
+}
+
+}  // namespace kllm
+
+using namespace kllm;
+
+static bool fl_aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+extern "C" long kllm_fused_linear_lds_bytes(int n, int k, int nsplit) {
+  if (n <= 0 || k <= 0 || nsplit <= 0) return -1;
+  const int kslice = ceil_div(ceil_div(k, nsplit), 32) * 32;
+  return (long)fl_lds_bytes(n, ceil_div(n, 16), kslice);
+}
+
+extern "C" int kllm_fused_linear(const KllmLinearIn* xin, const KllmLinearOut* yout, const void* w, int n,
+                                 int m, int k, int tiles_per_wg, hipStream_t stream) {
+  KLLM_REQUIRE(xin && yout && w && xin->x && yout->y, "fused_linear: null pointer");
+  KLLM_REQUIRE(n > 0 && n <= KLLM_FUSED_LINEAR_MAX_ROWS, "fused_linear: n=%d is outside [1, %d]", n,
+               KLLM_FUSED_LINEAR_MAX_ROWS);
+  KLLM_REQUIRE(m > 0 && k > 0 && k % 8 == 0, "fused_linear: bad sizes m=%d k=%d (K must be a multiple of 8)", m, k);
+  KLLM_REQUIRE((long)m * k < (1L << 40), "fused_linear: sizes overflow");
+  KLLM_REQUIRE(fl_aligned16(w) && fl_aligned16(xin->x), "fused_linear: operands must be 16-byte aligned");
+  KLLM_REQUIRE(tiles_per_wg >= 1 && tiles_per_wg <= 64, "fused_linear: %d tiles per workgroup", tiles_per_wg);
+  const int ep = yout->kind, xk = xin->kind;
+  KLLM_REQUIRE(xk == FL_X_BF16 || xk == FL_X_RESIDUAL, "fused_linear: unknown input kind %d", xk);
+  KLLM_REQUIRE(ep >= FL_PARTS && ep <= FL_ROPE, "fused_linear: unknown output kind %d", ep);
+  const int nsplit = yout->nsplit;
+  KLLM_REQUIRE(nsplit >= 1 && nsplit <= 64, "fused_linear: nsplit %d is outside [1, 64]", nsplit);
+  KLLM_REQUIRE(nsplit == 1 || (ep == FL_PARTS && xk == FL_X_BF16),
+               "fused_linear: K is split only between bfloat16 input and partial sums");
+  const int kslice = ceil_div(ceil_div(k, nsplit), 32) * 32;
+  KLLM_REQUIRE((long)kslice * (nsplit - 1) < k, "fused_linear: nsplit %d leaves an empty slice of K=%d", nsplit, k);
+  const int nt = ceil_div(n, 16);
+  KLLM_REQUIRE(fl_lds_bytes(n, nt, kslice) <= (size_t)FL_LDS_MAX,
+               "fused_linear: %d rows of K=%d need %zu bytes of LDS, more than %d", n, kslice,
+               fl_lds_bytes(n, nt, kslice), FL_LDS_MAX);
+
+  FlIn in = {};
+  in.x = xin->x;
+  int x_stride = xin->x_stride > 0 ? xin->x_stride : k;
+  KLLM_REQUIRE(x_stride >= k && x_stride % 8 == 0, "fused_linear: row stride %d of x does not fit K=%d", x_stride, k);
+  if (xk == FL_X_RESIDUAL) {
+    KLLM_REQUIRE(xin->norm_weight && fl_aligned16(xin->norm_weight), "fused_linear: the norm's weight is missing");
+    KLLM_REQUIRE(xin->delta_splits >= 0 && (xin->delta_splits == 0 || xin->delta),
+                 "fused_linear: %d partial sums without a pointer", xin->delta_splits);
+    KLLM_REQUIRE(!xin->delta_splits || (xin->x_out && xin->x_out != xin->x && fl_aligned16(xin->x_out) &&
+                                        fl_aligned16(xin->delta)),
+                 "fused_linear: partial sums need a separate, aligned x_out");
+    KLLM_REQUIRE(!xin->rows || !xin->delta_splits, "fused_linear: gathered rows take no partial sums");
+    in.delta = xin->delta_splits ? xin->delta : nullptr;
+    in.delta_splits = xin->delta_splits;
+    in.x_out = xin->delta_splits ? xin->x_out : nullptr;
+    in.norm_weight = xin->norm_weight;
+    in.rows = xin->rows;
+    in.eps = xin->eps;
+  }
+
+  FlOut out = {};
+  out.y = yout->y;
+  int tiles = ceil_div(m, 16);
+  if (ep == FL_SWIGLU || ep == FL_ROPE) {
+    KLLM_REQUIRE(m % 2 == 0, "fused_linear: m=%d must be even for a pair epilogue", m);
+    tiles = ceil_div(m / 2, 8);
+  }
+  if (ep == FL_ROPE) {
+    const int H = yout->H, KV = yout->KV, hd = yout->hd;
+    KLLM_REQUIRE(H > 0 && hd > 0 && hd % 2 == 0, "fused_linear: bad heads H=%d hd=%d", H, hd);
+    KLLM_REQUIRE((yout->cos_t == nullptr) == (yout->sin_t == nullptr), "fused_linear: cos and sin go together");
+    if (yout->cache)
+      KLLM_REQUIRE(KV > 0 && yout->positions && yout->span_of_token && yout->block_table &&
+                       yout->max_pages > 0 && yout->page_size > 0,
+                   "fused_linear: bad cache arguments");
+    KLLM_REQUIRE(m == H * hd + (yout->cache ? 2 * KV * hd : 0), "fused_linear: m=%d does not fit the heads", m);
+    out.cos_t = yout->cos_t;
+    out.sin_t = yout->sin_t;
+    out.cache = yout->cache;
+    out.positions = yout->positions;
+    out.span_of_token = yout->span_of_token;
+    out.block_table = yout->block_table;
+    out.max_pages = yout->max_pages;
+    out.page_size = yout->page_size;
+    out.H = H;
+    out.KV = KV;
+    out.hd = hd;
+  }
+
+  int rc;
+  if (nt == 1)
+    rc = xk == FL_X_BF16 ? fl_launch_ep<1, FL_X_BF16>(ep, in, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream)
+                         : fl_launch_ep<1, FL_X_RESIDUAL>(ep, in, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream);
+  else
+    rc = xk == FL_X_BF16 ? fl_launch_ep<2, FL_X_BF16>(ep, in, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream)
+                         : fl_launch_ep<2, FL_X_RESIDUAL>(ep, in, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream);
+  if (rc) return rc;
+  KLLM_CHECK_LAUNCH("fused_linear");
+  return 0;
+}

@@ -91,6 +91,56 @@ int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_out, const f
                           int page_size, int n, int H, int KV, int hd, int k, int dtype,
                           hipStream_t stream);
 
+/* Products of a decode batch (bfloat16, up to KLLM_FUSED_LINEAR_MAX_ROWS rows)
+ * on the matrix cores, fused with the step before and the step after.
+ * Input: bfloat16 activations [n][k] (row stride x_stride elements, 0 = k), or
+ * float32 residual rows that are normalised on the way (RMSNorm with
+ * norm_weight [k] and eps), optionally gathered through `rows`, optionally after
+ * adding partial sums delta [delta_splits][n][k]; the sum x + delta is then
+ * also written to x_out [n][k], which must not be x.
+ * Output, w being [m][k]:
+ *   PARTS   y float32 [nsplit][n][m]; only this one may split K (bfloat16 input)
+ *   ADD     y float32 [n][m] += x . w^T
+ *   SWIGLU  y bfloat16 [n][m/2] = silu(x . w[0:m/2]^T) * (x . w[m/2:m]^T)
+ *   ROPE    w = [q; k; v] rows (only q when cache is null): q and k rotated with
+ *           cos/sin [n][hd/2] (if given); y = q_out [n][H*hd], k and v go to the
+ *           tokens' pages of `cache`
+ * All of a workgroup's slice of K for all rows has to fit into LDS:
+ * kllm_fused_linear_lds_bytes says how much a call needs (160 KiB at most). */
+#define KLLM_FUSED_LINEAR_MAX_ROWS 32
+#define KLLM_LINEAR_IN_BF16 0
+#define KLLM_LINEAR_IN_RESIDUAL 1
+#define KLLM_LINEAR_OUT_PARTS 0
+#define KLLM_LINEAR_OUT_ADD 1
+#define KLLM_LINEAR_OUT_SWIGLU 2
+#define KLLM_LINEAR_OUT_ROPE 3
+typedef struct {
+  const void* x;
+  const float* delta;
+  float* x_out;
+  const float* norm_weight;
+  const int* rows;
+  int kind;
+  int x_stride;
+  int delta_splits;
+  float eps;
+} KllmLinearIn;
+typedef struct {
+  void* y;
+  const float* cos_t;
+  const float* sin_t;
+  void* cache;
+  const int* positions;
+  const int* span_of_token;
+  const int* block_table;
+  int kind;
+  int nsplit;
+  int max_pages, page_size, H, KV, hd;
+} KllmLinearOut;
+long kllm_fused_linear_lds_bytes(int n, int k, int nsplit);
+int kllm_fused_linear(const KllmLinearIn* in, const KllmLinearOut* out, const void* w, int n, int m,
+                      int k, int tiles_per_wg, hipStream_t stream);
+
 /* Causal attention of n tokens over the paged cache; any head size up to 256. */
 int kllm_attn_generic(const void* q, void* out, const void* cache, const int* positions,
                       const int* span_of_token, const int* block_table, int max_pages,
@@ -98,10 +148,11 @@ int kllm_attn_generic(const void* q, void* out, const void* cache, const int* po
                       int dtype, hipStream_t stream);
 
 /* Decode attention on the matrix cores (bfloat16): every token's keys are cut
- * into `nslices` slices (a multiple of 4) that run side by side; `part` is
- * float32 scratch of n*H*nslices*(hd+2) elements.  kllm_attn_decode_slices
- * proposes nslices for a batch.  With token_list only the n_listed tokens it
- * names are computed (q, out and part stay indexed by token row). */
+ * into `nslices` slices (1..256) that run side by side, four waves to a slice;
+ * `part` is float32 scratch of n*H*nslices*(hd+2) elements.
+ * kllm_attn_decode_slices proposes nslices for a batch.  With token_list only
+ * the n_listed tokens it names are computed (q, out and part stay indexed by
+ * token row). */
 int kllm_attn_decode_slices(int n, int KV, int H);
 int kllm_attn_decode(const void* q, void* out, float* part, long part_floats, const void* cache,
                      const int* positions, const int* span_of_token, const int* block_table,

@@ -77,12 +77,18 @@ class CausalSelfAttention(Part):
         if self.position is not None and hasattr(self.position, "tables"):
             cos, sin = self.position.tables(ctx)
         pages = cache.pages if writes else None
-        if (K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype)
-                and not self.runtime.options.get("no_fused_gemv")):
+        opts = self.runtime.options
+        if K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype) and not opts.get("no_fused_gemv"):
             # few tokens: projections, rotation and append in one launch
             K.gemv_rope_append(xn, self.w_in, q, cos, sin, pages, ctx.positions, ctx.span_of_token,
                                cache.block_table, cache.page_size, self.heads, self.kv_heads,
                                self.head_dim)
+        elif (dtype == torch.bfloat16 and K.fused_linear_fits(n, self.hidden)
+              and not opts.get("no_fused_linear")):
+            # a decode batch: the same on the matrix cores
+            K.fused_linear(self.w_in, q, K.LINEAR_ROPE, x=xn,
+                           rope=K.Rope(cos, sin, pages, ctx.positions, ctx.span_of_token, cache.block_table,
+                                       cache.page_size, self.heads, self.kv_heads, self.head_dim))
         else:
             qkv = linear(ctx, xn, self.w_in, "attn.qkv")
             K.rope_append(qkv, q, cos, sin, pages, ctx.positions, ctx.span_of_token,

@@ -34,14 +34,33 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   const int r = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const float* row = logits + (long)r * vocab;
   // Each thread owns one contiguous segment, so thread order is index order.
-  const int seg = (vocab + kSampleThreads - 1) / kSampleThreads;
+  // Segments are multiples of four logits, so that a row whose length is one too is read
+  // in 16-byte pieces, eight of them in flight per thread.
+  const int seg = (vocab + 4 * kSampleThreads - 1) / (4 * kSampleThreads) * 4;
   const int lo = min(tid * seg, vocab), hi = min(lo + seg, vocab);
 
   float bv = -INFINITY;
   int bi = vocab;  // "none": loses against every index
-  for (int i = lo; i < hi; ++i) {
-    const float v = row[i];
-    if (bi == vocab || v > bv) { bv = v; bi = i; }   // strict: the first maximum stays
+  if (vocab % 4 == 0 && ((uintptr_t)logits & 15) == 0) {
+    for (int i0 = lo; i0 < hi; i0 += 32) {
+      floatx4 v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        v[j] = i0 + 4 * j < hi ? *reinterpret_cast<const floatx4*>(row + i0 + 4 * j)
+                               : floatx4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = i0 + 4 * j + e;
+          if (i < hi && (bi == vocab || v[j][e] > bv)) { bv = v[j][e]; bi = i; }   // strict: the first maximum stays
+        }
+    }
+  } else {
+    for (int i = lo; i < hi; ++i) {
+      const float v = row[i];
+      if (bi == vocab || v > bv) { bv = v; bi = i; }
+    }
   }
 #pragma unroll
   for (int off = kWave / 2; off > 0; off >>= 1) {

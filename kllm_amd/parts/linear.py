@@ -8,7 +8,9 @@ rotary + append, SiLU gate); with the compute dtype as result it returns
   n <= 8    gemv with X in LDS and the whole of K in one wave (no partial
             sums), if the sizes fit; else the streaming or the general gemv
   float32   else: tiled FMA (true 32-bit)
-  bfloat16  n <= 64: MFMA skinny      else: MFMA tiles,
+  bfloat16  n <= 64: MFMA skinny (n <= 16 and one float32 result wanted: the
+            decode-batch kernel with all of K in a workgroup)
+            else: MFMA tiles,
             or the vendor library (torch.matmul) when the engine option
             ``gemm`` is "library" -- the reference uses its vendor library for
             every product (backend/model.cu:494-503)
@@ -78,6 +80,13 @@ def linear(ctx, x, w, tag, out_dtype=torch.float32, split=True):
     rt = ctx.runtime
     algo, nsplit = choose(x.dtype, n, m, k, rt.options)
     whole = not split or out_dtype != torch.float32
+    if (algo == K.GEMM_SKINNY_BF16 and whole and out_dtype == torch.float32 and n <= 16
+            and K.fused_linear_fits(n, k) and not rt.options.get("no_fused_linear")):
+        # one float32 result from a decode batch (the logits): all of K in one workgroup, so
+        # that no partial sums have to be added afterwards
+        y = ctx.buf(tag, (1, n, m), torch.float32)
+        K.fused_linear(w, y, K.LINEAR_PARTS, x=x, tiles_per_wg=4 if m >= 16384 else 1)
+        return y[0]
     if algo == "library":
         y = ctx.buf(tag, (n, m), x.dtype)
         torch.matmul(x, w.t(), out=y)

@@ -38,6 +38,7 @@ namespace kllm {
 constexpr int FL_AHEAD = 8;        // W loads per lane and round; two rounds are in flight
 constexpr int FL_PAD = 8;          // LDS row padding (elements): 16-byte reads without conflicts
 constexpr int FL_LDS_MAX = 160 * 1024;
+constexpr int FL_TILE = 16 * 17;    // floats of one wave's partial tile in LDS: [x row][w row], padded
 
 enum : int { FL_X_BF16 = 0, FL_X_RESIDUAL = 1 };
 enum : int { FL_PARTS = 0, FL_ADD = 1, FL_SWIGLU = 2, FL_ROPE = 3 };
@@ -93,8 +94,8 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   const int ld = kslice + FL_PAD;
   bf16_t* xs = reinterpret_cast<bf16_t*>(lds_raw);                            // [n][ld]
-  float* part = reinterpret_cast<float*>(lds_raw + (size_t)n * ld * sizeof(bf16_t));   // [2][4][NT][16][16]
-  float* inv = part + 2 * 4 * NT * 256;                                       // [NT * 16]
+  float* part = reinterpret_cast<float*>(lds_raw + (size_t)n * ld * sizeof(bf16_t));   // [2][4][NT][x row 16][17]
+  float* inv = part + 2 * 4 * NT * FL_TILE;                                   // [NT * 16]
 
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int g = lane / 16, c = lane % 16;
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
   const int rsteps = (steps + FL_AHEAD - 1) / FL_AHEAD * FL_AHEAD;   // a tile's steps in whole rounds
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  // ---- rotate-and-append epilogue: thread (pair tid / 16, token tid % 16) needs the token's
+  // ---- rotate-and-append epilogue: thread (pair tid % 8, token tid / 8) needs the token's
   // page and slot, and cos and sin of its pair.  Loads return in order, so the position and
   // the span are asked for before the weights, and what depends on them after X is on its
   // way: none of it then holds up the weights or X, and all of it is there at the epilogue.
@@ -117,7 +118,7 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
   if (EP == FL_ROPE) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      const int xr = t * 16 + tid % 16;
+      const int xr = t * 16 + tid / 8;
       const bool ok = out.cache && xr < n && tid < 128;
       ep_pos[t] = ok ? out.positions[xr] : 0;
       ep_span[t] = ok ? out.span_of_token[xr] : 0;
@@ -240,11 +241,11 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
   auto rope_angles = [&](int tile_index) {
     if (EP != FL_ROPE || tid >= 128) return;
     const int half = out.hd / 2;
-    const int pair = (tile0 + tile_index) * 8 + tid / 16;
+    const int pair = (tile0 + tile_index) * 8 + tid % 8;
     const int rot_pairs = (out.H + (out.cache ? out.KV : 0)) * half;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      const int xr = t * 16 + tid % 16;
+      const int xr = t * 16 + tid / 8;
       const bool ok = out.cos_t && xr < n && pair < rot_pairs && tile_index < my_tiles;
       ep_cos[t] = ok ? out.cos_t[(long)xr * half + pair % half] : 1.f;
       ep_sin[t] = ok ? out.sin_t[(long)xr * half + pair % half] : 0.f;
@@ -253,7 +254,7 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
   if (EP == FL_ROPE) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      const int xr = t * 16 + tid % 16;
+      const int xr = t * 16 + tid / 8;
       ep_page[t] = ep_slot[t] = 0;
       if (out.cache && xr < n && tid < 128) {
         ep_page[t] = out.block_table[(long)ep_span[t] * out.max_pages + ep_pos[t] / out.page_size];
@@ -296,25 +297,25 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
       }
     }
     // ---- the tile is complete in this wave: meet the other waves in LDS
-    float* pb = part + (tile & 1) * 4 * NT * 256;
+    float* pb = part + (tile & 1) * 4 * NT * FL_TILE;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) pb[((wave * NT + t) * 16 + 4 * g + i) * 16 + c] = acc[t][i];
+      for (int i = 0; i < 4; ++i) pb[(wave * NT + t) * FL_TILE + c * 17 + 4 * g + i] = acc[t][i];
       acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
     __syncthreads();
     const int tl = tile0 + tile;
-    const int xc = tid % 16;
+    // Neighbouring threads take neighbouring rows of W: their stores share cache lines.
     if (EP == FL_PARTS || EP == FL_ADD) {
-      const int r16 = tid / 16;
+      const int r16 = tid % 16, xc = tid / 16;
       const long row = (long)tl * 16 + r16;
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         const int xr = t * 16 + xc;
         float v = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) v += pb[((w * NT + t) * 16 + r16) * 16 + xc];
+        for (int w = 0; w < 4; ++w) v += pb[(w * NT + t) * FL_TILE + xc * 17 + r16];
         if (XKIND == FL_X_RESIDUAL && xr < n) v *= inv[xr];
         if (row < m && xr < n) {
           float* y = reinterpret_cast<float*>(out.y);
@@ -323,7 +324,7 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
         }
       }
     } else if (tid < 128) {
-      const int p8 = tid / 16;
+      const int p8 = tid % 8, xc = tid / 8;
       const int pair = tl * 8 + p8, pairs = m / 2;
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
@@ -331,8 +332,8 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
         float a = 0.f, b = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-          a += pb[((w * NT + t) * 16 + p8) * 16 + xc];
-          b += pb[((w * NT + t) * 16 + p8 + 8) * 16 + xc];
+          a += pb[(w * NT + t) * FL_TILE + xc * 17 + p8];
+          b += pb[(w * NT + t) * FL_TILE + xc * 17 + p8 + 8];
         }
         if (pair >= pairs || xr >= n) continue;
         if (XKIND == FL_X_RESIDUAL) {
@@ -374,7 +375,7 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
 }
 
 static size_t fl_lds_bytes(int n, int nt, int kslice) {
-  return (size_t)n * (kslice + FL_PAD) * sizeof(bf16_t) + (size_t)(2 * 4 * nt * 256 + nt * 16) * sizeof(float);
+  return (size_t)n * (kslice + FL_PAD) * sizeof(bf16_t) + (size_t)(2 * 4 * nt * FL_TILE + nt * 16) * sizeof(float);
 }
 
 template <int NT, int XKIND, int EP>

@@ -299,7 +299,7 @@ constexpr int SK_SLICE_MAX = 512;             // K per workgroup at most
 constexpr int SK_LD = SK_SLICE_MAX + 8;       // LDS row stride (elements): 16-byte reads conflict-free
 constexpr int SK_AHEAD = 8;                   // W loads in flight per lane
 
-template <int NT>
+template <int NT, int RT>   // NT: 16-row tiles of X; RT: 16-row tiles of W per wave (1 or 2)
 __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ X,
                                                                const bf16_t* __restrict__ W,
                                                                float* __restrict__ Y, int n, int m,
@@ -312,19 +312,28 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
   const int klen = kend - kbeg;                                  // a multiple of 8
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  // This wave's rows of W; their first loads go out before X is staged.
-  const long m0 = ((long)blockIdx.x * 4 + wave) * 16;
-  const long wrow = m0 + c;
-  const bool wok = wrow < m;
-  const bf16_t* wp = W + (wok ? wrow : 0) * k + kbeg + 8 * g;
-  const int steps = (klen + 31) / 32;
-  auto load_a = [&](int s) -> bf16x8 {
-    return (wok && s < steps && 32 * s + 8 * g < klen) ? *reinterpret_cast<const bf16x8*>(wp + 32 * s)
-                                                        : zero;
-  };
-  bf16x8 cur[SK_AHEAD], nxt[SK_AHEAD];
+  // This wave's rows of W; their first loads go out before X is staged.  With RT = 2 a
+  // wave multiplies every piece of X it reads from LDS with two tiles of W, and a
+  // workgroup stages X once for 128 rows of W instead of 64.
+  const long m0 = ((long)blockIdx.x * 4 + wave) * 16 * RT;
+  const bf16_t* wp[RT];
+  bool wok[RT];
 #pragma unroll
-  for (int u = 0; u < SK_AHEAD; ++u) cur[u] = load_a(u);
+  for (int rt = 0; rt < RT; ++rt) {
+    const long wrow = m0 + rt * 16 + c;
+    wok[rt] = wrow < m;
+    wp[rt] = W + (wok[rt] ? wrow : 0) * k + kbeg + 8 * g;
+  }
+  const int steps = (klen + 31) / 32;
+  auto load_a = [&](int rt, int s) -> bf16x8 {
+    return (wok[rt] && s < steps && 32 * s + 8 * g < klen) ? *reinterpret_cast<const bf16x8*>(wp[rt] + 32 * s)
+                                                            : zero;
+  };
+  bf16x8 cur[RT][SK_AHEAD], nxt[RT][SK_AHEAD];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int u = 0; u < SK_AHEAD; ++u) cur[rt][u] = load_a(rt, u);
 
   // Stage X[0..16*NT)[kbeg..kend) in LDS, eight 16-byte loads in flight per thread.
   const int chunks = (klen + 7) / 8;
@@ -349,13 +358,17 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
   __syncthreads();
   if (m0 >= m) return;
 
-  floatx4 acc[NT];
+  floatx4 acc[RT][NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[rt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   for (int s0 = 0; s0 < steps; s0 += SK_AHEAD) {
 #pragma unroll
-    for (int u = 0; u < SK_AHEAD; ++u) nxt[u] = load_a(s0 + SK_AHEAD + u);
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int u = 0; u < SK_AHEAD; ++u) nxt[rt][u] = load_a(rt, s0 + SK_AHEAD + u);
 #pragma unroll
     for (int u = 0; u < SK_AHEAD; ++u) {
       const int s1 = s0 + u;
@@ -365,23 +378,36 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __r
         for (int t = 0; t < NT; ++t) {
           const bf16x8 b = kin ? *reinterpret_cast<const bf16x8*>(&xs[(t * 16 + c) * SK_LD + 32 * s1 + 8 * g])
                                : zero;
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u], b, acc[t], 0, 0, 0);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[rt][u], b, acc[rt][t], 0, 0, 0);
         }
       }
     }
 #pragma unroll
-    for (int u = 0; u < SK_AHEAD; ++u) cur[u] = nxt[u];
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int u = 0; u < SK_AHEAD; ++u) cur[rt][u] = nxt[rt][u];
   }
 
+  // A lane holds four neighbouring columns of one row of X: one 16-byte store where the
+  // row length allows it.
   float* out = Y + (long)blockIdx.y * n * m;
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int xr = t * 16 + c;
-    if (xr >= n) continue;
+  for (int rt = 0; rt < RT; ++rt) {
+    const long col0 = m0 + rt * 16 + 4 * g;
+    const bool vec = m % 4 == 0 && col0 + 3 < m && ((uintptr_t)Y & 15) == 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const long col = m0 + 4 * g + i;
-      if (col < m) out[(long)xr * m + col] = acc[t][i];
+    for (int t = 0; t < NT; ++t) {
+      const int xr = t * 16 + c;
+      if (xr >= n) continue;
+      if (vec) {
+        *reinterpret_cast<floatx4*>(&out[(long)xr * m + col0]) = acc[rt][t];
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (col0 + i < m) out[(long)xr * m + col0 + i] = acc[rt][t][i];
+      }
     }
   }
 }
@@ -500,15 +526,19 @@ static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 // The 64-row variant of the skinny kernel stages 66,560 bytes of LDS, above the
 // default limit of a launch; raise it once per kernel.
-template <int NT>
-static int allow_skinny_lds() {
-  static int done = 0;
-  if (done) return 0;
-  hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_skinny_kernel<NT>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     NT * 16 * SK_LD * (int)sizeof(bf16_t));
-  if (e != hipSuccess) KLLM_FAIL((int)e, "gemm skinny: cannot raise the LDS limit: %s", hipGetErrorString(e));
-  done = 1;
+template <int NT, int RT>
+static int launch_skinny(const bf16_t* x, const bf16_t* w, float* y, int n, int m, int k, int kslice,
+                         int nsplit, hipStream_t stream) {
+  static int raised = 0;
+  const size_t lds = (size_t)NT * 16 * SK_LD * sizeof(bf16_t);
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_skinny_kernel<NT, RT>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) KLLM_FAIL((int)e, "gemm skinny: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = 1;
+  }
+  const dim3 grid(ceil_div(m, 64 * RT), nsplit);
+  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<NT, RT>), grid, dim3(256), lds, stream, x, w, y, n, m, k, kslice);
   return 0;
 }
 
@@ -573,21 +603,20 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
                  nsplit, SK_SLICE_MAX);
     KLLM_REQUIRE((long)kslice * (nsplit - 1) < k, "gemm skinny: nsplit %d leaves an empty slice of K=%d",
                  nsplit, k);
-    const dim3 grid(ceil_div(m, 64), nsplit);
     const bf16_t *xp = (const bf16_t*)x, *wp = (const bf16_t*)w;
     float* yp = (float*)y;
     const int nt = ceil_div(n, 16);
-    const size_t lds = (size_t)nt * 16 * SK_LD * sizeof(bf16_t);
-#define KLLM_SK(NT)                                                                              \
-  hipLaunchKernelGGL((gemm_bf16_skinny_kernel<NT>), grid, dim3(256), lds, stream, xp, wp, yp, n, m, k, kslice)
-    int rc = nt == 1 ? allow_skinny_lds<1>() : nt == 2 ? allow_skinny_lds<2>()
-             : nt == 3 ? allow_skinny_lds<3>() : allow_skinny_lds<4>();
+    // Many rows of X and of W: two tiles of W per wave, while that still leaves a workgroup
+    // for every CU (measured: a gain from 33 rows of X on, a loss below).
+    const bool wide = nt >= 3 && (long)ceil_div(m, 128) * nsplit >= 256;
+    int rc;
+    if (nt == 1) rc = launch_skinny<1, 1>(xp, wp, yp, n, m, k, kslice, nsplit, stream);
+    else if (nt == 2) rc = launch_skinny<2, 1>(xp, wp, yp, n, m, k, kslice, nsplit, stream);
+    else if (nt == 3) rc = wide ? launch_skinny<3, 2>(xp, wp, yp, n, m, k, kslice, nsplit, stream)
+                                : launch_skinny<3, 1>(xp, wp, yp, n, m, k, kslice, nsplit, stream);
+    else rc = wide ? launch_skinny<4, 2>(xp, wp, yp, n, m, k, kslice, nsplit, stream)
+                   : launch_skinny<4, 1>(xp, wp, yp, n, m, k, kslice, nsplit, stream);
     if (rc) return rc;
-    if (nt == 1) KLLM_SK(1);
-    else if (nt == 2) KLLM_SK(2);
-    else if (nt == 3) KLLM_SK(3);
-    else KLLM_SK(4);
-#undef KLLM_SK
     KLLM_CHECK_LAUNCH("gemm skinny");
     return 0;
   }

@@ -328,6 +328,12 @@ FUSED_LINEAR_LDS = 160 * 1024
 LINEAR_PARTS, LINEAR_ADD, LINEAR_SWIGLU, LINEAR_ROPE = 0, 1, 2, 3
 
 
+# Rows up to which the decode-batch kernel beats the split-K kernel plus a separate
+# elementwise launch (measured at widths 2048 -> 2560 and 2048 -> 11264).
+FUSED_ROPE_BEST_ROWS = 16
+FUSED_SWIGLU_BEST_ROWS = 8
+
+
 def fused_linear_fits(n, k, nsplit=1) -> bool:
     """Whether the decode-batch products take n rows of K: bfloat16 only, K a
     multiple of 8, and all rows of a workgroup's slice of K in LDS."""
@@ -335,7 +341,7 @@ def fused_linear_fits(n, k, nsplit=1) -> bool:
         return False
     kslice = -(-(-(-k // nsplit)) // 32) * 32
     nt = -(-n // 16)
-    return n * (kslice + 8) * 2 + (2 * 4 * nt * 256 + nt * 16) * 4 <= FUSED_LINEAR_LDS
+    return n * (kslice + 8) * 2 + (2 * 4 * nt * 16 * 17 + nt * 16) * 4 <= FUSED_LINEAR_LDS
 
 
 class Rope:

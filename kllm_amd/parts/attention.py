@@ -83,7 +83,7 @@ class CausalSelfAttention(Part):
             K.gemv_rope_append(xn, self.w_in, q, cos, sin, pages, ctx.positions, ctx.span_of_token,
                                cache.block_table, cache.page_size, self.heads, self.kv_heads,
                                self.head_dim)
-        elif (dtype == torch.bfloat16 and K.fused_linear_fits(n, self.hidden)
+        elif (dtype == torch.bfloat16 and n <= K.FUSED_ROPE_BEST_ROWS and K.fused_linear_fits(n, self.hidden)
               and not opts.get("no_fused_linear")):
             # a decode batch: the same on the matrix cores
             K.fused_linear(self.w_in, q, K.LINEAR_ROPE, x=xn,

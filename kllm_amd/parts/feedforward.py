@@ -46,7 +46,8 @@ class GatedFeedForward(Part):
         if (K.gemv_fits(n, 2 * self.intermediate, self.hidden, xn.dtype)
                 and not self.runtime.options.get("no_fused_gemv")):
             K.gemv_swiglu(xn, self.w_gu, h)          # few tokens: both products and the gate in one launch
-        elif (xn.dtype == torch.bfloat16 and K.fused_linear_fits(n, self.hidden)
+        elif (xn.dtype == torch.bfloat16 and n <= K.FUSED_SWIGLU_BEST_ROWS
+              and K.fused_linear_fits(n, self.hidden)
               and not self.runtime.options.get("no_fused_linear")):
             K.fused_linear(self.w_gu, h, K.LINEAR_SWIGLU, x=xn)    # a decode batch: the same on the matrix cores
         elif (n > 64 and xn.dtype == torch.bfloat16 and self.hidden % 8 == 0

@@ -37,13 +37,12 @@ def _gemv_split(dtype, n, m, k):
 
 def _skinny_split(n, m, k):
     """Slices of K for the skinny MFMA kernel: at most 512 of K per workgroup
-    (its LDS stage); more slices while the chip has no workgroup per CU, as
-    long as a slice keeps 128 of K and the partial sums stay small beside the
-    weights: every further slice is another row the consumer has to add."""
+    (its LDS stage); more slices while the chip has no workgroup per CU and a
+    slice keeps 128 of K.  Idle CUs cost more than the partial sums that a
+    further slice writes (measured up to 64 rows)."""
     nsplit = -(-k // 512)
     wgs = -(-m // 64)
-    most = max(nsplit, k // (16 * n))
-    while wgs * nsplit < 256 and nsplit * 2 <= most and k // (nsplit * 2) >= 128:
+    while wgs * nsplit < 256 and k // (nsplit * 2) >= 128:
         nsplit *= 2
     while (-(-(-(-k // nsplit)) // 32) * 32) * (nsplit - 1) >= k:   # no empty slice
         nsplit -= 1

@@ -1,33 +1,29 @@
-// Matrix products of a decode batch (up to 32 rows of X, bfloat16) on MFMA,
-// with the step before and the step after done in the same launch:
+// Matrix products of a decode batch (up to 32 rows of X, bfloat16) on MFMA, with
+// the step after the product done in the same launch.  Y = X . W^T, then
 //
-//   input    activations in bfloat16 [n, k], or the float32 residual rows, to
-//            which partial sums are added first and which are normalised on
-//            the way (RMSNorm: reference backend/model.cu:101-122, with the
-//            add: :144-165)
-//   output   float32 sums [nsplit, n, m]; or the sums added into float32 rows
-//            in place (the residual add); or silu(gate) * up in bfloat16
-//            (reference backend/model.cu:477-483); or rotated queries and
-//            keys, and values, written to q_out and to the tokens' pages
-//            (reference backend/model.cu:170-201).
+//   PARTS    float32 sums [nsplit, n, m] (only this one may split K);
+//   SWIGLU   silu(gate) * up in bfloat16 (reference backend/model.cu:477-483);
+//   ROPE     rotated queries and keys, and values, written to q_out and to
+//            the tokens' pages (reference backend/model.cu:170-201).
 //
 // A workgroup owns tiles of 16 rows of W and one slice of K (all of K unless
 // the caller splits).  It puts its slice of X, all rows, into LDS once.  Each
 // of its four waves takes a quarter of the slice: it streams its part of the 16
-// rows of W straight from memory, sixteen 16-byte loads per lane in flight,
-// the first of them before X is staged, and multiplies with X from LDS (MFMA
-// 16x16x32: A = W tile, B = X^T, D[w row][x row]).  The four partial tiles meet
-// in LDS, are added in a fixed order, and the epilogue runs on the sums; no
-// partial sum crosses memory unless the caller splits K.
-//
-// Normalisation commutes with the product: LDS holds bfloat16(x * weight) and
-// the epilogue multiplies row t's sums with rsqrt(mean(x_t^2) + eps) in
-// float32, so that one pass over x serves every size of K.
+// rows of W straight from memory, up to twenty-four 16-byte loads per lane in
+// flight, the first of them before X is staged, and multiplies with X from LDS
+// (MFMA 16x16x32: A = W tile, B = X^T, D[w row][x row]).  The four partial
+// tiles meet in LDS, are added in a fixed order, and the epilogue runs on the
+// sums; no partial sum crosses memory unless the caller splits K.
 //
 // What the 16 MFMA rows of a tile are depends on the epilogue: 16 consecutive
 // rows of W, or 8 pairs (gate row p and up row p; rows j and j + hd/2 of one
 // head; two neighbouring value rows) with the first members in MFMA rows 0-7
 // and the second in rows 8-15.
+//
+// The kernel is kept small on purpose (loops over rounds and tiles, one copy of
+// the epilogue): a decode step runs a few workgroups of it per CU between other
+// kernels, with a cold instruction cache every time, and a version with the
+// epilogue unrolled into every round (74 KB of code) took half as long again.
 #include <math.h>
 
 #include "common.hpp"
@@ -40,18 +36,7 @@ constexpr int FL_PAD = 8;          // LDS row padding (elements): 16-byte reads 
 constexpr int FL_LDS_MAX = 160 * 1024;
 constexpr int FL_TILE = 16 * 17;    // floats of one wave's partial tile in LDS: [x row][w row], padded
 
-enum : int { FL_X_BF16 = 0, FL_X_RESIDUAL = 1 };
-enum : int { FL_PARTS = 0, FL_ADD = 1, FL_SWIGLU = 2, FL_ROPE = 3 };
-
-struct FlIn {
-  const void* x;
-  const float* delta;
-  float* x_out;
-  const float* norm_weight;
-  const int* rows;
-  int delta_splits;
-  float eps;
-};
+enum : int { FL_PARTS = 0, FL_SWIGLU = 2, FL_ROPE = 3 };
 
 struct FlOut {
   void* y;
@@ -67,7 +52,7 @@ struct FlOut {
 // Row of W behind MFMA row c of a tile, or -1.  Pair epilogues: unit = pair.
 template <int EP>
 __device__ __forceinline__ long fl_row(int tile, int c, int m, const FlOut& o) {
-  if (EP == FL_PARTS || EP == FL_ADD) {
+  if (EP == FL_PARTS) {
     const long r = (long)tile * 16 + c;
     return r < m ? r : -1;
   }
@@ -86,8 +71,8 @@ __device__ __forceinline__ long fl_row(int tile, int c, int m, const FlOut& o) {
   return (long)(o.H + o.KV) * o.hd + e + (second ? 1 : 0);
 }
 
-template <int NT, int XKIND, int EP>
-__global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
+template <int NT, int EP>
+__global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restrict__ X, FlOut out,
                                                            const bf16_t* __restrict__ W, int n, int m,
                                                            int k, int kslice, int tiles, int tiles_per_wg,
                                                            int x_stride) {
@@ -95,7 +80,6 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
   const int ld = kslice + FL_PAD;
   bf16_t* xs = reinterpret_cast<bf16_t*>(lds_raw);                            // [n][ld]
   float* part = reinterpret_cast<float*>(lds_raw + (size_t)n * ld * sizeof(bf16_t));   // [2][4][NT][x row 16][17]
-  float* inv = part + 2 * 4 * NT * FL_TILE;                                   // [NT * 16]
 
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int g = lane / 16, c = lane % 16;
@@ -153,87 +137,25 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
   advance();
 
   // ---- X into LDS: wave w takes rows w, w + 4, ...; eight loads in flight per lane
-  constexpr int RPW = NT * 4;                               // rows per wave at most
-  if (XKIND == FL_X_BF16) {
-    const bf16_t* X = reinterpret_cast<const bf16_t*>(in.x);
-    const int chunks = klen / 8;
-    const int mine = (n - wave + 3) / 4;                    // rows of this wave
-    const int items = mine * chunks;
-    for (int base = lane; base < items; base += kWave * 8) {
-      bf16x8 v[8];
+  const int chunks = klen / 8;
+  const int mine = (n - wave + 3) / 4;                    // rows of this wave
+  const int items = mine * chunks;
+  for (int base = lane; base < items; base += kWave * 8) {
+    bf16x8 v[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int idx = base + j * kWave;
+    for (int j = 0; j < 8; ++j) {
+      const int idx = base + j * kWave;
+      const int ri = idx / chunks, ch = idx - ri * chunks;
+      v[j] = idx < items ? *reinterpret_cast<const bf16x8*>(X + (long)(wave + 4 * ri) * x_stride + kbeg + ch * 8)
+                         : zero;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int idx = base + j * kWave;
+      if (idx < items) {
         const int ri = idx / chunks, ch = idx - ri * chunks;
-        v[j] = idx < items ? *reinterpret_cast<const bf16x8*>(X + (long)(wave + 4 * ri) * x_stride + kbeg + ch * 8)
-                           : zero;
+        *reinterpret_cast<bf16x8*>(&xs[(wave + 4 * ri) * ld + ch * 8]) = v[j];
       }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int idx = base + j * kWave;
-        if (idx < items) {
-          const int ri = idx / chunks, ch = idx - ri * chunks;
-          *reinterpret_cast<bf16x8*>(&xs[(wave + 4 * ri) * ld + ch * 8]) = v[j];
-        }
-      }
-    }
-  } else {
-    // float32 residual rows (+ partial sums) -> x_out, sum of squares, bfloat16(x * weight)
-    const float* X = reinterpret_cast<const float*>(in.x);
-    const int chunks = klen / 4;                            // klen == k here
-    const int mine = (n - wave + 3) / 4;
-    const int items = mine * chunks;
-    const bool write_x = in.x_out != nullptr && blockIdx.x == 0;
-    float ss[RPW];
-#pragma unroll
-    for (int j = 0; j < RPW; ++j) ss[j] = 0.f;
-    for (int base = lane; base < items; base += kWave * 4) {
-      floatx4 v[4], wv[4];
-      int ri[4], ch[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int idx = base + j * kWave;
-        ri[j] = idx / chunks;
-        ch[j] = idx - ri[j] * chunks;
-        const bool ok = idx < items;
-        const int r = wave + 4 * ri[j];
-        const long src = (ok && in.rows) ? in.rows[r] : r;
-        v[j] = ok ? *reinterpret_cast<const floatx4*>(X + src * (long)x_stride + ch[j] * 4) : floatx4{0, 0, 0, 0};
-        wv[j] = ok ? *reinterpret_cast<const floatx4*>(in.norm_weight + ch[j] * 4) : floatx4{0, 0, 0, 0};
-      }
-      for (int s = 0; s < in.delta_splits; ++s) {
-        floatx4 d[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int idx = base + j * kWave;
-          d[j] = idx < items ? *reinterpret_cast<const floatx4*>(
-                                   in.delta + ((long)s * n + wave + 4 * ri[j]) * k + ch[j] * 4)
-                             : floatx4{0, 0, 0, 0};
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] += d[j];
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int idx = base + j * kWave;
-        if (idx < items) {
-          const int r = wave + 4 * ri[j];
-          if (write_x) *reinterpret_cast<floatx4*>(in.x_out + (long)r * k + ch[j] * 4) = v[j];
-          const float sq = v[j][0] * v[j][0] + v[j][1] * v[j][1] + v[j][2] * v[j][2] + v[j][3] * v[j][3];
-#pragma unroll
-          for (int q = 0; q < RPW; ++q) ss[q] += (ri[j] == q) ? sq : 0.f;
-          bf16x4 b;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) b[e] = from_f32<bf16_t>(v[j][e] * wv[j][e]);
-          *reinterpret_cast<bf16x4*>(&xs[r * ld + ch[j] * 4]) = b;
-        }
-      }
-    }
-#pragma unroll
-    for (int q = 0; q < RPW; ++q) {
-      const float s = wave_sum(ss[q]);
-      const int r = wave + 4 * q;
-      if (lane == 0 && r < n) inv[r] = rsqrtf(s / (float)k + in.eps);
     }
   }
   int ep_page[NT], ep_slot[NT];
@@ -307,7 +229,7 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
     __syncthreads();
     const int tl = tile0 + tile;
     // Neighbouring threads take neighbouring rows of W: their stores share cache lines.
-    if (EP == FL_PARTS || EP == FL_ADD) {
+    if (EP == FL_PARTS) {
       const int r16 = tid % 16, xc = tid / 16;
       const long row = (long)tl * 16 + r16;
 #pragma unroll
@@ -316,12 +238,7 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
         float v = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; ++w) v += pb[(w * NT + t) * FL_TILE + xc * 17 + r16];
-        if (XKIND == FL_X_RESIDUAL && xr < n) v *= inv[xr];
-        if (row < m && xr < n) {
-          float* y = reinterpret_cast<float*>(out.y);
-          if (EP == FL_ADD) y[(long)xr * m + row] += v;
-          else y[((long)blockIdx.y * n + xr) * m + row] = v;
-        }
+        if (row < m && xr < n) reinterpret_cast<float*>(out.y)[((long)blockIdx.y * n + xr) * m + row] = v;
       }
     } else if (tid < 128) {
       const int p8 = tid % 8, xc = tid / 8;
@@ -336,10 +253,6 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
           b += pb[(w * NT + t) * FL_TILE + xc * 17 + p8 + 8];
         }
         if (pair >= pairs || xr >= n) continue;
-        if (XKIND == FL_X_RESIDUAL) {
-          a *= inv[xr];
-          b *= inv[xr];
-        }
         if (EP == FL_SWIGLU) {
           bf16_t* h = reinterpret_cast<bf16_t*>(out.y);
           h[(long)xr * pairs + pair] = from_f32<bf16_t>((a / (1.f + expf(-a))) * b);
@@ -375,34 +288,33 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(FlIn in, FlOut out,
 }
 
 static size_t fl_lds_bytes(int n, int nt, int kslice) {
-  return (size_t)n * (kslice + FL_PAD) * sizeof(bf16_t) + (size_t)(2 * 4 * nt * FL_TILE + nt * 16) * sizeof(float);
+  return (size_t)n * (kslice + FL_PAD) * sizeof(bf16_t) + (size_t)(2 * 4 * nt * FL_TILE) * sizeof(float);
 }
 
-template <int NT, int XKIND, int EP>
-static int fl_launch(const FlIn& in, const FlOut& out, const void* w, int n, int m, int k, int kslice,
+template <int NT, int EP>
+static int fl_launch(const void* x, const FlOut& out, const void* w, int n, int m, int k, int kslice,
                      int nsplit, int tiles, int tiles_per_wg, int x_stride, hipStream_t stream) {
   const size_t lds = fl_lds_bytes(n, NT, kslice);
   static size_t allowed = 64 * 1024;
   if (lds > allowed) {
-    hipError_t e = hipFuncSetAttribute((const void*)fused_linear_kernel<NT, XKIND, EP>,
+    hipError_t e = hipFuncSetAttribute((const void*)fused_linear_kernel<NT, EP>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, FL_LDS_MAX);
     if (e != hipSuccess) KLLM_FAIL((int)e, "fused_linear: cannot raise the LDS limit: %s", hipGetErrorString(e));
     allowed = FL_LDS_MAX;
   }
   const dim3 grid(ceil_div(tiles, tiles_per_wg), nsplit);
-  hipLaunchKernelGGL((fused_linear_kernel<NT, XKIND, EP>), grid, dim3(256), lds, stream, in, out,
+  hipLaunchKernelGGL((fused_linear_kernel<NT, EP>), grid, dim3(256), lds, stream, (const bf16_t*)x, out,
                      (const bf16_t*)w, n, m, k, kslice, tiles, tiles_per_wg, x_stride);
   return 0;
 }
 
-template <int NT, int XKIND>
-static int fl_launch_ep(int ep, const FlIn& in, const FlOut& out, const void* w, int n, int m, int k,
+template <int NT>
+static int fl_launch_ep(int ep, const void* x, const FlOut& out, const void* w, int n, int m, int k,
                         int kslice, int nsplit, int tiles, int tpw, int xs, hipStream_t st) {
   switch (ep) {
-    case FL_PARTS: return fl_launch<NT, XKIND, FL_PARTS>(in, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
-    case FL_ADD: return fl_launch<NT, XKIND, FL_ADD>(in, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
-    case FL_SWIGLU: return fl_launch<NT, XKIND, FL_SWIGLU>(in, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
-    default: return fl_launch<NT, XKIND, FL_ROPE>(in, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+    case FL_PARTS: return fl_launch<NT, FL_PARTS>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+    case FL_SWIGLU: return fl_launch<NT, FL_SWIGLU>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+    default: return fl_launch<NT, FL_ROPE>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
   }
 }
 
@@ -418,48 +330,28 @@ extern "C" long kllm_fused_linear_lds_bytes(int n, int k, int nsplit) {
   return (long)fl_lds_bytes(n, ceil_div(n, 16), kslice);
 }
 
-extern "C" int kllm_fused_linear(const KllmLinearIn* xin, const KllmLinearOut* yout, const void* w, int n,
-                                 int m, int k, int tiles_per_wg, hipStream_t stream) {
-  KLLM_REQUIRE(xin && yout && w && xin->x && yout->y, "fused_linear: null pointer");
+extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOut* yout, const void* w,
+                                 int n, int m, int k, int tiles_per_wg, hipStream_t stream) {
+  KLLM_REQUIRE(x && yout && w && yout->y, "fused_linear: null pointer");
   KLLM_REQUIRE(n > 0 && n <= KLLM_FUSED_LINEAR_MAX_ROWS, "fused_linear: n=%d is outside [1, %d]", n,
                KLLM_FUSED_LINEAR_MAX_ROWS);
   KLLM_REQUIRE(m > 0 && k > 0 && k % 8 == 0, "fused_linear: bad sizes m=%d k=%d (K must be a multiple of 8)", m, k);
-  KLLM_REQUIRE((long)m * k < (1L << 40), "fused_linear: sizes overflow");
-  KLLM_REQUIRE(fl_aligned16(w) && fl_aligned16(xin->x), "fused_linear: operands must be 16-byte aligned");
+  KLLM_REQUIRE((long)m * k < (1L << 40) && m < (1 << 30), "fused_linear: sizes overflow");
+  KLLM_REQUIRE(fl_aligned16(w) && fl_aligned16(x), "fused_linear: operands must be 16-byte aligned");
   KLLM_REQUIRE(tiles_per_wg >= 1 && tiles_per_wg <= 64, "fused_linear: %d tiles per workgroup", tiles_per_wg);
-  const int ep = yout->kind, xk = xin->kind;
-  KLLM_REQUIRE(xk == FL_X_BF16 || xk == FL_X_RESIDUAL, "fused_linear: unknown input kind %d", xk);
-  KLLM_REQUIRE(ep >= FL_PARTS && ep <= FL_ROPE, "fused_linear: unknown output kind %d", ep);
+  const int ep = yout->kind;
+  KLLM_REQUIRE(ep == FL_PARTS || ep == FL_SWIGLU || ep == FL_ROPE, "fused_linear: unknown output kind %d", ep);
   const int nsplit = yout->nsplit;
   KLLM_REQUIRE(nsplit >= 1 && nsplit <= 64, "fused_linear: nsplit %d is outside [1, 64]", nsplit);
-  KLLM_REQUIRE(nsplit == 1 || (ep == FL_PARTS && xk == FL_X_BF16),
-               "fused_linear: K is split only between bfloat16 input and partial sums");
+  KLLM_REQUIRE(nsplit == 1 || ep == FL_PARTS, "fused_linear: K is split only for partial sums");
   const int kslice = ceil_div(ceil_div(k, nsplit), 32) * 32;
   KLLM_REQUIRE((long)kslice * (nsplit - 1) < k, "fused_linear: nsplit %d leaves an empty slice of K=%d", nsplit, k);
   const int nt = ceil_div(n, 16);
   KLLM_REQUIRE(fl_lds_bytes(n, nt, kslice) <= (size_t)FL_LDS_MAX,
                "fused_linear: %d rows of K=%d need %zu bytes of LDS, more than %d", n, kslice,
                fl_lds_bytes(n, nt, kslice), FL_LDS_MAX);
-
-  FlIn in = {};
-  in.x = xin->x;
-  int x_stride = xin->x_stride > 0 ? xin->x_stride : k;
+  if (x_stride <= 0) x_stride = k;
   KLLM_REQUIRE(x_stride >= k && x_stride % 8 == 0, "fused_linear: row stride %d of x does not fit K=%d", x_stride, k);
-  if (xk == FL_X_RESIDUAL) {
-    KLLM_REQUIRE(xin->norm_weight && fl_aligned16(xin->norm_weight), "fused_linear: the norm's weight is missing");
-    KLLM_REQUIRE(xin->delta_splits >= 0 && (xin->delta_splits == 0 || xin->delta),
-                 "fused_linear: %d partial sums without a pointer", xin->delta_splits);
-    KLLM_REQUIRE(!xin->delta_splits || (xin->x_out && xin->x_out != xin->x && fl_aligned16(xin->x_out) &&
-                                        fl_aligned16(xin->delta)),
-                 "fused_linear: partial sums need a separate, aligned x_out");
-    KLLM_REQUIRE(!xin->rows || !xin->delta_splits, "fused_linear: gathered rows take no partial sums");
-    in.delta = xin->delta_splits ? xin->delta : nullptr;
-    in.delta_splits = xin->delta_splits;
-    in.x_out = xin->delta_splits ? xin->x_out : nullptr;
-    in.norm_weight = xin->norm_weight;
-    in.rows = xin->rows;
-    in.eps = xin->eps;
-  }
 
   FlOut out = {};
   out.y = yout->y;
@@ -489,14 +381,8 @@ extern "C" int kllm_fused_linear(const KllmLinearIn* xin, const KllmLinearOut* y
     out.KV = KV;
     out.hd = hd;
   }
-
-  int rc;
-  if (nt == 1)
-    rc = xk == FL_X_BF16 ? fl_launch_ep<1, FL_X_BF16>(ep, in, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream)
-                         : fl_launch_ep<1, FL_X_RESIDUAL>(ep, in, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream);
-  else
-    rc = xk == FL_X_BF16 ? fl_launch_ep<2, FL_X_BF16>(ep, in, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream)
-                         : fl_launch_ep<2, FL_X_RESIDUAL>(ep, in, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream);
+  const int rc = nt == 1 ? fl_launch_ep<1>(ep, x, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream)
+                         : fl_launch_ep<2>(ep, x, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream);
   if (rc) return rc;
   KLLM_CHECK_LAUNCH("fused_linear");
   return 0;

@@ -92,15 +92,9 @@ int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_out, const f
                           hipStream_t stream);
 
 /* Products of a decode batch (bfloat16, up to KLLM_FUSED_LINEAR_MAX_ROWS rows)
- * on the matrix cores, fused with the step before and the step after.
- * Input: bfloat16 activations [n][k] (row stride x_stride elements, 0 = k), or
- * float32 residual rows that are normalised on the way (RMSNorm with
- * norm_weight [k] and eps), optionally gathered through `rows`, optionally after
- * adding partial sums delta [delta_splits][n][k]; the sum x + delta is then
- * also written to x_out [n][k], which must not be x.
- * Output, w being [m][k]:
- *   PARTS   y float32 [nsplit][n][m]; only this one may split K (bfloat16 input)
- *   ADD     y float32 [n][m] += x . w^T
+ * on the matrix cores, fused with the step after them.  x is [n][k] with a row
+ * stride of x_stride elements (0 = k), w is [m][k].  Output:
+ *   PARTS   y float32 [nsplit][n][m]; only this one may split K
  *   SWIGLU  y bfloat16 [n][m/2] = silu(x . w[0:m/2]^T) * (x . w[m/2:m]^T)
  *   ROPE    w = [q; k; v] rows (only q when cache is null): q and k rotated with
  *           cos/sin [n][hd/2] (if given); y = q_out [n][H*hd], k and v go to the
@@ -108,23 +102,9 @@ int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_out, const f
  * All of a workgroup's slice of K for all rows has to fit into LDS:
  * kllm_fused_linear_lds_bytes says how much a call needs (160 KiB at most). */
 #define KLLM_FUSED_LINEAR_MAX_ROWS 32
-#define KLLM_LINEAR_IN_BF16 0
-#define KLLM_LINEAR_IN_RESIDUAL 1
 #define KLLM_LINEAR_OUT_PARTS 0
-#define KLLM_LINEAR_OUT_ADD 1
 #define KLLM_LINEAR_OUT_SWIGLU 2
 #define KLLM_LINEAR_OUT_ROPE 3
-typedef struct {
-  const void* x;
-  const float* delta;
-  float* x_out;
-  const float* norm_weight;
-  const int* rows;
-  int kind;
-  int x_stride;
-  int delta_splits;
-  float eps;
-} KllmLinearIn;
 typedef struct {
   void* y;
   const float* cos_t;
@@ -138,7 +118,7 @@ typedef struct {
   int max_pages, page_size, H, KV, hd;
 } KllmLinearOut;
 long kllm_fused_linear_lds_bytes(int n, int k, int nsplit);
-int kllm_fused_linear(const KllmLinearIn* in, const KllmLinearOut* out, const void* w, int n, int m,
+int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOut* out, const void* w, int n, int m,
                       int k, int tiles_per_wg, hipStream_t stream);
 
 /* Causal attention of n tokens over the paged cache; any head size up to 256. */

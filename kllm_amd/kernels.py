@@ -88,7 +88,7 @@ def _declare(lib):
         "kllm_gemv_plain": [P, P, P, I, I, I, I, P],
         "kllm_gemv_swiglu": [P, P, P, I, I, I, I, P],
         "kllm_gemv_rope_append": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
-        "kllm_fused_linear": [P, P, P, I, I, I, I, P],
+        "kllm_fused_linear": [P, I, P, P, I, I, I, I, P],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
         "kllm_attn_decode_slices": [I, I, I],
@@ -310,12 +310,6 @@ def gemv_rope_append(x, w_qkv, q_out, cos, sin, cache, positions, span_of_token,
         n_kv_heads, head_dim, k, dtype_code(x.dtype), _stream()), "gemv_rope_append")
 
 
-class _LinearIn(ctypes.Structure):
-    _fields_ = [("x", c_void_p), ("delta", c_void_p), ("x_out", c_void_p), ("norm_weight", c_void_p),
-                ("rows", c_void_p), ("kind", c_int), ("x_stride", c_int), ("delta_splits", c_int),
-                ("eps", c_float)]
-
-
 class _LinearOut(ctypes.Structure):
     _fields_ = [("y", c_void_p), ("cos_t", c_void_p), ("sin_t", c_void_p), ("cache", c_void_p),
                 ("positions", c_void_p), ("span_of_token", c_void_p), ("block_table", c_void_p),
@@ -325,7 +319,7 @@ class _LinearOut(ctypes.Structure):
 
 FUSED_LINEAR_MAX_ROWS = 32
 FUSED_LINEAR_LDS = 160 * 1024
-LINEAR_PARTS, LINEAR_ADD, LINEAR_SWIGLU, LINEAR_ROPE = 0, 1, 2, 3
+LINEAR_PARTS, LINEAR_SWIGLU, LINEAR_ROPE = 0, 2, 3
 
 
 # Rows up to which the decode-batch kernel beats the split-K kernel plus a separate
@@ -341,7 +335,7 @@ def fused_linear_fits(n, k, nsplit=1) -> bool:
         return False
     kslice = -(-(-(-k // nsplit)) // 32) * 32
     nt = -(-n // 16)
-    return n * (kslice + 8) * 2 + (2 * 4 * nt * 16 * 17 + nt * 16) * 4 <= FUSED_LINEAR_LDS
+    return n * (kslice + 8) * 2 + 2 * 4 * nt * 16 * 17 * 4 <= FUSED_LINEAR_LDS
 
 
 class Rope:
@@ -354,47 +348,23 @@ class Rope:
         self.page_size, self.heads, self.kv_heads, self.head_dim = page_size, heads, kv_heads, head_dim
 
 
-def fused_linear(w, y, kind, x=None, residual=None, norm_weight=None, eps=0.0, delta=None, x_out=None,
-                 rows=None, nsplit=1, tiles_per_wg=1, rope=None):
-    """One launch for a decode batch's product with w [m, k] (bfloat16).
-
-    Input: ``x`` bfloat16 [n, k] (a view with a row stride is taken), or
-    ``residual`` float32 [*, k] with ``norm_weight``/``eps`` (normalised on the
-    way), either gathered through ``rows`` or after adding ``delta``
-    [splits, n, k], the sum then also going to ``x_out``.
-    Output by ``kind``: LINEAR_PARTS y float32 [nsplit, n, m]; LINEAR_ADD y
-    float32 [n, m] +=; LINEAR_SWIGLU y bfloat16 [n, m/2]; LINEAR_ROPE y = q_out
-    with ``rope`` describing rotation and cache."""
+def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None):
+    """One launch for a decode batch's product of x [n, k] (bfloat16; a view
+    with a row stride is taken) with w [m, k], and the step after it, by
+    ``kind``: LINEAR_PARTS y float32 [nsplit, n, m]; LINEAR_SWIGLU y bfloat16
+    [n, m/2]; LINEAR_ROPE y = q_out with ``rope`` describing rotation and
+    cache."""
     m, k = w.shape
-    li, lo = _LinearIn(), _LinearOut()
-    if (x is None) == (residual is None):
-        raise KernelError("fused_linear: give either x or residual")
+    lo = _LinearOut()
     if w.dtype != torch.bfloat16:
         raise KernelError("fused_linear: bfloat16 weights only")
-    if x is not None:
-        n = x.shape[0]
-        if x.dim() != 2 or x.shape[1] != k or x.dtype != torch.bfloat16 or x.stride(1) != 1 or not x.is_cuda:
-            raise KernelError(f"fused_linear: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)}")
-        li.x, li.kind, li.x_stride = x.data_ptr(), 0, x.stride(0) if n > 1 else k
-    else:
-        if residual.dim() != 2 or residual.shape[1] != k or norm_weight is None or norm_weight.numel() != k:
-            raise KernelError("fused_linear: residual or norm weight does not fit")
-        n = rows.numel() if rows is not None else residual.shape[0]
-        li.x, li.kind, li.x_stride = _ptr(residual, "fused_linear residual", torch.float32), 1, k
-        li.norm_weight = _ptr(norm_weight, "fused_linear norm weight", torch.float32)
-        li.eps = eps
-        li.rows = _ptr(rows, "fused_linear rows", torch.int32, True)
-        if delta is not None:
-            if delta.dim() != 3 or tuple(delta.shape[1:]) != (n, k) or x_out is None or tuple(x_out.shape) != (n, k):
-                raise KernelError("fused_linear: delta or x_out does not fit")
-            li.delta = _ptr(delta, "fused_linear delta", torch.float32)
-            li.delta_splits = delta.shape[0]
-            li.x_out = _ptr(x_out, "fused_linear x_out", torch.float32)
+    n = x.shape[0]
+    if x.dim() != 2 or x.shape[1] != k or x.dtype != torch.bfloat16 or x.stride(1) != 1 or not x.is_cuda:
+        raise KernelError(f"fused_linear: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)}")
+    x_stride = x.stride(0) if n > 1 else k
     lo.kind, lo.nsplit = kind, nsplit
     if kind == LINEAR_PARTS:
         want, dt = (nsplit, n, m), torch.float32
-    elif kind == LINEAR_ADD:
-        want, dt = (n, m), torch.float32
     elif kind == LINEAR_SWIGLU:
         want, dt = (n, m // 2), torch.bfloat16
     elif kind == LINEAR_ROPE:
@@ -423,7 +393,7 @@ def fused_linear(w, y, kind, x=None, residual=None, norm_weight=None, eps=0.0, d
     if tuple(y.shape) != want or y.dtype != dt:
         raise KernelError(f"fused_linear: output {tuple(y.shape)} {y.dtype}, expected {want} {dt}")
     lo.y = _ptr(y, "fused_linear y")
-    _check(library().kllm_fused_linear(ctypes.byref(li), ctypes.byref(lo), _ptr(w, "fused_linear w"), n, m, k,
+    _check(library().kllm_fused_linear(x.data_ptr(), x_stride, ctypes.byref(lo), _ptr(w, "fused_linear w"), n, m, k,
                                        tiles_per_wg, _stream()), "fused_linear")
 
 

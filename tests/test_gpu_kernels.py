@@ -266,83 +266,33 @@ def _bf(*shape, seed, scale):
 @pytest.mark.parametrize("n,m,k,nsplit,tpw", [(1, 48, 64, 1, 1), (8, 2048, 2048, 1, 1), (5, 100, 264, 1, 3),
                                               (16, 72, 520, 2, 1), (19, 33, 4104, 3, 2), (32, 257, 1000, 1, 4),
                                               (8, 176, 5632, 1, 1)])
-def test_fused_linear_parts_and_add(n, m, k, nsplit, tpw):
-    """bfloat16 rows in, partial sums out; and the sums added into float32 rows in place."""
+def test_fused_linear_parts(n, m, k, nsplit, tpw):
+    """bfloat16 rows in, float32 sums (or partial sums over slices of K) out."""
     k_ = K()
     x, w = _bf(n, k, seed=1, scale=0.5), _bf(m, k, seed=2, scale=0.1)
     want = P.linear(x.cpu().double(), w.cpu().double())
     bound = 1e-3 * math.sqrt(k) * 0.05 + 1e-4
     y = torch.full((nsplit, n, m), float("nan"), device=DEV)
-    k_.fused_linear(w, y, k_.LINEAR_PARTS, x=x, nsplit=nsplit, tiles_per_wg=tpw)
+    k_.fused_linear(w, y, k_.LINEAR_PARTS, x, nsplit=nsplit, tiles_per_wg=tpw)
     assert (y.cpu().double().sum(0) - want).abs().max() < bound
     if nsplit == 1:
-        base = rnd(n, m, seed=3)
-        acc = base.clone()
-        k_.fused_linear(w, acc, k_.LINEAR_ADD, x=x, tiles_per_wg=tpw)
-        assert (acc.cpu().double() - base.cpu().double() - want).abs().max() < bound
         # a view with a row stride (columns of a wider buffer)
         wide = torch.zeros(n, k + 16, dtype=torch.bfloat16, device=DEV)
         wide[:, 8:8 + k] = x
         y2 = torch.full((1, n, m), float("nan"), device=DEV)
-        k_.fused_linear(w, y2, k_.LINEAR_PARTS, x=wide[:, 8:8 + k], tiles_per_wg=tpw)
+        k_.fused_linear(w, y2, k_.LINEAR_PARTS, wide[:, 8:8 + k], tiles_per_wg=tpw)
         assert torch.equal(y2, y)
 
 
-@pytest.mark.parametrize("n,m,k,splits", [(1, 48, 64, 0), (8, 2560, 2048, 2), (7, 100, 264, 1), (16, 40, 1000, 0),
-                                          (21, 64, 520, 3)])
-def test_fused_linear_normalises_the_residual(n, m, k, splits):
-    """float32 residual (+ partial sums) in: x_out, and the product with the RMS-normalised rows."""
-    k_ = K()
-    eps = 1e-5
-    x, nw = rnd(n, k, seed=1, scale=3.0), (1 + 0.2 * rnd(k, seed=2))
-    w = _bf(m, k, seed=4, scale=0.1)
-    delta = rnd(splits, n, k, seed=3) if splits else None
-    x_out = torch.full((n, k), float("nan"), device=DEV) if splits else None
-    xs = x.cpu().double() + (delta.cpu().double().sum(0) if splits else 0)
-    want = P.linear(P.rmsnorm(xs, nw.cpu().double(), eps), w.cpu().double())
-    x0 = x.clone()
-    y = torch.full((1, n, m), float("nan"), device=DEV)
-    k_.fused_linear(w, y, k_.LINEAR_PARTS, residual=x0, norm_weight=nw, eps=eps, delta=delta, x_out=x_out)
-    assert torch.equal(x0, x)
-    if splits:
-        assert (x_out.cpu().double() - xs).abs().max() < 1e-5
-    assert (y[0].cpu().double() - want).abs().max() < 0.01 * want.abs().max() + 1e-3
-    # gathered rows
-    if not splits and n >= 3:
-        rows = torch.tensor([n - 1, 0, 2], dtype=torch.int32, device=DEV)
-        y3 = torch.full((1, 3, m), float("nan"), device=DEV)
-        k_.fused_linear(w, y3, k_.LINEAR_PARTS, residual=x0, norm_weight=nw, eps=eps, rows=rows)
-        assert (y3[0].cpu().double() - want[[n - 1, 0, 2]]).abs().max() < 0.01 * want.abs().max() + 1e-3
-
-
-def test_fused_linear_norm_catches_a_wrong_place_of_eps_and_weight():
-    """One row of tiny numbers: eps inside the root matters, and the weight multiplies after."""
-    k_ = K()
-    n, m, k, eps = 2, 32, 64, 1e-2
-    x = torch.cat([rnd(1, k, seed=1, scale=1e-2), rnd(1, k, seed=5, scale=2.0)])
-    nw = (1 + 0.5 * rnd(k, seed=2))
-    w = _bf(m, k, seed=4, scale=0.2)
-    want = P.linear(P.rmsnorm(x.cpu().double(), nw.cpu().double(), eps), w.cpu().double())
-    y = torch.empty(1, n, m, device=DEV)
-    k_.fused_linear(w, y, k_.LINEAR_PARTS, residual=x, norm_weight=nw, eps=eps)
-    assert (y[0].cpu().double() - want).abs().max() < 0.01 * want.abs().max()
-
-
-@pytest.mark.parametrize("n,f,k,norm", [(1, 176, 64, False), (3, 120, 88, True), (8, 5632, 2048, True),
-                                        (20, 33, 520, False), (16, 100, 264, True)])
-def test_fused_linear_swiglu(n, f, k, norm):
+@pytest.mark.parametrize("n,f,k,tpw", [(1, 176, 64, 1), (3, 120, 88, 2), (8, 5632, 2048, 1), (20, 33, 520, 1),
+                                       (16, 100, 264, 3)])
+def test_fused_linear_swiglu(n, f, k, tpw):
     k_ = K()
     w = _bf(2 * f, k, seed=2, scale=0.1)
     h = torch.full((n, f), float("nan"), dtype=torch.bfloat16, device=DEV)
-    if norm:
-        x, nw = rnd(n, k, seed=1, scale=2.0), (1 + 0.2 * rnd(k, seed=6))
-        k_.fused_linear(w, h, k_.LINEAR_SWIGLU, residual=x, norm_weight=nw, eps=1e-6, tiles_per_wg=2)
-        xd = P.rmsnorm(x.cpu().double(), nw.cpu().double(), 1e-6)
-    else:
-        x = _bf(n, k, seed=1, scale=0.5)
-        k_.fused_linear(w, h, k_.LINEAR_SWIGLU, x=x)
-        xd = x.cpu().double()
-    wd = w.cpu().double()
+    x = _bf(n, k, seed=1, scale=0.5)
+    k_.fused_linear(w, h, k_.LINEAR_SWIGLU, x, tiles_per_wg=tpw)
+    xd, wd = x.cpu().double(), w.cpu().double()
     want = P.silu(P.linear(xd, wd[:f])) * P.linear(xd, wd[f:])
     assert (h.cpu().double() - want).abs().max() < 0.01 * want.abs().max() + 1e-3
 
@@ -350,9 +300,9 @@ def test_fused_linear_swiglu(n, f, k, norm):
 @pytest.mark.parametrize("H,KV,hd,ps,d", [(4, 2, 16, 16, 64), (3, 1, 32, 16, 96), (5, 5, 48, 32, 88),
                                           (32, 4, 64, 16, 2048), (3, 3, 80, 16, 104)])
 def test_fused_linear_rope_append(H, KV, hd, ps, d):
-    """Norm, projections, rotation and append in one launch, against the plain functions."""
+    """Projections, rotation and append in one launch, against the plain functions."""
     k_ = K()
-    theta, eps = 10000.0, 1e-5
+    theta = 10000.0
     spans = [(37, 3), (0, 2), (ps - 1, 1), (5, 11)]       # seventeen tokens of four requests
     n = sum(l for _, l in spans)
     pos = torch.tensor([p0 + i for p0, l in spans for i in range(l)], dtype=torch.int32, device=DEV)
@@ -360,16 +310,15 @@ def test_fused_linear_rope_append(H, KV, hd, ps, d):
     tables = [[9, 4, 11], [2, -1, -1], [7, -1, -1], [3, -1, -1]]
     bt = torch.tensor(tables, dtype=torch.int32, device=DEV)
     qd, kvd = H * hd, KV * hd
-    x, nw = rnd(n, d, seed=3, scale=2.0), (1 + 0.2 * rnd(d, seed=6))
+    x = _bf(n, d, seed=3, scale=0.5)
     w = _bf(qd + 2 * kvd, d, seed=4, scale=0.1)
     cos = torch.empty(n, hd // 2, device=DEV)
     sin = torch.empty(n, hd // 2, device=DEV)
     k_.rope_tables(cos, sin, pos, hd, theta)
     cache = torch.full((12, 2, KV, ps * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
     q_out = torch.full((n, qd), float("nan"), dtype=torch.bfloat16, device=DEV)
-    k_.fused_linear(w, q_out, k_.LINEAR_ROPE, residual=x, norm_weight=nw, eps=eps,
-                    rope=k_.Rope(cos, sin, cache, pos, sot, bt, ps, H, KV, hd))
-    full = P.linear(P.rmsnorm(x.cpu().double(), nw.cpu().double(), eps), w.cpu().double())
+    k_.fused_linear(w, q_out, k_.LINEAR_ROPE, x, rope=k_.Rope(cos, sin, cache, pos, sot, bt, ps, H, KV, hd))
+    full = P.linear(x.cpu().double(), w.cpu().double())
     want_q = P.rope(full[:, :qd], pos.cpu().tolist(), H, hd, theta)
     want_k = P.rope(full[:, qd:qd + kvd], pos.cpu().tolist(), KV, hd, theta)
     want_v = full[:, qd + kvd:]
@@ -382,10 +331,10 @@ def test_fused_linear_rope_append(H, KV, hd, ps, d):
         assert (v[p0:].double() - want_v[off:off + l]).abs().max() < t
         assert torch.isnan(k[:p0]).all() and torch.isnan(v[:p0]).all()
         off += l
-    # query only (a run that reads another run's cache), without rotation, bfloat16 rows in
+    # query only (a run that reads another run's cache), without rotation
     xb = _bf(n, d, seed=8, scale=0.5)
     q2 = torch.full((n, qd), float("nan"), dtype=torch.bfloat16, device=DEV)
-    k_.fused_linear(w[:qd].contiguous(), q2, k_.LINEAR_ROPE, x=xb,
+    k_.fused_linear(w[:qd].contiguous(), q2, k_.LINEAR_ROPE, xb,
                     rope=k_.Rope(None, None, None, None, None, None, ps, H, KV, hd))
     want2 = P.linear(xb.cpu().double(), w[:qd].cpu().double())
     assert (q2.cpu().double() - want2).abs().max() < 0.01 * want2.abs().max() + 1e-3
@@ -396,16 +345,17 @@ def test_fused_linear_refuses_what_it_does_not_take():
     w = _bf(32, 64, seed=1, scale=0.1)
     y = torch.empty(1, 33, 32, device=DEV)
     with pytest.raises(k_.KernelError, match="outside"):
-        k_.fused_linear(w, y, k_.LINEAR_PARTS, x=_bf(33, 64, seed=2, scale=1.0))
+        k_.fused_linear(w, y, k_.LINEAR_PARTS, _bf(33, 64, seed=2, scale=1.0))
     with pytest.raises(k_.KernelError, match="multiple of 8"):
         k_.fused_linear(_bf(32, 60, seed=1, scale=0.1), torch.empty(1, 4, 32, device=DEV), k_.LINEAR_PARTS,
-                        x=_bf(4, 60, seed=2, scale=1.0))
+                        _bf(4, 60, seed=2, scale=1.0))
     with pytest.raises(k_.KernelError, match="LDS"):
         k_.fused_linear(_bf(16, 8192, seed=1, scale=0.1), torch.empty(1, 32, 16, device=DEV), k_.LINEAR_PARTS,
-                        x=_bf(32, 8192, seed=2, scale=1.0))
+                        _bf(32, 8192, seed=2, scale=1.0))
     assert not k_.fused_linear_fits(32, 8192) and k_.fused_linear_fits(32, 8192, 4) and k_.fused_linear_fits(8, 5632)
     with pytest.raises(k_.KernelError, match="split"):
-        k_.fused_linear(w, torch.empty(4, 32, device=DEV), k_.LINEAR_ADD, x=_bf(4, 64, seed=2, scale=1.0), nsplit=2)
+        k_.fused_linear(_bf(32, 64, seed=1, scale=0.1), torch.empty(4, 16, dtype=torch.bfloat16, device=DEV),
+                        k_.LINEAR_SWIGLU, _bf(4, 64, seed=2, scale=1.0), nsplit=2)
 
 
 def test_fused_gemv_refuses_what_it_does_not_take():

@@ -109,36 +109,57 @@ __global__ __launch_bounds__(256) void gemm_f32_tiled_kernel(const float* __rest
 }
 
 // ------------------------------------------------------------------ bf16 MFMA tiles
-// Workgroup tile 128 (rows of X) x 128 (rows of W), 32 of K per stage, two LDS
-// stages.  Four waves in 2 x 2, each 64 x 64 = 2 x 2 MFMA tiles of 32 x 32.
-// MFMA 32x32x16: lane l holds A[l%32][8*(l/32) .. +8], B[8*(l/32) .. +8][l%32]
-// and D[8*(i/4) + 4*(l/32) + i%4][l%32] for i = 0..15.
-constexpr int MBN = 128, MBK = 32;
-constexpr int MLD = MBK + 8;  // LDS row stride in elements (80 bytes: 16-byte reads stay conflict-free)
-
+// Workgroup tile 128 (rows of X) x 128 (rows of W), 64 of K per stage, two or
+// three LDS stages.  Four waves in 2 x 2, each 2 x 2 MFMA tiles of 32 x 32.
+// MFMA 32x32x16: lane l holds A[l%32][8*(l/32)..+7], B[l%32][...] likewise, and
+// D[8*(i/4) + 4*(l/32) + i%4][l%32] in accumulator register i.
+//
+// Operands go from memory to LDS directly (global_load_lds, 16 bytes per
+// lane), one or two stages ahead of the MFMAs, without passing through
+// registers: nothing waits on a register stage and no ds_write is issued.
+// Such a load puts lane l's 16 bytes at LDS base + 16 l, so a wave's
+// instruction fills 8 rows x 128 bytes of an unpadded tile -- whole cache
+// lines of both operands, which measured a third faster than 64-byte rows.
+// Bank conflicts of the 16-byte reads are avoided by a swizzle instead of
+// padding: row r keeps its chunk c (8 elements) in slot c ^ swz(r), which the
+// loading lane arranges by choosing which chunk it fetches.  Rows beyond the
+// matrices are clamped to the last row (their results are never stored) and
+// chunks beyond K come from a page of zeros.
+//
+// Stages: two (64 KB of LDS, two workgroups per CU) when the product has more
+// tiles than CUs; three (one workgroup per CU, a deeper queue of loads) when
+// every CU gets at most one tile.
+//
 // DUAL: W is [gate rows; up rows] = [2m, k]; a workgroup takes 64 gate rows and
 // the 64 up rows that belong to them, and writes silu(gate) * up for m columns
 // (reference: backend/model.cu:477-483, :1112-1114) -- the gated activation
 // never exists in 32-bit in memory.
 //
-// Global loads run three stages ahead of the MFMAs (three register sets in
-// rotation, two LDS stages), so that a stage's loads have two stages of
-// compute to arrive.  Workgroups are numbered so that the eight XCDs (which
-// take workgroups round-robin, each with an L2 of its own) each get a
-// contiguous run of tiles that share rows of X.
-template <typename TOUT, bool DUAL>
-__global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ X,
+// Workgroups are numbered so that the eight XCDs (which take workgroups
+// round-robin, each with an L2 of its own) each get a contiguous run of tiles
+// that share rows of X.
+constexpr int MBN = 128, MBK = 64;
+constexpr int MROW = MBK * 2;                 // bytes of a tile row in LDS
+
+__device__ __attribute__((aligned(16))) bf16_t g_zero_chunk[8];   // zero-initialised
+
+// Slot permutation of a row's eight chunks: rows of equal parity among 16 neighbours get
+// different slots, so that the 16-byte reads of 16 lanes spread over all 64 banks.
+__device__ __forceinline__ int mfma_swz(int row) { return (row >> 1) & 7; }
+
+template <typename TOUT, bool DUAL, int MSTAGES>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ X,
                                                              const bf16_t* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
                                                              int k, int tiles_x, int tiles_y) {
-  // 32-row MFMA tiles per wave.  4 (a 256-row workgroup tile) halves the traffic per flop
-  // but needs 268 registers, one wave per SIMD, and measured 15% slower than 2.
+  // 32-row MFMA tiles per wave.  4 (a 256-row workgroup tile) halves the traffic per flop but
+  // leaves one workgroup per CU, and measured 10% slower than 2.
   constexpr int WTM = 2;
   constexpr int BM = 64 * WTM;                  // rows of X per workgroup
-  constexpr int XPASS = BM / 64;                // loads of X per thread and stage
-  extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
-  bf16_t* Xs = lds;                             // [2][BM * MLD]
-  bf16_t* Ws = lds + 2 * BM * MLD;              // [2][MBN * MLD]
+  constexpr int XI = BM / 32;                   // load instructions of X per wave and stage (8 rows each)
+  constexpr int WI = MBN / 32;
+  constexpr int XBYTES = BM * MROW, WBYTES = MBN * MROW;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];   // [MSTAGES][X tile | W tile]
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int wr = wave / 2, wc = wave % 2;
   const long total = (long)tiles_x * tiles_y;
@@ -152,53 +173,42 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
   const long tcol = x_major ? id / tiles_y : id % tiles_x;
   const long row0 = trow * BM, col0 = tcol * (DUAL ? MBN / 2 : MBN);
 
-  // Loads of one stage: rows x 4 chunks of 8 elements per operand; each thread takes
-  // chunk (tid % 4) of rows tid/4 + 64h.  DUAL: LDS rows 0..63 of W are gate rows,
-  // 64..127 the up rows of the same columns.
-  const int lrow = tid / 4, lchunk = (tid % 4) * 8;
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  const bf16_t* xptr[XPASS];
-  const bf16_t* wptr[2];
-  bool xok[XPASS], wok[2];
+  // Wave w loads rows [8 XI w, 8 XI (w+1)) of the X tile and [32 w, 32 w + 32) of the W
+  // tile.  In one instruction lane l serves row l / 8 (of 8), slot l % 8.
+  const bf16_t* xsrc[XI];
+  const bf16_t* wsrc[WI];
+  int xchunk[XI], wchunk[WI];
 #pragma unroll
-  for (int h = 0; h < XPASS; ++h) {
-    const long xr = row0 + lrow + h * 64;
-    xok[h] = xr < n;
-    xptr[h] = X + (xok[h] ? xr : 0) * k + lchunk;
+  for (int i = 0; i < XI; ++i) {
+    const int r = 8 * (XI * wave + i) + lane / 8;
+    xchunk[i] = ((lane % 8) ^ mfma_swz(r)) * 8;
+    xsrc[i] = X + min(row0 + r, (long)n - 1) * k + xchunk[i];
   }
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const long wcol = DUAL ? col0 + lrow : col0 + lrow + h * 64;   // output column
-    const long wrow = DUAL ? wcol + (long)h * m : wcol;
-    wok[h] = wcol < m;
-    wptr[h] = W + (wok[h] ? wrow : 0) * k + lchunk;
+  for (int i = 0; i < WI; ++i) {
+    const int r = 32 * wave + 8 * i + lane / 8;               // DUAL: rows 0..63 gate, 64..127 up
+    wchunk[i] = ((lane % 8) ^ mfma_swz(r)) * 8;
+    const long col = DUAL ? col0 + r % 64 : col0 + r;
+    const long wrow = min(col, (long)m - 1) + (DUAL && r >= 64 ? m : 0);
+    wsrc[i] = W + wrow * k + wchunk[i];
   }
-  // Loads carry no branch and no select: rows and K offsets outside the matrices are
-  // clamped to valid addresses here and replaced by zeros when the stage is stored, so
-  // that the loop is straight-line code and a store waits only for its own, oldest loads.
-  struct Stage {
-    bf16x8 x[XPASS], w[2];
-  };
-  auto load_stage = [&](int kt) -> Stage {
-    Stage st;
+  auto issue = [&](int kt) {
+    unsigned char* base = lds + (kt % MSTAGES) * (XBYTES + WBYTES);
     const int kk = kt * MBK;
-    const int koff = (kk + lchunk < k) ? kk : 0;
 #pragma unroll
-    for (int h = 0; h < XPASS; ++h) st.x[h] = *reinterpret_cast<const bf16x8*>(xptr[h] + koff);
+    for (int i = 0; i < XI; ++i) {
+      const bf16_t* src = kk + xchunk[i] < k ? xsrc[i] + kk : g_zero_chunk;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(base + 8 * (XI * wave + i) * MROW),
+                                       16, 0, 0);
+    }
 #pragma unroll
-    for (int h = 0; h < 2; ++h) st.w[h] = *reinterpret_cast<const bf16x8*>(wptr[h] + koff);
-    return st;
-  };
-  auto store_stage = [&](const Stage& st, int kt, int buf) {
-    const bool kin = kt * MBK + lchunk < k;
-#pragma unroll
-    for (int h = 0; h < XPASS; ++h)
-      *reinterpret_cast<bf16x8*>(&Xs[buf * BM * MLD + (lrow + h * 64) * MLD + lchunk]) =
-          (xok[h] && kin) ? st.x[h] : zero;
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-      *reinterpret_cast<bf16x8*>(&Ws[buf * MBN * MLD + (lrow + h * 64) * MLD + lchunk]) =
-          (wok[h] && kin) ? st.w[h] : zero;
+    for (int i = 0; i < WI; ++i) {
+      const bf16_t* src = kk + wchunk[i] < k ? wsrc[i] + kk : g_zero_chunk;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(base + XBYTES + (32 * wave + 8 * i) * MROW),
+                                       16, 0, 0);
+    }
   };
 
   floatx16 acc[WTM][2];
@@ -209,47 +219,43 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  auto compute = [&](int cur) {
+  const int ktiles = (k + MBK - 1) / MBK;
+  issue(0);
+  if (MSTAGES > 2 && ktiles > 1) issue(1);
+  for (int kt = 0; kt < ktiles; ++kt) {
+    // This wave's loads of stage kt have landed when at most the newer stage's (XI + WI
+    // instructions, with three stages) are still in flight; after the barrier so have every
+    // wave's, and every wave is done reading the stage that the next loads overwrite.  The
+    // barrier is a bare s_barrier: a fence here would also wait for the newest loads.
+    if (MSTAGES > 2 && kt + 1 < ktiles) __builtin_amdgcn_s_waitcnt(0x0F70 | (XI + WI));   // vmcnt(XI + WI)
+    else __builtin_amdgcn_s_waitcnt(0x0F70);                                             // vmcnt(0)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (kt + MSTAGES - 1 < ktiles) issue(kt + MSTAGES - 1);
+    const unsigned char* xs = lds + (kt % MSTAGES) * (XBYTES + WBYTES);
+    const unsigned char* ws = xs + XBYTES;
 #pragma unroll
-    for (int ks = 0; ks < MBK; ks += 16) {
+    for (int ks = 0; ks < MBK / 16; ++ks) {
       bf16x8 a[WTM], b[2];
+      const int chunk = ks * 2 + lane / 32;
 #pragma unroll
-      for (int i = 0; i < WTM; ++i)
-        a[i] = *reinterpret_cast<const bf16x8*>(
-            &Xs[cur * BM * MLD + (wr * 32 * WTM + i * 32 + lane % 32) * MLD + ks + (lane / 32) * 8]);
+      for (int i = 0; i < WTM; ++i) {
+        const int r = wr * 32 * WTM + i * 32 + lane % 32;
+        a[i] = *reinterpret_cast<const bf16x8*>(xs + r * MROW + (chunk ^ mfma_swz(r)) * 16);
+      }
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        b[j] = *reinterpret_cast<const bf16x8*>(
-            &Ws[cur * MBN * MLD + ((DUAL ? j * 64 + wc * 32 : wc * 64 + j * 32) + lane % 32) * MLD + ks +
-                (lane / 32) * 8]);
+      for (int j = 0; j < 2; ++j) {
+        const int r = (DUAL ? j * 64 + wc * 32 : wc * 64 + j * 32) + lane % 32;
+        b[j] = *reinterpret_cast<const bf16x8*>(ws + r * MROW + (chunk ^ mfma_swz(r)) * 16);
+      }
 #pragma unroll
       for (int i = 0; i < WTM; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
     }
-  };
-
-  const int ktiles = (k + MBK - 1) / MBK;
-  Stage r0 = load_stage(0), r1 = load_stage(1), r2 = load_stage(2);
-  store_stage(r0, 0, 0);
-  __syncthreads();
-  // Stage kt: tile kt is in LDS[kt & 1]; SA holds tile kt+1, SL is free for tile kt+3.
-#define KLLM_GEMM_STAGE(kt_, SA, SL)                                                    \
-  if ((kt_) < ktiles) {                                                                 \
-    SL = load_stage((kt_) + 3);                                                         \
-    compute((kt_) & 1);                                                                 \
-    if ((kt_) + 1 < ktiles) {                                                           \
-      store_stage(SA, (kt_) + 1, ((kt_) + 1) & 1); /* read before the last barrier */   \
-      __syncthreads();                                                                  \
-    }                                                                                   \
   }
-  for (int kt = 0; kt < ktiles; kt += 3) {
-    KLLM_GEMM_STAGE(kt, r1, r0)
-    KLLM_GEMM_STAGE(kt + 1, r2, r1)
-    KLLM_GEMM_STAGE(kt + 2, r0, r2)
-  }
-#undef KLLM_GEMM_STAGE
 
   if (DUAL) {
     const long c = col0 + wc * 32 + lane % 32;
@@ -278,14 +284,28 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
     }
 }
 
-template <typename TOUT, bool DUAL>
-static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, hipStream_t stream) {
+template <typename TOUT, bool DUAL, int MSTAGES>
+static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m, int k, hipStream_t stream) {
   const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN), ty = ceil_div(n, 128);
   const dim3 grid(ceil_div((long)tx * ty, 8) * 8);   // padded so that every XCD gets as many
-  const size_t lds = (size_t)2 * (128 + MBN) * MLD * sizeof(bf16_t);
-  hipLaunchKernelGGL((gemm_bf16_mfma_kernel<TOUT, DUAL>), grid, dim3(256), lds, stream,
+  const size_t lds = (size_t)MSTAGES * (128 + MBN) * MROW;
+  static int raised = 0;
+  if (lds > 64 * 1024 && !raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_mfma_kernel<TOUT, DUAL, MSTAGES>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) KLLM_FAIL((int)e, "gemm mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = 1;
+  }
+  hipLaunchKernelGGL((gemm_bf16_mfma_kernel<TOUT, DUAL, MSTAGES>), grid, dim3(256), lds, stream,
                      (const bf16_t*)x, (const bf16_t*)w, (TOUT*)y, n, m, k, tx, ty);
   return 0;
+}
+
+template <typename TOUT, bool DUAL>
+static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, hipStream_t stream) {
+  const long tiles = (long)ceil_div(n, 128) * ceil_div(m, DUAL ? MBN / 2 : MBN);
+  if (tiles <= 256) return launch_mfma_tile<TOUT, DUAL, 3>(x, w, y, n, m, k, stream);   // one per CU at most
+  return launch_mfma_tile<TOUT, DUAL, 2>(x, w, y, n, m, k, stream);
 }
 
 // ------------------------------------------------------------------ bf16 MFMA skinny

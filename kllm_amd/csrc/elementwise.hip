@@ -211,6 +211,70 @@ __global__ void rope_append_kernel(const TIN* __restrict__ qkv, int nsplit, long
   }
 }
 
+// The same for whole float32 sums (one split) and head sizes that are multiples of 8: a
+// thread takes four neighbouring pairs, or four values, with 16-byte loads, and its loads go
+// out before the token's page is looked up, so that the two waits overlap.
+template <typename T>
+__global__ void rope_append_vec_kernel(const float* __restrict__ qkv, T* __restrict__ q_out,
+                                       const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                       T* __restrict__ cache, const int* __restrict__ positions,
+                                       const int* __restrict__ span_of_token,
+                                       const int* __restrict__ block_table, int max_pages,
+                                       int page_size, int H, int KV, int hd) {
+  typedef T tx4 __attribute__((ext_vector_type(4)));
+  const long t = blockIdx.x;
+  const int half = hd / 2;
+  const int qd = H * hd, kvd = cache ? KV * hd : 0;
+  const float* in = qkv + t * (qd + 2 * kvd);
+  const int q_items = H * half / 4, k_items = cache ? KV * half / 4 : 0;
+  const int items = q_items + k_items + kvd / 4;
+  const int item = blockIdx.y * blockDim.x + threadIdx.x;
+  if (item >= items) return;
+  const bool rotated = item < q_items + k_items;
+  const bool is_q = item < q_items;
+  int h, j;
+  floatx4 a, b = {0, 0, 0, 0}, cc = {1, 1, 1, 1}, sn = {0, 0, 0, 0};
+  if (rotated) {
+    const int idx = (is_q ? item : item - q_items) * 4;
+    h = idx / half;
+    j = idx % half;
+    const float* src = in + (is_q ? 0 : qd) + h * hd + j;
+    a = *reinterpret_cast<const floatx4*>(src);
+    b = *reinterpret_cast<const floatx4*>(src + half);
+    if (cos_t) {
+      cc = *reinterpret_cast<const floatx4*>(cos_t + t * half + j);
+      sn = *reinterpret_cast<const floatx4*>(sin_t + t * half + j);
+    }
+  } else {
+    const int idx = (item - q_items - k_items) * 4;
+    h = idx / hd;
+    j = idx % hd;
+    a = *reinterpret_cast<const floatx4*>(in + qd + kvd + idx);
+  }
+  int page = 0, slot = 0;
+  if (cache && !is_q) {
+    const int pos = positions[t];
+    page = block_table[(long)span_of_token[t] * max_pages + pos / page_size];
+    slot = pos % page_size;
+  }
+  const long block = (long)page_size * hd;
+  if (rotated) {
+    tx4 lo, hi;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      lo[e] = from_f32<T>(a[e] * cc[e] - b[e] * sn[e]);
+      hi[e] = from_f32<T>(b[e] * cc[e] + a[e] * sn[e]);
+    }
+    T* o = is_q ? q_out + t * qd + h * hd : cache + (((long)page * 2 + 0) * KV + h) * block + (long)slot * hd;
+    *reinterpret_cast<tx4*>(o + j) = lo;
+    *reinterpret_cast<tx4*>(o + j + half) = hi;
+  } else {
+    T* v = cache + (((long)page * 2 + 1) * KV + h) * block + slot;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[(long)(j + e) * page_size] = from_f32<T>(a[e]);
+  }
+}
+
 // out[t, i] = silu(gate[t, i]) * up[t, i], gate = cols [0, f), up = cols [f, 2f)
 // (reference: backend/model.cu:477-483)
 template <typename TIN, typename TOUT>
@@ -338,6 +402,15 @@ static int launch_rope_append(const void* qkv, int nsplit, long split_stride, vo
   const int items = H * (hd / 2) + (cache ? KV * (hd / 2) + KV * hd : 0);
   int chunks = ceil_div(items, kThreads);
   if ((long)n * chunks > 16384) chunks = ceil_div(16384, n);   // many tokens: fewer, longer workgroups
+  if (sizeof(TIN) == 4 && nsplit == 1 && hd % 8 == 0 && ((uintptr_t)qkv & 15) == 0 &&
+      ((uintptr_t)q_out & 15) == 0 && (!cache || ((uintptr_t)cache & 15) == 0) &&
+      (!cos_t || (((uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0)) {
+    hipLaunchKernelGGL((rope_append_vec_kernel<T>), dim3(n, ceil_div(items, 4 * kThreads)), dim3(kThreads), 0,
+                       stream, (const float*)qkv, (T*)q_out, cos_t, sin_t, (T*)cache, positions, span_of_token,
+                       block_table, max_pages, page_size, H, KV, hd);
+    KLLM_CHECK_LAUNCH("rope_append");
+    return 0;
+  }
   hipLaunchKernelGGL((rope_append_kernel<TIN, T>), dim3(n, chunks), dim3(kThreads), 0, stream,
                      (const TIN*)qkv, nsplit, split_stride, (T*)q_out, cos_t, sin_t, (T*)cache,
                      positions, span_of_token, block_table, max_pages, page_size, H, KV, hd);

@@ -147,17 +147,16 @@ __device__ __attribute__((aligned(16))) bf16_t g_zero_chunk[8];   // zero-initia
 // different slots, so that the 16-byte reads of 16 lanes spread over all 64 banks.
 __device__ __forceinline__ int mfma_swz(int row) { return (row >> 1) & 7; }
 
-template <typename TOUT, bool DUAL, int MSTAGES>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ X,
+template <typename TOUT, bool DUAL, int WR, int MSTAGES>   // WR: rows of waves (2 or 4), two waves a row
+__global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ X,
                                                              const bf16_t* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
                                                              int k, int tiles_x, int tiles_y) {
-  // 32-row MFMA tiles per wave.  4 (a 256-row workgroup tile) halves the traffic per flop but
-  // leaves one workgroup per CU, and measured 10% slower than 2.
-  constexpr int WTM = 2;
-  constexpr int BM = 64 * WTM;                  // rows of X per workgroup
-  constexpr int XI = BM / 32;                   // load instructions of X per wave and stage (8 rows each)
-  constexpr int WI = MBN / 32;
+  constexpr int WTM = 2;                        // 32-row MFMA tiles per wave, each way
+  constexpr int BM = 64 * WR;                   // rows of X per workgroup
+  constexpr int NW = 2 * WR;                    // waves
+  constexpr int XI = BM / 8 / NW;               // load instructions of X per wave and stage (8 rows each)
+  constexpr int WI = MBN / 8 / NW;
   constexpr int XBYTES = BM * MROW, WBYTES = MBN * MROW;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];   // [MSTAGES][X tile | W tile]
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
@@ -173,7 +172,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
   const long tcol = x_major ? id / tiles_y : id % tiles_x;
   const long row0 = trow * BM, col0 = tcol * (DUAL ? MBN / 2 : MBN);
 
-  // Wave w loads rows [8 XI w, 8 XI (w+1)) of the X tile and [32 w, 32 w + 32) of the W
+  // Wave w loads rows [8 XI w, 8 XI (w+1)) of the X tile and [8 WI w, 8 WI (w+1)) of the W
   // tile.  In one instruction lane l serves row l / 8 (of 8), slot l % 8.
   const bf16_t* xsrc[XI];
   const bf16_t* wsrc[WI];
@@ -186,7 +185,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
   }
 #pragma unroll
   for (int i = 0; i < WI; ++i) {
-    const int r = 32 * wave + 8 * i + lane / 8;               // DUAL: rows 0..63 gate, 64..127 up
+    const int r = 8 * (WI * wave + i) + lane / 8;             // DUAL: rows 0..63 gate, 64..127 up
     wchunk[i] = ((lane % 8) ^ mfma_swz(r)) * 8;
     const long col = DUAL ? col0 + r % 64 : col0 + r;
     const long wrow = min(col, (long)m - 1) + (DUAL && r >= 64 ? m : 0);
@@ -206,7 +205,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     for (int i = 0; i < WI; ++i) {
       const bf16_t* src = kk + wchunk[i] < k ? wsrc[i] + kk : g_zero_chunk;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(base + XBYTES + (32 * wave + 8 * i) * MROW),
+                                       (__attribute__((address_space(3))) void*)(base + XBYTES + 8 * (WI * wave + i) * MROW),
                                        16, 0, 0);
     }
   };
@@ -284,28 +283,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     }
 }
 
-template <typename TOUT, bool DUAL, int MSTAGES>
+template <typename TOUT, bool DUAL, int WR, int MSTAGES>
 static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m, int k, hipStream_t stream) {
-  const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN), ty = ceil_div(n, 128);
+  const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN), ty = ceil_div(n, 64 * WR);
   const dim3 grid(ceil_div((long)tx * ty, 8) * 8);   // padded so that every XCD gets as many
-  const size_t lds = (size_t)MSTAGES * (128 + MBN) * MROW;
+  const size_t lds = (size_t)MSTAGES * (64 * WR + MBN) * MROW;
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_mfma_kernel<TOUT, DUAL, MSTAGES>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_mfma_kernel<TOUT, DUAL, WR, MSTAGES>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) KLLM_FAIL((int)e, "gemm mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = 1;
   }
-  hipLaunchKernelGGL((gemm_bf16_mfma_kernel<TOUT, DUAL, MSTAGES>), grid, dim3(256), lds, stream,
+  hipLaunchKernelGGL((gemm_bf16_mfma_kernel<TOUT, DUAL, WR, MSTAGES>), grid, dim3(128 * WR), lds, stream,
                      (const bf16_t*)x, (const bf16_t*)w, (TOUT*)y, n, m, k, tx, ty);
   return 0;
 }
 
+// Tiles of 256 rows of X (eight waves) fetch a quarter less per flop than two tiles of 128;
+// they are taken when they still give every CU two rounds of work.
 template <typename TOUT, bool DUAL>
 static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, hipStream_t stream) {
-  const long tiles = (long)ceil_div(n, 128) * ceil_div(m, DUAL ? MBN / 2 : MBN);
-  if (tiles <= 256) return launch_mfma_tile<TOUT, DUAL, 3>(x, w, y, n, m, k, stream);   // one per CU at most
-  return launch_mfma_tile<TOUT, DUAL, 2>(x, w, y, n, m, k, stream);
+  const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN);
+  if ((long)ceil_div(n, 256) * tx >= 512) return launch_mfma_tile<TOUT, DUAL, 4, 2>(x, w, y, n, m, k, stream);
+  const long tiles = (long)ceil_div(n, 128) * tx;
+  if (tiles <= 256) return launch_mfma_tile<TOUT, DUAL, 2, 3>(x, w, y, n, m, k, stream);   // one per CU at most
+  return launch_mfma_tile<TOUT, DUAL, 2, 2>(x, w, y, n, m, k, stream);
 }
 
 // ------------------------------------------------------------------ bf16 MFMA skinny

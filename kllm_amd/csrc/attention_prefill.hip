@@ -1,11 +1,15 @@
 // Prompt attention over the paged cache on the matrix cores (bfloat16).
 //
-// One wave takes 32 consecutive tokens of one request (a query tile) and one
-// head, and walks the request's keys in tiles of 32, from the first key any of
-// its queries may read to the last: earlier pages of the cache and the rows
-// this step has just written alike, so a prompt's portion at a position > 0
-// needs no other path.  Running maximum and sum per query (online softmax), no
-// score matrix in memory, context bounded by pages only.  Formulas as in the
+// A workgroup takes 32 consecutive tokens of one request (a query tile) and one
+// head; its four waves share out the request's keys in tiles of 32, round
+// robin, from the first key any of the queries may read to the last: earlier
+// pages of the cache and the rows this step has just written alike, so a
+// prompt's portion at a position > 0 needs no other path.  Running maximum and
+// sum per query (online softmax) in every wave, merged in LDS at the end; no
+// score matrix in memory, context bounded by pages only.  Sharing a tile's keys
+// out over waves keeps the longest chain of dependent tiles short (a late
+// query tile of a long prompt has many) and gives the chip four times as many
+// workgroups as one wave per tile would, so that late and early tiles balance.  Formulas as in the
 // generic kernel (reference: backend/model.cu:343-408, window :224-225), in
 // 32-bit; probabilities are rounded to bfloat16 for the product with the values.
 //
@@ -29,7 +33,7 @@ constexpr int kPrefillWaves = 4;
 constexpr int kQueryTile = 32;
 
 template <int HDT>  // head_dim = 32 * HDT
-__global__ __launch_bounds__(64 * kPrefillWaves) void attn_prefill_mfma_kernel(
+__global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per_eu(HDT <= 2 ? 3 : 1))) void attn_prefill_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ query_tiles, int n_tiles, const int* __restrict__ span_start,
     const int* __restrict__ span_pos, const int* __restrict__ block_table, int max_pages,
@@ -38,13 +42,16 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void attn_prefill_mfma_kernel(
   constexpr int KS = hd / 16;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int g = lane / 32, c = lane % 32;
-  const long item = (long)blockIdx.x * kPrefillWaves + wave;   // (tile, head), head fastest
-  if (item >= (long)n_tiles * H) return;
+  const long item = blockIdx.x;                               // (tile, head), head fastest
   const int tile = n_tiles - 1 - (int)(item / H), h = item % H;   // later tiles read more keys: start them first
   const int kvh = h / (H / KV);
-  const int t0 = query_tiles[2 * tile], span = query_tiles[2 * tile + 1];
-  const int s_begin = span_start[span], s_end = span_start[span + 1];
-  const int pos0 = span_pos[span];
+  // The same for every lane: said so explicitly, which keeps the loop's page lookups and
+  // address arithmetic on the scalar unit.
+  const int t0 = __builtin_amdgcn_readfirstlane(query_tiles[2 * tile]);
+  const int span = __builtin_amdgcn_readfirstlane(query_tiles[2 * tile + 1]);
+  const int s_begin = __builtin_amdgcn_readfirstlane(span_start[span]);
+  const int s_end = __builtin_amdgcn_readfirstlane(span_start[span + 1]);
+  const int pos0 = __builtin_amdgcn_readfirstlane(span_pos[span]);
   const int kv_len = pos0 + (s_end - s_begin);              // keys of the request after this step
   const int nq = min(kQueryTile, s_end - t0);               // queries of this tile
   const int tq = t0 + min(c, nq - 1);                       // this lane's query (clamped)
@@ -69,55 +76,64 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void attn_prefill_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[r][i] = 0.f;
 
-  // One tile's operands.  The loads of tile i+1 go out before tile i is
-  // computed; its page ids were read one tile earlier still.
+  // One tile's operands.  Two tiles are in registers: while one is multiplied the loads of
+  // the wave's next one are on their way, and the page ids of the one after that.  Loads
+  // carry no branch (a page or a row that does not exist reads page 0 and is masked or
+  // zeroed where it is used), so that the waits count them exactly.
   struct Tile {
     bf16x8 k[KS];
     bf16x4 vlo[HDT][2], vhi[HDT][2];
-    bool row_ok, live[2];
+    bool live[2];
   };
   const int kb0 = lowest / 32 * 32;
-  const int first_page_key = lowest / page_size * page_size;   // pages before this may be gone
-  auto pages_of = [&](int kb, int& prow, int& p0, int& p1) {
-    const int key_row = kb + c;
-    const bool in = kb <= qpos_max;
-    prow = (in && key_row < kv_len && key_row >= first_page_key) ? table[key_row / page_size] : -1;
-    p0 = (in && kb < kv_len && kb + 16 > lowest) ? table[kb / page_size] : -1;
-    p1 = (in && kb + 16 < kv_len && kb + 32 > lowest) ? table[(kb + 16) / page_size] : -1;
+  // page and slot of a key: a shift and a mask when the page size is a power of two
+  const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+  auto page_index = [&](int key) { return page_shift >= 0 ? key >> page_shift : key / page_size; };
+  auto page_slot = [&](int key) { return page_shift >= 0 ? key & (page_size - 1) : key % page_size; };
+  const int first_page_key = page_index(lowest) * page_size;   // pages before this may be gone
+  struct Pages {
+    int row, p0, p1;
   };
-  auto fetch = [&](int kb, int prow, int p0, int p1) -> Tile {
-    Tile T;
+  auto pages_of = [&](int kb) -> Pages {
+    Pages P = {-1, -1, -1};
+    if (kb > qpos_max) return P;
     const int key_row = kb + c;
-    T.row_ok = prow >= 0;
-    const bf16_t* krow = cache + (((long)(T.row_ok ? prow : 0) * 2 + 0) * KV + kvh) * block +
-                         (long)(key_row % page_size) * hd;
+    const bool in = true;
+    const bool rok = in && key_row < kv_len && key_row >= first_page_key;
+    const bool ok0 = in && kb < kv_len && kb + 16 > lowest;
+    const bool ok1 = in && kb + 16 < kv_len && kb + 32 > lowest;
+    P.row = table[rok ? page_index(key_row) : 0];
+    P.p0 = table[ok0 ? page_index(kb) : 0];
+    P.p1 = table[ok1 ? page_index(kb + 16) : 0];
+    P.row = rok ? P.row : -1;
+    P.p0 = ok0 ? P.p0 : -1;
+    P.p1 = ok1 ? P.p1 : -1;
+    return P;
+  };
+  auto fetch = [&](int kb, const Pages& P) -> Tile {
+    Tile T = {};
+    if (kb > qpos_max) return T;                              // beyond the last tile: same for all lanes
+    const int key_row = kb + c;
+    const bf16_t* krow = cache + (((long)max(P.row, 0) * 2 + 0) * KV + kvh) * block +
+                         (long)page_slot(key_row) * hd;
 #pragma unroll
-    for (int kk = 0; kk < KS; ++kk)
-      T.k[kk] = T.row_ok ? *reinterpret_cast<const bf16x8*>(krow + 16 * kk + 8 * g) : zero8;
+    for (int kk = 0; kk < KS; ++kk) T.k[kk] = *reinterpret_cast<const bf16x8*>(krow + 16 * kk + 8 * g);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int vp = u ? p1 : p0;
-      const int k0 = kb + 16 * u;
+      const int vp = u ? P.p1 : P.p0;
       T.live[u] = vp >= 0;
-      const bf16_t* vbase = cache + (((long)(T.live[u] ? vp : 0) * 2 + 1) * KV + kvh) * block + (k0 % page_size);
+      const bf16_t* vbase = cache + (((long)max(vp, 0) * 2 + 1) * KV + kvh) * block + page_slot(kb + 16 * u);
 #pragma unroll
       for (int r = 0; r < HDT; ++r) {
         const bf16_t* vrow = vbase + (long)(32 * r + c) * page_size;
-        T.vlo[r][u] = T.live[u] ? *reinterpret_cast<const bf16x4*>(vrow + 4 * g) : bf16x4{0, 0, 0, 0};
-        T.vhi[r][u] = T.live[u] ? *reinterpret_cast<const bf16x4*>(vrow + 8 + 4 * g) : bf16x4{0, 0, 0, 0};
+        T.vlo[r][u] = *reinterpret_cast<const bf16x4*>(vrow + 4 * g);
+        T.vhi[r][u] = *reinterpret_cast<const bf16x4*>(vrow + 8 + 4 * g);
       }
     }
     return T;
   };
 
-  int prow, pg0, pg1;
-  pages_of(kb0, prow, pg0, pg1);
-  Tile nxt = fetch(kb0, prow, pg0, pg1);
-  pages_of(kb0 + 32, prow, pg0, pg1);
-  for (int kb = kb0; kb <= qpos_max; kb += 32) {
-    const Tile cur = nxt;
-    nxt = fetch(kb + 32, prow, pg0, pg1);
-    pages_of(kb + 64, prow, pg0, pg1);
+  auto compute = [&](const Tile& cur, int kb) {
     // ---- scores: this lane's key row is kb + c
     floatx16 s;
 #pragma unroll
@@ -190,10 +206,56 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void attn_prefill_mfma_kernel(
           acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[u], acc[r], 0, 0, 0);
         }
     }
+  };
+
+  // A and B take turns, so that no tile is copied from register to register.
+  constexpr int kStride = 32 * kPrefillWaves;                 // keys between a wave's tiles
+  const int kfirst = kb0 + 32 * wave;
+  Pages P = pages_of(kfirst);
+  Tile A = fetch(kfirst, P);
+  P = pages_of(kfirst + kStride);
+  for (int kb = kfirst; kb <= qpos_max; kb += 2 * kStride) {
+    const Tile B = fetch(kb + kStride, P);
+    P = pages_of(kb + 2 * kStride);
+    compute(A, kb);
+    if (kb + kStride > qpos_max) break;
+    A = fetch(kb + 2 * kStride, P);
+    P = pages_of(kb + 3 * kStride);
+    compute(B, kb + kStride);
   }
 
   l += __shfl_xor(l, 32, kWave);
-  if (c >= nq) return;
+
+  // ---- the waves meet: waves 1..3 leave maximum, sum and output in LDS (lane-contiguous),
+  // wave 0 adds them in a fixed order with weights exp(m_w - max m) and writes the tile.
+  extern __shared__ float red[];                              // [3][HDT*16 + 2][64]
+  constexpr int kRows = HDT * 16 + 2;
+  if (wave > 0) {
+    float* mine = red + (wave - 1) * kRows * kWave + lane;
+#pragma unroll
+    for (int r = 0; r < HDT; ++r)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mine[(16 * r + i) * kWave] = acc[r][i];
+    mine[(HDT * 16) * kWave] = m;
+    mine[(HDT * 16 + 1) * kWave] = l;
+  }
+  __syncthreads();
+  if (wave > 0 || c >= nq) return;
+  float mw[kPrefillWaves - 1], M = m;
+#pragma unroll
+  for (int w = 0; w < kPrefillWaves - 1; ++w) {
+    mw[w] = red[(w * kRows + HDT * 16) * kWave + lane];
+    M = fmaxf(M, mw[w]);
+  }
+  // M is finite: the wave that holds the query's own key has a finite maximum
+  const float w0 = __builtin_amdgcn_exp2f((m - M) * c2);      // exp2(-inf) = 0 for a wave without keys
+  float ww[kPrefillWaves - 1];
+  l *= w0;
+#pragma unroll
+  for (int w = 0; w < kPrefillWaves - 1; ++w) {
+    ww[w] = __builtin_amdgcn_exp2f((mw[w] - M) * c2);
+    l += ww[w] * red[(w * kRows + HDT * 16 + 1) * kWave + lane];
+  }
   const float inv = 1.f / l;
   bf16_t* orow = out + ((long)tq * H + h) * hd;
 #pragma unroll
@@ -202,7 +264,13 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void attn_prefill_mfma_kernel(
     for (int b = 0; b < 4; ++b) {
       bf16x4 v;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) v[j] = (bf16_t)(acc[r][4 * b + j] * inv);
+      for (int j = 0; j < 4; ++j) {
+        const int i = 4 * b + j;
+        float o = acc[r][i] * w0;
+#pragma unroll
+        for (int w = 0; w < kPrefillWaves - 1; ++w) o += ww[w] * red[(w * kRows + 16 * r + i) * kWave + lane];
+        v[j] = (bf16_t)(o * inv);
+      }
       *reinterpret_cast<bf16x4*>(orow + 32 * r + 8 * b + 4 * g) = v;
     }
 }
@@ -212,7 +280,14 @@ static void launch_prefill(int grid, hipStream_t stream, const void* q, void* ou
                            const int* query_tiles, int n_tiles, const int* span_start,
                            const int* span_pos, const int* block_table, int max_pages, int page_size,
                            int H, int KV, int window, float scale) {
-  hipLaunchKernelGGL(attn_prefill_mfma_kernel<HDT>, dim3(grid), dim3(64 * kPrefillWaves), 0, stream,
+  const size_t lds = (size_t)(kPrefillWaves - 1) * (HDT * 16 + 2) * kWave * sizeof(float);
+  static int raised = 0;
+  if (lds > 64 * 1024 && !raised) {
+    (void)hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<HDT>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    raised = 1;
+  }
+  hipLaunchKernelGGL(attn_prefill_mfma_kernel<HDT>, dim3(grid), dim3(64 * kPrefillWaves), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, query_tiles, n_tiles,
                      span_start, span_pos, block_table, max_pages, page_size, H, KV, window, scale);
 }
@@ -237,7 +312,7 @@ extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, co
   KLLM_REQUIRE(max_pages > 0 && window >= 0, "attn_prefill: bad table width or window");
   const long items = (long)n_tiles * H;
   KLLM_REQUIRE(items < (1L << 31), "attn_prefill: too many tiles");
-  const int grid = ceil_div(items, kPrefillWaves);
+  const int grid = (int)items;
 #define KLLM_PF(HDT)                                                                              \
   case HDT:                                                                                       \
     launch_prefill<HDT>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,  \

@@ -29,6 +29,8 @@ def main(argv=None):
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--gemm", default="hip", choices=["hip", "library"])
     ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill only (for profiles)")
+    ap.add_argument("--model", default="tinyllama-1.1b", choices=["tinyllama-1.1b", "llama2-7b", "llama3-8b"],
+                    help="whose sizes to run (the default is the headline configuration)")
     args = ap.parse_args(argv)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not built")
@@ -37,7 +39,7 @@ def main(argv=None):
     import torch
     from kllm_amd import benchmark as B
 
-    cfg = dict(B.TINYLLAMA_1_1B)
+    cfg = dict(B.PRESETS[args.model])
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -55,13 +57,14 @@ def main(argv=None):
     need = B.decode_step_bytes(cfg, args.batch, int(ctx), elem)
     achieved = need / (ms * 1e-3) / 1e9
     out = {
-        "metric": "decode tok/s, TinyLlama-1.1B sizes, random weights",
+        "metric": "decode tok/s, %s sizes, random weights" % {"tinyllama-1.1b": "TinyLlama-1.1B", "llama2-7b": "Llama-2-7B",
+                                                               "llama3-8b": "Llama-3-8B"}[args.model],
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "config": {
-            "model": "tinyllama-1.1b-sizes", "layers": cfg["num_hidden_layers"], "layers_full": full_layers,
+            "model": args.model + "-sizes", "layers": cfg["num_hidden_layers"], "layers_full": full_layers,
             "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
             "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
             "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],

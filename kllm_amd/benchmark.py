@@ -29,6 +29,25 @@ TINYLLAMA_1_1B = {
 }
 
 
+# The other sizes that the baseline names (Llama-2 7B: all heads keep keys; Llama-3 8B: groups
+# of four, a vocabulary of 128,256).
+LLAMA2_7B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 32,
+    "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 32, "head_dim": 128,
+    "intermediate_size": 11008, "vocab_size": 32000, "rope_theta": 10000.0,
+    "max_position_embeddings": 4096, "rms_norm_eps": 1e-5, "tie_word_embeddings": False,
+    "hidden_act": "silu",
+}
+LLAMA3_8B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 32,
+    "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+    "intermediate_size": 14336, "vocab_size": 128256, "rope_theta": 500000.0,
+    "max_position_embeddings": 8192, "rms_norm_eps": 1e-5, "tie_word_embeddings": False,
+    "hidden_act": "silu",
+}
+PRESETS = {"tinyllama-1.1b": TINYLLAMA_1_1B, "llama2-7b": LLAMA2_7B, "llama3-8b": LLAMA3_8B}
+
+
 def synthetic_ids(n: int, vocab: int, salt: int = 0) -> List[int]:
     """The reference's synthetic prompt (cmd/bench/main.go:61-64), salted per request."""
     return [((i + salt * 101) * 37 + 11) % vocab for i in range(n)]

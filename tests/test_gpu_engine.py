@@ -120,6 +120,24 @@ def test_all_families_agree_with_each_other(model_dirs, dtype):
             assert float(np.abs(other[key] - row).max()) < tol, key
 
 
+@pytest.mark.parametrize("options", [
+    {"extra": {"no_fused_gemv": True}},                              # few tokens through the split-K kernels
+    {"extra": {"no_fused_gemv": True, "no_fused_linear": True}},     # and without the decode-batch kernel
+    {"attention": "generic"},                                        # the attention kernel that takes every size
+    {"gemm": "library"},                                             # prompt-sized products from the vendor library
+    {"graphs": False},
+])
+def test_every_choice_of_kernels_gives_the_same_logits(model_dirs, options):
+    """The engine picks kernels by the number of tokens; each alternative path, forced here,
+    must agree with the plain implementation just as well (bfloat16, where the choices are)."""
+    cfg, d = tiny.CONFIGS["B"], model_dirs("B")
+    reqs = make_requests(cfg, [150, 33, 70], 9)
+    want = expected(d, cfg, reqs, "bfloat16")
+    for steps in (traces.portions(reqs, 3), traces.mixed(reqs, seed=4)[0]):
+        rows, _ = replay(d, "bfloat16", steps, traces.peak_tokens(steps), **options)
+        compare(rows, want, "bfloat16", reqs)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(model_dirs, dtype):
     """One token per step for 400 steps, past several pages and past the

@@ -109,6 +109,34 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
     }
   }
 
+  // ---- X: wave w stages rows w, w + 4, ... of the slice, eight 16-byte loads a lane at a time.
+  // Loads return in order, so the first batch goes out before the weights: X is then in LDS
+  // and the workgroup past its barrier while the weights are still arriving.
+  const int chunks = klen / 8;
+  const int mine = (n - wave + 3) / 4;                    // rows of this wave
+  const int items = mine * chunks;
+  auto x_load = [&](int base, bf16x8 (&v)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int idx = base + j * kWave;
+      const int ri = idx / chunks, ch = idx - ri * chunks;
+      v[j] = idx < items ? *reinterpret_cast<const bf16x8*>(X + (long)(wave + 4 * ri) * x_stride + kbeg + ch * 8)
+                         : zero;
+    }
+  };
+  auto x_store = [&](int base, const bf16x8 (&v)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int idx = base + j * kWave;
+      if (idx < items) {
+        const int ri = idx / chunks, ch = idx - ri * chunks;
+        *reinterpret_cast<bf16x8*>(&xs[(wave + 4 * ri) * ld + ch * 8]) = v[j];
+      }
+    }
+  };
+  bf16x8 xv[8];
+  x_load(lane, xv);
+
   // ---- W loads.  A tile's steps are padded to whole rounds of FL_AHEAD, so that a round
   // belongs to one tile; three rounds are in registers (being multiplied, next, far).
   auto tile_ptr = [&](int t) -> const bf16_t* {
@@ -136,27 +164,11 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
   for (int u = 0; u < FL_AHEAD; ++u) nxt[u] = load_a(far_ptr, far_s0 + u);
   advance();
 
-  // ---- X into LDS: wave w takes rows w, w + 4, ...; eight loads in flight per lane
-  const int chunks = klen / 8;
-  const int mine = (n - wave + 3) / 4;                    // rows of this wave
-  const int items = mine * chunks;
-  for (int base = lane; base < items; base += kWave * 8) {
-    bf16x8 v[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int idx = base + j * kWave;
-      const int ri = idx / chunks, ch = idx - ri * chunks;
-      v[j] = idx < items ? *reinterpret_cast<const bf16x8*>(X + (long)(wave + 4 * ri) * x_stride + kbeg + ch * 8)
-                         : zero;
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int idx = base + j * kWave;
-      if (idx < items) {
-        const int ri = idx / chunks, ch = idx - ri * chunks;
-        *reinterpret_cast<bf16x8*>(&xs[(wave + 4 * ri) * ld + ch * 8]) = v[j];
-      }
-    }
+  // ---- X into LDS: the first batch was asked for before the weights and has arrived first
+  x_store(lane, xv);
+  for (int base = lane + kWave * 8; base < items; base += kWave * 8) {
+    x_load(base, xv);
+    x_store(base, xv);
   }
   int ep_page[NT], ep_slot[NT];
   float ep_cos[NT], ep_sin[NT];

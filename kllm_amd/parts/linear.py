@@ -5,8 +5,10 @@ it returns partial sums [nsplit, n, m] that the consuming kernel adds (norm,
 rotary + append, SiLU gate); with the compute dtype as result it returns
 [n, m].  Which kernel runs depends only on the dtype and on n:
 
-  n <= 8    gemv with X in LDS and the whole of K in one wave (no partial
-            sums), if the sizes fit; else the streaming or the general gemv
+  n <= 8    float32: gemv with X in LDS and the whole of K in one wave (no
+            partial sums), if the sizes fit; bfloat16 up to 4 rows: the streaming
+            gemv, K cut into slices for long rows (measured faster than the
+            former for a plain product; the fused epilogues are another matter)
   float32   else: tiled FMA (true 32-bit)
   bfloat16  n <= 64: MFMA skinny (n <= 16 and one float32 result wanted: the
             decode-batch kernel with all of K in a workgroup)
@@ -55,7 +57,7 @@ def choose(dtype, n, m, k, options=None):
     forced = options.get("gemm_algo")
     if forced is not None:
         return forced, 1
-    if K.gemv_fits(n, m, k, dtype) and not options.get("no_fused_gemv"):
+    if dtype == torch.float32 and K.gemv_fits(n, m, k, dtype) and not options.get("no_fused_gemv"):
         return K.GEMM_GEMV_LDS, 1
     if n <= 4 or (n <= 8 and dtype == torch.float32):
         return K.GEMM_GEMV, _gemv_split(dtype, n, m, k)

@@ -389,7 +389,8 @@ def test_linear_chooses_a_kernel_for_every_size():
     k_ = K()
     assert choose(torch.float32, 1, 64, 64)[0] == k_.GEMM_GEMV_LDS
     assert choose(torch.float32, 1, 65, 64)[0] == k_.GEMM_GEMV          # odd number of rows of W
-    assert choose(torch.bfloat16, 4, 2560, 2048) == (k_.GEMM_GEMV_LDS, 1)
+    assert choose(torch.bfloat16, 4, 2560, 2048) == (k_.GEMM_GEMV, 1)
+    assert choose(torch.bfloat16, 1, 2048, 5632) == (k_.GEMM_GEMV, 3)
     assert choose(torch.float32, 8, 2560, 2048) == (k_.GEMM_GEMV_LDS, 1)
     assert choose(torch.bfloat16, 8, 2560, 2048) == (k_.GEMM_SKINNY_BF16, 8)
     assert choose(torch.float32, 100, 64, 64)[0] == k_.GEMM_TILED_F32

@@ -14,7 +14,7 @@ from typing import Dict, List
 
 import torch
 
-from .engine import Engine, EngineOptions, StepEntry
+from .engine import Engine, EngineOptions, StepEntry, TokenRef
 
 # Published peaks of MI355X.
 PEAK_HBM_GBS = 8000.0
@@ -131,11 +131,25 @@ def measure_decode(engine: Engine, batch: int, context_end: int, steps: int, war
         raise ValueError("context too short for the steps asked for")
     rids, toks = fill_context(engine, batch, start)
     zeros = [0.0] * batch
+    ahead = engine.can_sample_ahead([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)])
 
     def run(k):
+        """k steps, each fed with the ids of the one before.  Where the engine can queue a
+        step ahead (as its scheduler does), the ids go from step to step on the device and
+        are read on the host one step late; every step's ids are read."""
         nonlocal toks
+        before = None
         for _ in range(k):
-            toks = engine.step_sample([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)], zeros, zeros)
+            if not ahead:
+                toks = engine.step_sample([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)], zeros, zeros)
+                continue
+            ids = toks if before is None else [TokenRef(before, i) for i in range(batch)]
+            handle = engine.step_sample_ahead([StepEntry(r, [t], [0]) for r, t in zip(rids, ids)], zeros, zeros)
+            if before is not None:
+                before.tokens()
+            before = handle
+        if before is not None:
+            toks = before.tokens()
     run(warmup)
     _sync()
     t0 = time.perf_counter()

@@ -12,12 +12,16 @@ namespace kllm {
 
 constexpr int kThreads = 256;
 
-// x[t, :] = table[ids[t], :]   (reference: backend/model.cu:89-95)
+// x[t, :] = table[ids[t], :]   (reference: backend/model.cu:89-95).  With `from`, token t
+// whose from[t] >= 0 takes its id from sampled[from[t]] instead: the id that the last step's
+// sampling left on the device, so that a step can be queued before that id has reached the host.
 template <typename T>
 __global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ table,
-                             const int* __restrict__ ids, int d, int vocab) {
+                             const int* __restrict__ ids, const int* __restrict__ from,
+                             const int* __restrict__ sampled, int d, int vocab) {
   const long t = blockIdx.x;
   int id = ids[t];
+  if (from && from[t] >= 0) id = sampled[from[t]];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // the host has checked the range
   const T* src = table + (long)id * d;
   float* dst = out + t * d;
@@ -321,17 +325,18 @@ extern "C" int kllm_sum_splits(const float* in, int nsplit, long count, void* ou
   return 0;
 }
 
-extern "C" int kllm_embed(float* out, const void* table, const int* ids, int n, int d, int vocab,
-                          int dtype, hipStream_t stream) {
+extern "C" int kllm_embed(float* out, const void* table, const int* ids, const int* from,
+                          const int* sampled, int n, int d, int vocab, int dtype, hipStream_t stream) {
   KLLM_REQUIRE(out && table && ids, "embed: null pointer");
+  KLLM_REQUIRE((from == nullptr) == (sampled == nullptr), "embed: from and sampled go together");
   KLLM_REQUIRE(n > 0 && d > 0 && vocab > 0, "embed: bad sizes n=%d d=%d vocab=%d", n, d, vocab);
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "embed: unknown dtype %d", dtype);
   if (dtype == DT_F32)
     hipLaunchKernelGGL(embed_kernel<float>, dim3(n), dim3(kThreads), 0, stream, out,
-                       (const float*)table, ids, d, vocab);
+                       (const float*)table, ids, from, sampled, d, vocab);
   else
     hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(n), dim3(kThreads), 0, stream, out,
-                       (const bf16_t*)table, ids, d, vocab);
+                       (const bf16_t*)table, ids, from, sampled, d, vocab);
   KLLM_CHECK_LAUNCH("embed");
   return 0;
 }

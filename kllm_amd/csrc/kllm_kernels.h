@@ -34,8 +34,10 @@ int kllm_device_info(int device, char* buf, int len);
 /* ABI version, bumped when a signature changes. */
 int kllm_abi_version(void);
 
-int kllm_embed(float* out, const void* table, const int* ids, int n, int d, int vocab, int dtype,
-               hipStream_t stream);
+/* out[t] = table[ids[t]]; with `from` (and `sampled`), token t whose from[t] >= 0 takes its id
+ * from sampled[from[t]], a token id that an earlier launch left on the device. */
+int kllm_embed(float* out, const void* table, const int* ids, const int* from, const int* sampled,
+               int n, int d, int vocab, int dtype, hipStream_t stream);
 
 /* v = x[src] + sum of the nsplit partial deltas (delta may be null);
  * x[src] = v when write_x; out[r] = rmsnorm(v) * w when out is not null.

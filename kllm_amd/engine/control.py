@@ -39,7 +39,7 @@ class ControlLayout:
              ("span_start", self.spans + 1), ("span_pos", self.spans), ("slots", self.spans),
              ("logit_rows", max(self.rows, 1))]
         s += [(f"table{g}", self.spans * m) for g, m in enumerate(self.pages)]
-        s += [("temperature", self.samples), ("uniform", self.samples)]
+        s += [("temperature", self.samples), ("uniform", self.samples), ("token_from", self.samples)]
         s += [("short_tokens", self.short), ("query_tiles", 2 * self.tiles)]
         return s
 
@@ -65,9 +65,12 @@ def layout_for(lens: Sequence[int], rows: int, pages: tuple, samples: int = 0) -
 
 def fill(host: np.ndarray, layout: ControlLayout, tokens: Sequence[Sequence[int]],
          pos0: Sequence[int], slots: Sequence[int], rows: Sequence[int],
-         tables: Sequence[Sequence[Sequence[int]]], temperatures=None, uniforms=None):
+         tables: Sequence[Sequence[Sequence[int]]], temperatures=None, uniforms=None,
+         token_from=None):
     """Write one step into ``host`` (int32).  ``tables[g][s]`` is span s's
-    table in group g."""
+    table in group g.  ``token_from[t] >= 0`` (sampled steps only) says that
+    token t's id is not ``tokens`` but the id the last sampled step left on
+    the device at that index."""
     offs, _ = layout.offsets()
 
     def sec(name):
@@ -102,6 +105,7 @@ def fill(host: np.ndarray, layout: ControlLayout, tokens: Sequence[Sequence[int]
     if layout.samples:
         sec("temperature").view(np.float32)[:] = np.asarray(temperatures, dtype=np.float32)
         sec("uniform").view(np.float32)[:] = np.asarray(uniforms, dtype=np.float32)
+        sec("token_from")[:] = -1 if token_from is None else np.asarray(token_from, dtype=np.int32)
     return starts
 
 
@@ -122,7 +126,8 @@ def context(dev: torch.Tensor, layout: ControlLayout, runtime, starts, pos0, len
         runtime=runtime, max_span_len=max(lens), all_decode=all(l == 1 for l in lens),
         short_tokens=sec("short_tokens") if layout.short else None, n_short=layout.short,
         query_tiles=sec("query_tiles").view(layout.tiles, 2) if layout.tiles else None,
-        n_tiles=layout.tiles)
+        n_tiles=layout.tiles,
+        token_from=sec("token_from") if layout.samples and layout.samples == layout.n else None)
 
 
 def sampling_views(dev: torch.Tensor, layout: ControlLayout):

@@ -23,6 +23,7 @@ from ..config import ModelConfig, config_from_dict, load_config, resolve_archite
 from ..parts.base import PagedCacheView, Runtime, StateCacheView, StepContext
 from ..weights import load_weights, random_weights
 from . import control
+from .graph import DecodeGraphs, SampledTokens, TokenRef
 from .model import Model
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16,
@@ -98,7 +99,6 @@ class Engine:
         self._control = None
         self.steps_run = 0
         self.tokens_run = 0
-        from .graph import DecodeGraphs
         self._graphs = DecodeGraphs(self)
 
     # ------------------------------------------------------------------ construction
@@ -219,7 +219,7 @@ class Engine:
             if e.request_id in seen:
                 raise StepError(f"request {e.request_id!r} appears twice in one step")
             seen.add(e.request_id)
-            toks = np.asarray(e.tokens, dtype=np.int64)
+            toks = np.asarray([0 if isinstance(t, TokenRef) else t for t in e.tokens], dtype=np.int64)
             if toks.ndim != 1 or toks.size == 0:
                 raise StepError(f"request {e.request_id!r}: a step needs at least one token")
             if toks.min() < 0 or toks.max() >= self.vocab_size:
@@ -289,6 +289,8 @@ class Engine:
         device, in the order of the entries and of their ``want`` lists, or
         None if nothing is wanted.  Raises OutOfPages (and changes nothing) if
         the cache cannot hold the step's tokens."""
+        if any(isinstance(t, TokenRef) for e in entries for t in e.tokens):
+            raise StepError("a TokenRef can only stand in a batch of single decode tokens that is sampled")
         self._validate(entries)
         opened, reserved = self._reserve(entries)
         try:
@@ -312,14 +314,29 @@ class Engine:
         self._commit(entries)
         return logits
 
+    def can_sample_ahead(self, entries: Sequence[StepEntry]) -> bool:
+        """Whether ``step_sample_ahead`` takes these entries: single decode
+        tokens of a model whose parts can be replayed as a HIP graph."""
+        return (self.options.graphs and self.model.graph_safe
+                and 0 < len(entries) <= self.options.max_graph_batch
+                and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
+
+    def step_sample_ahead(self, entries: Sequence[StepEntry], temperatures, uniforms) -> SampledTokens:
+        """Queue a step of single decode tokens and return without waiting for
+        it.  The sampled ids are read from the handle; the *next* step may be
+        queued before that, with ``TokenRef(handle, i)`` in place of the ids."""
+        if not self.can_sample_ahead(entries):
+            raise StepError("only batches of single decode tokens can be queued ahead")
+        return self._graphs.decode(entries, temperatures, uniforms)
+
     def step_sample(self, entries: Sequence[StepEntry], temperatures, uniforms) -> List[int]:
         """A step whose wanted places are sampled on the device: one token per
         wanted place, as host ints.  Batches of single decode tokens are
         replayed as a HIP graph (forward pass and sampling in one launch)."""
-        if (self.options.graphs and self.model.graph_safe
-                and len(entries) <= self.options.max_graph_batch
-                and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)):
-            return self._graphs.decode(entries, temperatures, uniforms)
+        if self.can_sample_ahead(entries):
+            return self._graphs.decode(entries, temperatures, uniforms).tokens()
+        if any(isinstance(t, TokenRef) for e in entries for t in e.tokens):
+            raise StepError("a TokenRef can only stand in a batch of single decode tokens")
         logits = self.step(entries)
         if logits is None:
             return []

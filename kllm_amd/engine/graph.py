@@ -7,6 +7,13 @@ docs/JOURNAL.md:90-101).  A batch of B single tokens is therefore recorded
 once -- forward pass and sampling -- and replayed: per step the host fills one
 control buffer, copies it, launches the graph and reads B token ids back.
 
+The ids need not be read back before the next step is queued.  A step's ids
+stay in ``engine``-wide device memory where the next step's embedding finds
+them (an entry names its token as a ``TokenRef`` to the previous step's
+result), and the copy to the host is queued between the two graphs; the caller
+takes the ids from the ``SampledTokens`` handle when it wants them.  Queued
+one step ahead, the device does not wait for the host between steps.
+
 What makes a step replayable: every array a kernel reads lives at a fixed
 address (the control buffer's layout depends only on B and on the width of the
 block tables, which grows in powers of two), scratch tensors come from a
@@ -35,11 +42,38 @@ def _bucket(pages: int) -> int:
     return b
 
 
+class SampledTokens:
+    """The token ids of a sampled step, on their way to the host."""
+
+    def __init__(self, host: torch.Tensor, event: torch.cuda.Event, count: int):
+        self._host, self._event, self.count = host, event, count
+        self._ids = None
+
+    def ready(self) -> bool:
+        return self._ids is not None or self._event.query()
+
+    def tokens(self) -> List[int]:
+        """Waits for the step and returns its ids."""
+        if self._ids is None:
+            self._event.synchronize()
+            self._ids = self._host[:self.count].tolist()
+            self._host = None
+        return self._ids
+
+
+class TokenRef:
+    """In place of a token id in a step's entry: "what ``source`` chose at
+    ``index``", for a source that is the step sampled last."""
+    __slots__ = ("source", "index")
+
+    def __init__(self, source: SampledTokens, index: int):
+        self.source, self.index = source, int(index)
+
+
 class _Recording:
     def __init__(self, engine, batch: int, caps: tuple):
         self.layout = control.layout_for([1] * batch, batch, caps, samples=batch)
         self.control = torch.zeros(self.layout.total, dtype=torch.int32, device=engine.device)
-        self.tokens = torch.zeros(batch, dtype=torch.int32, device=engine.device)
         self.workspace = Workspace(engine.device)
         self.graph = None
         self.replays = 0
@@ -52,19 +86,42 @@ class DecodeGraphs:
         self.engine = engine
         self.recordings: "OrderedDict[tuple, _Recording]" = OrderedDict()
         self.captures = 0
+        # Every recording samples into the same place, so that the next step, whichever
+        # recording it is, finds the ids there.
+        self.sampled = torch.zeros(max(engine.options.max_graph_batch, 1), dtype=torch.int32,
+                                   device=engine.device)
+        self.last: "SampledTokens | None" = None
+        self._host_ring = [torch.empty(self.sampled.numel(), dtype=torch.int32, pin_memory=True)
+                           for _ in range(4)]
+        self._host_owner = [None] * len(self._host_ring)   # the handle that reads from each
+        self._host_next = 0
 
     def _run(self, rec: _Recording, lens, pos0):
         eng = self.engine
         starts = list(range(rec.layout.n + 1))
         ctx = control.context(rec.control, rec.layout, eng.runtime, starts, pos0, lens)
         ctx.workspace = rec.workspace
+        ctx.sampled = self.sampled
         logits = eng.model.run(ctx, eng._cache_views(ctx))
         temps, uniforms = control.sampling_views(rec.control, rec.layout)
-        K.sample(rec.tokens, logits, temps, uniforms)
+        K.sample(self.sampled[:rec.layout.n], logits, temps, uniforms)
 
-    def decode(self, entries, temperatures: Sequence[float], uniforms: Sequence[float]) -> List[int]:
-        """One token for every entry (each entry is a single decode token)."""
+    def decode(self, entries, temperatures: Sequence[float], uniforms: Sequence[float]) -> SampledTokens:
+        """One token for every entry (each entry is a single decode token, given
+        as an id or as a TokenRef to the step sampled last).  Returns at once;
+        the ids are read from the handle."""
         eng = self.engine
+        token_from, tokens = [], []
+        for e in entries:
+            t = e.tokens[0]
+            if isinstance(t, TokenRef):
+                if t.source is not self.last or not 0 <= t.index < t.source.count:
+                    raise ValueError("a TokenRef must name a token of the step that was sampled last")
+                token_from.append(t.index)
+                tokens.append([0])
+            else:
+                token_from.append(-1)
+                tokens.append([int(t)])
         eng._validate(entries)
         opened, reserved = eng._reserve(entries)
         try:
@@ -82,12 +139,13 @@ class DecodeGraphs:
                 self.recordings.move_to_end(key)
             host = eng._staging(rec.layout.total)
             pos0 = [rc.length for rc in rcs]
-            control.fill(host.numpy(), rec.layout, [e.tokens for e in entries], pos0,
-                         [rc.slot for rc in rcs], rows, tables, temperatures, uniforms)
+            control.fill(host.numpy(), rec.layout, tokens, pos0, [rc.slot for rc in rcs], rows, tables,
+                         temperatures, uniforms, token_from)
             eng._send(host, rec.control, rec.layout.total)
             if rec.graph is None:
                 self._run(rec, lens, pos0)              # the step itself, and the warm-up
-                out = rec.tokens.tolist()
+                out = self._read_back(batch)
+                out.tokens()                            # before the capture's second run of the kernels
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph, capture_error_mode="thread_local"):
                     self._run(rec, lens, pos0)          # recorded, not executed
@@ -96,9 +154,23 @@ class DecodeGraphs:
             else:
                 rec.graph.replay()
                 rec.replays += 1
-                out = rec.tokens.tolist()
+                out = self._read_back(batch)
         except Exception:
             eng._undo(opened, reserved)
             raise
         eng._commit(entries)
+        self.last = out
         return out
+
+    def _read_back(self, batch: int) -> SampledTokens:
+        """Queue the copy of the sampled ids to the host behind the step."""
+        i = self._host_next
+        self._host_next = (i + 1) % len(self._host_ring)
+        if self._host_owner[i] is not None:
+            self._host_owner[i].tokens()                # an old handle nobody has read yet: read it now
+        host = self._host_ring[i]
+        host[:batch].copy_(self.sampled[:batch], non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        self._host_owner[i] = SampledTokens(host, event, batch)
+        return self._host_owner[i]

@@ -24,6 +24,15 @@ Where this scheduler decides differently, and why:
   the tokens it has generated; it is later recomputed from prompt + generated
   tokens.  A request that could not fit the pool even alone is refused at
   submit.
+* One step ahead.  While every running request is decoding and nothing waits
+  for a place, a step is queued before the ids of the step before it have
+  reached the host: the engine feeds them to the next step on the device
+  (``Engine.step_sample_ahead``), and the device does not stand still while the
+  host reads ids and prepares the next batch.  The price is that an
+  end-of-sequence id is seen one step late: the request has then taken one
+  more step, whose token is thrown away; its pages are given back when that
+  step is over.  Anything else -- a prompt portion, an admission, a shortage
+  of pages -- first settles the step in flight and then takes the plain path.
 """
 
 from __future__ import annotations
@@ -34,6 +43,8 @@ from typing import Callable, Dict, Hashable, List, Optional
 
 from ..sampling import uniform
 from .engine import StepEntry
+
+PENDING = -1     # in Request.generated: a token that is sampled but has not reached the host yet
 
 
 @dataclass
@@ -50,6 +61,7 @@ class Request:
     error: Optional[str] = None
     preemptions: int = 0
     admitted_at: int = -1    # admission counter: larger = younger
+    overrun: bool = False    # ended on an end-of-sequence id while one more step was in flight
 
     @property
     def tokens(self) -> List[int]:
@@ -104,6 +116,7 @@ class Scheduler:
         self.requests: Dict[int, Request] = {}
         self._next_id = 0
         self._admissions = 0
+        self._in_flight = None   # (handle, [(request, place in generated)]) of a step queued ahead
         self.stats = {"steps": 0, "tokens": 0, "prefill_tokens": 0, "decode_tokens": 0,
                       "preemptions": 0, "max_batch_seen": 0}
 
@@ -239,9 +252,13 @@ class Scheduler:
     def step(self) -> List[tuple]:
         """One iteration: plan, run, sample, finish.  Returns the
         (request id, token) pairs produced."""
+        ahead = self._decode_batch_ahead()
+        if ahead is not None:
+            return self._queue_ahead(ahead)
+        produced = self._settle()                # nothing is in flight below this line
         plan = self.plan()
         if not plan.entries:
-            return []
+            return produced
         entries = []
         for pe in plan.entries:
             toks = pe.request.all_tokens()[pe.start:pe.start + pe.count]
@@ -272,7 +289,6 @@ class Scheduler:
             pe.request.cursor += pe.count
             key = "decode_tokens" if (pe.count == 1 and pe.request.generated) else "prefill_tokens"
             self.stats[key] += pe.count
-        produced = []
         if wanting:
             eos = set(getattr(self.engine, "eos_token_ids", ()) or ())
             for pe, tok in zip(wanting, toks):
@@ -287,18 +303,116 @@ class Scheduler:
                     self.running.remove(r)
         return produced
 
+    # ------------------------------------------------------------------ one step ahead
+    def _decode_batch_ahead(self):
+        """The running requests, if the next step is one decode token for each
+        of them and can be queued without any decision: nothing to admit,
+        nothing to cut, pages for all.  Looks, changes nothing."""
+        eng = self.engine
+        if not hasattr(eng, "step_sample_ahead") or not self.running:
+            return None
+        if self.waiting and len(self.running) < self.max_batch:
+            return None
+        if len(self.running) > self.max_step_tokens:
+            return None
+        free = [p.free_pages for p in eng.cache.pools]
+        for r in self.running:
+            if not (r.pending() == 1 and r.generated):
+                return None
+            need = eng.cache.pages_needed(self._key(r), 1)
+            if any(a > b for a, b in zip(need, free)):
+                return None
+            free = [b - a for a, b in zip(need, free)]
+        entries = [StepEntry(self._key(r), [0], [0]) for r in self.running]
+        return list(self.running) if eng.can_sample_ahead(entries) else None
+
+    def _queue_ahead(self, requests: List[Request]) -> List[tuple]:
+        """Queue one decode token for each of ``requests``, then take in the
+        ids of the step before."""
+        from .graph import TokenRef
+        before = self._in_flight
+        place_before = {id(r): i for i, (r, _) in enumerate(before[1])} if before else {}
+        entries, temps, us = [], [], []
+        for r in requests:
+            last = r.generated[-1]
+            tok = TokenRef(before[0], place_before[id(r)]) if last == PENDING else last
+            entries.append(StepEntry(self._key(r), [tok], [0]))
+            temps.append(r.temperature)
+            us.append(uniform(r.seed, len(r.generated)))
+        try:
+            handle = self.engine.step_sample_ahead(entries, temps, us)
+        except Exception as exc:
+            self._fail_all(requests, exc)
+            raise
+        self.stats["steps"] += 1
+        self.stats["tokens"] += len(requests)
+        self.stats["decode_tokens"] += len(requests)
+        self.stats["max_batch_seen"] = max(self.stats["max_batch_seen"], len(requests))
+        places = []
+        for r in requests:
+            r.cursor += 1
+            places.append((r, len(r.generated)))
+            r.generated.append(PENDING)
+            if len(r.generated) >= r.max_new_tokens:
+                self.running.remove(r)           # its last token is on its way; it takes no further step
+        self._in_flight = (handle, places)
+        return self._take_in(before) if before else []
+
+    def _take_in(self, flight) -> List[tuple]:
+        """Wait for a queued step and book its ids."""
+        handle, places = flight
+        toks = handle.tokens()
+        eos = set(getattr(self.engine, "eos_token_ids", ()) or ())
+        newer = {id(r) for r, _ in self._in_flight[1]} if self._in_flight and self._in_flight is not flight else set()
+        produced = []
+        for (r, at), tok in zip(places, toks):
+            if r.overrun:                        # it had ended already: this step was one too many
+                del r.generated[at:]
+                self.engine.release(self._key(r))
+                continue
+            r.generated[at] = int(tok)
+            produced.append((r.id, int(tok)))
+            if r.on_token is not None:
+                r.on_token(r.id, int(tok))
+            if int(tok) in eos or at + 1 >= r.max_new_tokens:
+                r.done = True
+                if r in self.running:
+                    self.running.remove(r)
+                if id(r) in newer:
+                    r.overrun = True             # pages go back when the newer step is over
+                else:
+                    self.engine.release(self._key(r))
+        return produced
+
+    def _settle(self) -> List[tuple]:
+        """Take in whatever is in flight."""
+        flight, self._in_flight = self._in_flight, None
+        return self._take_in(flight) if flight else []
+
+    def _fail_all(self, requests, exc):
+        try:
+            self._settle()
+        except Exception:
+            self._in_flight = None
+        for r in requests:
+            r.done, r.error = True, f"step failed: {exc}"
+            if self._key(r) in self.engine.cache:
+                self.engine.release(self._key(r))
+            if r in self.running:
+                self.running.remove(r)
+
     def has_work(self) -> bool:
-        return bool(self.running or self.waiting)
+        return bool(self.running or self.waiting or self._in_flight)
 
     def run_until_done(self, max_steps: int = 10_000_000) -> Dict[int, Request]:
         steps = 0
         while self.has_work():
             tokens_before = self.stats["tokens"]
-            n_before = len(self.running) + len(self.waiting)
+            n_before = len(self.running) + len(self.waiting) + (self._in_flight is not None)
             self.step()
             steps += 1
             if (self.stats["tokens"] == tokens_before
-                    and len(self.running) + len(self.waiting) == n_before):
+                    and len(self.running) + len(self.waiting) + (self._in_flight is not None) == n_before):
                 raise SchedulerError("scheduler stands still: no request can take a step")
             if steps > max_steps:
                 raise SchedulerError("scheduler did not finish")
@@ -307,6 +421,10 @@ class Scheduler:
     def stop(self):
         """Fail everything in flight and give its pages back
         (engine/scheduler.go:130-134)."""
+        try:
+            self._settle()                       # the device is done with the pages after this
+        except Exception:
+            self._in_flight = None
         for r in list(self.running):
             r.done, r.error = True, "scheduler stopped"
             self.engine.release(self._key(r))

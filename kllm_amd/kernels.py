@@ -20,7 +20,7 @@ DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS = 0, 1, 2, 3, 4, 5
 GEMV_MAX_ROWS = 8          # what the fused kernels take
 GEMV_BEST_ROWS = 4         # up to here they beat the MFMA kernel with split K
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class KernelError(RuntimeError):
@@ -77,7 +77,7 @@ def _declare(lib):
     sigs = {
         "kllm_last_error": [c_char_p, I],
         "kllm_device_info": [I, c_char_p, I],
-        "kllm_embed": [P, P, P, I, I, I, I, P],
+        "kllm_embed": [P, P, P, P, P, I, I, I, I, P],
         "kllm_add_rmsnorm": [P, P, I, I, L, P, P, I, P, I, I, F, I, P],
         "kllm_rope_tables": [P, P, P, I, I, D, P],
         "kllm_rope_append": [P, I, I, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
@@ -143,14 +143,19 @@ def device_info(device: int = 0) -> str:
 
 # ----------------------------------------------------------------------------- wrappers
 
-def embed(out, table, ids):
+def embed(out, table, ids, from_sampled=None, sampled=None):
+    """out [n, d] = table[ids]; where ``from_sampled[t] >= 0`` the id is
+    ``sampled[from_sampled[t]]``, a token id still on the device."""
     n, d = out.shape
     if ids.numel() < n or table.shape[1] != d:
         raise KernelError(f"embed: out {tuple(out.shape)}, table {tuple(table.shape)}, "
                           f"{ids.numel()} ids do not fit")
+    if (from_sampled is None) != (sampled is None) or (from_sampled is not None and from_sampled.numel() < n):
+        raise KernelError("embed: from_sampled and sampled go together, one entry per token")
     _check(library().kllm_embed(
         _ptr(out, "embed out", torch.float32), _ptr(table, "embed table"),
-        _ptr(ids, "embed ids", torch.int32), n, d, table.shape[0], dtype_code(table.dtype),
+        _ptr(ids, "embed ids", torch.int32), _ptr(from_sampled, "embed from", torch.int32, True),
+        _ptr(sampled, "embed sampled", torch.int32, True), n, d, table.shape[0], dtype_code(table.dtype),
         _stream()), "embed")
 
 

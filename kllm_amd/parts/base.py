@@ -194,6 +194,10 @@ class StepContext:
     n_short: int = 0
     query_tiles: Optional[torch.Tensor] = None              # [n_tiles, 2]: (first row, span), longer spans
     n_tiles: int = 0
+    # Token ids that never reached the host: token t with token_from[t] >= 0 is
+    # sampled[token_from[t]], what the last sampled step chose (both or neither are set).
+    token_from: Optional[torch.Tensor] = None
+    sampled: Optional[torch.Tensor] = None
 
     def buf(self, tag, shape, dtype):
         return (self.workspace or self.runtime.workspace).get(tag, shape, dtype)

@@ -35,7 +35,10 @@ class TokenEmbedding(Part):
 
     def forward(self, ctx, token_ids):
         x = ctx.buf("x", (ctx.n, self.hidden), torch.float32)
-        K.embed(x, self.table, token_ids)
+        if ctx.sampled is not None and ctx.token_from is not None:
+            K.embed(x, self.table, token_ids, ctx.token_from, ctx.sampled)
+        else:
+            K.embed(x, self.table, token_ids)
         return x
 
 

@@ -139,6 +139,46 @@ def test_every_choice_of_kernels_gives_the_same_logits(model_dirs, options):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_a_step_queued_ahead_takes_its_ids_from_the_device(model_dirs, dtype):
+    """Decode steps queued one ahead, fed by TokenRef, give the ids that steps fed from the
+    host give; a reference to an older step is refused and changes nothing."""
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry, TokenRef, StepError
+    cfg, d = tiny.CONFIGS["A"], model_dirs("A")
+    prompts = [tiny.tokens(cfg, n, 70 + i) for i, n in enumerate([9, 33, 4])]
+    runs = []
+    for ahead in (False, True):
+        eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=512))
+        firsts = eng.step_sample([StepEntry(i, p, [len(p) - 1]) for i, p in enumerate(prompts)],
+                                 [0.0] * 3, [0.0] * 3)
+        out, ids, before, handles = [list(firsts)], list(firsts), None, []
+        for _ in range(20):
+            if not ahead:
+                ids = eng.step_sample([StepEntry(i, [t], [0]) for i, t in enumerate(ids)], [0.0] * 3, [0.0] * 3)
+                out.append(list(ids))
+                continue
+            feed = ids if before is None else [TokenRef(before, i) for i in range(3)]
+            h = eng.step_sample_ahead([StepEntry(i, [t], [0]) for i, t in enumerate(feed)], [0.0] * 3, [0.0] * 3)
+            if before is not None:
+                out.append(before.tokens())
+            before = h
+            handles.append(h)
+        if ahead:
+            out.append(before.tokens())
+            lengths = [eng.cache.get(i).length for i in range(3)]
+            with pytest.raises(ValueError, match="sampled last"):
+                eng.step_sample_ahead([StepEntry(i, [TokenRef(handles[0], i)], [0]) for i in range(3)],
+                                      [0.0] * 3, [0.0] * 3)
+            assert [eng.cache.get(i).length for i in range(3)] == lengths
+            with pytest.raises(StepError, match="TokenRef"):
+                eng.step([StepEntry(0, [TokenRef(before, 0), 5], [1])])
+        runs.append(out)
+    assert runs[0] == runs[1]
+    want = [P.generate_greedy(tiny.read_weights(d, as_stored_in=dtype), cfg, p, 21) for p in prompts]
+    if dtype == "float32":
+        assert [[step[i] for step in runs[1]] for i in range(3)] == want
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(model_dirs, dtype):
     """One token per step for 400 steps, past several pages and past the
     model's max_position_embeddings (positions are computed, not looked up)."""

@@ -215,3 +215,113 @@ def test_a_failed_step_fails_its_requests():
         s.step()
     assert "device lost" in s.requests[a].error and not s.running
     assert eng.cache.slots.free_slots == 16
+
+
+# ------------------------------------------------------------------ one step ahead
+
+class FakeHandle:
+    """What a queued step returns: its ids exist only after tokens() is called,
+    and until then the "device" still works on the step's requests."""
+
+    def __init__(self, engine, compute, rids):
+        self.engine, self._compute, self.rids, self._ids = engine, compute, rids, None
+        self.count = len(rids)
+        engine.in_flight.append(self)
+
+    def tokens(self):
+        if self._ids is None:
+            self._ids = self._compute()
+            self.engine.in_flight.remove(self)
+        return self._ids
+
+
+class StandInAhead(StandIn):
+    """A stand-in that can queue a step of decode tokens before the ids of the
+    step before are known, as the engine does with its HIP graphs."""
+
+    def __init__(self, *a, **k):
+        super().__init__(*a, **k)
+        self.in_flight = []
+        self.last = None
+        self.ahead_steps = 0
+
+    def can_sample_ahead(self, entries):
+        return bool(entries) and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
+
+    def step_sample_ahead(self, entries, temps, us):
+        from kllm_amd.engine.graph import TokenRef
+        for e in entries:
+            t = e.tokens[0]
+            assert not isinstance(t, TokenRef) or t.source is self.last, "a reference to an older step"
+        for e in entries:
+            self.cache.reserve(e.request_id, 1)
+        for e in entries:
+            self.cache.commit(e.request_id, 1)      # the engine commits when it queues
+        before, refs = self.last, [e.tokens[0] for e in entries]
+
+        def compute():
+            out = []
+            for e, t in zip(entries, refs):
+                tok = before.tokens()[t.index] if isinstance(t, TokenRef) else t
+                have = self.seen.setdefault(e.request_id, [])
+                have.append(tok)
+                out.append(next_token(have))
+            return out
+        self.steps.append([(e.request_id, 1) for e in entries])
+        self.ahead_steps += 1
+        self.last = FakeHandle(self, compute, [e.request_id for e in entries])
+        return self.last
+
+    def step_sample(self, entries, temps, us):
+        assert not self.in_flight, "a plain step while another is in flight"
+        rows = self.step(entries)
+        return self.sample(rows, temps, us) if rows else []
+
+    def release(self, rid):
+        assert all(rid not in h.rids for h in self.in_flight), "pages given back under a running step"
+        super().release(rid)
+
+
+@pytest.mark.parametrize("eos", [(), (7, 21, 33)])
+def test_one_step_ahead_gives_the_same_tokens_and_returns_every_page(eos):
+    ps = prompts(11, 10, lo=1, hi=30)
+    news = [1, 2, 3, 17, 40, 9, 25, 6, 31, 12]
+    eng = StandInAhead(num_pages=400, eos=eos)
+    s = Scheduler(eng, max_batch=4, max_step_tokens=32)
+    seen = {}
+    ids = [s.submit(p, n, on_token=lambda i, t: seen.setdefault(i, []).append(t)) for p, n in zip(ps, news)]
+    res = s.run_until_done()
+    assert eng.ahead_steps > 5 and not eng.in_flight
+    for i, p, n in zip(ids, ps, news):
+        want = alone(p, n, eos)
+        assert res[i].tokens == want and res[i].done and res[i].error is None, (i, res[i].tokens, want)
+        assert seen[i] == want                      # callbacks saw every token once, in order
+    assert eng.cache.pools[0].free_pages == 400 and eng.cache.slots.free_slots == 16
+    eng.cache.check_invariants()
+
+
+def test_an_end_of_sequence_id_is_seen_one_step_late_and_the_extra_token_dropped():
+    p = [3, 1, 4]
+    first = alone(p, 50)
+    eos_at = 5
+    eos = (first[eos_at],)
+    assert first[eos_at] not in first[:eos_at]
+    eng = StandInAhead(eos=eos)
+    s = Scheduler(eng, max_batch=2, max_step_tokens=16)
+    i = s.submit(p, 50)
+    res = s.run_until_done()
+    assert res[i].tokens == first[:eos_at + 1]
+    decode_steps = sum(1 for st in eng.steps if st == [(("sched", id(s), i), 1)])
+    assert decode_steps == eos_at + 1               # one step more than the tokens after the first
+    assert eng.cache.pools[0].free_pages == 64
+
+
+def test_stop_with_a_step_in_flight():
+    eng = StandInAhead()
+    s = Scheduler(eng, max_batch=2, max_step_tokens=16)
+    i = s.submit([1, 2, 3], 30)
+    for _ in range(4):
+        s.step()
+    assert eng.in_flight
+    s.stop()
+    assert not eng.in_flight and eng.cache.pools[0].free_pages == 64 and s.requests[i].done

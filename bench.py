@@ -29,6 +29,7 @@ def main(argv=None):
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--gemm", default="hip", choices=["hip", "library"])
     ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill only (for profiles)")
+    ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--model", default="tinyllama-1.1b", choices=["tinyllama-1.1b", "llama2-7b", "llama3-8b"],
                     help="whose sizes to run (the default is the headline configuration)")
     args = ap.parse_args(argv)
@@ -46,7 +47,7 @@ def main(argv=None):
     elem = 2 if args.dtype == "bfloat16" else 4
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     eng = B.make_engine(cfg, args.dtype, max_tokens=max_batch * args.context + 4096,
-                        max_model_len=args.context + 64, gemm=args.gemm)
+                        max_model_len=args.context + 64, gemm=args.gemm, page_size=args.page_size)
 
     if args.prefill_only:
         pms = B.measure_prefill(eng, 2048, reps=max(1, args.steps), warmup=args.warmup)

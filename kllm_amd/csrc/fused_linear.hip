@@ -9,8 +9,8 @@
 // A workgroup owns tiles of 16 rows of W and one slice of K (all of K unless
 // the caller splits).  It puts its slice of X, all rows, into LDS once.  Each
 // of its four waves takes a quarter of the slice: it streams its part of the 16
-// rows of W straight from memory, up to twenty-four 16-byte loads per lane in
-// flight, the first of them before X is staged, and multiplies with X from LDS
+// rows of W straight from memory, sixteen 16-byte loads per lane in flight, the
+// first of them before X is staged, and multiplies with X from LDS
 // (MFMA 16x16x32: A = W tile, B = X^T, D[w row][x row]).  The four partial
 // tiles meet in LDS, are added in a fixed order, and the epilogue runs on the
 // sums; no partial sum crosses memory unless the caller splits K.
@@ -31,8 +31,8 @@
 
 namespace kllm {
 
-constexpr int FL_AHEAD = 8;        // W loads per lane and round; two rounds are in flight
-constexpr int FL_PAD = 8;          // LDS row padding (elements): 16-byte reads without conflicts
+constexpr int FL_AHEAD = 8;        // W loads per lane in one of the two buffers
+constexpr int FL_PAD = 136;        // LDS row padding (elements): 128 of zeros behind K, 8 to shift banks
 constexpr int FL_LDS_MAX = 160 * 1024;
 constexpr int FL_TILE = 16 * 17;    // floats of one wave's partial tile in LDS: [x row][w row], padded
 
@@ -71,6 +71,15 @@ __device__ __forceinline__ long fl_row(int tile, int c, int m, const FlOut& o) {
   return (long)(o.H + o.KV) * o.hd + e + (second ? 1 : 0);
 }
 
+// A workgroup barrier for data in LDS.  Unlike __syncthreads it does not wait for loads from
+// memory: the weights asked for ahead stay in flight while the waves meet.
+__device__ __forceinline__ void fl_lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0): this wave's LDS operations are done
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 template <int NT, int EP>
 __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restrict__ X, FlOut out,
                                                            const bf16_t* __restrict__ W, int n, int m,
@@ -91,7 +100,7 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
   const int steps = kw / 32;
   const int tile0 = blockIdx.x * tiles_per_wg;
   const int my_tiles = min(tiles_per_wg, tiles - tile0);
-  const int rsteps = (steps + FL_AHEAD - 1) / FL_AHEAD * FL_AHEAD;   // a tile's steps in whole rounds
+  const int rsteps = (steps + 2 * FL_AHEAD - 1) / (2 * FL_AHEAD) * (2 * FL_AHEAD);   // whole turns of both buffers
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
   // ---- rotate-and-append epilogue: thread (pair tid % 8, token tid / 8) needs the token's
@@ -109,19 +118,21 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
     }
   }
 
-  // ---- X: wave w stages rows w, w + 4, ... of the slice, eight 16-byte loads a lane at a time.
-  // Loads return in order, so the first batch goes out before the weights: X is then in LDS
-  // and the workgroup past its barrier while the weights are still arriving.
+  // ---- X: wave w stages rows w, w + 4, ... of the slice, eight 16-byte loads a lane at a
+  // time.  Loads return in order, so the last batch goes out before the weights: X is
+  // then in LDS and the workgroup past its barrier while the weights are still arriving.
+  // No load carries a branch (an index beyond the wave's share reads its last item again), so
+  // that the compiler can count what is in flight and wait for X alone.
   const int chunks = klen / 8;
   const int mine = (n - wave + 3) / 4;                    // rows of this wave
   const int items = mine * chunks;
   auto x_load = [&](int base, bf16x8 (&v)[8]) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int idx = base + j * kWave;
+      const int idx = min(base + j * kWave, max(items - 1, 0));
       const int ri = idx / chunks, ch = idx - ri * chunks;
-      v[j] = idx < items ? *reinterpret_cast<const bf16x8*>(X + (long)(wave + 4 * ri) * x_stride + kbeg + ch * 8)
-                         : zero;
+      const int row = min(wave + 4 * ri, n - 1);          // a wave without rows reads the last row
+      v[j] = *reinterpret_cast<const bf16x8*>(X + (long)row * x_stride + kbeg + ch * 8);
     }
   };
   auto x_store = [&](int base, const bf16x8 (&v)[8]) {
@@ -134,41 +145,53 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
       }
     }
   };
-  bf16x8 xv[8];
-  x_load(lane, xv);
+  bf16x8 xv0[8];
+  int xbase = lane;
+  for (; xbase + kWave * 8 < items; xbase += kWave * 8) {   // all but the last batch (more than eight rows)
+    x_load(xbase, xv0);
+    x_store(xbase, xv0);
+  }
+  x_load(xbase, xv0);
 
-  // ---- W loads.  A tile's steps are padded to whole rounds of FL_AHEAD, so that a round
-  // belongs to one tile; three rounds are in registers (being multiplied, next, far).
-  auto tile_ptr = [&](int t) -> const bf16_t* {
-    if (t >= my_tiles) return nullptr;
-    const long r = fl_row<EP>((int)tile0 + t, c, m, out);
-    return r >= 0 ? W + r * k + kbeg + wk0 + 8 * g : nullptr;
+  // ---- W: two buffers of FL_AHEAD loads each, used in turn: while one is multiplied the
+  // other is on its way, and it is asked for again as soon as it has been used.  No register
+  // is copied from one buffer to the other (a copy would have to wait for its load).  A tile's
+  // steps are padded to whole turns of both buffers.  A row, a tile or a K that does not exist
+  // reads the first K of a row that does (finite numbers): the X beside it in LDS is zero, or
+  // the output row is ignored.
+  const bf16_t* far_row;                                    // first K of this lane's row of W
+  int far_lane_off;                                         // this lane's offset in it, or -1: no such row
+  int far_tile = 0, far_s0 = 0;                             // the steps that are loaded next
+  auto tile_ptr = [&](int t) {
+    const long r = t < my_tiles ? fl_row<EP>((int)tile0 + t, c, m, out) : -1;
+    far_row = W + (r >= 0 ? r : 0) * k + kbeg;
+    far_lane_off = r >= 0 ? wk0 + 8 * g : -1;
   };
-  auto load_a = [&](const bf16_t* ptr, int s) -> bf16x8 {
-    return (ptr && s < steps && 32 * s + 8 * g < wlen) ? *reinterpret_cast<const bf16x8*>(ptr + 32 * s) : zero;
-  };
-  int far_tile = 0, far_s0 = 0;                             // the round that is loaded next
-  const bf16_t* far_ptr = tile_ptr(0);
-  auto advance = [&]() {
+  auto fill = [&](bf16x8 (&buf)[FL_AHEAD]) {
+#pragma unroll
+    for (int i = 0; i < FL_AHEAD; ++i) {
+      const int s = far_s0 + i;
+      const bool valid = far_lane_off >= 0 && s < steps && 32 * s + 8 * g < wlen;
+      buf[i] = *reinterpret_cast<const bf16x8*>(far_row + (valid ? far_lane_off + 32 * s : 0));
+    }
     far_s0 += FL_AHEAD;
     if (far_s0 == rsteps) {
       far_s0 = 0;
-      far_ptr = tile_ptr(++far_tile);
+      tile_ptr(++far_tile);
     }
   };
-  bf16x8 cur[FL_AHEAD], nxt[FL_AHEAD];
-#pragma unroll
-  for (int u = 0; u < FL_AHEAD; ++u) cur[u] = load_a(far_ptr, far_s0 + u);
-  advance();
-#pragma unroll
-  for (int u = 0; u < FL_AHEAD; ++u) nxt[u] = load_a(far_ptr, far_s0 + u);
-  advance();
+  bf16x8 bufa[FL_AHEAD], bufb[FL_AHEAD];
+  tile_ptr(0);
+  fill(bufa);
+  fill(bufb);
 
-  // ---- X into LDS: the first batch was asked for before the weights and has arrived first
-  x_store(lane, xv);
-  for (int base = lane + kWave * 8; base < items; base += kWave * 8) {
-    x_load(base, xv);
-    x_store(base, xv);
+  // ---- X into LDS: what was asked for before the weights has arrived first
+  x_store(xbase, xv0);
+  {   // zeros in X's columns [klen, klen + 128): what the waves' slices of K reach beyond klen
+    const int r = tid / 16, ch = tid % 16;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      if (t * 16 + r < n) *reinterpret_cast<bf16x8*>(&xs[(t * 16 + r) * ld + klen + 8 * ch]) = zero;
   }
   int ep_page[NT], ep_slot[NT];
   float ep_cos[NT], ep_sin[NT];
@@ -197,38 +220,34 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
     }
     rope_angles(0);
   }
-  __syncthreads();
+  fl_lds_barrier();
 
   floatx4 acc[NT];
+  const bf16_t* xrow[NT];                                   // rows beyond n are ignored: they read row n - 1
 #pragma unroll
-  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  for (int tile = 0; tile < my_tiles; ++tile) {
-    for (int s0 = 0; s0 < rsteps; s0 += FL_AHEAD) {
-      bf16x8 far[FL_AHEAD];
+  for (int t = 0; t < NT; ++t) {
+    acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    xrow[t] = xs + min(t * 16 + c, n - 1) * ld + wk0 + 8 * g;
+  }
+  auto multiply = [&](const bf16x8 (&buf)[FL_AHEAD], int s0) {
 #pragma unroll
-      for (int u = 0; u < FL_AHEAD; ++u) far[u] = load_a(far_ptr, far_s0 + u);
-      advance();
+    for (int i = 0; i < FL_AHEAD; ++i) {
+      if (s0 + i < steps) {
 #pragma unroll
-      for (int u = 0; u < FL_AHEAD; ++u) {
-        const int s = s0 + u;
-        if (s < steps) {
-          const bool kin = 32 * s + 8 * g < wlen;
-#pragma unroll
-          for (int t = 0; t < NT; ++t) {
-            const int xr = t * 16 + c;
-            const bf16x8 b = (kin && xr < n)
-                                 ? *reinterpret_cast<const bf16x8*>(&xs[xr * ld + wk0 + 32 * s + 8 * g])
-                                 : zero;
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u], b, acc[t], 0, 0, 0);
-          }
+        for (int t = 0; t < NT; ++t) {
+          const bf16x8 b = *reinterpret_cast<const bf16x8*>(xrow[t] + 32 * (s0 + i));
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf[i], b, acc[t], 0, 0, 0);
         }
       }
-#pragma unroll
-      for (int u = 0; u < FL_AHEAD; ++u) {
-        cur[u] = nxt[u];
-        nxt[u] = far[u];
-      }
+    }
+  };
+
+  for (int tile = 0; tile < my_tiles; ++tile) {
+    for (int s0 = 0; s0 < rsteps; s0 += 2 * FL_AHEAD) {
+      multiply(bufa, s0);
+      fill(bufa);
+      multiply(bufb, s0 + FL_AHEAD);
+      fill(bufb);
     }
     // ---- the tile is complete in this wave: meet the other waves in LDS
     float* pb = part + (tile & 1) * 4 * NT * FL_TILE;
@@ -238,7 +257,7 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
       for (int i = 0; i < 4; ++i) pb[(wave * NT + t) * FL_TILE + c * 17 + 4 * g + i] = acc[t][i];
       acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
-    __syncthreads();
+    fl_lds_barrier();
     const int tl = tile0 + tile;
     // Neighbouring threads take neighbouring rows of W: their stores share cache lines.
     if (EP == FL_PARTS) {

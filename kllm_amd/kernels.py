@@ -340,7 +340,7 @@ def fused_linear_fits(n, k, nsplit=1) -> bool:
         return False
     kslice = -(-(-(-k // nsplit)) // 32) * 32
     nt = -(-n // 16)
-    return n * (kslice + 8) * 2 + 2 * 4 * nt * 16 * 17 * 4 <= FUSED_LINEAR_LDS
+    return n * (kslice + 136) * 2 + 2 * 4 * nt * 16 * 17 * 4 <= FUSED_LINEAR_LDS
 
 
 class Rope:

@@ -1,27 +1,37 @@
 // Prompt attention over the paged cache on the matrix cores (bfloat16).
 //
-// A workgroup takes 32 consecutive tokens of one request (a query tile) and one
-// head; its four waves share out the request's keys in tiles of 32, round
-// robin, from the first key any of the queries may read to the last: earlier
-// pages of the cache and the rows this step has just written alike, so a
-// prompt's portion at a position > 0 needs no other path.  Running maximum and
-// sum per query (online softmax) in every wave, merged in LDS at the end; no
-// score matrix in memory, context bounded by pages only.  Sharing a tile's keys
-// out over waves keeps the longest chain of dependent tiles short (a late
-// query tile of a long prompt has many) and gives the chip four times as many
-// workgroups as one wave per tile would, so that late and early tiles balance.  Formulas as in the
+// A workgroup takes up to 128 consecutive tokens of one request (a query block)
+// and one head; 32 of the queries belong to one wave of each of its two groups
+// of four waves, and the groups take the tiles of keys in turn (a wave's chain
+// of dependent steps per tile is long, and the last block of a long prompt has
+// many tiles: two chains of half the length), meeting in LDS at the end.  The request's
+// keys and values pass through LDS, from the first key any
+// of the queries may read to the last -- earlier pages of the cache and the
+// rows this step has just written alike, so a prompt's portion at a position
+// > 0 needs no other path -- in tiles of 64 keys (two blocks of 32: a wave's chain of
+// dependent steps per tile -- LDS, scores, maximum, exponentials, values, barrier -- is long, and
+// 64 keys share one chain), and every tile is read from memory once for the
+// 128 queries (one wave per 32 queries reading its own keys took four times the
+// traffic between L2 and the CUs, and that traffic was the kernel's bound).
+// The tiles after the one being multiplied are on their way: the next one
+// being written to the other LDS buffer, two more in registers; the page ids
+// two tiles before their loads.  Running maximum and sum per query (online softmax), no
+// score matrix in memory, context bounded by pages only.  Formulas as in the
 // generic kernel (reference: backend/model.cu:343-408, window :224-225), in
 // 32-bit; probabilities are rounded to bfloat16 for the product with the values.
 //
 // The scores are computed transposed, S^T = K Q^T, so that a query is a
 // column: MFMA 32x32x16, lane l (g = l/32, c = l%32) holds A[c][8g..8g+7],
 // B[8g..8g+7][c] and D[8(i/4) + 4g + i%4][c], i = 0..15.  A = 32 keys x 16 of
-// hd, one key row per lane straight from its page; B = q of 32 tokens.  A lane
-// then holds 16 scores of one query, its partner lane (l ^ 32) the other 16:
-// maximum and sum need one exchange.  For the values, O^T += V^T P^T, the 16 k
-// slots of MFMA u are the keys 16u + 8(j/4) + 4g + j%4, j = 0..7 -- exactly the
-// scores D[8u + j] a lane holds -- and A = values [hd row c][those keys], two
-// 8-byte reads from the [hd][slot] value layout of one page.
+// hd, one key row per lane from LDS; B = q of 32 tokens.  A lane then holds 16
+// scores of one query, its partner lane (l ^ 32) the other 16: maximum and sum
+// need one exchange.  For the values, O^T += V^T P^T, the 16 k slots of MFMA u
+// are the keys 16u + 8(j/4) + 4g + j%4, j = 0..7 -- exactly the scores
+// D[8u + j] a lane holds -- and A = values [hd row c][those keys], two 8-byte
+// reads from the [hd][key] tile in LDS.
+//
+// LDS rows are padded so that the lanes of a read fall into different banks:
+// keys [64][hd + 8], values [hd][64 + 4] (tiles of 32 keys for head sizes above 128).
 #include <math.h>
 
 #include "common.hpp"
@@ -30,10 +40,333 @@
 namespace kllm {
 
 constexpr int kPrefillWaves = 4;
+constexpr int kQueryBlock = 32 * kPrefillWaves;   // queries of a workgroup
+
+template <int HDT>
+struct PrefillShape {
+  static constexpr int hd = 32 * HDT;
+  static constexpr int KS = hd / 16;
+  static constexpr int NB = HDT <= 4 ? 2 : 1;       // blocks of 32 keys in a tile (large heads leave registers for one)
+  static constexpr int KT = 32 * NB;                // keys of a tile
+  static constexpr int KLD = hd + 8;                // elements of a key row in LDS
+  static constexpr int VLD = KT + 4;                // elements of a value row in LDS
+  static constexpr int kBuf = KT * KLD + hd * VLD;  // elements of one buffer: a tile's keys, then its values
+  static constexpr int kPieces = KT * hd / 8;       // 16-byte pieces of a tile's keys, and of its values
+  static constexpr int CPT = kPieces / 256;         // pieces per thread
+  static constexpr int kMaxPar = HDT <= 4 ? 2 : 1;  // groups of four waves that may take the tiles in turn (registers)
+};
+
+template <int HDT, int PAR>  // head_dim = 32 * HDT; PAR groups of four waves
+__global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_waves_per_eu(HDT <= 4 ? 2 : 1))) void attn_prefill_mfma_kernel(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
+    const int* __restrict__ query_tiles, int n_tiles, const int* __restrict__ span_start,
+    const int* __restrict__ span_pos, const int* __restrict__ block_table, int max_pages,
+    int page_size, int H, int KV, int window, float scale) {
+  typedef PrefillShape<HDT> S;
+  constexpr int hd = S::hd, KS = S::KS, NB = S::NB, KT = S::KT, KLD = S::KLD, VLD = S::VLD, CPT = S::CPT;
+  extern __shared__ __attribute__((aligned(16))) bf16_t tiles_lds[];   // [PAR][2][kBuf]
+  const int lane = threadIdx.x % kWave;
+  const int tid = threadIdx.x % 256;                          // within the group of four waves
+  const int par = PAR == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x / 256) : 0;   // the group: tiles par, par + PAR, ...
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave) % kPrefillWaves;
+  const int g = lane / 32, c = lane % 32;
+  const long item = blockIdx.x;                               // (block, head), head fastest
+  // Later blocks read more keys.  The later half of the list is started first, longest block
+  // first, then the earlier half, shortest first: a CU that holds one workgroup of each half
+  // gets a long and a short one, and all CUs about the same number of keys.
+  const int j_ = (int)(item / H), h = item % H, n_late = (n_tiles + 1) / 2;
+  const int blk = j_ < n_late ? n_tiles - 1 - j_ : j_ - n_late;
+  const int kvh = h / (H / KV);
+  // The same for every lane: said so explicitly, which keeps the loop's address arithmetic on
+  // the scalar unit.
+  const int t0 = __builtin_amdgcn_readfirstlane(query_tiles[2 * blk]);
+  const int span = __builtin_amdgcn_readfirstlane(query_tiles[2 * blk + 1]);
+  const int s_begin = __builtin_amdgcn_readfirstlane(span_start[span]);
+  const int s_end = __builtin_amdgcn_readfirstlane(span_start[span + 1]);
+  const int pos0 = __builtin_amdgcn_readfirstlane(span_pos[span]);
+  const int kv_len = pos0 + (s_end - s_begin);              // keys of the request after this step
+  // the block's queries, and this wave's
+  const int nq_blk = min(kQueryBlock, s_end - t0);
+  const int blk_qmin = pos0 + (t0 - s_begin), blk_qmax = blk_qmin + nq_blk - 1;
+  const int wq0 = t0 + 32 * wave;
+  const int nq = max(0, min(32, s_end - wq0));
+  const bool active = nq > 0;
+  const int tq = active ? wq0 + min(c, nq - 1) : t0;        // this lane's query (clamped)
+  const int qpos = pos0 + (tq - s_begin);
+  const int w_qmin = pos0 + (wq0 - s_begin), w_qmax = w_qmin + nq - 1;
+  const int lowest = (window > 0) ? max(0, blk_qmin - window + 1) : 0;   // first key any query reads
+  const int w_lowest = (window > 0) ? max(0, w_qmin - window + 1) : 0;   // ... any query of this wave
+  const int my_start = (window > 0) ? max(0, qpos - window + 1) : 0;
+  const int* table = block_table + (long)span * max_pages;
+  const long block = (long)page_size * hd;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const float c2 = scale * 1.4426950408889634f;             // scale * log2(e)
+
+  bf16x8 qb[KS];
+#pragma unroll
+  for (int kk = 0; kk < KS; ++kk)
+    qb[kk] = *reinterpret_cast<const bf16x8*>(q + ((long)tq * H + h) * hd + 16 * kk + 8 * g);
+
+  float m = -INFINITY, l = 0.f;
+  floatx16 acc[HDT];
+#pragma unroll
+  for (int r = 0; r < HDT; ++r)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[r][i] = 0.f;
+
+  const int kb0 = lowest / 32 * 32;
+  const int ntiles_all = (blk_qmax - kb0) / KT + 1;
+  const int ntiles = (ntiles_all + PAR - 1) / PAR;          // steps of the loop: the same for both groups
+  auto tile_key = [&](int t) { return kb0 + KT * (PAR * t + par); };   // first key of this group's t-th tile
+  // page and slot of a key: a shift and a mask when the page size is a power of two
+  const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+  auto page_index = [&](int key) { return page_shift >= 0 ? key >> page_shift : key / page_size; };
+  auto page_slot = [&](int key) { return page_shift >= 0 ? key & (page_size - 1) : key % page_size; };
+  const int first_page_key = page_index(lowest) * page_size;   // pages before this may be gone
+
+  // ---- a tile's way from memory to LDS.  Thread tid moves the same pieces of every tile:
+  // piece i = tid + 256 j of the keys is 16 bytes of key row i / (hd/8); piece i of the values
+  // is 8 keys of one hd row of one half of the tile.  A half (16 keys) lies in one page, and
+  // the pieces of one wave lie in one half: page, slot and base address are the same for the
+  // whole wave and are worked out on the scalar unit; what differs between lanes is constant
+  // over the tiles and kept in registers.  Loads carry no branch: a half that does not exist
+  // reads page 0 and is masked (keys) or zeroed (values).
+  int half_of[CPT], k_off[CPT], v_off[CPT], k_lds[CPT], v_lds[CPT], v_key[CPT];
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) {
+    const int i = tid + 256 * j;
+    half_of[j] = __builtin_amdgcn_readfirstlane(i / (2 * hd));
+    const int krow = i / (hd / 8), kcol = i % (hd / 8) * 8;
+    const int rest = i % (2 * hd), d = rest / 2, part = rest % 2;
+    k_off[j] = (krow % 16) * hd + kcol;                     // from the half's first key row in its page
+    v_off[j] = d * page_size + 8 * part;                    // from the half's first slot of the page's values
+    k_lds[j] = krow * KLD + kcol;
+    v_lds[j] = KT * KLD + d * VLD + 16 * half_of[j] + 8 * part;
+    v_key[j] = 16 * half_of[j] + 8 * part;                  // first key of the values piece, from the tile's
+  }
+  struct Pages {
+    int page[CPT];
+  };
+  struct Stage {
+    bf16x8 k[CPT], v[CPT];
+  };
+  auto key_ok = [&](int key) { return key < kv_len && key >= first_page_key; };
+  auto lookup = [&](int t) -> Pages {
+    Pages P;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      const int key0 = tile_key(t) + 16 * half_of[j];
+      const bool ok = PAR * t + par < ntiles_all && key_ok(key0);
+      // A vector load although the address is the same in every lane: a scalar load would be
+      // counted together with the LDS operations, and every wait for LDS would wait for it.
+      int index = ok ? page_index(key0) : 0;
+      asm volatile("" : "+v"(index));
+      P.page[j] = table[index];                             // made uniform, and clamped, in fetch
+    }
+    return P;
+  };
+  auto fetch = [&](int t, const Pages& P) -> Stage {
+    Stage T;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      const int slot0 = page_slot(tile_key(t) + 16 * half_of[j]);
+      const int page = max(__builtin_amdgcn_readfirstlane(P.page[j]), 0);
+      const bf16_t* kbase = cache + (((long)page * 2 + 0) * KV + kvh) * block + (long)slot0 * hd;
+      const bf16_t* vbase = cache + (((long)page * 2 + 1) * KV + kvh) * block + slot0;
+      T.k[j] = *reinterpret_cast<const bf16x8*>(kbase + k_off[j]);
+      T.v[j] = *reinterpret_cast<const bf16x8*>(vbase + v_off[j]);
+    }
+    return T;
+  };
+  auto stash = [&](const Stage& T, int t, bf16_t* buf) {
+    if (PAR * t + par >= ntiles_all) return;
+    const int kb = tile_key(t);
+    const bool v_edge = kb < first_page_key || kb + KT > kv_len;   // slots that may hold anything
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      {
+        *reinterpret_cast<bf16x8*>(&buf[k_lds[j]]) = T.k[j];
+        bf16x8 v = T.v[j];
+        if (v_edge) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = key_ok(kb + v_key[j] + e) ? v[e] : (bf16_t)0.f;
+        }
+        bf16_t* dst = &buf[v_lds[j]];                                   // 8-byte aligned
+        bf16x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+        *reinterpret_cast<bf16x4*>(dst) = lo;
+        *reinterpret_cast<bf16x4*>(dst + 4) = hi;
+      }
+    }
+  };
+  auto lds_barrier = [&]() {   // for data in LDS only: loads from memory stay in flight
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+
+  auto compute = [&](int t, const bf16_t* buf) {
+    const int kb = tile_key(t);
+    if (!active || kb > w_qmax || kb + KT <= w_lowest) return;   // nothing here for this wave's queries
+    const bool two = NB == 2 && kb + 32 <= w_qmax;            // the second block of 32 keys has keys to read
+    // ---- scores: this lane's key rows are kb + c and kb + 32 + c
+    floatx16 s[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[b][i] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) {
+      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(&buf[c * KLD + 16 * kk + 8 * g]);
+      s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qb[kk], s[0], 0, 0, 0);
+      if (two) {
+        const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(&buf[(32 + c) * KLD + 16 * kk + 8 * g]);
+        s[NB - 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qb[kk], s[NB - 1], 0, 0, 0);
+      }
+    }
+    // ---- mask (only where a tile touches an edge), maximum, probabilities.
+    // exp(x) is taken as exp2(x * log2 e) with the hardware's exp2.
+    const bool inner = kb >= my_start && kb + KT - 1 <= qpos && kb + KT <= kv_len;   // no mask needed
+    if (__any(!inner)) {
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = kb + 32 * b + 8 * (i / 4) + 4 * g + i % 4;
+          const bool ok = inner || (key <= qpos && key >= my_start);
+          s[b][i] = ok ? s[b][i] : -INFINITY;
+        }
+    }
+    float tmax = fmaxf(s[0][0], s[NB - 1][0]);
+#pragma unroll
+    for (int i = 1; i < 16; ++i) tmax = fmaxf(tmax, fmaxf(s[0][i], s[NB - 1][i]));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+    const float m_new = fmaxf(m, tmax);                       // in units of raw scores
+    const float mc = (m_new == -INFINITY) ? 0.f : m_new * c2;
+    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m * c2 - mc);
+    bf16x8 pb[NB][2];
+    float psum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[b][i], c2, -mc));   // exp2(-inf) = 0
+        pb[b][i / 8][i % 8] = (bf16_t)p;
+        psum[i % 4] += p;
+      }
+    l = l * alpha + ((psum[0] + psum[1]) + (psum[2] + psum[3]));
+    m = m_new;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int r = 0; r < HDT; ++r)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[r][i] *= alpha;
+    }
+    // ---- values: half u of block b holds keys kb + 32b + 16u .. + 15
+    const bf16_t* vt = buf + KT * KLD;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      if (b == 1 && !two) break;
+#pragma unroll
+      for (int r = 0; r < HDT; ++r)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const bf16_t* vrow = vt + (32 * r + c) * VLD + 32 * b + 16 * u + 4 * g;
+          const bf16x4 lo = *reinterpret_cast<const bf16x4*>(vrow);
+          const bf16x4 hi = *reinterpret_cast<const bf16x4*>(vrow + 8);
+          const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[b][u], acc[r], 0, 0, 0);
+        }
+    }
+  };
+
+  constexpr int kAhead = HDT <= 3 ? 2 : 1;                  // large heads leave registers for one
+  constexpr int kRound = kAhead > 2 ? kAhead : 2;            // steps of a round: even, so that buffers alternate
+  bf16_t* const bufs[2] = {tiles_lds + (2 * par) * S::kBuf, tiles_lds + (2 * par + 1) * S::kBuf};
+  Pages pg[2];                                              // pg[x % 2]: the pages of tile x, then of x + 2
+  Stage st[kAhead];
+  pg[0] = lookup(0);
+  pg[1] = lookup(1);
+#pragma unroll
+  for (int i = 0; i < kAhead; ++i) {
+    st[i] = fetch(i, pg[i % 2]);
+    pg[i % 2] = lookup(i + 2);
+  }
+  stash(st[0], 0, bufs[0]);
+  lds_barrier();
+  st[0] = fetch(kAhead, pg[kAhead % 2]);
+  pg[kAhead % 2] = lookup(kAhead + 2);
+  // Whole rounds, every step of every round the same for all waves and without a branch
+  // around a load, so that the compiler can count the loads in flight: a tile beyond the last
+  // is asked for (a valid address) and dropped.
+  for (int t0_ = 0; t0_ < ntiles; t0_ += kRound) {
+#pragma unroll
+    for (int i = 0; i < kRound; ++i) {
+      const int t = t0_ + i;
+      compute(t, bufs[i % 2]);
+      stash(st[(i + 1) % kAhead], t + 1, bufs[(i + 1) % 2]);
+      lds_barrier();
+      st[(i + 1) % kAhead] = fetch(t + 1 + kAhead, pg[(i + 1 + kAhead) % 2]);
+      pg[(i + 1 + kAhead) % 2] = lookup(t + 3 + kAhead);
+    }
+  }
+
+  // ---- the two groups meet: the second leaves maximum, sum and output in LDS (lane-contiguous,
+  // in place of the tiles), the first adds them with weights exp(m - max m) and writes.
+  if (PAR == 2) {
+    float* red = reinterpret_cast<float*>(tiles_lds);         // [4 waves][HDT*16 + 2][64]
+    constexpr int kRows = HDT * 16 + 2;
+    lds_barrier();                                            // the last tiles have been read
+    float* mine = red + (wave * kRows) * kWave + lane;
+    if (par == 1) {
+#pragma unroll
+      for (int r = 0; r < HDT; ++r)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mine[(16 * r + i) * kWave] = acc[r][i];
+      mine[(HDT * 16) * kWave] = m;
+      mine[(HDT * 16 + 1) * kWave] = l;
+    }
+    lds_barrier();
+    if (par == 1) return;
+    const float m1 = mine[(HDT * 16) * kWave], l1 = mine[(HDT * 16 + 1) * kWave];
+    const float M = fmaxf(m, m1);
+    // M is finite for a lane with a query: one of the groups holds the query's own key
+    const float w0 = (M == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m - M) * c2);   // exp2(-inf) = 0
+    const float w1 = (M == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m1 - M) * c2);
+    l = l * w0 + l1 * w1;
+#pragma unroll
+    for (int r = 0; r < HDT; ++r)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[r][i] = acc[r][i] * w0 + mine[(16 * r + i) * kWave] * w1;
+  }
+  if (!active || c >= nq) return;
+  l += __shfl_xor(l, 32, kWave);
+  const float inv = 1.f / l;                                  // finite: a query reads its own key
+  bf16_t* orow = out + ((long)tq * H + h) * hd;
+#pragma unroll
+  for (int r = 0; r < HDT; ++r)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      bf16x4 v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = (bf16_t)(acc[r][4 * b + j] * inv);
+      *reinterpret_cast<bf16x4*>(orow + 32 * r + 8 * b + 4 * g) = v;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// The same attention for steps with few query blocks (short prompts, a portion
+// of a prompt at a long context, few heads): there the longest chain of key
+// tiles bounds the time, not the traffic, and the keys are better shared out
+// more finely.  A workgroup takes 32 of a block's queries and one head; its
+// four waves share out the request's keys in tiles of 32, round robin, each
+// streaming its tiles straight from the pages into registers (no LDS on the
+// way), and meet in LDS at the end.  Four times the workgroups, a quarter of
+// the chain, four times the reads from L2.
 constexpr int kQueryTile = 32;
 
 template <int HDT>  // head_dim = 32 * HDT
-__global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per_eu(HDT <= 2 ? 3 : 1))) void attn_prefill_mfma_kernel(
+__global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per_eu(HDT <= 2 ? 3 : 1))) void attn_prefill_split_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ query_tiles, int n_tiles, const int* __restrict__ span_start,
     const int* __restrict__ span_pos, const int* __restrict__ block_table, int max_pages,
@@ -42,17 +375,20 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
   constexpr int KS = hd / 16;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int g = lane / 32, c = lane % 32;
-  const long item = blockIdx.x;                               // (tile, head), head fastest
-  const int tile = n_tiles - 1 - (int)(item / H), h = item % H;   // later tiles read more keys: start them first
+  const long item = blockIdx.x;                               // (block, tile of 32 in it, head), head fastest
+  const int tiles32 = kQueryBlock / kQueryTile;
+  const int tile = n_tiles - 1 - (int)(item / ((long)H * tiles32));   // later blocks read more keys: start them first
+  const int sub = tiles32 - 1 - (int)(item / H % tiles32), h = item % H;
   const int kvh = h / (H / KV);
   // The same for every lane: said so explicitly, which keeps the loop's page lookups and
   // address arithmetic on the scalar unit.
-  const int t0 = __builtin_amdgcn_readfirstlane(query_tiles[2 * tile]);
+  const int t0 = __builtin_amdgcn_readfirstlane(query_tiles[2 * tile]) + kQueryTile * sub;
   const int span = __builtin_amdgcn_readfirstlane(query_tiles[2 * tile + 1]);
   const int s_begin = __builtin_amdgcn_readfirstlane(span_start[span]);
   const int s_end = __builtin_amdgcn_readfirstlane(span_start[span + 1]);
   const int pos0 = __builtin_amdgcn_readfirstlane(span_pos[span]);
   const int kv_len = pos0 + (s_end - s_begin);              // keys of the request after this step
+  if (t0 >= s_end) return;                                  // the block ends before this tile
   const int nq = min(kQueryTile, s_end - t0);               // queries of this tile
   const int tq = t0 + min(c, nq - 1);                       // this lane's query (clamped)
   const int qpos = pos0 + (tq - s_begin);
@@ -275,21 +611,67 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
     }
 }
 
+template <int HDT, int PAR>
+static void launch_prefill_par(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
+                               const int* query_tiles, int n_tiles, const int* span_start,
+                               const int* span_pos, const int* block_table, int max_pages, int page_size,
+                               int H, int KV, int window, float scale) {
+  typedef PrefillShape<HDT> S;
+  const size_t lds = (size_t)PAR * 2 * S::kBuf * sizeof(bf16_t);   // also holds the groups' merge
+  static int raised = 0;
+  if (lds > 64 * 1024 && !raised) {
+    (void)hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<HDT, PAR>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    raised = 1;
+  }
+  hipLaunchKernelGGL((attn_prefill_mfma_kernel<HDT, PAR>), dim3(grid), dim3(64 * kPrefillWaves * PAR), lds, stream,
+                     (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, query_tiles, n_tiles,
+                     span_start, span_pos, block_table, max_pages, page_size, H, KV, window, scale);
+}
+
+template <int HDT>
+static void launch_prefill_split(int n_tiles, hipStream_t stream, const void* q, void* out, const void* cache,
+                                 const int* query_tiles, const int* span_start, const int* span_pos,
+                                 const int* block_table, int max_pages, int page_size, int H, int KV,
+                                 int window, float scale) {
+  const size_t lds = (size_t)(kPrefillWaves - 1) * (HDT * 16 + 2) * kWave * sizeof(float);
+  static int raised = 0;
+  if (lds > 64 * 1024 && !raised) {
+    (void)hipFuncSetAttribute((const void*)attn_prefill_split_kernel<HDT>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    raised = 1;
+  }
+  const int grid = n_tiles * (kQueryBlock / kQueryTile) * H;
+  hipLaunchKernelGGL(attn_prefill_split_kernel<HDT>, dim3(grid), dim3(64 * kPrefillWaves), lds, stream,
+                     (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, query_tiles, n_tiles,
+                     span_start, span_pos, block_table, max_pages, page_size, H, KV, window, scale);
+}
+
+// Which kernel: with more than one query block per CU the CUs are full either way and the
+// traffic decides (keys through LDS, one group of waves); with fewer the chain of tiles
+// decides (keys shared out over the waves of small workgroups; for head sizes from 128 on,
+// whose tiles are heavy, through LDS with two groups of waves).
 template <int HDT>
 static void launch_prefill(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
                            const int* query_tiles, int n_tiles, const int* span_start,
                            const int* span_pos, const int* block_table, int max_pages, int page_size,
                            int H, int KV, int window, float scale) {
-  const size_t lds = (size_t)(kPrefillWaves - 1) * (HDT * 16 + 2) * kWave * sizeof(float);
-  static int raised = 0;
-  if (lds > 64 * 1024 && !raised) {
-    (void)hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<HDT>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    raised = 1;
+  if constexpr (HDT >= 4) {
+    if (grid > 256 || PrefillShape<HDT>::kMaxPar == 1)
+      launch_prefill_par<HDT, 1>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,
+                                 block_table, max_pages, page_size, H, KV, window, scale);
+    else
+      launch_prefill_par<HDT, PrefillShape<HDT>::kMaxPar>(grid, stream, q, out, cache, query_tiles, n_tiles,
+                                                          span_start, span_pos, block_table, max_pages, page_size,
+                                                          H, KV, window, scale);
+  } else {
+    if (grid > 256)
+      launch_prefill_par<HDT, 1>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,
+                                 block_table, max_pages, page_size, H, KV, window, scale);
+    else
+      launch_prefill_split<HDT>(n_tiles, stream, q, out, cache, query_tiles, span_start, span_pos, block_table,
+                                max_pages, page_size, H, KV, window, scale);
   }
-  hipLaunchKernelGGL(attn_prefill_mfma_kernel<HDT>, dim3(grid), dim3(64 * kPrefillWaves), lds, stream,
-                     (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, query_tiles, n_tiles,
-                     span_start, span_pos, block_table, max_pages, page_size, H, KV, window, scale);
 }
 
 }  // namespace kllm

@@ -143,7 +143,7 @@ int kllm_attn_decode(const void* q, void* out, float* part, long part_floats, co
                      hipStream_t stream);
 
 /* Prompt attention on the matrix cores (bfloat16).  query_tiles holds
- * (first token row, span) pairs: up to 32 consecutive tokens of one span. */
+ * (first token row, span) pairs: up to 128 consecutive tokens of one span. */
 int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                       int n_tiles, const int* span_start, const int* span_pos,
                       const int* block_table, int max_pages, int page_size, int H, int KV, int hd,

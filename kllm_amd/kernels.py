@@ -439,11 +439,13 @@ def attn_decode_slices(n, n_kv_heads, n_heads) -> int:
 
 
 PREFILL_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
+PREFILL_QUERY_BLOCK = 128      # tokens of one request that a workgroup of the prompt kernel takes
 
 
 def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, block_table, page_size,
                  n_heads, n_kv_heads, head_dim, window, scale):
-    """query_tiles [n_tiles, 2] int32: (first token row, span) of each tile of 32 tokens."""
+    """query_tiles [n_tiles, 2] int32: (first token row, span) of each block of up to
+    PREFILL_QUERY_BLOCK consecutive tokens of one span."""
     n = q.shape[0]
     if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape)
             or q.dtype != cache.dtype or out.dtype != q.dtype):

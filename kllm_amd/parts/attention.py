@@ -102,7 +102,7 @@ class CausalSelfAttention(Part):
         """Choose the attention kernels by dtype and by the spans' lengths:
         in bfloat16, tokens of short spans (decode tokens) go to the kernel
         that splits a token's keys over many waves, longer spans to the prompt
-        kernel in tiles of 32 queries; float32, and sizes those kernels do not
+        kernel in blocks of 128 queries; float32, and sizes those kernels do not
         take, go to the kernel that takes every size."""
         mode = self.runtime.options.get("attention", "auto")
         fast = (mode != "generic" and q.dtype == torch.bfloat16 and cache.page_size % 16 == 0

@@ -148,7 +148,7 @@ class StateCacheView:
 # How a step's spans are listed for the attention kernels: tokens of spans of at
 # most SHORT_SPAN tokens one by one, longer spans in tiles of QUERY_TILE tokens.
 SHORT_SPAN = 4
-QUERY_TILE = 32
+QUERY_TILE = 128       # = kernels.PREFILL_QUERY_BLOCK
 
 
 def span_lists(starts, lens):

@@ -461,7 +461,7 @@ def run_prefill(c, min_len=1):
     start = 0
     for s, (_, b) in enumerate(c["spans"]):
         if b >= min_len:
-            tiles += [(t, s) for t in range(start, start + b, 32)]
+            tiles += [(t, s) for t in range(start, start + b, K().PREFILL_QUERY_BLOCK)]
             rows[start:start + b] = True
         start += b
     qt = torch.tensor(tiles, dtype=torch.int32, device=DEV)
@@ -520,6 +520,22 @@ def test_attention_prefill(H, KV, hd, ps, window):
     # only the listed spans are touched
     out2, rows2 = run_prefill(c, min_len=33)
     assert torch.isnan(out2.cpu()[~rows2]).all() and torch.equal(out2.cpu()[rows2], out.cpu()[rows2])
+
+
+@pytest.mark.parametrize("H,KV,hd,ps", [(24, 4, 32, 16), (24, 3, 64, 16), (22, 2, 96, 32), (22, 11, 128, 16)])
+@pytest.mark.parametrize("window", [0, 150])
+def test_attention_prefill_many_blocks(H, KV, hd, ps, window):
+    """More query blocks than CUs: the kernel that passes the keys through LDS,
+    with blocks of 128 queries that end inside a tile, long chains of tiles,
+    portions behind cached keys, and a window that ends inside a block."""
+    spans = [(0, 300), (500, 260), (100, 129), (37, 70), (5, 1), (16, 32), (31, 33)]
+    c = attention_case(H, KV, hd, ps, torch.bfloat16, window, spans, seed=6)
+    blocks = sum(-(-b // K().PREFILL_QUERY_BLOCK) for _, b in spans)
+    assert blocks * H > 256
+    out, rows = run_prefill(c)
+    assert rows.all() and torch.isfinite(out).all()
+    err = (out.cpu().double() - c["want"]).abs().max()
+    assert err < 2e-2, float(err)
 
 
 def test_attention_prefill_refuses_what_it_does_not_take():

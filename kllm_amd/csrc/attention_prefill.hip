@@ -1,24 +1,28 @@
-// Prompt attention over the paged cache on the matrix cores (bfloat16).
+// Prompt attention over the paged cache on the matrix cores (bfloat16), two
+// kernels with the same arithmetic; which one runs is decided per launch (see
+// launch_prefill at the end of this file).
 //
-// A workgroup takes up to 128 consecutive tokens of one request (a query block)
-// and one head; 32 of the queries belong to one wave of each of its two groups
-// of four waves, and the groups take the tiles of keys in turn (a wave's chain
-// of dependent steps per tile is long, and the last block of a long prompt has
-// many tiles: two chains of half the length), meeting in LDS at the end.  The request's
-// keys and values pass through LDS, from the first key any
-// of the queries may read to the last -- earlier pages of the cache and the
-// rows this step has just written alike, so a prompt's portion at a position
-// > 0 needs no other path -- in tiles of 64 keys (two blocks of 32: a wave's chain of
-// dependent steps per tile -- LDS, scores, maximum, exponentials, values, barrier -- is long, and
-// 64 keys share one chain), and every tile is read from memory once for the
-// 128 queries (one wave per 32 queries reading its own keys took four times the
-// traffic between L2 and the CUs, and that traffic was the kernel's bound).
-// The tiles after the one being multiplied are on their way: the next one
-// being written to the other LDS buffer, two more in registers; the page ids
-// two tiles before their loads.  Running maximum and sum per query (online softmax), no
-// score matrix in memory, context bounded by pages only.  Formulas as in the
-// generic kernel (reference: backend/model.cu:343-408, window :224-225), in
-// 32-bit; probabilities are rounded to bfloat16 for the product with the values.
+// Both read a request's keys from the first key any of a workgroup's queries
+// may read to the last -- earlier pages of the cache and the rows this step
+// has just written alike, so a prompt's portion at a position > 0 needs no
+// other path.  Running maximum and sum per query (online softmax), no score
+// matrix in memory, context bounded by pages only.  Formulas as in the generic
+// kernel (reference: backend/model.cu:343-408, window :224-225), in 32-bit;
+// probabilities are rounded to bfloat16 for the product with the values.
+//
+// The first kernel (attn_prefill_mfma_kernel): a workgroup takes up to 128
+// consecutive tokens of one request (a query block) and one head; each wave of
+// a group of four owns 32 of the queries.  Keys and values pass through LDS in
+// tiles of 64 keys (two blocks of 32; 32 keys for head sizes above 128, for
+// registers), and every tile is read from memory once for the 128 queries: one
+// workgroup per 32 queries reading its own keys takes four times the traffic
+// between L2 and the CUs, and with many workgroups that traffic bounds the
+// kernel.  The tiles after the one being multiplied are on their way: the next
+// one being written to the other LDS buffer, two more in registers, the page
+// ids two tiles before their loads.  A wave's chain of dependent steps per tile
+// is long (LDS, scores, maximum across lanes, exponentials, values, barrier), so
+// 64 keys share one chain, and with PAR = 2 two groups of four waves take the
+// tiles in turn and meet in LDS at the end: two chains of half the length.
 //
 // The scores are computed transposed, S^T = K Q^T, so that a query is a
 // column: MFMA 32x32x16, lane l (g = l/32, c = l%32) holds A[c][8g..8g+7],

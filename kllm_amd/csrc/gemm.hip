@@ -151,7 +151,7 @@ template <typename TOUT, bool DUAL, int WR, int MSTAGES>   // WR: rows of waves 
 __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ X,
                                                              const bf16_t* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
-                                                             int k, int tiles_x, int tiles_y) {
+                                                             int k, int tiles_x, int tiles_y, int kslice) {
   constexpr int WTM = 2;                        // 32-row MFMA tiles per wave, each way
   constexpr int BM = 64 * WR;                   // rows of X per workgroup
   constexpr int NW = 2 * WR;                    // waves
@@ -191,19 +191,22 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
     const long wrow = min(col, (long)m - 1) + (DUAL && r >= 64 ? m : 0);
     wsrc[i] = W + wrow * k + wchunk[i];
   }
+  // blockIdx.y: a slice of K (kslice a multiple of 64); its sums go to Y[blockIdx.y]
+  const int kbeg = blockIdx.y * kslice, kend = min(k, kbeg + kslice);
+  Y += (long)blockIdx.y * n * m;
   auto issue = [&](int kt) {
     unsigned char* base = lds + (kt % MSTAGES) * (XBYTES + WBYTES);
-    const int kk = kt * MBK;
+    const int kk = kbeg + kt * MBK;
 #pragma unroll
     for (int i = 0; i < XI; ++i) {
-      const bf16_t* src = kk + xchunk[i] < k ? xsrc[i] + kk : g_zero_chunk;
+      const bf16_t* src = kk + xchunk[i] < kend ? xsrc[i] + kk : g_zero_chunk;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(base + 8 * (XI * wave + i) * MROW),
                                        16, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < WI; ++i) {
-      const bf16_t* src = kk + wchunk[i] < k ? wsrc[i] + kk : g_zero_chunk;
+      const bf16_t* src = kk + wchunk[i] < kend ? wsrc[i] + kk : g_zero_chunk;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(base + XBYTES + 8 * (WI * wave + i) * MROW),
                                        16, 0, 0);
@@ -218,7 +221,7 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int ktiles = (k + MBK - 1) / MBK;
+  const int ktiles = (kend - kbeg + MBK - 1) / MBK;
   issue(0);
   if (MSTAGES > 2 && ktiles > 1) issue(1);
   for (int kt = 0; kt < ktiles; ++kt) {
@@ -234,25 +237,31 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
     if (kt + MSTAGES - 1 < ktiles) issue(kt + MSTAGES - 1);
     const unsigned char* xs = lds + (kt % MSTAGES) * (XBYTES + WBYTES);
     const unsigned char* ws = xs + XBYTES;
-#pragma unroll
-    for (int ks = 0; ks < MBK / 16; ++ks) {
-      bf16x8 a[WTM], b[2];
+    // The operands of step ks + 1 are asked for before the MFMAs of step ks are issued, so
+    // that LDS answers while the matrix unit works.
+    bf16x8 a[2][WTM], b[2][2];
+    auto read_step = [&](int ks, bf16x8 (&ar)[WTM], bf16x8 (&br)[2]) {
       const int chunk = ks * 2 + lane / 32;
 #pragma unroll
       for (int i = 0; i < WTM; ++i) {
         const int r = wr * 32 * WTM + i * 32 + lane % 32;
-        a[i] = *reinterpret_cast<const bf16x8*>(xs + r * MROW + (chunk ^ mfma_swz(r)) * 16);
+        ar[i] = *reinterpret_cast<const bf16x8*>(xs + r * MROW + (chunk ^ mfma_swz(r)) * 16);
       }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int r = (DUAL ? j * 64 + wc * 32 : wc * 64 + j * 32) + lane % 32;
-        b[j] = *reinterpret_cast<const bf16x8*>(ws + r * MROW + (chunk ^ mfma_swz(r)) * 16);
+        br[j] = *reinterpret_cast<const bf16x8*>(ws + r * MROW + (chunk ^ mfma_swz(r)) * 16);
       }
+    };
+    read_step(0, a[0], b[0]);
+#pragma unroll
+    for (int ks = 0; ks < MBK / 16; ++ks) {
+      if (ks + 1 < MBK / 16) read_step(ks + 1, a[(ks + 1) & 1], b[(ks + 1) & 1]);
 #pragma unroll
       for (int i = 0; i < WTM; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks & 1][i], b[ks & 1][j], acc[i][j], 0, 0, 0);
     }
   }
 
@@ -284,9 +293,11 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
 }
 
 template <typename TOUT, bool DUAL, int WR, int MSTAGES>
-static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m, int k, hipStream_t stream) {
+static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m, int k, int nsplit,
+                            hipStream_t stream) {
   const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN), ty = ceil_div(n, 64 * WR);
-  const dim3 grid(ceil_div((long)tx * ty, 8) * 8);   // padded so that every XCD gets as many
+  const int kslice = ceil_div(ceil_div(k, nsplit), MBK) * MBK;
+  const dim3 grid(ceil_div((long)tx * ty, 8) * 8, nsplit);   // padded so that every XCD gets as many
   const size_t lds = (size_t)MSTAGES * (64 * WR + MBN) * MROW;
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
@@ -296,19 +307,20 @@ static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m,
     raised = 1;
   }
   hipLaunchKernelGGL((gemm_bf16_mfma_kernel<TOUT, DUAL, WR, MSTAGES>), grid, dim3(128 * WR), lds, stream,
-                     (const bf16_t*)x, (const bf16_t*)w, (TOUT*)y, n, m, k, tx, ty);
+                     (const bf16_t*)x, (const bf16_t*)w, (TOUT*)y, n, m, k, tx, ty, kslice);
   return 0;
 }
 
 // Tiles of 256 rows of X (eight waves) fetch a quarter less per flop than two tiles of 128;
 // they are taken when they still give every CU two rounds of work.
 template <typename TOUT, bool DUAL>
-static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, hipStream_t stream) {
+static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, hipStream_t stream) {
   const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN);
-  if ((long)ceil_div(n, 256) * tx >= 512) return launch_mfma_tile<TOUT, DUAL, 4, 2>(x, w, y, n, m, k, stream);
-  const long tiles = (long)ceil_div(n, 128) * tx;
-  if (tiles <= 256) return launch_mfma_tile<TOUT, DUAL, 2, 3>(x, w, y, n, m, k, stream);   // one per CU at most
-  return launch_mfma_tile<TOUT, DUAL, 2, 2>(x, w, y, n, m, k, stream);
+  if ((long)ceil_div(n, 256) * tx * nsplit >= 512)
+    return launch_mfma_tile<TOUT, DUAL, 4, 2>(x, w, y, n, m, k, nsplit, stream);
+  const long tiles = (long)ceil_div(n, 128) * tx * nsplit;
+  if (tiles <= 256) return launch_mfma_tile<TOUT, DUAL, 2, 3>(x, w, y, n, m, k, nsplit, stream);   // one per CU at most
+  return launch_mfma_tile<TOUT, DUAL, 2, 2>(x, w, y, n, m, k, nsplit, stream);
 }
 
 // ------------------------------------------------------------------ bf16 MFMA skinny
@@ -605,11 +617,13 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
 
   if (algo == KLLM_GEMM_MFMA_BF16) {
     KLLM_REQUIRE(dtype == DT_BF16, "gemm mfma: bfloat16 only");
-    KLLM_REQUIRE(nsplit == 1, "gemm mfma: no split");
+    KLLM_REQUIRE(nsplit == 1 || out_dtype == DT_F32, "gemm mfma: K is split only for float32 partial sums");
+    KLLM_REQUIRE(nsplit <= 16 && (long)(ceil_div(ceil_div(k, nsplit), MBK) * MBK) * (nsplit - 1) < k,
+                 "gemm mfma: nsplit %d leaves an empty slice of K=%d", nsplit, k);
     KLLM_REQUIRE(k % 8 == 0 && aligned16(x) && aligned16(w),
                  "gemm mfma: K=%d must be a multiple of 8 and the operands 16-byte aligned", k);
-    int rc = out_dtype == DT_F32 ? launch_mfma<float, false>(x, w, y, n, m, k, stream)
-                                 : launch_mfma<bf16_t, false>(x, w, y, n, m, k, stream);
+    int rc = out_dtype == DT_F32 ? launch_mfma<float, false>(x, w, y, n, m, k, nsplit, stream)
+                                 : launch_mfma<bf16_t, false>(x, w, y, n, m, k, 1, stream);
     if (rc) return rc;
     KLLM_CHECK_LAUNCH("gemm mfma");
     return 0;
@@ -704,7 +718,7 @@ extern "C" int kllm_gemm_swiglu(const void* x, const void* w_gate_up, void* h, i
   KLLM_REQUIRE(k % 8 == 0 && aligned16(x) && aligned16(w_gate_up),
                "gemm_swiglu: K=%d must be a multiple of 8 and the operands 16-byte aligned", k);
   KLLM_REQUIRE((long)n * f < (1L << 31), "gemm_swiglu: sizes overflow");
-  if (int rc = launch_mfma<bf16_t, true>(x, w_gate_up, h, n, f, k, stream)) return rc;
+  if (int rc = launch_mfma<bf16_t, true>(x, w_gate_up, h, n, f, k, 1, stream)) return rc;
   KLLM_CHECK_LAUNCH("gemm_swiglu");
   return 0;
 }

@@ -178,6 +178,8 @@ def test_gemm_kernels_against_plain(n, m, k, dtype):
         algos.append((k_.GEMM_TILED_F32, 1))
     elif k % 8 == 0:
         algos.append((k_.GEMM_MFMA_BF16, 1))
+        if k >= 128:
+            algos += [(k_.GEMM_MFMA_BF16, 2)] + ([(k_.GEMM_MFMA_BF16, 3)] if k >= 200 else [])
         if n <= 64:
             base = -(-k // 512)
             algos += [(k_.GEMM_SKINNY_BF16, base)] + ([(k_.GEMM_SKINNY_BF16, base * 2)] if k >= 256 else [])
@@ -402,7 +404,9 @@ def test_linear_chooses_a_kernel_for_every_size():
         ns = choose(torch.bfloat16, n, m, k)[1]
         kslice = -(-(-(-k // ns)) // 32) * 32
         assert kslice <= 512 and kslice * (ns - 1) < k, (n, m, k, ns)
-    assert choose(torch.bfloat16, 400, 64, 64)[0] == k_.GEMM_MFMA_BF16
+    assert choose(torch.bfloat16, 400, 64, 64) == (k_.GEMM_MFMA_BF16, 1)
+    assert choose(torch.bfloat16, 2048, 2048, 5632) == (k_.GEMM_MFMA_BF16, 2)     # long K, few tiles
+    assert choose(torch.bfloat16, 2048, 11264, 2048) == (k_.GEMM_MFMA_BF16, 1)
     assert choose(torch.bfloat16, 400, 64, 64, {"gemm": "library"})[0] == "library"
     a, ns = choose(torch.bfloat16, 1, 2049, 5632)
     assert a == k_.GEMM_GEMV and 1 <= ns <= 16

@@ -69,6 +69,17 @@ def test_alone_and_whole(model_dirs, name, lengths, dtype):
     compare(rows, expected(d, cfg, reqs, dtype), dtype, reqs)
 
 
+def test_a_long_prompt_with_more_query_blocks_than_cus(model_dirs):
+    """2,300 tokens of a model with 16 heads in one step (the prompt kernel that passes
+    keys through LDS), then its last 32 tokens one by one over the long context."""
+    cfg, d = tiny.CONFIGS["E"], model_dirs("E")
+    reqs = make_requests(cfg, [2300], 5)
+    want = expected(d, cfg, reqs, "bfloat16")
+    for steps in (traces.whole(reqs), traces.bulk_then_tail(reqs, 32)):
+        rows, _ = replay(d, "bfloat16", steps, traces.peak_tokens(steps))
+        compare(rows, want, "bfloat16", reqs)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name,lengths", [("A", [33, 100]), ("B", [40, 129]), ("C", [50]), ("D", [45])])
 def test_bulk_then_last_32_one_by_one(model_dirs, name, lengths, dtype):

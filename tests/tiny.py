@@ -5,7 +5,8 @@ option: layers, width, heads and groups (GQA / MQA), head size, feed-forward
 width, vocabulary, rotary base, context, eps, tying.  C is multi-head
 (KV = H) with a head size that is not hidden/heads, a width and a vocabulary
 that are not powers of two.  D has sizes the fast kernels refuse (they must
-fall back, never give a wrong result).  R is the reference's own tiny model
+fall back, never give a wrong result).  E has many heads and room for long
+prompts.  R is the reference's own tiny model
 (tools/make_test_model.py:47-100).
 """
 
@@ -38,6 +39,10 @@ CONFIGS = {
     "D": _cfg(num_hidden_layers=2, hidden_size=100, num_attention_heads=5, head_dim=80,
               intermediate_size=172, vocab_size=257, rope_theta=20000.0,
               max_position_embeddings=64, rms_norm_eps=1e-3, tie_word_embeddings=True),
+    # many heads and a long context: prompts of this model fill the GPU with query blocks
+    "E": _cfg(num_hidden_layers=1, hidden_size=64, num_attention_heads=16, num_key_value_heads=4,
+              head_dim=32, intermediate_size=96, vocab_size=96, rope_theta=10000.0,
+              max_position_embeddings=4096, rms_norm_eps=1e-5, tie_word_embeddings=False),
     "R": _cfg(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2,
               head_dim=16, intermediate_size=128, vocab_size=512, rope_theta=10000.0,
               max_position_embeddings=256, rms_norm_eps=1e-6, tie_word_embeddings=False,

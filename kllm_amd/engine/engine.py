@@ -75,6 +75,7 @@ class Engine:
             raise RuntimeError("kllm_amd runs on a GPU only; torch sees none")
         from .. import kernels
         kernels.library()  # fail now, and loudly, if the kernels are missing
+        self.kernels = kernels
         self.options = options
         self.config = config
         self.device = torch.device("cuda", options.device)
@@ -307,7 +308,8 @@ class Engine:
             self._send(host, self._control, total)
             ctx = control.context(self._control, layout, self.runtime, starts, pos0, lens)
             ctx.taps = taps
-            logits = self.model.run(ctx, self._cache_views(ctx))
+            with self.kernels.stream_scope():
+                logits = self.model.run(ctx, self._cache_views(ctx))
         except Exception:
             self._undo(opened, reserved)
             raise

@@ -102,9 +102,10 @@ class DecodeGraphs:
         ctx = control.context(rec.control, rec.layout, eng.runtime, starts, pos0, lens)
         ctx.workspace = rec.workspace
         ctx.sampled = self.sampled
-        logits = eng.model.run(ctx, eng._cache_views(ctx))
-        temps, uniforms = control.sampling_views(rec.control, rec.layout)
-        K.sample(self.sampled[:rec.layout.n], logits, temps, uniforms)
+        with K.stream_scope():                   # the capture's stream while recording
+            logits = eng.model.run(ctx, eng._cache_views(ctx))
+            temps, uniforms = control.sampling_views(rec.control, rec.layout)
+            K.sample(self.sampled[:rec.layout.n], logits, temps, uniforms)
 
     def decode(self, entries, temperatures: Sequence[float], uniforms: Sequence[float]) -> SampledTokens:
         """One token for every entry (each entry is a single decode token, given

@@ -117,8 +117,28 @@ def _check(rc: int, what: str):
     raise KernelError(f"{what}: {buf.value.decode(errors='replace')} (code {rc})")
 
 
+_scoped = threading.local()
+
+
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    s = getattr(_scoped, "stream", None)
+    return s if s is not None else torch.cuda.current_stream().cuda_stream
+
+
+class stream_scope:
+    """Within the scope every launch of this thread goes to the stream that was
+    current when the scope was entered, looked up once instead of once per
+    launch (a step is a few hundred launches, and the lookup costs as much as
+    a launch).  The caller must not switch streams inside the scope."""
+
+    def __enter__(self):
+        self._outer = getattr(_scoped, "stream", None)
+        _scoped.stream = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        _scoped.stream = self._outer
+        return False
 
 
 def _ptr(t, name, dtype=None, allow_none=False):

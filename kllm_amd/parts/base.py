@@ -85,18 +85,28 @@ class Workspace:
 
     def __init__(self, device):
         self.device = device
-        self._bufs: Dict[str, torch.Tensor] = {}
+        self._bufs: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self._views: Dict[Tuple[str, tuple, torch.dtype], torch.Tensor] = {}   # handed out before
 
     def get(self, tag: str, shape, dtype) -> torch.Tensor:
+        shape = tuple(shape)
+        view = self._views.get((tag, shape, dtype))
+        if view is not None:
+            return view
         numel = 1
         for s in shape:
             numel *= int(s)
-        key = f"{tag}:{dtype}"
+        key = (tag, dtype)
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < numel:
             buf = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
             self._bufs[key] = buf
-        return buf[:numel].view(*shape)
+            for k in [k for k in self._views if k[0] == tag and k[2] == dtype]:   # views of the old buffer
+                del self._views[k]
+        view = buf[:numel].view(*shape)
+        if len(self._views) < 4096:
+            self._views[(tag, shape, dtype)] = view
+        return view
 
     def bytes(self) -> int:
         return sum(b.numel() * b.element_size() for b in self._bufs.values())

@@ -12,7 +12,7 @@ rotary + append, SiLU gate); with the compute dtype as result it returns
   float32   else: tiled FMA (true 32-bit)
   bfloat16  n <= 64: MFMA skinny (n <= 16 and one float32 result wanted: the
             decode-batch kernel with all of K in a workgroup)
-            else: MFMA tiles (K in two slices for a long K with few tiles),
+            else: MFMA tiles (K in slices where the tiles alone do not fill the chip),
             or the vendor library (torch.matmul) when the engine option
             ``gemm`` is "library" -- the reference uses its vendor library for
             every product (backend/model.cu:494-503)
@@ -51,6 +51,23 @@ def _skinny_split(n, m, k):
     return int(nsplit)
 
 
+def _mfma_split(n, m, k):
+    """Slices of K for the tiled MFMA kernel.  A product with fewer 128 x 128
+    tiles than the chip has room for workgroups (a portion of a prompt, a
+    projection to a narrow output) is bound by how many workgroups stream the
+    weights: up to 8 slices of at least 256 of K bring it to about 512
+    workgroups (measured, 72 rows: 2048 -> 2560 in 9 us instead of 26 us,
+    5632 -> 2048 in 13 us instead of 62 us; 2048 rows, 5632 -> 2048: 57 us
+    instead of 68 us with two slices, the second sum's traffic included)."""
+    tiles = -(-n // 128) * -(-m // 128)
+    nsplit = 1
+    while nsplit * 2 <= min(8, 512 // tiles, k // 256):
+        nsplit *= 2
+    while nsplit > 1 and (-(-(-(-k // nsplit)) // 64) * 64) * (nsplit - 1) >= k:   # no empty slice
+        nsplit -= 1
+    return nsplit
+
+
 def choose(dtype, n, m, k, options=None):
     """(algorithm, nsplit) for a product of these sizes."""
     options = options or {}
@@ -69,10 +86,7 @@ def choose(dtype, n, m, k, options=None):
         return K.GEMM_SKINNY_BF16, _skinny_split(n, m, k)
     if options.get("gemm") == "library":
         return "library", 1
-    # A long K with no more tiles than CUs: two slices of K give every CU a second workgroup
-    # (measured: 57 us against 68 us for 2048 x 5632 -> 2048, the second sum's traffic included).
-    tiles = -(-n // 128) * -(-m // 128)
-    return K.GEMM_MFMA_BF16, (2 if tiles <= 256 and k >= 4096 else 1)
+    return K.GEMM_MFMA_BF16, _mfma_split(n, m, k)
 
 
 def linear(ctx, x, w, tag, out_dtype=torch.float32, split=True):

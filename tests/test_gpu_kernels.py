@@ -405,8 +405,13 @@ def test_linear_chooses_a_kernel_for_every_size():
         kslice = -(-(-(-k // ns)) // 32) * 32
         assert kslice <= 512 and kslice * (ns - 1) < k, (n, m, k, ns)
     assert choose(torch.bfloat16, 400, 64, 64) == (k_.GEMM_MFMA_BF16, 1)
-    assert choose(torch.bfloat16, 2048, 2048, 5632) == (k_.GEMM_MFMA_BF16, 2)     # long K, few tiles
+    assert choose(torch.bfloat16, 2048, 2048, 5632) == (k_.GEMM_MFMA_BF16, 2)     # few tiles: slices of K
+    assert choose(torch.bfloat16, 72, 2048, 5632) == (k_.GEMM_MFMA_BF16, 8)
+    assert choose(torch.bfloat16, 512, 2560, 2048) == (k_.GEMM_MFMA_BF16, 4)
     assert choose(torch.bfloat16, 2048, 11264, 2048) == (k_.GEMM_MFMA_BF16, 1)
+    for n, m, k in [(65, 130, 40), (130, 515, 1032), (300, 257, 520), (70, 64, 4104), (100, 2048, 264)]:
+        ns = choose(torch.bfloat16, n, m, k)[1]
+        assert ns >= 1 and (-(-(-(-k // ns)) // 64) * 64) * (ns - 1) < k, (n, m, k, ns)
     assert choose(torch.bfloat16, 400, 64, 64, {"gemm": "library"})[0] == "library"
     a, ns = choose(torch.bfloat16, 1, 2049, 5632)
     assert a == k_.GEMM_GEMV and 1 <= ns <= 16

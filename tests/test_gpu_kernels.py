@@ -515,7 +515,8 @@ def test_attention_generic(H, KV, hd, ps, dtype, window):
 
 
 @pytest.mark.parametrize("H,KV,hd,ps", [(4, 2, 32, 16), (3, 1, 64, 16), (8, 2, 64, 32), (5, 5, 96, 16),
-                                        (2, 1, 128, 16), (2, 2, 192, 16), (2, 1, 256, 16), (32, 4, 64, 16)])
+                                        (2, 1, 128, 16), (2, 2, 192, 16), (2, 1, 256, 16), (32, 4, 64, 16),
+                                        (4, 2, 64, 48), (2, 1, 128, 48), (2, 2, 192, 80)])
 @pytest.mark.parametrize("window", [0, 37, 200])
 def test_attention_prefill(H, KV, hd, ps, window):
     """Whole prompts of ragged lengths, portions behind cached keys that start
@@ -531,7 +532,8 @@ def test_attention_prefill(H, KV, hd, ps, window):
     assert torch.isnan(out2.cpu()[~rows2]).all() and torch.equal(out2.cpu()[rows2], out.cpu()[rows2])
 
 
-@pytest.mark.parametrize("H,KV,hd,ps", [(24, 4, 32, 16), (24, 3, 64, 16), (22, 2, 96, 32), (22, 11, 128, 16)])
+@pytest.mark.parametrize("H,KV,hd,ps", [(24, 4, 32, 16), (24, 3, 64, 16), (22, 2, 96, 32), (22, 11, 128, 16),
+                                        (24, 6, 64, 48)])
 @pytest.mark.parametrize("window", [0, 150])
 def test_attention_prefill_many_blocks(H, KV, hd, ps, window):
     """More query blocks than CUs: the kernel that passes the keys through LDS,

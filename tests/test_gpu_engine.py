@@ -323,6 +323,35 @@ def test_greedy_generation_through_the_entry_point(model_dirs, name, dtype):
     assert not eng.cache.requests
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_generation_when_pages_run_out(model_dirs, dtype):
+    """A pool too small for the requests together: the scheduler gives the youngest one's
+    pages back and starts it again later, decode steps are queued ahead in between, and
+    every request still gets the plain implementation's tokens."""
+    from kllm_amd.engine import Engine, EngineOptions
+    from kllm_amd.engine.scheduler import Scheduler
+    cfg, d = tiny.CONFIGS["A"], model_dirs("A")
+    prompts = [tiny.tokens(cfg, n, 50 + n) for n in (40, 33, 50, 20)]
+    new = 30
+    eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=176, poison_freed_pages=True))
+    sched = Scheduler(eng, max_batch=4, max_step_tokens=64)
+    ids = [sched.submit(list(p), new, seed=i) for i, p in enumerate(prompts)]
+    results = sched.run_until_done()
+    assert sched.stats["preemptions"] > 0
+    assert not eng.cache.requests and all(p.free_pages == p.num_pages for p in eng.cache.pools)
+    w = tiny.read_weights(d, as_stored_in=dtype)
+    for i, p in zip(ids, prompts):
+        assert results[i].error is None
+        g, want = results[i].tokens, P.generate_greedy(w, cfg, p, new)
+        if dtype == "float32":
+            assert g == want
+        else:                                            # bfloat16 may part ways at a near-tie
+            agree = next((k for k, (x, y) in enumerate(zip(g, want)) if x != y), len(want))
+            if agree < len(want):
+                top2 = torch.topk(P.forward(w, cfg, p + want[:agree])[-1], 2).values
+                assert float(top2[0] - top2[1]) < tiny.TOL[dtype], (agree, g, want)
+
+
 def test_temperature_generation_matches_the_plain_sampler(model_dirs):
     """Config B, temperature 0.8, seeded: the same tokens as the plain
     implementation drawing with the same uniforms, alone and in a batch."""

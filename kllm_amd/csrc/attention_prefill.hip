@@ -78,8 +78,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
   // Later blocks read more keys.  The later half of the list is started first, longest block
   // first, then the earlier half, shortest first: a CU that holds one workgroup of each half
   // gets a long and a short one, and all CUs about the same number of keys.
-  const int j_ = (int)(item / H), h = item % H, n_late = (n_tiles + 1) / 2;
-  const int blk = j_ < n_late ? n_tiles - 1 - j_ : j_ - n_late;
+  const int place = (int)(item / H), h = item % H, n_late = (n_tiles + 1) / 2;
+  const int blk = place < n_late ? n_tiles - 1 - place : place - n_late;
   const int kvh = h / (H / KV);
   // The same for every lane: said so explicitly, which keeps the loop's address arithmetic on
   // the scalar unit.
@@ -303,10 +303,10 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
   // Whole rounds, every step of every round the same for all waves and without a branch
   // around a load, so that the compiler can count the loads in flight: a tile beyond the last
   // is asked for (a valid address) and dropped.
-  for (int t0_ = 0; t0_ < ntiles; t0_ += kRound) {
+  for (int round0 = 0; round0 < ntiles; round0 += kRound) {
 #pragma unroll
     for (int i = 0; i < kRound; ++i) {
-      const int t = t0_ + i;
+      const int t = round0 + i;
       compute(t, bufs[i % 2]);
       stash(st[(i + 1) % kAhead], t + 1, bufs[(i + 1) % 2]);
       lds_barrier();

@@ -45,9 +45,13 @@ def _bucket(pages: int) -> int:
 class SampledTokens:
     """The token ids of a sampled step, on their way to the host."""
 
-    def __init__(self, host: torch.Tensor, event: torch.cuda.Event, count: int):
+    def __init__(self, host: torch.Tensor, event: torch.cuda.Event, count: int, logits=None):
         self._host, self._event, self.count = host, event, count
         self._ids = None
+        # The step's float32 logits [count, vocab] on the device, in the recording's own
+        # buffer: they are what was sampled from, and hold until a step of the same batch
+        # size and table width is queued again.
+        self.logits = logits
 
     def ready(self) -> bool:
         return self._ids is not None or self._event.query()
@@ -77,6 +81,7 @@ class _Recording:
         self.workspace = Workspace(engine.device)
         self.graph = None
         self.replays = 0
+        self.logits = None
 
 
 class DecodeGraphs:
@@ -104,6 +109,7 @@ class DecodeGraphs:
         ctx.sampled = self.sampled
         with K.stream_scope():                   # the capture's stream while recording
             logits = eng.model.run(ctx, eng._cache_views(ctx))
+            rec.logits = logits
             temps, uniforms = control.sampling_views(rec.control, rec.layout)
             K.sample(self.sampled[:rec.layout.n], logits, temps, uniforms)
 
@@ -145,7 +151,7 @@ class DecodeGraphs:
             eng._send(host, rec.control, rec.layout.total)
             if rec.graph is None:
                 self._run(rec, lens, pos0)              # the step itself, and the warm-up
-                out = self._read_back(batch)
+                out = self._read_back(batch, rec.logits)
                 out.tokens()                            # before the capture's second run of the kernels
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph, capture_error_mode="thread_local"):
@@ -155,7 +161,7 @@ class DecodeGraphs:
             else:
                 rec.graph.replay()
                 rec.replays += 1
-                out = self._read_back(batch)
+                out = self._read_back(batch, rec.logits)
         except Exception:
             eng._undo(opened, reserved)
             raise
@@ -163,7 +169,7 @@ class DecodeGraphs:
         self.last = out
         return out
 
-    def _read_back(self, batch: int) -> SampledTokens:
+    def _read_back(self, batch: int, logits=None) -> SampledTokens:
         """Queue the copy of the sampled ids to the host behind the step."""
         i = self._host_next
         self._host_next = (i + 1) % len(self._host_ring)
@@ -173,5 +179,5 @@ class DecodeGraphs:
         host[:batch].copy_(self.sampled[:batch], non_blocking=True)
         event = torch.cuda.Event()
         event.record()
-        self._host_owner[i] = SampledTokens(host, event, batch)
+        self._host_owner[i] = SampledTokens(host, event, batch, logits)
         return self._host_owner[i]

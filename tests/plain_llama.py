@@ -63,7 +63,7 @@ def rope(x, positions, n_heads, head_dim, theta):
     return out.reshape(T, n_heads * head_dim)
 
 
-def attention(q, k, v, q_positions, n_heads, n_kv_heads, head_dim, window=0):
+def attention(q, k, v, q_positions, n_heads, n_kv_heads, head_dim, window=0, store=None):
     """Causal softmax attention of one sequence over its own keys.
 
     q is [T, H*hd] at absolute positions ``q_positions``; k and v are
@@ -72,7 +72,9 @@ def attention(q, k, v, q_positions, n_heads, n_kv_heads, head_dim, window=0):
     [0, p] (backend/model.cu:361), or the last ``window`` of them when
     window > 0 (backend/model.cu:224-225, :362).  score = (q.k) * 1/sqrt(hd)
     (backend/model.cu:1063-1064); softmax with the maximum subtracted
-    (backend/model.cu:365-407; tools/gen_reference_numpy_moe.py:105-118)."""
+    (backend/model.cu:365-407; tools/gen_reference_numpy_moe.py:105-118).
+    ``store`` (see ``forward``) rounds the exponentials before they meet the
+    values; their sum is then taken over the rounded numbers."""
     T, S = q.shape[0], k.shape[0]
     group = n_heads // n_kv_heads
     qpos = torch.as_tensor(q_positions, dtype=torch.long)
@@ -91,6 +93,10 @@ def attention(q, k, v, q_positions, n_heads, n_kv_heads, head_dim, window=0):
         sc = torch.where(mask, sc, torch.full_like(sc, float("-inf")))
         sc = sc - sc.max(dim=1, keepdim=True).values
         p = torch.exp(sc)
+        if store is not None:
+            p = store(p)
+            out[:, h * head_dim:(h + 1) * head_dim] = (p @ vh) / p.sum(dim=1, keepdim=True)
+            continue
         p = p / p.sum(dim=1, keepdim=True)
         out[:, h * head_dim:(h + 1) * head_dim] = p @ vh
     return out
@@ -101,9 +107,10 @@ def silu(x):
     return x / (1.0 + torch.exp(-x))
 
 
-def swiglu(xn, w_gate, w_up, w_down):
+def swiglu(xn, w_gate, w_up, w_down, store=None):
     """down(silu(gate(x)) * up(x)) (backend/model.cu:1112-1115)."""
-    return linear(silu(linear(xn, w_gate)) * linear(xn, w_up), w_down)
+    h = silu(linear(xn, w_gate)) * linear(xn, w_up)
+    return linear(h if store is None else store(h), w_down)
 
 
 # --------------------------------------------------------------------------- model
@@ -123,39 +130,46 @@ def _cfg(cfg):
     )
 
 
-def attention_sublayer(w, prefix, xn, positions, c, window=0, kv=None):
+def attention_sublayer(w, prefix, xn, positions, c, window=0, kv=None, store=None):
     """q, k, v projections, rotary on q and k before they are kept, attention,
     output projection (backend/model.cu:1090-1104).  With ``kv`` given (the
     rotated keys and the values another layer made) only q is projected.
     Returns (output, (k, v))."""
+    keep = store if store is not None else (lambda t: t)
     q = linear(xn, w[prefix + "self_attn.q_proj.weight"])
-    q = rope(q, positions, c["H"], c["hd"], c["theta"])
+    q = keep(rope(q, positions, c["H"], c["hd"], c["theta"]))
     if kv is None:
         k = linear(xn, w[prefix + "self_attn.k_proj.weight"])
-        v = linear(xn, w[prefix + "self_attn.v_proj.weight"])
-        k = rope(k, positions, c["KV"], c["hd"], c["theta"])
+        v = keep(linear(xn, w[prefix + "self_attn.v_proj.weight"]))
+        k = keep(rope(k, positions, c["KV"], c["hd"], c["theta"]))
     else:
         k, v = kv
-    a = attention(q, k, v, torch.arange(len(positions)), c["H"], c["KV"], c["hd"], window)
+    a = keep(attention(q, k, v, torch.arange(len(positions)), c["H"], c["KV"], c["hd"], window, store))
     return linear(a, w[prefix + "self_attn.o_proj.weight"]), (k, v)
 
 
-def decoder_layer(w, layer, x, positions, c, window=0, kv=None):
+def decoder_layer(w, layer, x, positions, c, window=0, kv=None, store=None):
     """a = h + Attn(Norm_in(h)); h' = a + FFN(Norm_post(a))
     (backend/model.cu:1083-1117; the reference defers the second add into the
     next norm, which does not change the sum)."""
     p = f"model.layers.{layer}."
-    xn = rmsnorm(x, w[p + "input_layernorm.weight"], c["eps"])
-    a, kv_out = attention_sublayer(w, p, xn, positions, c, window, kv)
+    keep = store if store is not None else (lambda t: t)
+    xn = keep(rmsnorm(x, w[p + "input_layernorm.weight"], c["eps"]))
+    a, kv_out = attention_sublayer(w, p, xn, positions, c, window, kv, store)
     x = x + a
-    xn = rmsnorm(x, w[p + "post_attention_layernorm.weight"], c["eps"])
+    xn = keep(rmsnorm(x, w[p + "post_attention_layernorm.weight"], c["eps"]))
     x = x + swiglu(xn, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
-                   w[p + "mlp.down_proj.weight"])
+                   w[p + "mlp.down_proj.weight"], store)
     return x, kv_out
 
 
+def round_bfloat16(t):
+    """A value as an engine with bfloat16 storage keeps it: rounded to nearest even."""
+    return t.to(torch.bfloat16).to(t.dtype)
+
+
 def forward(w, cfg, ids, dtype=torch.float32, return_hidden=False, schedule=None, pos0=0,
-            windows=None, kv_from=None):
+            windows=None, kv_from=None, store=None):
     """Logits [T, vocab] at every position of one whole sequence whose first
     token stands at position ``pos0`` (0 for a real sequence; another value
     only shifts every rotary angle, which must not change anything).
@@ -164,7 +178,12 @@ def forward(w, cfg, ids, dtype=torch.float32, return_hidden=False, schedule=None
     :1085, :1123-1124; engine/e2e/e2e_test.go:117-131).  ``schedule`` is the
     order in which layers run (default 0..L-1); ``windows`` maps a layer to
     its attention window; ``kv_from`` maps a run of the schedule to the earlier
-    run whose keys and values it reads."""
+    run whose keys and values it reads.  ``store`` (for instance
+    ``round_bfloat16``) is applied wherever an engine with narrower storage
+    keeps an activation: the normalised rows that feed a product, rotated
+    queries, kept keys and values, attention's exponentials and output, the
+    gated activation.  The residual stream, every sum and the logits stay in
+    ``dtype``; weights are rounded by the caller."""
     c = _cfg(cfg)
     w = {k: v.to(dtype) for k, v in w.items()}
     T = len(ids)
@@ -176,9 +195,11 @@ def forward(w, cfg, ids, dtype=torch.float32, return_hidden=False, schedule=None
     for run, layer in enumerate(order):
         kv = kept[kv_from[run]] if kv_from and run in kv_from else None
         win = (windows or {}).get(layer, 0)
-        x, kept[run] = decoder_layer(w, layer, x, positions, c, win, kv)
+        x, kept[run] = decoder_layer(w, layer, x, positions, c, win, kv, store)
         hidden.append(x.clone())
     xn = rmsnorm(x, w["model.norm.weight"], c["eps"])
+    if store is not None:
+        xn = store(xn)
     hidden.append(xn.clone())
     head = w["model.embed_tokens.weight"] if c["tied"] else w["lm_head.weight"]
     logits = linear(xn, head)

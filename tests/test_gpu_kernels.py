@@ -39,37 +39,59 @@ def test_embed(dtype):
     assert torch.equal(out.cpu(), P.embedding(ids.cpu().tolist(), table.cpu().float()))
 
 
-@pytest.mark.parametrize("d", [72, 100, 2048, 4100])
-@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-def test_add_rmsnorm(d, out_dtype):
-    n, eps = 7, 1e-5
+SPLITS = [1, 3, 4, 7, 8, 11, 12, 15, 16]
+
+
+@pytest.mark.parametrize("n,d", [(7, 72), (7, 100), (5, 1000), (7, 2048), (3, 3000), (7, 4100), (2, 9000), (300, 2048)])
+@pytest.mark.parametrize("out_dtype,delta_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.float32),
+                                                   (torch.bfloat16, torch.bfloat16)])
+def test_add_rmsnorm(n, d, out_dtype, delta_dtype):
+    """Every number of partial sums that a split product hands over (the consumer's 8-wide,
+    4-wide and one-by-one branches), at row lengths a thread keeps 2, 4 or 8 elements of (and
+    longer ones), with 256 and with 1024 threads a row."""
+    eps = 1e-5
     x, w = rnd(n, d, seed=1, scale=3.0), (1 + 0.2 * rnd(d, seed=2))
-    delta = rnd(3, n, d, seed=3)
-    want_x = x.cpu().double() + delta.cpu().double().sum(0)
-    want = P.rmsnorm(want_x, w.cpu().double(), eps)
-    # norm only
     out = torch.empty(n, d, dtype=out_dtype, device=DEV)
+    # norm only
     x0 = x.clone()
     K().add_rmsnorm(x0, weight=w, out=out, eps=eps)
     assert torch.equal(x0, x)
     ref0 = P.rmsnorm(x.cpu().double(), w.cpu().double(), eps)
     assert (out.cpu().double() - ref0).abs().max() < tol(out_dtype) * 3
-    # add (three partial sums) + norm, x updated
-    x1 = x.clone()
-    K().add_rmsnorm(x1, delta=delta, weight=w, out=out, eps=eps)
-    assert (x1.cpu().double() - want_x).abs().max() < 1e-5
-    assert (out.cpu().double() - want).abs().max() < tol(out_dtype) * 3
-    # add only
-    x2 = x.clone()
-    K().add_rmsnorm(x2, delta=delta[0], write_x=True)
-    assert torch.allclose(x2, x + delta[0])
-    # gathered rows: x untouched
-    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
-    x3 = x.clone()
-    out3 = torch.empty(3, d, dtype=out_dtype, device=DEV)
-    K().add_rmsnorm(x3, delta=delta, weight=w, out=out3, rows=rows, eps=eps)
-    assert torch.equal(x3, x)
-    assert (out3.cpu().double() - want[[6, 0, 3]]).abs().max() < tol(out_dtype) * 3
+    rows = torch.tensor([n - 1, 0, n // 2], dtype=torch.int32, device=DEV)
+    for nsplit in SPLITS:
+        delta = rnd(nsplit, n, d, seed=3 + nsplit, dtype=delta_dtype)
+        want_x = x.cpu().double() + delta.cpu().double().sum(0)
+        want = P.rmsnorm(want_x, w.cpu().double(), eps)
+        # add (partial sums) + norm, x updated
+        x1 = x.clone()
+        out.fill_(float("nan"))
+        K().add_rmsnorm(x1, delta=delta, weight=w, out=out, eps=eps)
+        assert (x1.cpu().double() - want_x).abs().max() < 2e-5, nsplit
+        assert (out.cpu().double() - want).abs().max() < tol(out_dtype) * 3, nsplit
+        # add only (all partial sums, and a single one given as a matrix)
+        x2 = x.clone()
+        K().add_rmsnorm(x2, delta=delta, write_x=True)
+        assert torch.equal(x2, x1), nsplit
+        x2 = x.clone()
+        K().add_rmsnorm(x2, delta=delta[0], write_x=True)
+        assert torch.allclose(x2, x + delta[0].float())
+        # gathered rows: x untouched
+        x3 = x.clone()
+        out3 = torch.empty(3, d, dtype=out_dtype, device=DEV)
+        K().add_rmsnorm(x3, delta=delta, weight=w, out=out3, rows=rows, eps=eps)
+        assert torch.equal(x3, x)
+        assert (out3.cpu().double() - want[rows.cpu().long()]).abs().max() < tol(out_dtype) * 3, nsplit
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_sum_splits(out_dtype):
+    for nsplit, shape in [(1, (3, 130)), (4, (8, 257)), (7, (5, 100)), (8, (64, 515)), (11, (64, 2048)), (16, (2, 33))]:
+        parts = rnd(nsplit, *shape, seed=nsplit)
+        out = torch.full(shape, float("nan"), dtype=out_dtype, device=DEV)
+        K().sum_splits(parts, out)
+        want = parts.cpu().double().sum(0)
+        assert (out.cpu().double() - want).abs().max() < tol(out_dtype) * 3, nsplit
 
 
 def test_rmsnorm_zero_row_and_eps_inside_the_root():
@@ -109,8 +131,9 @@ def read_cache(cache, table, length, KV, hd, ps):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,KV,hd,ps", [(4, 2, 16, 16), (3, 1, 32, 16), (5, 5, 48, 32), (6, 3, 80, 16)])
-def test_rope_append(dtype, H, KV, hd, ps):
-    theta, nsplit = 10000.0, 2
+@pytest.mark.parametrize("nsplit", [1, 2, 4, 7, 8, 11, 16])
+def test_rope_append(dtype, H, KV, hd, ps, nsplit):
+    theta = 10000.0
     # two spans: positions 30..36 of request 0 and 0..4 of request 1, scattered pages
     spans = [(30, 7), (0, 5)]
     n = sum(l for _, l in spans)
@@ -147,16 +170,18 @@ def test_rope_append(dtype, H, KV, hd, ps):
 # ------------------------------------------------------------------ silu gate
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-def test_silu_mul(out_dtype):
+@pytest.mark.parametrize("nsplit", [1, 2, 4, 7, 8, 11, 16])
+def test_silu_mul(out_dtype, nsplit):
     n, f = 5, 176
-    gu = rnd(2, n, 2 * f, seed=4, scale=3.0)
-    gu[0, 0, 0], gu[1, 0, 0] = -60.0, -60.0       # far negative gate: 0, not NaN
+    gu = rnd(nsplit, n, 2 * f, seed=4, scale=3.0 / nsplit ** 0.5)
+    gu[:, 0, 0] = -60.0 / nsplit                  # far negative gate: 0, not NaN
     out = torch.empty(n, f, dtype=out_dtype, device=DEV)
     K().silu_mul(gu, out)
     s = gu.cpu().double().sum(0)
     want = P.silu(s[:, :f]) * s[:, f:]
     assert torch.isfinite(out).all()
-    assert (out.cpu().double() - want).abs().max() < tol(out_dtype) * 10
+    bound = 1e-4 if out_dtype == torch.float32 else 0.01 * want.abs().max()    # eight bits of the largest value
+    assert (out.cpu().double() - want).abs().max() < bound
 
 
 # ------------------------------------------------------------------ matrix products
@@ -196,6 +221,83 @@ def test_gemm_kernels_against_plain(n, m, k, dtype):
         y = torch.empty(n, m, dtype=dtype, device=DEV)
         k_.gemm(x, w, y, k_.GEMM_MFMA_BF16)
         assert (y.cpu().double() - want).abs().max() < 0.01 * want.abs().max()
+
+
+def _gpu_reference(x, w):
+    """x . w^T in double on the GPU with the library's product: the yardstick for
+    sizes at which the CPU would take minutes.  (The library is the reference
+    here, never the product path.)"""
+    return x.double() @ w.double().t()
+
+
+@pytest.mark.parametrize("n,m,k,nsplit", [
+    (2048, 2560, 2048, 1),      # more tiles than CUs: two stages, 128-row tiles
+    (2048, 2048, 5632, 2),      # two slices of K
+    (2048, 2048, 5632, 1),
+    (2048, 11264, 2048, 1),     # 256-row tiles, eight waves
+    (1000, 5000, 2056, 1),      # ragged in every direction, 256-row tiles
+    (1000, 5000, 2056, 3),
+    (700, 2100, 264, 1),        # two stages, ragged
+    (4096, 4096, 4096, 1),
+    (2048, 32000, 2048, 1),     # the logits of a whole prompt
+])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_gemm_mfma_at_prompt_sizes(n, m, k, nsplit, out_dtype):
+    """The tile variants that only products of prompt size reach (256-row tiles with eight
+    waves; two stages when there are more tiles than CUs), whole and in slices of K."""
+    if out_dtype == torch.bfloat16 and nsplit > 1:
+        pytest.skip("K is split only for float32 partial sums")
+    k_ = K()
+    x, w = rnd(n, k, seed=1, dtype=torch.bfloat16), rnd(m, k, seed=2, dtype=torch.bfloat16)
+    want = _gpu_reference(x, w)
+    y = torch.full((nsplit, n, m), float("nan"), dtype=out_dtype, device=DEV)
+    k_.gemm(x, w, y if nsplit > 1 or out_dtype == torch.float32 else y[0], k_.GEMM_MFMA_BF16, nsplit)
+    err = (y.double().sum(0) - want).abs().max()
+    if out_dtype == torch.float32:
+        assert err < 1e-5 * k ** 0.5 * 8, float(err)
+    else:
+        assert err < 0.01 * want.abs().max(), float(err)
+    # one row and one column against the plain kernel's way of summing, on the CPU in double
+    r, c = n - 1, m - 1
+    assert abs(float(y.double().sum(0)[r, c]) - float(P.linear(x[r:r + 1].cpu().double(), w[c:c + 1].cpu().double()))) < \
+        (1e-3 if out_dtype == torch.float32 else 0.01 * float(want.abs().max()))
+
+
+@pytest.mark.parametrize("n,f,k", [(2048, 5632, 2048), (1000, 2500, 2056), (2048, 14336, 4096), (300, 5632, 2048)])
+def test_gemm_swiglu_at_prompt_sizes(n, f, k):
+    dtype = torch.bfloat16
+    x, w = rnd(n, k, seed=1, dtype=dtype, scale=0.5), rnd(2 * f, k, seed=2, dtype=dtype, scale=0.05)
+    h = torch.full((n, f), float("nan"), dtype=dtype, device=DEV)
+    K().gemm_swiglu(x, w, h)
+    g, u = _gpu_reference(x, w[:f]), _gpu_reference(x, w[f:])
+    want = P.silu(g) * u
+    assert (h.double() - want).abs().max() < 0.01 * want.abs().max() + 1e-3
+
+
+@pytest.mark.parametrize("n", [5, 8, 16, 33, 64])
+@pytest.mark.parametrize("m,k", [(2048, 2048), (2048, 5632), (4096, 14336), (2560, 2048)])
+def test_split_product_into_its_consumers(n, m, k):
+    """A decode batch's product with K in as many slices as the engine chooses at these sizes
+    (8 at K = 2048, 11 at 5632), consumed by the norm and by the sum kernel."""
+    from kllm_amd.parts.linear import choose
+    k_ = K()
+    algo, nsplit = choose(torch.bfloat16, n, m, k)
+    assert algo == k_.GEMM_SKINNY_BF16 and nsplit >= 4
+    x, w = rnd(n, k, seed=1, dtype=torch.bfloat16, scale=0.5), rnd(m, k, seed=2, dtype=torch.bfloat16, scale=0.05)
+    parts = torch.full((nsplit, n, m), float("nan"), device=DEV)
+    k_.gemm(x, w, parts, algo, nsplit)
+    want = _gpu_reference(x, w).cpu()
+    assert (parts.cpu().double().sum(0) - want).abs().max() < 1e-5 * k ** 0.5 * 8
+    res, nw = rnd(n, m, seed=3), 1 + 0.2 * rnd(m, seed=4)
+    out = torch.empty(n, m, dtype=torch.bfloat16, device=DEV)
+    x1 = res.clone()
+    k_.add_rmsnorm(x1, delta=parts, weight=nw, out=out, eps=1e-5)
+    want_x = res.cpu().double() + want
+    assert (x1.cpu().double() - want_x).abs().max() < 1e-4
+    assert (out.cpu().double() - P.rmsnorm(want_x, nw.cpu().double(), 1e-5)).abs().max() < 6e-2
+    y = torch.empty(n, m, device=DEV)
+    k_.sum_splits(parts, y)
+    assert (y.cpu().double() - want).abs().max() < 1e-5 * k ** 0.5 * 8
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

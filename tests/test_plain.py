@@ -278,3 +278,19 @@ def test_sampling_reference():
     assert P.sample_inverse_cdf(row, 0, 0.0) == 2
     # temperature sharpens: at T = 0.5 the weights are squared (1, 4, 25)/30
     assert P.sample_inverse_cdf(row, 0.5, 0.034) == 1
+
+
+def test_storage_rounding_changes_little_and_nothing_when_it_is_the_identity():
+    """``store`` marks where an engine with narrower storage keeps activations: the
+    identity must give the default's logits (but for the order of the softmax's division),
+    bfloat16 rounding logits that differ by rounding noise only (far less than the
+    logits' own size)."""
+    import tiny
+    cfg = tiny.CONFIGS["A"]
+    w = P.random_weights(cfg, 2, std=0.05, norm_std=0.1)
+    ids = tiny.tokens(cfg, 40, 1)
+    base = P.forward(w, cfg, ids)
+    assert float((P.forward(w, cfg, ids, store=lambda t: t) - base).abs().max()) < 2e-6
+    rounded = P.forward(w, cfg, ids, store=P.round_bfloat16)
+    err = float((rounded - base).abs().max())
+    assert 0 < err < 0.02 * float(base.abs().max())

@@ -21,6 +21,8 @@
 // [hd row c][those keys], two 8-byte reads from the [hd][slot] value layout.
 #include <math.h>
 
+#include <mutex>
+
 #include "common.hpp"
 #include "kllm_kernels.h"
 
@@ -319,25 +321,28 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H) {
   return wg;
 }
 
-extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part_floats,
-                                const void* cache, const int* positions, const int* span_of_token,
-                                const int* block_table, int max_pages, int page_size, int n, int H,
-                                int KV, int hd, int window, float scale, int nslices, int dtype,
-                                const int* token_list, int n_listed, hipStream_t stream) {
+// Checks and launches shared by both entry points; `part` holds at least part_floats floats.
+static int attn_decode_run(const char* who, const void* q, void* out, float* part, long part_floats,
+                           const void* cache, const int* positions, const int* span_of_token,
+                           const int* block_table, int max_pages, int page_size, int n, int H, int KV,
+                           int hd, int window, float scale, int nslices, int dtype,
+                           const int* token_list, int n_listed, hipStream_t stream) {
   KLLM_REQUIRE(q && out && part && cache && positions && span_of_token && block_table,
-               "attn_decode: null pointer");
-  KLLM_REQUIRE(dtype == DT_BF16, "attn_decode: bfloat16 only (float32 uses the generic kernel)");
-  KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && H % KV == 0, "attn_decode: bad heads n=%d H=%d KV=%d", n, H, KV);
+               "%s: null pointer", who);
+  KLLM_REQUIRE(dtype == DT_BF16, "%s: bfloat16 only (float32 uses the generic kernel)", who);
+  KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && H % KV == 0, "%s: bad heads n=%d H=%d KV=%d", who, n, H, KV);
   KLLM_REQUIRE(hd % 16 == 0 && hd >= 16 && hd <= 256 && (hd <= 128 || hd == 192 || hd == 256),
-               "attn_decode: head_dim %d is not built (16..128 in steps of 16, 192, 256)", hd);
+               "%s: head_dim %d is not built (16..128 in steps of 16, 192, 256)", who, hd);
   KLLM_REQUIRE(page_size % 16 == 0 && page_size > 0 && max_pages > 0,
-               "attn_decode: page_size %d must be a multiple of 16", page_size);
-  KLLM_REQUIRE(nslices >= 1 && nslices <= 256, "attn_decode: nslices %d is outside [1, 256]", nslices);
-  KLLM_REQUIRE(window >= 0, "attn_decode: negative window");
-  KLLM_REQUIRE(part_floats >= (long)n * H * nslices * (hd + 2), "attn_decode: workspace too small");
+               "%s: page_size %d must be a multiple of 16", who, page_size);
+  KLLM_REQUIRE(nslices >= 1 && nslices <= 256, "%s: nslices %d is outside [1, 256]", who, nslices);
+  KLLM_REQUIRE(window >= 0, "%s: negative window", who);
+  KLLM_REQUIRE(part_floats >= (long)n * H * nslices * (hd + 2),
+               "%s: the partial results of n=%d H=%d nslices=%d head_dim=%d need %ld floats, the workspace has %ld",
+               who, n, H, nslices, hd, (long)n * H * nslices * (hd + 2), part_floats);
   const int head_tiles = (H / KV + 15) / 16;
-  KLLM_REQUIRE((long)KV * head_tiles <= 65535 && H <= 65535, "attn_decode: too many heads for the grid");
-  KLLM_REQUIRE(!token_list || (n_listed > 0 && n_listed <= n), "attn_decode: bad token list");
+  KLLM_REQUIRE((long)KV * head_tiles <= 65535 && H <= 65535, "%s: too many heads for the grid", who);
+  KLLM_REQUIRE(!token_list || (n_listed > 0 && n_listed <= n), "%s: bad token list", who);
   const int count = token_list ? n_listed : n;     // part and out are indexed by token, not by list place
   const dim3 grid(count, KV * head_tiles, nslices);
 #define KLLM_DEC(HDT)                                                                             \
@@ -348,12 +353,74 @@ extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part
   switch (hd / 16) {
     KLLM_DEC(1); KLLM_DEC(2); KLLM_DEC(3); KLLM_DEC(4); KLLM_DEC(5); KLLM_DEC(6); KLLM_DEC(7);
     KLLM_DEC(8); KLLM_DEC(12); KLLM_DEC(16);
-    default: KLLM_FAIL(ERR_ARG, "attn_decode: head_dim %d is not built", hd);
+    default: KLLM_FAIL(ERR_ARG, "%s: head_dim %d is not built", who, hd);
   }
 #undef KLLM_DEC
-  KLLM_CHECK_LAUNCH("attn_decode");
+  KLLM_CHECK_LAUNCH(who);
   hipLaunchKernelGGL(attn_merge_kernel<bf16_t>, dim3(count, H), dim3(64), 0, stream, (bf16_t*)out, part,
                      H, hd, nslices, token_list);
   KLLM_CHECK_LAUNCH("attn_merge");
   return 0;
+}
+
+extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part_floats,
+                                const void* cache, const int* positions, const int* span_of_token,
+                                const int* block_table, int max_pages, int page_size, int n, int H,
+                                int KV, int hd, int window, float scale, int nslices, int dtype,
+                                const int* token_list, int n_listed, hipStream_t stream) {
+  return attn_decode_run("attn_decode", q, out, part, part_floats, cache, positions, span_of_token,
+                         block_table, max_pages, page_size, n, H, KV, hd, window, scale, nslices, dtype,
+                         token_list, n_listed, stream);
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------------
+// The partial results of the slices live in this array instead of a workspace of the caller's.
+// Every GPU that the library runs on holds its own copy (4 MiB) until the process ends.  In
+// host code the array's name is only a stand-in: its address on the current device comes
+// from hipGetSymbolAddress, once per device, and only that pointer is ever handed to a kernel.
+static __device__ __align__(256) float scratch[KLLM_ATTN_DECODE_STATIC_FLOATS];
+
+constexpr int kMaxDevices = 64;
+static float* g_scratch_ptr[kMaxDevices];        // per device, null until looked up
+static std::mutex g_scratch_mutex;
+
+// The array's address on the current device (looked up at the first call there).
+static int scratch_on_current_device(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) KLLM_FAIL((int)e, "attn_decode_static: hipGetDevice: %s", hipGetErrorString(e));
+  KLLM_REQUIRE(dev >= 0 && dev < kMaxDevices, "attn_decode_static: device %d is outside [0, %d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      KLLM_FAIL(e != hipSuccess ? (int)e : ERR_STATE, "attn_decode_static: hipGetSymbolAddress on device %d: %s",
+                dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int kllm_attn_decode_static(const void* q, void* out, const void* cache, const int* positions,
+                                       const int* span_of_token, const int* block_table, int max_pages,
+                                       int page_size, int n, int H, int KV, int hd, int window, float scale,
+                                       int nslices, int dtype, const int* token_list, int n_listed,
+                                       hipStream_t stream) {
+  KLLM_REQUIRE(n > 0 && H > 0 && nslices >= 1 && hd > 0, "attn_decode_static: bad sizes n=%d H=%d nslices=%d hd=%d",
+               n, H, nslices, hd);
+  const long need = (long)n * H * nslices * (hd + 2);
+  KLLM_REQUIRE(need <= (long)KLLM_ATTN_DECODE_STATIC_FLOATS,
+               "attn_decode_static: n=%d tokens x H=%d heads x nslices=%d slices x (head_dim=%d + 2) = %ld floats of "
+               "partial results exceed the built-in scratch of %ld floats; use fewer slices or kllm_attn_decode "
+               "with a workspace",
+               n, H, nslices, hd, need, (long)KLLM_ATTN_DECODE_STATIC_FLOATS);
+  float* part = nullptr;
+  if (int rc = scratch_on_current_device(&part)) return rc;
+  // Nothing in the scratch has to start at zero: the first kernel writes every partial result
+  // (maximum, sum, output of each token, head and slice) that the second one reads.
+  return attn_decode_run("attn_decode_static", q, out, part, (long)KLLM_ATTN_DECODE_STATIC_FLOATS, cache,
+                         positions, span_of_token, block_table, max_pages, page_size, n, H, KV, hd, window,
+                         scale, nslices, dtype, token_list, n_listed, stream);
 }

@@ -142,6 +142,23 @@ int kllm_attn_decode(const void* q, void* out, float* part, long part_floats, co
                      float scale, int nslices, int dtype, const int* token_list, int n_listed,
                      hipStream_t stream);
 
+/* kllm_attn_decode without a workspace argument and without any allocation: for callers
+ * that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The partial
+ * results go to an array that the library holds on every GPU it runs on
+ * (KLLM_ATTN_DECODE_STATIC_FLOATS floats = 4 MiB, kept until the process ends); a call whose
+ * n * H * nslices * (hd + 2) exceeds that is refused.  The array's address is looked up at
+ * the first call on a device, which must be the current device (and the stream's).  All
+ * calls on one GPU share the array and it keeps the last call's contents: calls that
+ * overlap on one GPU (two streams, two threads) race; nothing in it needs clearing
+ * between calls.  Same kernels, same results as kllm_attn_decode. */
+#define KLLM_ATTN_DECODE_STATIC_FLOATS (1 << 20)
+int kllm_attn_decode_static(const void* q, void* out, const void* cache, const int* positions,
+                            const int* span_of_token, const int* block_table, int max_pages,
+                            int page_size, int n, int H, int KV, int hd, int window, float scale,
+                            int nslices, int dtype, const int* token_list, int n_listed,
+                            hipStream_t stream);
+
 /* Prompt attention on the matrix cores (bfloat16).  query_tiles holds
  * (first token row, span) pairs: up to 128 consecutive tokens of one span. */
 int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,

@@ -23,6 +23,8 @@
 
 #include <mutex>
 
+#include "attention_f32.hpp"
+#include "attention_merge.hpp"
 #include "common.hpp"
 #include "kllm_kernels.h"
 
@@ -258,43 +260,6 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
   }
 }
 
-// out[t, h, :] = sum_s w_s o_s / sum_s w_s l_s with w_s = exp(m_s - max m).
-// One wave per (token, head); eight slices are read at a time.
-template <typename T>
-__global__ __launch_bounds__(64) void attn_merge_kernel(T* __restrict__ out,
-                                                        const float* __restrict__ part, int H, int hd,
-                                                        int nslices, const int* __restrict__ token_list) {
-  const int t = token_list ? token_list[blockIdx.x] : blockIdx.x;
-  const int h = blockIdx.y, lane = threadIdx.x;
-  const int stride = hd + 2;
-  const float* p = part + ((long)t * H + h) * nslices * stride;
-  float M = -INFINITY;
-  for (int s = lane; s < nslices; s += kWave) M = fmaxf(M, p[(long)s * stride + hd]);
-  M = wave_max(M);
-  float denom = 0.f;
-  for (int s = lane; s < nslices; s += kWave) {
-    const float ms = p[(long)s * stride + hd];
-    if (ms != -INFINITY) denom += expf(ms - M) * p[(long)s * stride + hd + 1];
-  }
-  denom = wave_sum(denom);
-  for (int d = lane; d < hd; d += kWave) {
-    float o = 0.f;
-    for (int s0 = 0; s0 < nslices; s0 += 8) {
-      float ms[8], os[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const bool ok = s0 + j < nslices;
-        ms[j] = ok ? p[(long)(s0 + j) * stride + hd] : -INFINITY;
-        os[j] = ok ? p[(long)(s0 + j) * stride + d] : 0.f;
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        if (ms[j] != -INFINITY) o += expf(ms[j] - M) * os[j];
-    }
-    out[((long)t * H + h) * hd + d] = from_f32<T>(o / denom);
-  }
-}
-
 template <int HDT>
 static void launch_decode(dim3 grid, hipStream_t stream, const void* q, float* part, const void* cache,
                           const int* positions, const int* span_of_token, const int* block_table,
@@ -309,12 +274,14 @@ static void launch_decode(dim3 grid, hipStream_t stream, const void* q, float* p
 
 using namespace kllm;
 
-extern "C" int kllm_attn_decode_slices(int n, int KV, int H) {
-  // About 2048 waves across the chip, shared out over tokens x KV heads x head tiles; a
-  // workgroup is four waves and leaves one partial result.
+extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int dtype) {
+  if (KV <= 0 || H <= 0 || n <= 0) return 1;
+  if (dtype == DT_F32) return attn_f32_slices(n, KV, H);
+  // About eight waves per CU across the chip, shared out over tokens x KV heads x head tiles;
+  // a workgroup is four waves and leaves one partial result.
   const int head_tiles = (H / KV + 15) / 16;
   long groups = (long)n * KV * head_tiles;
-  long want = 2048 / (groups > 0 ? groups : 1);
+  long want = 8L * device_cus() / (groups > 0 ? groups : 1);
   int wg = (int)((want + kDecodeWaves - 1) / kDecodeWaves);
   if (wg < 1) wg = 1;
   if (wg > 16) wg = 16;
@@ -329,8 +296,19 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
                            const int* token_list, int n_listed, hipStream_t stream) {
   KLLM_REQUIRE(q && out && part && cache && positions && span_of_token && block_table,
                "%s: null pointer", who);
-  KLLM_REQUIRE(dtype == DT_BF16, "%s: bfloat16 only (float32 uses the generic kernel)", who);
+  KLLM_REQUIRE(dtype == DT_BF16 || dtype == DT_F32, "%s: unknown dtype %d", who, dtype);
   KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && H % KV == 0, "%s: bad heads n=%d H=%d KV=%d", who, n, H, KV);
+  if (dtype == DT_F32) {
+    KLLM_REQUIRE(max_pages > 0 && window >= 0, "%s: bad table width or window", who);
+    KLLM_REQUIRE(nslices >= 1 && part_floats >= (long)n * H * nslices * (hd + 2),
+                 "%s: the partial results of n=%d H=%d nslices=%d head_dim=%d need %ld floats, the workspace has %ld",
+                 who, n, H, nslices, hd, (long)n * H * nslices * (hd + 2), part_floats);
+    KLLM_REQUIRE(H <= 65535, "%s: too many heads for the grid", who);
+    KLLM_REQUIRE(!token_list || (n_listed > 0 && n_listed <= n), "%s: bad token list", who);
+    return attn_f32_decode((const float*)q, (float*)out, part, (const float*)cache, positions, span_of_token,
+                           block_table, max_pages, page_size, H, KV, hd, window, scale, nslices, token_list,
+                           token_list ? n_listed : n, stream);
+  }
   KLLM_REQUIRE(hd % 16 == 0 && hd >= 16 && hd <= 256 && (hd <= 128 || hd == 192 || hd == 256),
                "%s: head_dim %d is not built (16..128 in steps of 16, 192, 256)", who, hd);
   KLLM_REQUIRE(page_size % 16 == 0 && page_size > 0 && max_pages > 0,

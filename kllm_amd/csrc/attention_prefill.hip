@@ -38,6 +38,7 @@
 // keys [64][hd + 8], values [hd][64 + 4] (tiles of 32 keys for head sizes above 128).
 #include <math.h>
 
+#include "attention_f32.hpp"
 #include "common.hpp"
 #include "kllm_kernels.h"
 
@@ -661,7 +662,7 @@ static void launch_prefill(int grid, hipStream_t stream, const void* q, void* ou
                            const int* span_pos, const int* block_table, int max_pages, int page_size,
                            int H, int KV, int window, float scale) {
   if constexpr (HDT >= 4) {
-    if (grid > 256 || PrefillShape<HDT>::kMaxPar == 1)
+    if (grid > device_cus() || PrefillShape<HDT>::kMaxPar == 1)
       launch_prefill_par<HDT, 1>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,
                                  block_table, max_pages, page_size, H, KV, window, scale);
     else
@@ -669,7 +670,7 @@ static void launch_prefill(int grid, hipStream_t stream, const void* q, void* ou
                                                           span_start, span_pos, block_table, max_pages, page_size,
                                                           H, KV, window, scale);
   } else {
-    if (grid > 256)
+    if (grid > device_cus())
       launch_prefill_par<HDT, 1>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,
                                  block_table, max_pages, page_size, H, KV, window, scale);
     else
@@ -688,9 +689,14 @@ extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, co
                                  int hd, int window, float scale, int dtype, hipStream_t stream) {
   KLLM_REQUIRE(q && out && cache && query_tiles && span_start && span_pos && block_table,
                "attn_prefill: null pointer");
-  KLLM_REQUIRE(dtype == DT_BF16, "attn_prefill: bfloat16 only (float32 uses the generic kernel)");
+  KLLM_REQUIRE(dtype == DT_BF16 || dtype == DT_F32, "attn_prefill: unknown dtype %d", dtype);
   KLLM_REQUIRE(n_tiles > 0 && H > 0 && KV > 0 && H % KV == 0, "attn_prefill: bad sizes tiles=%d H=%d KV=%d",
                n_tiles, H, KV);
+  if (dtype == DT_F32) {
+    KLLM_REQUIRE(max_pages > 0 && window >= 0, "attn_prefill: bad table width or window");
+    return attn_f32_prefill((const float*)q, (float*)out, (const float*)cache, query_tiles, n_tiles, span_start,
+                            span_pos, block_table, max_pages, page_size, H, KV, hd, window, scale, stream);
+  }
   KLLM_REQUIRE(hd % 32 == 0 && hd >= 32 && hd <= 256 && (hd <= 128 || hd == 192 || hd == 256),
                "attn_prefill: head_dim %d is not built (32, 64, 96, 128, 192, 256)", hd);
   KLLM_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_prefill: page_size %d must be a multiple of 16",

@@ -93,6 +93,9 @@ void set_error(const char* fmt, ...);
       KLLM_FAIL((int)e_, "%s: launch failed: %s", name, hipGetErrorString(e_));   \
   } while (0)
 
+// Compute units of the current device (cached); 256 if it cannot be asked.
+int device_cus();
+
 inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
 
 }  // namespace kllm

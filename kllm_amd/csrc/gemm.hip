@@ -5,7 +5,8 @@
 //   plain   one thread per output; any size; the yardstick the others are
 //           tested against
 //   tiled   true 32-bit FMA tiles through LDS, for the float32 engine
-//   mfma    bfloat16 MFMA 32x32x16 tiles through LDS, for prompts
+//   mfma    MFMA tiles through LDS, for prompts: bfloat16 on 32x32x16, float32 on
+//           32x32x2 (32-bit operands, products and sums: no reduced precision)
 //   skinny  bfloat16 MFMA 16x16x32, weights streamed straight from memory,
 //           for up to 64 rows of X (decode batches); K may be split
 //   gemv    one wave per weight row, up to 8 rows of X; K may be split
@@ -108,11 +109,18 @@ __global__ __launch_bounds__(256) void gemm_f32_tiled_kernel(const float* __rest
   }
 }
 
-// ------------------------------------------------------------------ bf16 MFMA tiles
-// Workgroup tile 128 (rows of X) x 128 (rows of W), 64 of K per stage, two or
-// three LDS stages.  Four waves in 2 x 2, each 2 x 2 MFMA tiles of 32 x 32.
-// MFMA 32x32x16: lane l holds A[l%32][8*(l/32)..+7], B[l%32][...] likewise, and
-// D[8*(i/4) + 4*(l/32) + i%4][l%32] in accumulator register i.
+// ------------------------------------------------------------------ MFMA tiles
+// Workgroup tile 128 (rows of X) x 128 (rows of W), 128 bytes of K per stage
+// (64 bfloat16 or 32 float32), two or three LDS stages.  Four waves in 2 x 2,
+// each 2 x 2 MFMA tiles of 32 x 32.
+// MFMA 32x32x16 (bfloat16): lane l holds A[l%32][8*(l/32)..+7], B[l%32][...]
+// likewise, and D[8*(i/4) + 4*(l/32) + i%4][l%32] in accumulator register i.
+// MFMA 32x32x2 (float32): lane l holds A[l%32][l/32] and B[l%32][l/32], D as
+// above.  Which element of K a lane's operand stands for is free as long as A
+// and B agree, so a lane reads the same 16 bytes as in bfloat16 -- four
+// consecutive floats, lanes 0..31 the first four of eight and lanes 32..63 the
+// second four -- and issues four MFMAs, one per float: the tile loads, the LDS
+// layout and the reads are the same code for both types.
 //
 // Operands go from memory to LDS directly (global_load_lds, 16 bytes per
 // lane), one or two stages ahead of the MFMAs, without passing through
@@ -138,20 +146,37 @@ __global__ __launch_bounds__(256) void gemm_f32_tiled_kernel(const float* __rest
 // Workgroups are numbered so that the eight XCDs (which take workgroups
 // round-robin, each with an L2 of its own) each get a contiguous run of tiles
 // that share rows of X.
-constexpr int MBN = 128, MBK = 64;
-constexpr int MROW = MBK * 2;                 // bytes of a tile row in LDS
+constexpr int MBN = 128;
+constexpr int MROW = 128;                     // bytes of a tile row in LDS: one stage of K
 
-__device__ __attribute__((aligned(16))) bf16_t g_zero_chunk[8];   // zero-initialised
+__device__ __attribute__((aligned(16))) unsigned char g_zero_chunk[16];   // zero-initialised
+
+template <typename T> struct MfmaOperand;
+template <> struct MfmaOperand<bf16_t> { typedef bf16x8 type; };
+template <> struct MfmaOperand<float> { typedef floatx4 type; };
+
+// One step of 32 bytes of K per row: acc += A . B^T for a 32 x 32 tile.
+__device__ __forceinline__ floatx16 mfma_tile_step(bf16x8 a, bf16x8 b, floatx16 acc) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+}
+__device__ __forceinline__ floatx16 mfma_tile_step(floatx4 a, floatx4 b, floatx16 acc) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], acc, 0, 0, 0);
+  return acc;
+}
 
 // Slot permutation of a row's eight chunks: rows of equal parity among 16 neighbours get
 // different slots, so that the 16-byte reads of 16 lanes spread over all 64 banks.
 __device__ __forceinline__ int mfma_swz(int row) { return (row >> 1) & 7; }
 
-template <typename TOUT, bool DUAL, int WR, int MSTAGES>   // WR: rows of waves (2 or 4), two waves a row
-__global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ X,
-                                                             const bf16_t* __restrict__ W,
+template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES>   // WR: rows of waves (1, 2 or 4), two waves a row
+__global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) void gemm_mfma_kernel(const T* __restrict__ X,
+                                                             const T* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
                                                              int k, int tiles_x, int tiles_y, int kslice) {
+  typedef typename MfmaOperand<T>::type op_t;   // 16 bytes of a row
+  constexpr int EPC = 16 / sizeof(T);           // elements of a 16-byte chunk
+  constexpr int MBK = MROW / sizeof(T);         // elements of K per stage
   constexpr int WTM = 2;                        // 32-row MFMA tiles per wave, each way
   constexpr int BM = 64 * WR;                   // rows of X per workgroup
   constexpr int NW = 2 * WR;                    // waves
@@ -174,24 +199,24 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
 
   // Wave w loads rows [8 XI w, 8 XI (w+1)) of the X tile and [8 WI w, 8 WI (w+1)) of the W
   // tile.  In one instruction lane l serves row l / 8 (of 8), slot l % 8.
-  const bf16_t* xsrc[XI];
-  const bf16_t* wsrc[WI];
+  const T* xsrc[XI];
+  const T* wsrc[WI];
   int xchunk[XI], wchunk[WI];
 #pragma unroll
   for (int i = 0; i < XI; ++i) {
     const int r = 8 * (XI * wave + i) + lane / 8;
-    xchunk[i] = ((lane % 8) ^ mfma_swz(r)) * 8;
+    xchunk[i] = ((lane % 8) ^ mfma_swz(r)) * EPC;
     xsrc[i] = X + min(row0 + r, (long)n - 1) * k + xchunk[i];
   }
 #pragma unroll
   for (int i = 0; i < WI; ++i) {
     const int r = 8 * (WI * wave + i) + lane / 8;             // DUAL: rows 0..63 gate, 64..127 up
-    wchunk[i] = ((lane % 8) ^ mfma_swz(r)) * 8;
+    wchunk[i] = ((lane % 8) ^ mfma_swz(r)) * EPC;
     const long col = DUAL ? col0 + r % 64 : col0 + r;
     const long wrow = min(col, (long)m - 1) + (DUAL && r >= 64 ? m : 0);
     wsrc[i] = W + wrow * k + wchunk[i];
   }
-  // blockIdx.y: a slice of K (kslice a multiple of 64); its sums go to Y[blockIdx.y]
+  // blockIdx.y: a slice of K (kslice a multiple of a stage); its sums go to Y[blockIdx.y]
   const int kbeg = blockIdx.y * kslice, kend = min(k, kbeg + kslice);
   Y += (long)blockIdx.y * n * m;
   auto issue = [&](int kt) {
@@ -199,14 +224,14 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
     const int kk = kbeg + kt * MBK;
 #pragma unroll
     for (int i = 0; i < XI; ++i) {
-      const bf16_t* src = kk + xchunk[i] < kend ? xsrc[i] + kk : g_zero_chunk;
+      const T* src = kk + xchunk[i] < kend ? xsrc[i] + kk : reinterpret_cast<const T*>(g_zero_chunk);
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(base + 8 * (XI * wave + i) * MROW),
                                        16, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < WI; ++i) {
-      const bf16_t* src = kk + wchunk[i] < kend ? wsrc[i] + kk : g_zero_chunk;
+      const T* src = kk + wchunk[i] < kend ? wsrc[i] + kk : reinterpret_cast<const T*>(g_zero_chunk);
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(base + XBYTES + 8 * (WI * wave + i) * MROW),
                                        16, 0, 0);
@@ -239,29 +264,29 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
     const unsigned char* ws = xs + XBYTES;
     // The operands of step ks + 1 are asked for before the MFMAs of step ks are issued, so
     // that LDS answers while the matrix unit works.
-    bf16x8 a[2][WTM], b[2][2];
-    auto read_step = [&](int ks, bf16x8 (&ar)[WTM], bf16x8 (&br)[2]) {
+    op_t a[2][WTM], b[2][2];
+    auto read_step = [&](int ks, op_t (&ar)[WTM], op_t (&br)[2]) {
       const int chunk = ks * 2 + lane / 32;
 #pragma unroll
       for (int i = 0; i < WTM; ++i) {
         const int r = wr * 32 * WTM + i * 32 + lane % 32;
-        ar[i] = *reinterpret_cast<const bf16x8*>(xs + r * MROW + (chunk ^ mfma_swz(r)) * 16);
+        ar[i] = *reinterpret_cast<const op_t*>(xs + r * MROW + (chunk ^ mfma_swz(r)) * 16);
       }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int r = (DUAL ? j * 64 + wc * 32 : wc * 64 + j * 32) + lane % 32;
-        br[j] = *reinterpret_cast<const bf16x8*>(ws + r * MROW + (chunk ^ mfma_swz(r)) * 16);
+        br[j] = *reinterpret_cast<const op_t*>(ws + r * MROW + (chunk ^ mfma_swz(r)) * 16);
       }
     };
     read_step(0, a[0], b[0]);
 #pragma unroll
-    for (int ks = 0; ks < MBK / 16; ++ks) {
-      if (ks + 1 < MBK / 16) read_step(ks + 1, a[(ks + 1) & 1], b[(ks + 1) & 1]);
+    for (int ks = 0; ks < MROW / 32; ++ks) {
+      if (ks + 1 < MROW / 32) read_step(ks + 1, a[(ks + 1) & 1], b[(ks + 1) & 1]);
 #pragma unroll
       for (int i = 0; i < WTM; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks & 1][i], b[ks & 1][j], acc[i][j], 0, 0, 0);
+          acc[i][j] = mfma_tile_step(a[ks & 1][i], b[ks & 1][j], acc[i][j]);
     }
   }
 
@@ -292,35 +317,40 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
     }
 }
 
-template <typename TOUT, bool DUAL, int WR, int MSTAGES>
+template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES>
 static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m, int k, int nsplit,
                             hipStream_t stream) {
+  constexpr int MBK = MROW / sizeof(T);
   const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN), ty = ceil_div(n, 64 * WR);
   const int kslice = ceil_div(ceil_div(k, nsplit), MBK) * MBK;
   const dim3 grid(ceil_div((long)tx * ty, 8) * 8, nsplit);   // padded so that every XCD gets as many
   const size_t lds = (size_t)MSTAGES * (64 * WR + MBN) * MROW;
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_mfma_kernel<TOUT, DUAL, WR, MSTAGES>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) KLLM_FAIL((int)e, "gemm mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = 1;
   }
-  hipLaunchKernelGGL((gemm_bf16_mfma_kernel<TOUT, DUAL, WR, MSTAGES>), grid, dim3(128 * WR), lds, stream,
-                     (const bf16_t*)x, (const bf16_t*)w, (TOUT*)y, n, m, k, tx, ty, kslice);
+  hipLaunchKernelGGL((gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES>), grid, dim3(128 * WR), lds, stream,
+                     (const T*)x, (const T*)w, (TOUT*)y, n, m, k, tx, ty, kslice);
   return 0;
 }
 
 // Tiles of 256 rows of X (eight waves) fetch a quarter less per flop than two tiles of 128;
-// they are taken when they still give every CU two rounds of work.
-template <typename TOUT, bool DUAL>
+// they are taken when they still give every CU two rounds of work.  The thresholds follow
+// the chip's number of CUs.
+template <typename T, typename TOUT, bool DUAL>
 static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, hipStream_t stream) {
+  const int cus = device_cus();
   const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN);
-  if ((long)ceil_div(n, 256) * tx * nsplit >= 512)
-    return launch_mfma_tile<TOUT, DUAL, 4, 2>(x, w, y, n, m, k, nsplit, stream);
+  if (sizeof(T) == 4 && n <= 64)   // a decode batch in float32: tiles of 64 rows, half the products of 128
+    return launch_mfma_tile<T, TOUT, DUAL, 1, 2>(x, w, y, n, m, k, nsplit, stream);
+  if ((long)ceil_div(n, 256) * tx * nsplit >= 2L * cus)
+    return launch_mfma_tile<T, TOUT, DUAL, 4, 2>(x, w, y, n, m, k, nsplit, stream);
   const long tiles = (long)ceil_div(n, 128) * tx * nsplit;
-  if (tiles <= 256) return launch_mfma_tile<TOUT, DUAL, 2, 3>(x, w, y, n, m, k, nsplit, stream);   // one per CU at most
-  return launch_mfma_tile<TOUT, DUAL, 2, 2>(x, w, y, n, m, k, nsplit, stream);
+  if (tiles <= cus) return launch_mfma_tile<T, TOUT, DUAL, 2, 3>(x, w, y, n, m, k, nsplit, stream);   // one per CU at most
+  return launch_mfma_tile<T, TOUT, DUAL, 2, 2>(x, w, y, n, m, k, nsplit, stream);
 }
 
 // ------------------------------------------------------------------ bf16 MFMA skinny
@@ -615,15 +645,18 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
     return 0;
   }
 
-  if (algo == KLLM_GEMM_MFMA_BF16) {
-    KLLM_REQUIRE(dtype == DT_BF16, "gemm mfma: bfloat16 only");
+  if (algo == KLLM_GEMM_MFMA_BF16 || algo == KLLM_GEMM_MFMA_F32) {
+    const bool f32 = algo == KLLM_GEMM_MFMA_F32;
+    const int stage = f32 ? MROW / 4 : MROW / 2, chunk = f32 ? 4 : 8;   // elements of K per stage, per 16 bytes
+    KLLM_REQUIRE(dtype == (f32 ? DT_F32 : DT_BF16), "gemm mfma: algorithm %d does not take dtype %d", algo, dtype);
     KLLM_REQUIRE(nsplit == 1 || out_dtype == DT_F32, "gemm mfma: K is split only for float32 partial sums");
-    KLLM_REQUIRE(nsplit <= 16 && (long)(ceil_div(ceil_div(k, nsplit), MBK) * MBK) * (nsplit - 1) < k,
+    KLLM_REQUIRE(nsplit <= 16 && (long)(ceil_div(ceil_div(k, nsplit), stage) * stage) * (nsplit - 1) < k,
                  "gemm mfma: nsplit %d leaves an empty slice of K=%d", nsplit, k);
-    KLLM_REQUIRE(k % 8 == 0 && aligned16(x) && aligned16(w),
-                 "gemm mfma: K=%d must be a multiple of 8 and the operands 16-byte aligned", k);
-    int rc = out_dtype == DT_F32 ? launch_mfma<float, false>(x, w, y, n, m, k, nsplit, stream)
-                                 : launch_mfma<bf16_t, false>(x, w, y, n, m, k, 1, stream);
+    KLLM_REQUIRE(k % chunk == 0 && aligned16(x) && aligned16(w),
+                 "gemm mfma: K=%d must be a multiple of %d and the operands 16-byte aligned", k, chunk);
+    int rc = f32 ? launch_mfma<float, float, false>(x, w, y, n, m, k, nsplit, stream)
+             : out_dtype == DT_F32 ? launch_mfma<bf16_t, float, false>(x, w, y, n, m, k, nsplit, stream)
+                                   : launch_mfma<bf16_t, bf16_t, false>(x, w, y, n, m, k, 1, stream);
     if (rc) return rc;
     KLLM_CHECK_LAUNCH("gemm mfma");
     return 0;
@@ -714,11 +747,14 @@ extern "C" int kllm_gemm_swiglu(const void* x, const void* w_gate_up, void* h, i
                                 int dtype, hipStream_t stream) {
   KLLM_REQUIRE(x && w_gate_up && h, "gemm_swiglu: null pointer");
   KLLM_REQUIRE(n > 0 && f > 0 && k > 0, "gemm_swiglu: bad sizes n=%d f=%d k=%d", n, f, k);
-  KLLM_REQUIRE(dtype == DT_BF16, "gemm_swiglu: bfloat16 only");
-  KLLM_REQUIRE(k % 8 == 0 && aligned16(x) && aligned16(w_gate_up),
-               "gemm_swiglu: K=%d must be a multiple of 8 and the operands 16-byte aligned", k);
+  KLLM_REQUIRE(dtype == DT_BF16 || dtype == DT_F32, "gemm_swiglu: unknown dtype %d", dtype);
+  const int chunk = dtype == DT_F32 ? 4 : 8;
+  KLLM_REQUIRE(k % chunk == 0 && aligned16(x) && aligned16(w_gate_up),
+               "gemm_swiglu: K=%d must be a multiple of %d and the operands 16-byte aligned", k, chunk);
   KLLM_REQUIRE((long)n * f < (1L << 31), "gemm_swiglu: sizes overflow");
-  if (int rc = launch_mfma<bf16_t, true>(x, w_gate_up, h, n, f, k, 1, stream)) return rc;
+  if (int rc = dtype == DT_F32 ? launch_mfma<float, float, true>(x, w_gate_up, h, n, f, k, 1, stream)
+                               : launch_mfma<bf16_t, bf16_t, true>(x, w_gate_up, h, n, f, k, 1, stream))
+    return rc;
   KLLM_CHECK_LAUNCH("gemm_swiglu");
   return 0;
 }

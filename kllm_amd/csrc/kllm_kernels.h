@@ -26,6 +26,7 @@ extern "C" {
 #define KLLM_GEMM_SKINNY_BF16 3
 #define KLLM_GEMM_GEMV 4
 #define KLLM_GEMM_GEMV_LDS 5 /* kllm_gemv_plain, reached through the Python wrapper */
+#define KLLM_GEMM_MFMA_F32 6 /* MFMA 32x32x2 with 32-bit operands: no reduced precision */
 
 /* Copies the calling thread's last error text; returns its length. */
 int kllm_last_error(char* buf, int len);
@@ -33,6 +34,8 @@ int kllm_last_error(char* buf, int len);
 int kllm_device_info(int device, char* buf, int len);
 /* ABI version, bumped when a signature changes. */
 int kllm_abi_version(void);
+/* Compute units of the current device (the launch heuristics scale with it). */
+int kllm_device_cus(void);
 
 /* out[t] = table[ids[t]]; with `from` (and `sampled`), token t whose from[t] >= 0 takes its id
  * from sampled[from[t]], a token id that an earlier launch left on the device. */
@@ -71,7 +74,7 @@ int kllm_sum_splits(const float* in, int nsplit, long count, void* out, int out_
 int kllm_gemm(const void* x, const void* w, void* y, int n, int m, int k, int dtype, int out_dtype,
               int algo, int nsplit, hipStream_t stream);
 
-/* h[n][f] = silu(x . w[0:f]^T) * (x . w[f:2f]^T) on the MFMA tiles, bfloat16. */
+/* h[n][f] = silu(x . w[0:f]^T) * (x . w[f:2f]^T) on the MFMA tiles, h in dtype. */
 int kllm_gemm_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f, int k, int dtype,
                      hipStream_t stream);
 
@@ -129,13 +132,15 @@ int kllm_attn_generic(const void* q, void* out, const void* cache, const int* po
                       int page_size, int n, int H, int KV, int hd, int window, float scale,
                       int dtype, hipStream_t stream);
 
-/* Decode attention on the matrix cores (bfloat16): every token's keys are cut
- * into `nslices` slices (1..256) that run side by side, four waves to a slice;
- * `part` is float32 scratch of n*H*nslices*(hd+2) elements.
+/* Decode attention on the matrix cores: every token's keys are cut into
+ * `nslices` slices (1..256) that run side by side (bfloat16: four waves to a
+ * slice, head sizes 16..128 in steps of 16, 192, 256, pages a multiple of 16;
+ * float32: one wave to a slice, 32-bit MFMA, head sizes in steps of 8, pages a
+ * multiple of 4); `part` is float32 scratch of n*H*nslices*(hd+2) elements.
  * kllm_attn_decode_slices proposes nslices for a batch.  With token_list only
  * the n_listed tokens it names are computed (q, out and part stay indexed by
  * token row). */
-int kllm_attn_decode_slices(int n, int KV, int H);
+int kllm_attn_decode_slices(int n, int KV, int H, int dtype);
 int kllm_attn_decode(const void* q, void* out, float* part, long part_floats, const void* cache,
                      const int* positions, const int* span_of_token, const int* block_table,
                      int max_pages, int page_size, int n, int H, int KV, int hd, int window,
@@ -159,8 +164,9 @@ int kllm_attn_decode_static(const void* q, void* out, const void* cache, const i
                             int nslices, int dtype, const int* token_list, int n_listed,
                             hipStream_t stream);
 
-/* Prompt attention on the matrix cores (bfloat16).  query_tiles holds
- * (first token row, span) pairs: up to 128 consecutive tokens of one span. */
+/* Prompt attention on the matrix cores (bfloat16, or float32 with 32-bit MFMA).
+ * query_tiles holds (first token row, span) pairs: up to 128 consecutive tokens
+ * of one span. */
 int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                       int n_tiles, const int* span_start, const int* span_pos,
                       const int* block_table, int max_pages, int page_size, int H, int KV, int hd,

@@ -17,7 +17,22 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
+// Compute units of the current device, asked once per device.
+int device_cus() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    cached[dev] = cus;
+  }
+  return cached[dev];
+}
+
 }  // namespace kllm
+
+extern "C" int kllm_device_cus(void) { return kllm::device_cus(); }
 
 extern "C" int kllm_last_error(char* buf, int len) {
   if (!buf || len <= 0) return 0;
@@ -26,7 +41,7 @@ extern "C" int kllm_last_error(char* buf, int len) {
   return (int)strlen(buf);
 }
 
-extern "C" int kllm_abi_version(void) { return 2; }
+extern "C" int kllm_abi_version(void) { return 3; }
 
 // Reference: te_device_info, backend/shim.cu:25-34.
 extern "C" int kllm_device_info(int device, char* buf, int len) {

@@ -17,10 +17,10 @@ from ctypes import c_char_p, c_double, c_float, c_int, c_long, c_void_p
 import torch
 
 DT_F32, DT_BF16 = 0, 1
-GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS = 0, 1, 2, 3, 4, 5
+GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
 GEMV_MAX_ROWS = 8          # what the fused kernels take
 GEMV_BEST_ROWS = 4         # up to here they beat the MFMA kernel with split K
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class KernelError(RuntimeError):
@@ -91,7 +91,8 @@ def _declare(lib):
         "kllm_fused_linear": [P, I, P, P, I, I, I, I, P],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
-        "kllm_attn_decode_slices": [I, I, I],
+        "kllm_attn_decode_slices": [I, I, I, I],
+        "kllm_device_cus": [],
         "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, P],
         "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
     }
@@ -290,7 +291,7 @@ def gemv_fits(n, m, k, dtype) -> bool:
 
 
 def gemm_swiglu(x, w_gate_up, h):
-    """h [n, f] = silu(x . gate^T) * (x . up^T) on the MFMA tiles (bfloat16, any n)."""
+    """h [n, f] = silu(x . gate^T) * (x . up^T) on the MFMA tiles (any n; float32 with 32-bit MFMA)."""
     n, k = x.shape
     f = h.shape[1]
     if tuple(w_gate_up.shape) != (2 * f, k) or h.shape[0] != n or x.dtype != w_gate_up.dtype or h.dtype != x.dtype:
@@ -454,8 +455,26 @@ def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size
 DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
 
 
-def attn_decode_slices(n, n_kv_heads, n_heads) -> int:
-    return library().kllm_attn_decode_slices(n, n_kv_heads, n_heads)
+def attn_decode_slices(n, n_kv_heads, n_heads, dtype=torch.bfloat16) -> int:
+    return library().kllm_attn_decode_slices(n, n_kv_heads, n_heads, dtype_code(dtype))
+
+
+def attn_f32_fits(head_dim, page_size) -> bool:
+    """Sizes the float32 attention on the matrix cores takes; the rest goes to
+    the generic kernel."""
+    return 8 <= head_dim <= 256 and head_dim % 8 == 0 and page_size > 0 and page_size % 4 == 0
+
+
+_cus = None
+
+
+def device_cus() -> int:
+    """Compute units of the current device; the choice of kernels and of
+    slices of K scales with it."""
+    global _cus
+    if _cus is None:
+        _cus = int(library().kllm_device_cus())
+    return _cus
 
 
 PREFILL_HEAD_DIMS = (32, 64, 96, 128, 192, 256)

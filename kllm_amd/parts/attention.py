@@ -99,14 +99,18 @@ class CausalSelfAttention(Part):
         return linear(ctx, out, self.w_o, "attn.proj")
 
     def attend(self, ctx, q, out, cache):
-        """Choose the attention kernels by dtype and by the spans' lengths:
-        in bfloat16, tokens of short spans (decode tokens) go to the kernel
-        that splits a token's keys over many waves, longer spans to the prompt
-        kernel in blocks of 128 queries; float32, and sizes those kernels do not
-        take, go to the kernel that takes every size."""
+        """Choose the attention kernels by the spans' lengths: tokens of short
+        spans (decode tokens) go to the kernel that splits a token's keys over
+        many waves, longer spans to the prompt kernel in blocks of 128 queries
+        (both on the matrix cores, in bfloat16 or with 32-bit operands); sizes
+        those kernels do not take go to the kernel that takes every size."""
         mode = self.runtime.options.get("attention", "auto")
-        fast = (mode != "generic" and q.dtype == torch.bfloat16 and cache.page_size % 16 == 0
-                and self.head_dim in K.DECODE_HEAD_DIMS)
+        if q.dtype == torch.bfloat16:
+            fast = cache.page_size % 16 == 0 and self.head_dim in K.DECODE_HEAD_DIMS
+            prompt_ok = self.head_dim in K.PREFILL_HEAD_DIMS
+        else:
+            fast = prompt_ok = K.attn_f32_fits(self.head_dim, cache.page_size)
+        fast = fast and mode != "generic"
         if not fast:
             K.attn_generic(q, out, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                            cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
@@ -114,7 +118,7 @@ class CausalSelfAttention(Part):
             return
         n = q.shape[0]
         listed = ctx.n_short + ctx.n_tiles > 0          # a context built by hand may carry no lists
-        if not listed or (ctx.n_tiles and self.head_dim not in K.PREFILL_HEAD_DIMS):
+        if not listed or (ctx.n_tiles and not prompt_ok):
             self._decode(ctx, q, out, cache, None, n)   # token by token
             return
         if ctx.n_short:
@@ -126,7 +130,7 @@ class CausalSelfAttention(Part):
 
     def _decode(self, ctx, q, out, cache, token_list, count):
         n = q.shape[0]
-        nslices = K.attn_decode_slices(count, self.kv_heads, self.heads)
+        nslices = K.attn_decode_slices(count, self.kv_heads, self.heads, q.dtype)
         part = ctx.buf("attn.part", (n * self.heads * nslices * (self.head_dim + 2),), torch.float32)
         K.attn_decode(q, out, part, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                       cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,

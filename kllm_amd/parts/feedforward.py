@@ -50,8 +50,8 @@ class GatedFeedForward(Part):
               and K.fused_linear_fits(n, self.hidden)
               and not self.runtime.options.get("no_fused_linear")):
             K.fused_linear(self.w_gu, h, K.LINEAR_SWIGLU, x=xn)    # a decode batch: the same on the matrix cores
-        elif (n > 128 and xn.dtype == torch.bfloat16 and self.hidden % 8 == 0
-              and self.runtime.options.get("gemm") != "library"):
+        elif (n > 128 and self.runtime.options.get("gemm") != "library"
+              and self.hidden % (8 if xn.dtype == torch.bfloat16 else 4) == 0):
             # prompts: the gate in the product's epilogue (up to 128 rows the product with K
             # in slices and a separate gate is faster: the epilogue cannot split K)
             K.gemm_swiglu(xn, self.w_gu, h)

@@ -9,7 +9,9 @@ rotary + append, SiLU gate); with the compute dtype as result it returns
             partial sums), if the sizes fit; bfloat16 up to 4 rows: the streaming
             gemv, K cut into slices for long rows (measured faster than the
             former for a plain product; the fused epilogues are another matter)
-  float32   else: tiled FMA (true 32-bit)
+  float32   else: MFMA tiles with 32-bit operands (true 32-bit; K in slices for
+            few rows, where one wave's chain of products bounds the time), or
+            tiled FMA where K is no multiple of 4
   bfloat16  n <= 64: MFMA skinny (n <= 16 and one float32 result wanted: the
             decode-batch kernel with all of K in a workgroup)
             else: MFMA tiles (K in slices where the tiles alone do not fill the chip),
@@ -44,7 +46,7 @@ def _skinny_split(n, m, k):
     further slice writes (measured up to 64 rows)."""
     nsplit = -(-k // 512)
     wgs = -(-m // 64)
-    while wgs * nsplit < 256 and k // (nsplit * 2) >= 128:
+    while wgs * nsplit < K.device_cus() and k // (nsplit * 2) >= 128:
         nsplit *= 2
     while (-(-(-(-k // nsplit)) // 32) * 32) * (nsplit - 1) >= k:   # no empty slice
         nsplit -= 1
@@ -61,11 +63,26 @@ def _mfma_split(n, m, k):
     instead of 68 us with two slices, the second sum's traffic included)."""
     tiles = -(-n // 128) * -(-m // 128)
     nsplit = 1
-    while nsplit * 2 <= min(8, 512 // tiles, k // 256):
+    while nsplit * 2 <= min(8, 2 * K.device_cus() // tiles, k // 256):
         nsplit *= 2
     while nsplit > 1 and (-(-(-(-k // nsplit)) // 64) * 64) * (nsplit - 1) >= k:   # no empty slice
         nsplit -= 1
     return nsplit
+
+
+def _mfma_f32_split(n, m, k):
+    """Slices of K for the float32 MFMA kernel.  With 32-bit operands a wave's
+    own chain of products bounds the time (64 cycles for 32 x 32 x 2), not the
+    loads, so a product should give every SIMD a wave or two: up to 16 slices
+    of at least 128 of K."""
+    if n <= 64:
+        waves = -(-m // 128) * 2                      # tiles of 64 rows, two waves
+    else:
+        waves = -(-n // 128) * -(-m // 128) * 4
+    nsplit = max(1, min(16, k // 128, -(-4 * K.device_cus() // waves)))
+    while nsplit > 1 and (-(-(-(-k // nsplit)) // 32) * 32) * (nsplit - 1) >= k:   # no empty slice
+        nsplit -= 1
+    return int(nsplit)
 
 
 def choose(dtype, n, m, k, options=None):
@@ -79,6 +96,8 @@ def choose(dtype, n, m, k, options=None):
     if n <= 4 or (n <= 8 and dtype == torch.float32):
         return K.GEMM_GEMV, _gemv_split(dtype, n, m, k)
     if dtype == torch.float32:
+        if k % 4 == 0 and not options.get("no_mfma_f32"):
+            return K.GEMM_MFMA_F32, _mfma_f32_split(n, m, k)
         return K.GEMM_TILED_F32, 1
     if k % 8 != 0:
         return (K.GEMM_GEMV, 1) if n <= 8 else (K.GEMM_PLAIN, 1)
@@ -113,7 +132,8 @@ def linear(ctx, x, w, tag, out_dtype=torch.float32, split=True):
             y32[0].copy_(y)
             return y32[0] if whole else y32
         return y
-    if algo == K.GEMM_MFMA_BF16 or algo == K.GEMM_PLAIN:      # write either dtype themselves
+    if (algo == K.GEMM_MFMA_BF16 or algo == K.GEMM_PLAIN
+            or (algo == K.GEMM_MFMA_F32 and (nsplit == 1 or not whole))):   # write either dtype themselves
         if whole:
             y = ctx.buf(tag, (n, m), out_dtype)
             K.gemm(x, w, y, algo, 1)

@@ -201,6 +201,12 @@ def test_gemm_kernels_against_plain(n, m, k, dtype):
     algos = [(k_.GEMM_PLAIN, 1)]
     if dtype == torch.float32:
         algos.append((k_.GEMM_TILED_F32, 1))
+        if k % 4 == 0:
+            algos.append((k_.GEMM_MFMA_F32, 1))
+            if k >= 64:
+                algos += [(k_.GEMM_MFMA_F32, 2)] + ([(k_.GEMM_MFMA_F32, 3)] if k >= 100 else [])
+            if k >= 2048 and (-(-(-(-k // 16)) // 32) * 32) * 15 < k:     # 16 slices, none empty
+                algos.append((k_.GEMM_MFMA_F32, 16))
     elif k % 8 == 0:
         algos.append((k_.GEMM_MFMA_BF16, 1))
         if k >= 128:
@@ -241,17 +247,20 @@ def _gpu_reference(x, w):
     (4096, 4096, 4096, 1),
     (2048, 32000, 2048, 1),     # the logits of a whole prompt
 ])
-@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-def test_gemm_mfma_at_prompt_sizes(n, m, k, nsplit, out_dtype):
+@pytest.mark.parametrize("dtype,out_dtype", [(torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                             (torch.float32, torch.float32)])
+def test_gemm_mfma_at_prompt_sizes(n, m, k, nsplit, dtype, out_dtype):
     """The tile variants that only products of prompt size reach (256-row tiles with eight
-    waves; two stages when there are more tiles than CUs), whole and in slices of K."""
+    waves; two stages when there are more tiles than CUs), whole and in slices of K, with
+    bfloat16 and with 32-bit operands."""
     if out_dtype == torch.bfloat16 and nsplit > 1:
         pytest.skip("K is split only for float32 partial sums")
     k_ = K()
-    x, w = rnd(n, k, seed=1, dtype=torch.bfloat16), rnd(m, k, seed=2, dtype=torch.bfloat16)
+    x, w = rnd(n, k, seed=1, dtype=dtype), rnd(m, k, seed=2, dtype=dtype)
     want = _gpu_reference(x, w)
     y = torch.full((nsplit, n, m), float("nan"), dtype=out_dtype, device=DEV)
-    k_.gemm(x, w, y if nsplit > 1 or out_dtype == torch.float32 else y[0], k_.GEMM_MFMA_BF16, nsplit)
+    algo = k_.GEMM_MFMA_BF16 if dtype == torch.bfloat16 else k_.GEMM_MFMA_F32
+    k_.gemm(x, w, y if nsplit > 1 or out_dtype == torch.float32 else y[0], algo, nsplit)
     err = (y.double().sum(0) - want).abs().max()
     if out_dtype == torch.float32:
         assert err < 1e-5 * k ** 0.5 * 8, float(err)
@@ -263,15 +272,16 @@ def test_gemm_mfma_at_prompt_sizes(n, m, k, nsplit, out_dtype):
         (1e-3 if out_dtype == torch.float32 else 0.01 * float(want.abs().max()))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("n,f,k", [(2048, 5632, 2048), (1000, 2500, 2056), (2048, 14336, 4096), (300, 5632, 2048)])
-def test_gemm_swiglu_at_prompt_sizes(n, f, k):
-    dtype = torch.bfloat16
+def test_gemm_swiglu_at_prompt_sizes(n, f, k, dtype):
     x, w = rnd(n, k, seed=1, dtype=dtype, scale=0.5), rnd(2 * f, k, seed=2, dtype=dtype, scale=0.05)
     h = torch.full((n, f), float("nan"), dtype=dtype, device=DEV)
     K().gemm_swiglu(x, w, h)
     g, u = _gpu_reference(x, w[:f]), _gpu_reference(x, w[f:])
     want = P.silu(g) * u
-    assert (h.double() - want).abs().max() < 0.01 * want.abs().max() + 1e-3
+    assert (h.double() - want).abs().max() < (0.01 * want.abs().max() + 1e-3 if dtype == torch.bfloat16
+                                              else 1e-5 * want.abs().max() + 1e-5)
 
 
 @pytest.mark.parametrize("n", [5, 8, 16, 33, 64])
@@ -311,15 +321,16 @@ def test_gemv_swiglu(dtype, n, f, k):
     assert (h.cpu().double() - want).abs().max() < (1e-4 if dtype == torch.float32 else 0.01 * want.abs().max() + 1e-3)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("n,f,k", [(65, 176, 64), (130, 120, 88), (300, 515, 264), (128, 5632, 2048)])
-def test_gemm_swiglu(n, f, k):
-    dtype = torch.bfloat16
+def test_gemm_swiglu(n, f, k, dtype):
     x, w = rnd(n, k, seed=1, dtype=dtype, scale=0.5), rnd(2 * f, k, seed=2, dtype=dtype, scale=0.1)
     h = torch.full((n, f), float("nan"), dtype=dtype, device=DEV)
     K().gemm_swiglu(x, w, h)
     xd, wd = x.cpu().double(), w.cpu().double()
     want = P.silu(P.linear(xd, wd[:f])) * P.linear(xd, wd[f:])
-    assert (h.cpu().double() - want).abs().max() < 0.01 * want.abs().max() + 1e-3
+    assert (h.cpu().double() - want).abs().max() < (1e-5 * want.abs().max() + 1e-5 if dtype == torch.float32
+                                                    else 0.01 * want.abs().max() + 1e-3)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -497,7 +508,12 @@ def test_linear_chooses_a_kernel_for_every_size():
     assert choose(torch.bfloat16, 1, 2048, 5632) == (k_.GEMM_GEMV, 3)
     assert choose(torch.float32, 8, 2560, 2048) == (k_.GEMM_GEMV_LDS, 1)
     assert choose(torch.bfloat16, 8, 2560, 2048) == (k_.GEMM_SKINNY_BF16, 8)
-    assert choose(torch.float32, 100, 64, 64)[0] == k_.GEMM_TILED_F32
+    assert choose(torch.float32, 100, 64, 64) == (k_.GEMM_MFMA_F32, 1)
+    assert choose(torch.float32, 100, 64, 66)[0] == k_.GEMM_TILED_F32        # K not a multiple of 4
+    assert choose(torch.float32, 64, 2048, 5632) == (k_.GEMM_MFMA_F32, 16)   # few rows: many slices of K
+    for n, m, k in [(9, 100, 72), (64, 2048, 5632), (300, 257, 520), (70, 64, 4104), (2048, 2048, 5632)]:
+        ns = choose(torch.float32, n, m, k)[1]
+        assert 1 <= ns <= 16 and (-(-(-(-k // ns)) // 32) * 32) * (ns - 1) < k, (n, m, k, ns)
     assert choose(torch.bfloat16, 40, 64, 64)[0] == k_.GEMM_SKINNY_BF16
     assert choose(torch.bfloat16, 40, 64, 60)[0] == k_.GEMM_PLAIN          # K not a multiple of 8
     assert choose(torch.bfloat16, 64, 2048, 5632) == (k_.GEMM_SKINNY_BF16, 11)
@@ -588,14 +604,18 @@ def run_attention(kernel, q, cache, pos, sot, bt, ps, H, KV, hd, window, scale, 
         K().attn_generic(q, out, cache, pos, sot, bt, ps, H, KV, hd, window, scale)
     else:
         n = q.shape[0]
-        ns = nslices or K().attn_decode_slices(n, KV, H)
+        ns = nslices or K().attn_decode_slices(n, KV, H, q.dtype)
         part = torch.full((n * H * ns * (hd + 2),), float("nan"), device=DEV)
         K().attn_decode(q, out, part, cache, pos, sot, bt, ps, H, KV, hd, window, scale, ns)
     return out
 
 
 def kernels_for(dtype):
-    return ["generic", "decode"] if dtype == torch.bfloat16 else ["generic"]
+    return ["generic", "decode"]
+
+
+def attn_tol(dtype):
+    return 2e-5 if dtype == torch.float32 else 2e-2
 
 
 ATTN_SHAPES = [(4, 2, 16, 16), (3, 1, 32, 16), (5, 5, 48, 16), (8, 2, 64, 16), (6, 3, 80, 32),
@@ -620,15 +640,16 @@ def test_attention_generic(H, KV, hd, ps, dtype, window):
                                         (2, 1, 128, 16), (2, 2, 192, 16), (2, 1, 256, 16), (32, 4, 64, 16),
                                         (4, 2, 64, 48), (2, 1, 128, 48), (2, 2, 192, 80)])
 @pytest.mark.parametrize("window", [0, 37, 200])
-def test_attention_prefill(H, KV, hd, ps, window):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_attention_prefill(H, KV, hd, ps, window, dtype):
     """Whole prompts of ragged lengths, portions behind cached keys that start
     and end inside pages and query tiles, and a one-token span, in one launch."""
-    c = attention_case(H, KV, hd, ps, torch.bfloat16, window,
+    c = attention_case(H, KV, hd, ps, dtype, window,
                        [(0, 45), (300, 9), (0, 100), (37, 70), (5, 1), (16, 32), (31, 33)], seed=5)
     out, rows = run_prefill(c)
     assert rows.all() and torch.isfinite(out).all()
     err = (out.cpu().double() - c["want"]).abs().max()
-    assert err < 2e-2, float(err)
+    assert err < attn_tol(dtype), float(err)
     # only the listed spans are touched
     out2, rows2 = run_prefill(c, min_len=33)
     assert torch.isnan(out2.cpu()[~rows2]).all() and torch.equal(out2.cpu()[rows2], out.cpu()[rows2])
@@ -637,18 +658,37 @@ def test_attention_prefill(H, KV, hd, ps, window):
 @pytest.mark.parametrize("H,KV,hd,ps", [(24, 4, 32, 16), (24, 3, 64, 16), (22, 2, 96, 32), (22, 11, 128, 16),
                                         (24, 6, 64, 48)])
 @pytest.mark.parametrize("window", [0, 150])
-def test_attention_prefill_many_blocks(H, KV, hd, ps, window):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_attention_prefill_many_blocks(H, KV, hd, ps, window, dtype):
     """More query blocks than CUs: the kernel that passes the keys through LDS,
     with blocks of 128 queries that end inside a tile, long chains of tiles,
     portions behind cached keys, and a window that ends inside a block."""
     spans = [(0, 300), (500, 260), (100, 129), (37, 70), (5, 1), (16, 32), (31, 33)]
-    c = attention_case(H, KV, hd, ps, torch.bfloat16, window, spans, seed=6)
+    c = attention_case(H, KV, hd, ps, dtype, window, spans, seed=6)
     blocks = sum(-(-b // K().PREFILL_QUERY_BLOCK) for _, b in spans)
     assert blocks * H > 256
     out, rows = run_prefill(c)
     assert rows.all() and torch.isfinite(out).all()
     err = (out.cpu().double() - c["want"]).abs().max()
-    assert err < 2e-2, float(err)
+    assert err < attn_tol(dtype), float(err)
+
+
+@pytest.mark.parametrize("H,KV,hd,ps", [(5, 5, 48, 16), (6, 3, 80, 32), (3, 1, 40, 12), (2, 1, 8, 4), (2, 2, 136, 20),
+                                        (70, 2, 16, 16)])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_float32_takes_head_sizes_in_steps_of_8(H, KV, hd, ps, window):
+    """Head sizes that are no multiple of 32, pages that are no multiple of 16 and more than
+    32 heads to a KV head, on the prompt and on the decode path of the float32 kernel."""
+    spans = [(0, 45), (300, 9), (0, 100), (37, 70), (5, 1), (16, 32), (31, 33), (ps * 3, 1), (ps * 2 - 1, 1), (0, 1)]
+    c = attention_case(H, KV, hd, ps, torch.float32, window, spans, seed=8)
+    out, rows = run_prefill(c)
+    assert rows.all() and torch.isfinite(out).all()
+    assert (out.cpu().double() - c["want"]).abs().max() < 2e-5
+    for nslices in (None, 1, 5):
+        out = run_attention("decode", c["q"], c["cache"], c["pos"], c["sot"], c["bt"], ps, H, KV, hd, window,
+                            c["scale"], nslices)
+        assert torch.isfinite(out).all()
+        assert (out.cpu().double() - c["want"]).abs().max() < 2e-5, nslices
 
 
 def test_attention_prefill_refuses_what_it_does_not_take():
@@ -660,13 +700,14 @@ def test_attention_prefill_refuses_what_it_does_not_take():
 
 @pytest.mark.parametrize("H,KV,hd,ps", [(40, 2, 32, 16), (17, 1, 64, 16), (12, 4, 192, 16), (8, 8, 112, 48)])
 @pytest.mark.parametrize("nslices", [4, 8, 64])
-def test_attention_decode_many_heads_and_slices(H, KV, hd, ps, nslices):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_attention_decode_many_heads_and_slices(H, KV, hd, ps, nslices, dtype):
     """More than 16 query heads per KV head (several head tiles), odd groups,
     more slices than there are keys."""
-    c = attention_case(H, KV, hd, ps, torch.bfloat16, 0, [(700, 1), (ps - 1, 1), (0, 1), (33, 2)], seed=3)
+    c = attention_case(H, KV, hd, ps, dtype, 0, [(700, 1), (ps - 1, 1), (0, 1), (33, 2)], seed=3)
     out = run_attention("decode", c["q"], c["cache"], c["pos"], c["sot"], c["bt"], ps, H, KV, hd, 0, c["scale"], nslices)
     assert torch.isfinite(out).all()
-    assert (out.cpu().double() - c["want"]).abs().max() < 2e-2
+    assert (out.cpu().double() - c["want"]).abs().max() < attn_tol(dtype)
 
 
 def standout_case(H, KV, hd, key_pos, ctx_len):

@@ -38,6 +38,17 @@ class GroupSpec:
     window: int = 0  # 0: all keys are kept
 
 
+def window_pages(n_tokens: int, step_tokens: int, page_size: int, window: int) -> int:
+    """Most pages a request of up to n_tokens holds in a group: all of its
+    pages without a window; with one, the pages from the first key that the
+    oldest token still to come may read to the end of the step being reserved:
+    at most ceil((step + window - 1) / page_size) + 1."""
+    whole = -(-n_tokens // page_size)
+    if window <= 0:
+        return whole
+    return min(whole, -(-(step_tokens + window - 1) // page_size) + 1)
+
+
 @dataclass
 class RequestCache:
     request_id: Hashable
@@ -98,13 +109,13 @@ class CacheManager:
         need = self.pages_needed(request_id, n_tokens)
         return all(n <= p.free_pages for n, p in zip(need, self.pools))
 
-    def pages_for_tokens(self, n_tokens: int) -> List[int]:
-        """Pages per group that a fresh request of n_tokens holds at most at
-        one time (a windowed group never holds more than its window spans)."""
-        out = []
-        for grp in self.groups:
-            out.append(-(-n_tokens // grp.page_size))
-        return out
+    def pages_for_tokens(self, n_tokens: int, step_tokens: Optional[int] = None) -> List[int]:
+        """Pages per group that a request growing to n_tokens holds at most at
+        one time, when no step brings it more than ``step_tokens`` tokens
+        (default: all of them at once).  A windowed group never holds more
+        than its window and one step's tokens span."""
+        step = n_tokens if step_tokens is None else max(1, min(int(step_tokens), n_tokens))
+        return [window_pages(n_tokens, step, grp.page_size, grp.window) for grp in self.groups]
 
     # ------------------------------------------------------------ protocol
     def reserve(self, request_id: Hashable, n_tokens: int) -> None:

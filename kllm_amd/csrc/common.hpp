@@ -28,6 +28,19 @@ template <> __device__ __forceinline__ float from_f32<float>(float v) { return v
 // float -> bfloat16 rounds to nearest even (the hardware conversion of gfx950).
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }
 
+// The gate's activation of a gated feed-forward, the value of the `act` argument of the
+// entry points that apply one.  Another activation is another value here and another case
+// in gate_act; every kernel with a gate in its epilogue calls this one function.
+enum : int { ACT_SILU = 0, ACT_GELU_TANH = 1, ACT_COUNT = 2 };
+
+__device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == ACT_GELU_TANH) {   // 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
+    const float u = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return 0.5f * g * (1.f + tanhf(u));
+  }
+  return g / (1.f + expf(-g));  // SiLU (reference: backend/model.cu:477-483)
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);

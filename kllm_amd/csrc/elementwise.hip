@@ -279,11 +279,11 @@ __global__ void rope_append_vec_kernel(const float* __restrict__ qkv, T* __restr
   }
 }
 
-// out[t, i] = silu(gate[t, i]) * up[t, i], gate = cols [0, f), up = cols [f, 2f)
+// out[t, i] = act(gate[t, i]) * up[t, i], gate = cols [0, f), up = cols [f, 2f)
 // (reference: backend/model.cu:477-483)
 template <typename TIN, typename TOUT>
 __global__ void silu_mul_kernel(const TIN* __restrict__ gu, int nsplit, long split_stride,
-                                TOUT* __restrict__ out, long n, int f) {
+                                TOUT* __restrict__ out, long n, int f, int act) {
   const long total = n * f;
   for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (long)gridDim.x * blockDim.x) {
@@ -292,7 +292,7 @@ __global__ void silu_mul_kernel(const TIN* __restrict__ gu, int nsplit, long spl
     const TIN* row = gu + t * 2 * f;
     const float g = sum_splits(row + i, nsplit, split_stride);
     const float u = sum_splits(row + f + i, nsplit, split_stride);
-    out[idx] = from_f32<TOUT>((g / (1.f + expf(-g))) * u);
+    out[idx] = from_f32<TOUT>(gate_act(g, act) * u);
   }
 }
 
@@ -453,8 +453,9 @@ extern "C" int kllm_rope_append(const void* qkv, int in_dtype, int nsplit, long 
 }
 
 extern "C" int kllm_silu_mul(const void* gu, int in_dtype, int nsplit, long split_stride, void* out,
-                             int out_dtype, int n, int f, hipStream_t stream) {
+                             int out_dtype, int n, int f, int act, hipStream_t stream) {
   KLLM_REQUIRE(gu && out, "silu_mul: null pointer");
+  KLLM_REQUIRE(act >= 0 && act < ACT_COUNT, "silu_mul: unknown activation %d", act);
   KLLM_REQUIRE(n > 0 && f > 0 && nsplit >= 1, "silu_mul: bad sizes n=%d f=%d nsplit=%d", n, f,
                nsplit);
   const long total = (long)n * f;
@@ -462,7 +463,7 @@ extern "C" int kllm_silu_mul(const void* gu, int in_dtype, int nsplit, long spli
   if (grid > 8192) grid = 8192;
 #define KLLM_SM(TIN, TOUT)                                                                      \
   hipLaunchKernelGGL((silu_mul_kernel<TIN, TOUT>), dim3(grid), dim3(kThreads), 0, stream,       \
-                     (const TIN*)gu, nsplit, split_stride, (TOUT*)out, (long)n, f)
+                     (const TIN*)gu, nsplit, split_stride, (TOUT*)out, (long)n, f, act)
   if (in_dtype == DT_F32 && out_dtype == DT_F32) KLLM_SM(float, float);
   else if (in_dtype == DT_F32 && out_dtype == DT_BF16) KLLM_SM(float, bf16_t);
   else if (in_dtype == DT_BF16 && out_dtype == DT_BF16) KLLM_SM(bf16_t, bf16_t);

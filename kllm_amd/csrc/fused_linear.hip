@@ -47,6 +47,7 @@ struct FlOut {
   const int* span_of_token;
   const int* block_table;
   int max_pages, page_size, H, KV, hd;
+  int act;                      // the gate's activation (FL_SWIGLU)
 };
 
 // Row of W behind MFMA row c of a tile, or -1.  Pair epilogues: unit = pair.
@@ -286,7 +287,7 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
         if (pair >= pairs || xr >= n) continue;
         if (EP == FL_SWIGLU) {
           bf16_t* h = reinterpret_cast<bf16_t*>(out.y);
-          h[(long)xr * pairs + pair] = from_f32<bf16_t>((a / (1.f + expf(-a))) * b);
+          h[(long)xr * pairs + pair] = from_f32<bf16_t>(gate_act(a, out.act) * b);
         } else {
           const int half = out.hd / 2;
           const int q_pairs = out.H * half, k_pairs = out.cache ? out.KV * half : 0;
@@ -386,6 +387,8 @@ extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOu
 
   FlOut out = {};
   out.y = yout->y;
+  out.act = yout->act;
+  KLLM_REQUIRE(ep != FL_SWIGLU || (out.act >= 0 && out.act < ACT_COUNT), "fused_linear: unknown activation %d", out.act);
   int tiles = ceil_div(m, 16);
   if (ep == FL_SWIGLU || ep == FL_ROPE) {
     KLLM_REQUIRE(m % 2 == 0, "fused_linear: m=%d must be even for a pair epilogue", m);

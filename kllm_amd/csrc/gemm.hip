@@ -139,7 +139,7 @@ __global__ __launch_bounds__(256) void gemm_f32_tiled_kernel(const float* __rest
 // every CU gets at most one tile.
 //
 // DUAL: W is [gate rows; up rows] = [2m, k]; a workgroup takes 64 gate rows and
-// the 64 up rows that belong to them, and writes silu(gate) * up for m columns
+// the 64 up rows that belong to them, and writes act(gate) * up for m columns
 // (reference: backend/model.cu:477-483, :1112-1114) -- the gated activation
 // never exists in 32-bit in memory.
 //
@@ -173,7 +173,7 @@ template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES>   // WR: ro
 __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) void gemm_mfma_kernel(const T* __restrict__ X,
                                                              const T* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
-                                                             int k, int tiles_x, int tiles_y, int kslice) {
+                                                             int k, int tiles_x, int tiles_y, int kslice, int act) {
   typedef typename MfmaOperand<T>::type op_t;   // 16 bytes of a row
   constexpr int EPC = 16 / sizeof(T);           // elements of a 16-byte chunk
   constexpr int MBK = MROW / sizeof(T);         // elements of K per stage
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
       for (int e = 0; e < 16; ++e) {
         const long r = row0 + wr * 32 * WTM + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
         const float gate = acc[i][0][e], up = acc[i][1][e];
-        if (r < n) Y[r * m + c] = from_f32<TOUT>((gate / (1.f + expf(-gate))) * up);
+        if (r < n) Y[r * m + c] = from_f32<TOUT>(gate_act(gate, act) * up);
       }
     return;
   }
@@ -318,7 +318,7 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
 }
 
 template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES>
-static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m, int k, int nsplit,
+static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, int act,
                             hipStream_t stream) {
   constexpr int MBK = MROW / sizeof(T);
   const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN), ty = ceil_div(n, 64 * WR);
@@ -333,7 +333,7 @@ static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m,
     raised = 1;
   }
   hipLaunchKernelGGL((gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES>), grid, dim3(128 * WR), lds, stream,
-                     (const T*)x, (const T*)w, (TOUT*)y, n, m, k, tx, ty, kslice);
+                     (const T*)x, (const T*)w, (TOUT*)y, n, m, k, tx, ty, kslice, act);
   return 0;
 }
 
@@ -341,16 +341,17 @@ static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m,
 // they are taken when they still give every CU two rounds of work.  The thresholds follow
 // the chip's number of CUs.
 template <typename T, typename TOUT, bool DUAL>
-static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, hipStream_t stream) {
+static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, int act,
+                       hipStream_t stream) {
   const int cus = device_cus();
   const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN);
   if (sizeof(T) == 4 && n <= 64)   // a decode batch in float32: tiles of 64 rows, half the products of 128
-    return launch_mfma_tile<T, TOUT, DUAL, 1, 2>(x, w, y, n, m, k, nsplit, stream);
+    return launch_mfma_tile<T, TOUT, DUAL, 1, 2>(x, w, y, n, m, k, nsplit, act, stream);
   if ((long)ceil_div(n, 256) * tx * nsplit >= 2L * cus)
-    return launch_mfma_tile<T, TOUT, DUAL, 4, 2>(x, w, y, n, m, k, nsplit, stream);
+    return launch_mfma_tile<T, TOUT, DUAL, 4, 2>(x, w, y, n, m, k, nsplit, act, stream);
   const long tiles = (long)ceil_div(n, 128) * tx * nsplit;
-  if (tiles <= cus) return launch_mfma_tile<T, TOUT, DUAL, 2, 3>(x, w, y, n, m, k, nsplit, stream);   // one per CU at most
-  return launch_mfma_tile<T, TOUT, DUAL, 2, 2>(x, w, y, n, m, k, nsplit, stream);
+  if (tiles <= cus) return launch_mfma_tile<T, TOUT, DUAL, 2, 3>(x, w, y, n, m, k, nsplit, act, stream);   // one per CU at most
+  return launch_mfma_tile<T, TOUT, DUAL, 2, 2>(x, w, y, n, m, k, nsplit, act, stream);
 }
 
 // ------------------------------------------------------------------ bf16 MFMA skinny
@@ -654,9 +655,9 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
                  "gemm mfma: nsplit %d leaves an empty slice of K=%d", nsplit, k);
     KLLM_REQUIRE(k % chunk == 0 && aligned16(x) && aligned16(w),
                  "gemm mfma: K=%d must be a multiple of %d and the operands 16-byte aligned", k, chunk);
-    int rc = f32 ? launch_mfma<float, float, false>(x, w, y, n, m, k, nsplit, stream)
-             : out_dtype == DT_F32 ? launch_mfma<bf16_t, float, false>(x, w, y, n, m, k, nsplit, stream)
-                                   : launch_mfma<bf16_t, bf16_t, false>(x, w, y, n, m, k, 1, stream);
+    int rc = f32 ? launch_mfma<float, float, false>(x, w, y, n, m, k, nsplit, 0, stream)
+             : out_dtype == DT_F32 ? launch_mfma<bf16_t, float, false>(x, w, y, n, m, k, nsplit, 0, stream)
+                                   : launch_mfma<bf16_t, bf16_t, false>(x, w, y, n, m, k, 1, 0, stream);
     if (rc) return rc;
     KLLM_CHECK_LAUNCH("gemm mfma");
     return 0;
@@ -744,16 +745,17 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
 }
 
 extern "C" int kllm_gemm_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f, int k,
-                                int dtype, hipStream_t stream) {
+                                int dtype, int act, hipStream_t stream) {
   KLLM_REQUIRE(x && w_gate_up && h, "gemm_swiglu: null pointer");
+  KLLM_REQUIRE(act >= 0 && act < ACT_COUNT, "gemm_swiglu: unknown activation %d", act);
   KLLM_REQUIRE(n > 0 && f > 0 && k > 0, "gemm_swiglu: bad sizes n=%d f=%d k=%d", n, f, k);
   KLLM_REQUIRE(dtype == DT_BF16 || dtype == DT_F32, "gemm_swiglu: unknown dtype %d", dtype);
   const int chunk = dtype == DT_F32 ? 4 : 8;
   KLLM_REQUIRE(k % chunk == 0 && aligned16(x) && aligned16(w_gate_up),
                "gemm_swiglu: K=%d must be a multiple of %d and the operands 16-byte aligned", k, chunk);
   KLLM_REQUIRE((long)n * f < (1L << 31), "gemm_swiglu: sizes overflow");
-  if (int rc = dtype == DT_F32 ? launch_mfma<float, float, true>(x, w_gate_up, h, n, f, k, 1, stream)
-                               : launch_mfma<bf16_t, bf16_t, true>(x, w_gate_up, h, n, f, k, 1, stream))
+  if (int rc = dtype == DT_F32 ? launch_mfma<float, float, true>(x, w_gate_up, h, n, f, k, 1, act, stream)
+                               : launch_mfma<bf16_t, bf16_t, true>(x, w_gate_up, h, n, f, k, 1, act, stream))
     return rc;
   KLLM_CHECK_LAUNCH("gemm_swiglu");
   return 0;

@@ -38,6 +38,7 @@ struct GvRope {
   const int* span_of_token;
   const int* block_table;
   int max_pages, page_size, H, KV, hd;
+  int act;                      // the gate's activation (GV_SWIGLU)
 };
 
 template <typename T, int NT, int MODE>
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(64 * GV_WAVES) void gemv_fused_kernel(
     y[(long)t * m + row_b] = mine_b;
   } else if (MODE == GV_SWIGLU) {
     T* h = reinterpret_cast<T*>(Y);
-    h[(long)t * f + pair] = from_f32<T>((mine_a / (1.f + expf(-mine_a))) * mine_b);
+    h[(long)t * f + pair] = from_f32<T>(gate_act(mine_a, rp.act) * mine_b);
   } else {
     const int half = rp.hd / 2;
     int page = 0, slot = 0;
@@ -260,9 +261,11 @@ extern "C" int kllm_gemv_plain(const void* x, const void* w, float* y, int n, in
 }
 
 extern "C" int kllm_gemv_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f, int k,
-                                int dtype, hipStream_t stream) {
+                                int dtype, int act, hipStream_t stream) {
   if (int rc = check_common("gemv_swiglu", x, w_gate_up, h, n, 2 * f, k, dtype)) return rc;
+  KLLM_REQUIRE(act >= 0 && act < ACT_COUNT, "gemv_swiglu: unknown activation %d", act);
   GvRope rp = {};
+  rp.act = act;
   if (dtype == DT_F32) launch_gv<float, GV_SWIGLU>(x, w_gate_up, h, n, 2 * f, k, f, rp, stream);
   else launch_gv<bf16_t, GV_SWIGLU>(x, w_gate_up, h, n, 2 * f, k, f, rp, stream);
   KLLM_CHECK_LAUNCH("gemv_swiglu");
@@ -282,7 +285,7 @@ extern "C" int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_o
     KLLM_REQUIRE(KV > 0 && positions && span_of_token && block_table && max_pages > 0 && page_size > 0,
                  "gemv_rope_append: bad cache arguments");
   GvRope rp = {q_out, cos_t, sin_t, cache, positions, span_of_token, block_table,
-               max_pages, page_size, H, KV, hd};
+               max_pages, page_size, H, KV, hd, 0};
   if (dtype == DT_F32) launch_gv<float, GV_ROPE>(x, w_qkv, q_out, n, m, k, 0, rp, stream);
   else launch_gv<bf16_t, GV_ROPE>(x, w_qkv, q_out, n, m, k, 0, rp, stream);
   KLLM_CHECK_LAUNCH("gemv_rope_append");

@@ -62,9 +62,13 @@ int kllm_rope_append(const void* qkv, int in_dtype, int nsplit, long split_strid
                      const int* span_of_token, const int* block_table, int max_pages,
                      int page_size, int n, int H, int KV, int hd, int dtype, hipStream_t stream);
 
-/* out[n][f] = silu(gu[:, :f]) * gu[:, f:], gu = [nsplit][n][2f]. */
+/* The gate's activation of a gated feed-forward (`act` below). */
+#define KLLM_ACT_SILU 0
+#define KLLM_ACT_GELU_TANH 1
+
+/* out[n][f] = act(gu[:, :f]) * gu[:, f:], gu = [nsplit][n][2f]. */
 int kllm_silu_mul(const void* gu, int in_dtype, int nsplit, long split_stride, void* out,
-                  int out_dtype, int n, int f, hipStream_t stream);
+                  int out_dtype, int n, int f, int act, hipStream_t stream);
 
 /* out[count] = sum over s of in[s][count], rounded to out_dtype. */
 int kllm_sum_splits(const float* in, int nsplit, long count, void* out, int out_dtype,
@@ -74,22 +78,22 @@ int kllm_sum_splits(const float* in, int nsplit, long count, void* out, int out_
 int kllm_gemm(const void* x, const void* w, void* y, int n, int m, int k, int dtype, int out_dtype,
               int algo, int nsplit, hipStream_t stream);
 
-/* h[n][f] = silu(x . w[0:f]^T) * (x . w[f:2f]^T) on the MFMA tiles, h in dtype. */
+/* h[n][f] = act(x . w[0:f]^T) * (x . w[f:2f]^T) on the MFMA tiles, h in dtype. */
 int kllm_gemm_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f, int k, int dtype,
-                     hipStream_t stream);
+                     int act, hipStream_t stream);
 
 /* Products for up to 8 rows of x with the whole of K in one wave (no partial
  * sums) and the next elementwise step in the epilogue.  m even, K a multiple
  * of 8 (bfloat16) or 4 (float32).
  *   plain:       y[n][m] float32 = x . w^T
- *   swiglu:      h[n][f] = silu(x . w[0:f]^T) * (x . w[f:2f]^T), h in dtype
+ *   swiglu:      h[n][f] = act(x . w[0:f]^T) * (x . w[f:2f]^T), h in dtype
  *   rope_append: w = [q; k; v] rows (only q when cache is null); rotates q and k
  *                with cos/sin [n][hd/2] (if given), writes q_out [n][H*hd] and
  *                puts k, v into the pages of `cache` */
 int kllm_gemv_plain(const void* x, const void* w, float* y, int n, int m, int k, int dtype,
                     hipStream_t stream);
 int kllm_gemv_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f, int k, int dtype,
-                     hipStream_t stream);
+                     int act, hipStream_t stream);
 int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_out, const float* cos_t,
                           const float* sin_t, void* cache, const int* positions,
                           const int* span_of_token, const int* block_table, int max_pages,
@@ -100,7 +104,7 @@ int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_out, const f
  * on the matrix cores, fused with the step after them.  x is [n][k] with a row
  * stride of x_stride elements (0 = k), w is [m][k].  Output:
  *   PARTS   y float32 [nsplit][n][m]; only this one may split K
- *   SWIGLU  y bfloat16 [n][m/2] = silu(x . w[0:m/2]^T) * (x . w[m/2:m]^T)
+ *   SWIGLU  y bfloat16 [n][m/2] = act(x . w[0:m/2]^T) * (x . w[m/2:m]^T)
  *   ROPE    w = [q; k; v] rows (only q when cache is null): q and k rotated with
  *           cos/sin [n][hd/2] (if given); y = q_out [n][H*hd], k and v go to the
  *           tokens' pages of `cache`
@@ -121,6 +125,7 @@ typedef struct {
   int kind;
   int nsplit;
   int max_pages, page_size, H, KV, hd;
+  int act;
 } KllmLinearOut;
 long kllm_fused_linear_lds_bytes(int n, int k, int nsplit);
 int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOut* out, const void* w, int n, int m,

@@ -2,8 +2,8 @@
 
 Everything a step needs besides weights and cache -- token ids, positions,
 which span a token belongs to, span offsets, state slots, the rows whose
-logits are wanted, one block table per cache group, and the sampling
-parameters -- is packed into one int32 buffer and sent with a single copy
+logits are wanted, one block table per cache group, the sampling parameters,
+and the index lists that parts ask for (how a mixer tiles the spans) -- is packed into one int32 buffer and sent with a single copy
 (the reference sends five, backend/model.cu:1048-1054).  The layout is fixed
 by (tokens, spans, wanted rows, pages per table), so a recorded HIP graph
 finds every array at the same address on every replay.
@@ -17,7 +17,7 @@ from typing import List, Sequence
 import numpy as np
 import torch
 
-from ..parts.base import StepContext, span_lists
+from ..parts.base import StepContext
 
 
 def _pad4(n: int) -> int:
@@ -31,8 +31,7 @@ class ControlLayout:
     rows: int              # wanted logit rows
     pages: tuple           # table width per cache group
     samples: int = 0       # rows of sampling parameters (temperature, uniform)
-    short: int = 0         # tokens of short spans, listed for the decode attention kernel
-    tiles: int = 0         # query tiles of longer spans, for the prompt attention kernel
+    lists: tuple = ()      # (name, count) of the index lists that parts asked for
 
     def sections(self):
         s = [("token_ids", self.n), ("positions", self.n), ("span_of_token", self.n),
@@ -40,7 +39,7 @@ class ControlLayout:
              ("logit_rows", max(self.rows, 1))]
         s += [(f"table{g}", self.spans * m) for g, m in enumerate(self.pages)]
         s += [("temperature", self.samples), ("uniform", self.samples), ("token_from", self.samples)]
-        s += [("short_tokens", self.short), ("query_tiles", 2 * self.tiles)]
+        s += [("list:" + name, count) for name, count in self.lists]
         return s
 
     def offsets(self):
@@ -55,18 +54,17 @@ class ControlLayout:
         return self.offsets()[1]
 
 
-def layout_for(lens: Sequence[int], rows: int, pages: tuple, samples: int = 0) -> ControlLayout:
-    starts = [0]
-    for l in lens:
-        starts.append(starts[-1] + l)
-    short, tiles = span_lists(starts, lens)
-    return ControlLayout(sum(lens), len(lens), rows, tuple(pages), samples, len(short), len(tiles))
+def layout_for(lens: Sequence[int], rows: int, pages: tuple, samples: int = 0, lists=None) -> ControlLayout:
+    """``lists``: name -> list of ints, the parts' index lists for these spans
+    (only their lengths enter the layout)."""
+    sizes = tuple((name, len(v)) for name, v in (lists or {}).items())
+    return ControlLayout(sum(lens), len(lens), rows, tuple(pages), samples, sizes)
 
 
 def fill(host: np.ndarray, layout: ControlLayout, tokens: Sequence[Sequence[int]],
          pos0: Sequence[int], slots: Sequence[int], rows: Sequence[int],
          tables: Sequence[Sequence[Sequence[int]]], temperatures=None, uniforms=None,
-         token_from=None):
+         token_from=None, lists=None):
     """Write one step into ``host`` (int32).  ``tables[g][s]`` is span s's
     table in group g.  ``token_from[t] >= 0`` (sampled steps only) says that
     token t's id is not ``tokens`` but the id the last sampled step left on
@@ -95,13 +93,13 @@ def fill(host: np.ndarray, layout: ControlLayout, tokens: Sequence[Sequence[int]
         bt.fill(-1)
         for s, t in enumerate(tables[g]):
             bt[s, :len(t)] = t
-    short, tiles = span_lists(starts, [len(t) for t in tokens])
-    if len(short) != layout.short or len(tiles) != layout.tiles:
-        raise ValueError("control layout does not fit the step's spans")
-    if layout.short:
-        sec("short_tokens")[:] = short
-    if layout.tiles:
-        sec("query_tiles")[:] = np.asarray(tiles, dtype=np.int32).reshape(-1)
+    lists = lists or {}
+    for name, count in layout.lists:
+        values = lists.get(name)
+        if values is None or len(values) != count:
+            raise ValueError(f"control layout does not fit the step's list {name!r}")
+        if count:
+            sec("list:" + name)[:] = np.asarray(values, dtype=np.int32)
     if layout.samples:
         sec("temperature").view(np.float32)[:] = np.asarray(temperatures, dtype=np.float32)
         sec("uniform").view(np.float32)[:] = np.asarray(uniforms, dtype=np.float32)
@@ -124,9 +122,7 @@ def context(dev: torch.Tensor, layout: ControlLayout, runtime, starts, pos0, len
         h_span_start=list(starts), h_span_pos=list(pos0), h_span_len=list(lens),
         block_tables=[sec(f"table{g}").view(layout.spans, m) for g, m in enumerate(layout.pages)],
         runtime=runtime, max_span_len=max(lens), all_decode=all(l == 1 for l in lens),
-        short_tokens=sec("short_tokens") if layout.short else None, n_short=layout.short,
-        query_tiles=sec("query_tiles").view(layout.tiles, 2) if layout.tiles else None,
-        n_tiles=layout.tiles,
+        lists={name: sec("list:" + name) for name, _ in layout.lists},
         token_from=sec("token_from") if layout.samples and layout.samples == layout.n else None)
 
 

@@ -19,6 +19,7 @@ import numpy as np
 import torch
 
 from ..cache import CacheManager, GroupSpec, OutOfPages
+from ..cache.manager import window_pages
 from ..config import ModelConfig, config_from_dict, load_config, resolve_architecture
 from ..parts.base import PagedCacheView, Runtime, StateCacheView, StepContext
 from ..weights import load_weights, random_weights
@@ -28,6 +29,13 @@ from .model import Model
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16,
            "bf16": torch.bfloat16}
+
+
+def _numel(shape) -> int:
+    n = 1
+    for d in shape:
+        n *= int(d)
+    return n
 
 
 class StepError(ValueError):
@@ -44,6 +52,8 @@ class EngineOptions:
     page_size: int = 16                   # tokens per page (reference default: 16)
     max_tokens: Optional[int] = None      # cache capacity in tokens (per group)
     num_pages: Optional[int] = None       # ... or directly in pages
+    memory_bytes: Optional[int] = None    # ... and never more than fits into this many bytes
+    max_step_tokens: Optional[int] = None  # most tokens one request brings in one step (None: any)
     max_requests: int = 64                # live requests (state slots)
     max_model_len: Optional[int] = None   # longest request; default max_position_embeddings
     gemm: str = "hip"                     # "hip" or "library" (vendor GEMM for large prompts)
@@ -133,33 +143,88 @@ class Engine:
 
     # ------------------------------------------------------------------ cache
     def _alloc_cache(self):
+        """Pools and device tensors of every cache group.
+
+        Capacity rule: the pool holds ``num_pages`` pages (or ``max_tokens``
+        tokens; by default four longest requests, engine/engine.go:30-32), but
+        never more than fit into ``memory_bytes`` beside the state slots -- the
+        reference's lesson that a pool must be sized from the model's
+        dimensions under a byte budget, not by a fixed count
+        (docs/JOURNAL.md:364-367, tools/modal_lab.py:232-240).  A group whose
+        layers read only a window of keys gets no more pages than
+        ``max_requests`` requests can hold at one time."""
         o = self.options
         plan = self.model.cache_plan
+        elem = torch.empty((), dtype=self.dtype).element_size()
+        if o.page_size <= 0:
+            raise ValueError(f"page_size {o.page_size} must be positive")
+        for part in self.model.all_parts():
+            part.check_cache(o.page_size)
         if o.num_pages is not None:
-            num_pages = int(o.num_pages)
+            asked = int(o.num_pages)
         else:
             tokens = o.max_tokens
             if tokens is None:
-                # The reference's default pool fits about four longest requests
-                # (engine/engine.go:30-32).
                 tokens = 4 * (self.max_model_len or 2048)
-            num_pages = -(-int(tokens) // o.page_size)
-        self.num_pages = num_pages
+            asked = -(-int(tokens) // o.page_size)
+        paged = [(g, gp) for g, gp in enumerate(plan.groups) if gp.need.kind == "paged"]
+        for g, gp in enumerate(plan.groups):
+            if gp.need.kind not in ("paged", "state"):
+                raise ValueError(f"unknown cache kind {gp.need.kind!r}")
+        state_bytes = sum(gp.entries * o.max_requests * _numel(gp.need.state_shape) * 4
+                          for gp in plan.groups if gp.need.kind == "state")
+        page_bytes = {g: gp.entries * 2 * gp.need.kv_heads * o.page_size * gp.need.head_dim * elem
+                      for g, gp in paged}
+        step = o.max_step_tokens or self.max_model_len or 0
+        want = {}
+        for g, gp in paged:
+            want[g] = asked
+            if gp.need.window > 0 and self.max_model_len:
+                per_request = window_pages(self.max_model_len, step, o.page_size, gp.need.window)
+                want[g] = min(asked, o.max_requests * per_request)
+        if o.memory_bytes is not None and paged:
+            budget = int(o.memory_bytes) - state_bytes
+            # shrink all groups by the same factor until they fit
+            need = sum(want[g] * page_bytes[g] for g, _ in paged)
+            if need > budget:
+                scale = max(budget, 0) / need
+                want = {g: int(want[g] * scale) for g in want}
+            if min(want.values()) < 1:
+                raise ValueError(
+                    f"memory_bytes={o.memory_bytes} leaves no room for a cache page in every group "
+                    f"(a page of each group takes {sum(page_bytes.values())} bytes, state slots "
+                    f"{state_bytes})")
+        self.num_pages = max(want.values()) if want else 0
         groups, self._paged_group_of, self.kv, self.state = [], {}, {}, {}
+        self._capacity = []
         for g, gp in enumerate(plan.groups):
             need = gp.need
             if need.kind == "paged":
                 self._paged_group_of[g] = len(groups)
-                groups.append(GroupSpec(f"group{g}", o.page_size, num_pages, need.window))
+                groups.append(GroupSpec(f"group{g}", o.page_size, want[g], need.window))
                 self.kv[g] = torch.zeros(
-                    gp.entries, num_pages, 2, need.kv_heads, o.page_size * need.head_dim,
+                    gp.entries, want[g], 2, need.kv_heads, o.page_size * need.head_dim,
                     dtype=self.dtype, device=self.device)
-            elif need.kind == "state":
+                self._capacity.append(
+                    f"group{g}: {gp.entries} layers, {need.kv_heads} KV heads of {need.head_dim}"
+                    + (f", window {need.window}" if need.window else "")
+                    + f": {want[g]} pages of {o.page_size} tokens = {want[g] * o.page_size} tokens, "
+                    f"{want[g] * page_bytes[g] / 2**20:.1f} MiB"
+                    + (f" (asked for {asked} pages)" if want[g] != asked else ""))
+            else:
                 self.state[g] = torch.zeros(gp.entries, o.max_requests, *need.state_shape,
                                             dtype=torch.float32, device=self.device)
-            else:
-                raise ValueError(f"unknown cache kind {need.kind!r}")
+                self._capacity.append(
+                    f"group{g}: {gp.entries} layers with state {tuple(need.state_shape)} in "
+                    f"{o.max_requests} slots, {self.state[g].numel() * 4 / 2**20:.1f} MiB")
         self.cache = CacheManager(groups, o.max_requests)
+
+    def capacity_report(self) -> str:
+        """What the cache was sized to, one line per group: for printing at start."""
+        head = f"cache: {self.cache_bytes() / 2**20:.1f} MiB"
+        if self.options.memory_bytes is not None:
+            head += f" of a budget of {self.options.memory_bytes / 2**20:.1f} MiB"
+        return "\n".join([head] + ["  " + line for line in self._capacity])
 
     def cache_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in list(self.kv.values()) + list(self.state.values()))
@@ -246,6 +311,10 @@ class Engine:
                     raise StepError(
                         f"request {e.request_id!r} would reach {rc.length + len(e.tokens)} tokens, "
                         f"the longest allowed is {self.max_model_len}")
+                if self.options.max_step_tokens and len(e.tokens) > self.options.max_step_tokens:
+                    raise StepError(
+                        f"request {e.request_id!r} brings {len(e.tokens)} tokens in one step, the engine "
+                        f"was sized for {self.options.max_step_tokens} (EngineOptions.max_step_tokens)")
                 self.cache.reserve(e.request_id, len(e.tokens))
                 reserved.append(e.request_id)
         except Exception:
@@ -297,12 +366,16 @@ class Engine:
         try:
             rcs, lens, rows, tables = self._describe(entries)
             pages = tuple(max(1, max(len(t) for t in tg)) for tg in tables)
-            layout = control.layout_for(lens, len(rows), pages)
+            span_starts = [0]
+            for l in lens:
+                span_starts.append(span_starts[-1] + l)
+            lists = self.model.step_lists(span_starts, lens)
+            layout = control.layout_for(lens, len(rows), pages, lists=lists)
             total = layout.total
             host = self._staging(total)
             pos0 = [rc.length for rc in rcs]
             starts = control.fill(host.numpy(), layout, [e.tokens for e in entries], pos0,
-                                  [rc.slot for rc in rcs], rows, tables)
+                                  [rc.slot for rc in rcs], rows, tables, lists=lists)
             if self._control is None or self._control.numel() < total:
                 self._control = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
             self._send(host, self._control, total)

@@ -76,7 +76,9 @@ class TokenRef:
 
 class _Recording:
     def __init__(self, engine, batch: int, caps: tuple):
-        self.layout = control.layout_for([1] * batch, batch, caps, samples=batch)
+        # the parts' index lists depend on the spans only: the same on every replay
+        self.lists = engine.model.step_lists(list(range(batch + 1)), [1] * batch)
+        self.layout = control.layout_for([1] * batch, batch, caps, samples=batch, lists=self.lists)
         self.control = torch.zeros(self.layout.total, dtype=torch.int32, device=engine.device)
         self.workspace = Workspace(engine.device)
         self.graph = None
@@ -147,7 +149,7 @@ class DecodeGraphs:
             host = eng._staging(rec.layout.total)
             pos0 = [rc.length for rc in rcs]
             control.fill(host.numpy(), rec.layout, tokens, pos0, [rc.slot for rc in rcs], rows, tables,
-                         temperatures, uniforms, token_from)
+                         temperatures, uniforms, token_from, lists=rec.lists)
             eng._send(host, rec.control, rec.layout.total)
             if rec.graph is None:
                 self._run(rec, lens, pos0)              # the step itself, and the warm-up

@@ -44,6 +44,7 @@ class Model:
         self.head = make_part("head", spec.head, runtime)
         self.schedule = list(spec.schedule)
         self.cache_plan = self._plan_cache()
+        self._list_providers = None
 
     # ------------------------------------------------------------------ cache plan
     def _plan_cache(self) -> CachePlan:
@@ -91,6 +92,33 @@ class Model:
     def bind(self, weights: Dict[str, torch.Tensor]) -> None:
         for p in self.parts():
             p.bind(weights)
+
+    def all_parts(self):
+        """Every part of the model, those inside arrangements and the shared ones included."""
+        out, todo = [], self.parts() + [p for _, p in self.runtime.shared.values()]
+        while todo:
+            p = todo.pop(0)
+            if any(p is q for q in out):
+                continue
+            out.append(p)
+            todo.extend(p.children())
+        return out
+
+    def step_lists(self, starts, lens) -> Dict[str, list]:
+        """The index lists that the model's parts want for a step with these spans:
+        "<key>.<name>" -> list of ints, one set per key."""
+        if self._list_providers is None:
+            seen = {}
+            for p in self.all_parts():
+                key = getattr(p, "step_lists_key", None)
+                if key is not None and key not in seen:
+                    seen[key] = p
+            self._list_providers = seen
+        out = {}
+        for key, part in self._list_providers.items():
+            for name, values in part.step_lists(list(starts), list(lens)).items():
+                out[f"{key}.{name}"] = values
+        return out
 
     @property
     def graph_safe(self) -> bool:

@@ -109,6 +109,9 @@ class Scheduler:
         self.max_batch = int(max_batch) if max_batch else 8
         self.max_step_tokens = int(max_step_tokens) if max_step_tokens else 2048
         self.chunk_size = int(chunk_size) if chunk_size else self.max_step_tokens
+        sized_for = getattr(getattr(engine, "options", None), "max_step_tokens", None)
+        if sized_for:                        # the engine takes no larger portion of one request
+            self.chunk_size = min(self.chunk_size, int(sized_for))
         if self.max_batch <= 0 or self.max_step_tokens <= 0 or self.chunk_size <= 0:
             raise SchedulerError("batch, token budget and chunk size must be positive")
         self.waiting: deque = deque()
@@ -136,7 +139,8 @@ class Scheduler:
                 f"prompt of {len(prompt)} tokens plus {max_new_tokens} new ones exceeds the "
                 f"longest request allowed ({limit})")
         cache = self.engine.cache
-        for need, pool in zip(cache.pages_for_tokens(total), cache.pools):
+        step = min(self.chunk_size, self.max_step_tokens)
+        for need, pool in zip(cache.pages_for_tokens(total, step), cache.pools):
             if need > pool.num_pages:
                 raise SchedulerError(
                     f"a request of {total} tokens needs {need} pages, the pool has "

@@ -81,12 +81,12 @@ def _declare(lib):
         "kllm_add_rmsnorm": [P, P, I, I, L, P, P, I, P, I, I, F, I, P],
         "kllm_rope_tables": [P, P, P, I, I, D, P],
         "kllm_rope_append": [P, I, I, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
-        "kllm_silu_mul": [P, I, I, L, P, I, I, I, P],
+        "kllm_silu_mul": [P, I, I, L, P, I, I, I, I, P],
         "kllm_gemm": [P, P, P, I, I, I, I, I, I, I, P],
         "kllm_sum_splits": [P, I, L, P, I, P],
-        "kllm_gemm_swiglu": [P, P, P, I, I, I, I, P],
+        "kllm_gemm_swiglu": [P, P, P, I, I, I, I, I, P],
         "kllm_gemv_plain": [P, P, P, I, I, I, I, P],
-        "kllm_gemv_swiglu": [P, P, P, I, I, I, I, P],
+        "kllm_gemv_swiglu": [P, P, P, I, I, I, I, I, P],
         "kllm_gemv_rope_append": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "kllm_fused_linear": [P, I, P, P, I, I, I, I, P],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
@@ -248,7 +248,12 @@ def rope_append(qkv, q_out, cos, sin, cache, positions, span_of_token, block_tab
         n_heads, n_kv_heads, head_dim, dtype_code(q_out.dtype), _stream()), "rope_append")
 
 
-def silu_mul(gu, out):
+ACT_SILU, ACT_GELU_TANH = 0, 1
+ACTIVATIONS = {"silu": ACT_SILU, "swish": ACT_SILU, "gelu_tanh": ACT_GELU_TANH, "gelu_pytorch_tanh": ACT_GELU_TANH}
+
+
+def silu_mul(gu, out, act=ACT_SILU):
+    """out [n, f] = act(gu[:, :f]) * gu[:, f:] (the gate of a gated feed-forward)."""
     n, f = out.shape
     nsplit, stride = 1, 0
     if gu.dim() == 3:
@@ -257,7 +262,7 @@ def silu_mul(gu, out):
         raise KernelError(f"silu_mul: input {tuple(gu.shape)} does not fit output {tuple(out.shape)}")
     _check(library().kllm_silu_mul(
         _ptr(gu, "silu_mul in"), dtype_code(gu.dtype), nsplit, stride, _ptr(out, "silu_mul out"),
-        dtype_code(out.dtype), n, f, _stream()), "silu_mul")
+        dtype_code(out.dtype), n, f, int(act), _stream()), "silu_mul")
 
 
 def gemm(x, w, y, algo, nsplit=1):
@@ -290,24 +295,24 @@ def gemv_fits(n, m, k, dtype) -> bool:
     return n <= most and m % 2 == 0 and k % v == 0
 
 
-def gemm_swiglu(x, w_gate_up, h):
+def gemm_swiglu(x, w_gate_up, h, act=ACT_SILU):
     """h [n, f] = silu(x . gate^T) * (x . up^T) on the MFMA tiles (any n; float32 with 32-bit MFMA)."""
     n, k = x.shape
     f = h.shape[1]
     if tuple(w_gate_up.shape) != (2 * f, k) or h.shape[0] != n or x.dtype != w_gate_up.dtype or h.dtype != x.dtype:
         raise KernelError("gemm_swiglu: shapes or dtypes do not fit")
     _check(library().kllm_gemm_swiglu(_ptr(x, "gemm x"), _ptr(w_gate_up, "gemm w"), _ptr(h, "gemm h"), n, f, k,
-                                      dtype_code(x.dtype), _stream()), "gemm_swiglu")
+                                      dtype_code(x.dtype), int(act), _stream()), "gemm_swiglu")
 
 
-def gemv_swiglu(x, w_gate_up, h):
+def gemv_swiglu(x, w_gate_up, h, act=ACT_SILU):
     """h [n, f] = silu(x . gate^T) * (x . up^T); w_gate_up is [2f, k], gate rows first."""
     n, k = x.shape
     f = h.shape[1]
     if tuple(w_gate_up.shape) != (2 * f, k) or h.shape[0] != n or x.dtype != w_gate_up.dtype or h.dtype != x.dtype:
         raise KernelError("gemv_swiglu: shapes or dtypes do not fit")
     _check(library().kllm_gemv_swiglu(_ptr(x, "gemv x"), _ptr(w_gate_up, "gemv w"), _ptr(h, "gemv h"), n, f, k,
-                                      dtype_code(x.dtype), _stream()), "gemv_swiglu")
+                                      dtype_code(x.dtype), int(act), _stream()), "gemv_swiglu")
 
 
 def gemv_rope_append(x, w_qkv, q_out, cos, sin, cache, positions, span_of_token, block_table, page_size,
@@ -340,7 +345,7 @@ class _LinearOut(ctypes.Structure):
     _fields_ = [("y", c_void_p), ("cos_t", c_void_p), ("sin_t", c_void_p), ("cache", c_void_p),
                 ("positions", c_void_p), ("span_of_token", c_void_p), ("block_table", c_void_p),
                 ("kind", c_int), ("nsplit", c_int), ("max_pages", c_int), ("page_size", c_int),
-                ("H", c_int), ("KV", c_int), ("hd", c_int)]
+                ("H", c_int), ("KV", c_int), ("hd", c_int), ("act", c_int)]
 
 
 FUSED_LINEAR_MAX_ROWS = 32
@@ -374,7 +379,7 @@ class Rope:
         self.page_size, self.heads, self.kv_heads, self.head_dim = page_size, heads, kv_heads, head_dim
 
 
-def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None):
+def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None, act=ACT_SILU):
     """One launch for a decode batch's product of x [n, k] (bfloat16; a view
     with a row stride is taken) with w [m, k], and the step after it, by
     ``kind``: LINEAR_PARTS y float32 [nsplit, n, m]; LINEAR_SWIGLU y bfloat16
@@ -388,7 +393,7 @@ def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None):
     if x.dim() != 2 or x.shape[1] != k or x.dtype != torch.bfloat16 or x.stride(1) != 1 or not x.is_cuda:
         raise KernelError(f"fused_linear: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)}")
     x_stride = x.stride(0) if n > 1 else k
-    lo.kind, lo.nsplit = kind, nsplit
+    lo.kind, lo.nsplit, lo.act = kind, nsplit, int(act)
     if kind == LINEAR_PARTS:
         want, dt = (nsplit, n, m), torch.float32
     elif kind == LINEAR_SWIGLU:
@@ -452,6 +457,7 @@ def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size
         "attn_generic")
 
 
+GENERIC_MAX_PAGE_SIZE = 256     # pages of the kernel that takes every size
 DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
 
 

@@ -28,6 +28,23 @@ from .spec import CacheNeed, WeightSpec
 @register_part("mixer", "attention")
 class CausalSelfAttention(Part):
     graph_safe = True
+    # How the attention kernels want a step's spans listed: the tokens of spans of at most
+    # SHORT_SPAN tokens one by one (for the kernel that cuts a token's keys into slices),
+    # longer spans in blocks of QUERY_BLOCK tokens (for the prompt kernel).
+    step_lists_key = "attention.spans"
+    SHORT_SPAN = 4
+    QUERY_BLOCK = K.PREFILL_QUERY_BLOCK
+
+    def step_lists(self, starts, lens):
+        short, blocks = [], []
+        for s, n in enumerate(lens):
+            a = starts[s]
+            if n <= self.SHORT_SPAN:
+                short.extend(range(a, a + n))
+            else:
+                for t in range(a, a + n, self.QUERY_BLOCK):
+                    blocks += [t, s]
+        return {"short": short, "blocks": blocks}
 
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)
@@ -65,6 +82,13 @@ class CausalSelfAttention(Part):
 
     def cache_need(self):
         return CacheNeed("paged", kv_heads=self.kv_heads, head_dim=self.head_dim, window=self.window)
+
+    def check_cache(self, page_size):
+        # The kernel that takes every size walks a chunk of up to 256 keys at a time, whole
+        # pages of them; the faster kernels are chosen per step where the sizes fit them.
+        if not 1 <= page_size <= K.GENERIC_MAX_PAGE_SIZE:
+            raise ValueError(f"attention: pages of {page_size} tokens are not built "
+                             f"(1 to {K.GENERIC_MAX_PAGE_SIZE})")
 
     def forward(self, ctx, xn, cache):
         n = xn.shape[0]
@@ -117,14 +141,17 @@ class CausalSelfAttention(Part):
                            self.scale)
             return
         n = q.shape[0]
-        listed = ctx.n_short + ctx.n_tiles > 0          # a context built by hand may carry no lists
-        if not listed or (ctx.n_tiles and not prompt_ok):
+        short = ctx.lists.get("attention.spans.short")
+        blocks = ctx.lists.get("attention.spans.blocks")
+        n_short = short.numel() if short is not None else 0
+        n_blocks = blocks.numel() // 2 if blocks is not None else 0
+        if n_short + n_blocks == 0 or (n_blocks and not prompt_ok):   # a context built by hand may carry no lists
             self._decode(ctx, q, out, cache, None, n)   # token by token
             return
-        if ctx.n_short:
-            self._decode(ctx, q, out, cache, None if ctx.n_short == n else ctx.short_tokens, ctx.n_short)
-        if ctx.n_tiles:
-            K.attn_prefill(q, out, cache.pages, ctx.query_tiles, ctx.n_tiles, ctx.span_start,
+        if n_short:
+            self._decode(ctx, q, out, cache, None if n_short == n else short, n_short)
+        if n_blocks:
+            K.attn_prefill(q, out, cache.pages, blocks, n_blocks, ctx.span_start,
                            ctx.span_pos, cache.block_table, cache.page_size, self.heads,
                            self.kv_heads, self.head_dim, self.window, self.scale)
 

@@ -155,24 +155,6 @@ class StateCacheView:
     write: bool = True
 
 
-# How a step's spans are listed for the attention kernels: tokens of spans of at
-# most SHORT_SPAN tokens one by one, longer spans in tiles of QUERY_TILE tokens.
-SHORT_SPAN = 4
-QUERY_TILE = 128       # = kernels.PREFILL_QUERY_BLOCK
-
-
-def span_lists(starts, lens):
-    """(token rows of short spans, (first row, span) of the long spans' tiles)."""
-    short, tiles = [], []
-    for s, n in enumerate(lens):
-        a = starts[s]
-        if n <= SHORT_SPAN:
-            short.extend(range(a, a + n))
-        else:
-            tiles.extend((t, s) for t in range(a, a + n, QUERY_TILE))
-    return short, tiles
-
-
 @dataclass
 class StepContext:
     """One step's batch as the parts see it.  All index tensors are int32 on
@@ -200,10 +182,9 @@ class StepContext:
     scratch: Dict[Any, Any] = field(default_factory=dict)   # per-step values of parts
     taps: Optional[List[torch.Tensor]] = None               # residual-stream captures
     workspace: Optional["Workspace"] = None                 # scratch of this step (default: the runtime's)
-    short_tokens: Optional[torch.Tensor] = None             # token rows of spans of <= SHORT_SPAN tokens
-    n_short: int = 0
-    query_tiles: Optional[torch.Tensor] = None              # [n_tiles, 2]: (first row, span), longer spans
-    n_tiles: int = 0
+    # Index lists that parts asked for through ``Part.step_lists``: "<key>.<name>" -> int32
+    # tensor on the device (as long as the host list was, possibly empty).
+    lists: Dict[str, torch.Tensor] = field(default_factory=dict)
     # Token ids that never reached the host: token t with token_from[t] >= 0 is
     # sampled[token_from[t]], what the last sampled step chose (both or neither are set).
     token_from: Optional[torch.Tensor] = None
@@ -222,6 +203,13 @@ class Part:
     # part can be recorded in a HIP graph.  A part that reads device values on
     # the host, or loops over host-side span data, leaves this False.
     graph_safe = False
+    # A part whose kernels want index lists that depend on how the step's tokens are cut
+    # into spans (which tokens are decode tokens, where tiles of queries begin) names a
+    # key here and builds the lists on the host in ``step_lists``; the engine packs them
+    # into the step's one control buffer and the part finds them as
+    # ``ctx.lists["<key>.<name>"]``.  Parts with the same key share one set of lists.  The
+    # lists may depend on nothing but ``starts`` and ``lens`` (a recorded step replays them).
+    step_lists_key: Optional[str] = None
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
         self.spec = spec
@@ -249,3 +237,16 @@ class Part:
 
     def cache_need(self) -> Optional[CacheNeed]:
         return None
+
+    def check_cache(self, page_size: int) -> None:
+        """Raise ValueError if this part's kernels do not take a cache with pages of
+        ``page_size`` tokens; the engine asks every part before it allocates."""
+
+    def children(self) -> List["Part"]:
+        """Parts this part is made of (an arrangement's norms, mixer, feed-forward)."""
+        return []
+
+    def step_lists(self, starts: List[int], lens: List[int]) -> Dict[str, List[int]]:
+        """name -> list of ints for a step whose span s covers rows
+        ``starts[s] .. starts[s] + lens[s]``; only called when ``step_lists_key`` is set."""
+        return {}

@@ -25,6 +25,9 @@ class PreNormBlock(Part):
     def parts(self):
         return [self.norm_mixer, self.mixer, self.norm_ff, self.feed_forward]
 
+    def children(self):
+        return self.parts()
+
     @property
     def graph_safe(self):
         return all(p.graph_safe for p in self.parts())

@@ -1,7 +1,8 @@
 """Gated feed-forward: down(act(gate(x)) * up(x)), no biases
 (backend/model.cu:1112-1115; SiLU: :477-483).
 
-Parameters: ``hidden``, ``intermediate``, ``activation`` ("silu").  Tensors:
+Parameters: ``hidden``, ``intermediate``, ``activation`` ("silu"; also
+"gelu_tanh": every kernel with a gate takes the activation as an argument).  Tensors:
 ``<prefix>.{gate,up,down}_proj.weight``.  Gate and up are kept as one matrix
 [2*intermediate, hidden] (gate rows first).
 """
@@ -25,8 +26,9 @@ class GatedFeedForward(Part):
         self.hidden = int(self.param("hidden"))
         self.intermediate = int(self.param("intermediate"))
         act = self.param("activation", "silu")
-        if act not in ("silu", "swish"):
-            raise ValueError(f"gated_mlp: activation {act!r} is not built (silu only)")
+        if act not in K.ACTIVATIONS:
+            raise ValueError(f"gated_mlp: activation {act!r} is not built (one of {sorted(K.ACTIVATIONS)})")
+        self.act = K.ACTIVATIONS[act]
         self.w_gu = None
         self.w_down = None
 
@@ -45,17 +47,17 @@ class GatedFeedForward(Part):
         h = ctx.buf("ffn.h", (n, self.intermediate), self.runtime.dtype)
         if (K.gemv_fits(n, 2 * self.intermediate, self.hidden, xn.dtype)
                 and not self.runtime.options.get("no_fused_gemv")):
-            K.gemv_swiglu(xn, self.w_gu, h)          # few tokens: both products and the gate in one launch
+            K.gemv_swiglu(xn, self.w_gu, h, self.act)          # few tokens: both products and the gate in one launch
         elif (xn.dtype == torch.bfloat16 and n <= K.FUSED_SWIGLU_BEST_ROWS
               and K.fused_linear_fits(n, self.hidden)
               and not self.runtime.options.get("no_fused_linear")):
-            K.fused_linear(self.w_gu, h, K.LINEAR_SWIGLU, x=xn)    # a decode batch: the same on the matrix cores
+            K.fused_linear(self.w_gu, h, K.LINEAR_SWIGLU, x=xn, act=self.act)    # a decode batch: the same on the matrix cores
         elif (n > 128 and self.runtime.options.get("gemm") != "library"
               and self.hidden % (8 if xn.dtype == torch.bfloat16 else 4) == 0):
             # prompts: the gate in the product's epilogue (up to 128 rows the product with K
             # in slices and a separate gate is faster: the epilogue cannot split K)
-            K.gemm_swiglu(xn, self.w_gu, h)
+            K.gemm_swiglu(xn, self.w_gu, h, self.act)
         else:
             gu = linear(ctx, xn, self.w_gu, "ffn.gu")
-            K.silu_mul(gu, h)
+            K.silu_mul(gu, h, self.act)
         return linear(ctx, h, self.w_down, "ffn.down")

@@ -107,6 +107,13 @@ def silu(x):
     return x / (1.0 + torch.exp(-x))
 
 
+def gelu_tanh(x):
+    """0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) (backend/model.cu:131-139): the
+    gate of the reference's other gated feed-forward; here for the kernels' activation
+    argument, no model in this package uses it."""
+    return 0.5 * x * (1.0 + torch.tanh(0.7978845608028654 * (x + 0.044715 * x * x * x)))
+
+
 def swiglu(xn, w_gate, w_up, w_down, store=None):
     """down(silu(gate(x)) * up(x)) (backend/model.cu:1112-1115)."""
     h = silu(linear(xn, w_gate)) * linear(xn, w_up)

@@ -192,3 +192,28 @@ def test_random_orders_lose_no_page(seed):
     for r in list(live):
         m.release(r)
     assert all(p.free_pages == p.num_pages for p in m.pools) and m.slots.free_slots == 5
+
+
+@pytest.mark.parametrize("page_size,window,step", [(4, 5, 1), (4, 6, 5), (8, 9, 13), (16, 20, 64), (16, 1, 2), (4, 16, 3)])
+def test_a_windowed_request_never_holds_more_than_pages_for_tokens_says(page_size, window, step):
+    """The bound that sizes a windowed group's pool and admits long requests:
+    random portions of at most ``step`` tokens, pages counted while reserved."""
+    from kllm_amd.cache.manager import window_pages
+    rng = random.Random(page_size * 1000 + window * 10 + step)
+    total = 40 * page_size
+    bound = window_pages(total, step, page_size, window)
+    assert bound <= -(-(step + window - 1) // page_size) + 1 and bound < -(-total // page_size)
+    m = CacheManager([GroupSpec("win", page_size, bound, window=window)], 2)
+    assert m.pages_for_tokens(total, step) == [bound] and m.pages_for_tokens(total) == [-(-total // page_size)]
+    m.open("r")
+    done, most = 0, 0
+    while done < total:
+        n = min(rng.randint(1, step), total - done)
+        m.reserve("r", n)                       # never OutOfPages: the pool is exactly the bound
+        most = max(most, m.pools[0].used_pages)
+        m.commit("r", n)
+        done += n
+        m.check_invariants()
+    assert most <= bound
+    assert most >= bound - 1                    # and the bound is not loose by more than a page
+    assert window_pages(total, step, page_size, 0) == -(-total // page_size)

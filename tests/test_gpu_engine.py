@@ -38,7 +38,7 @@ def replay(model_dir, dtype, steps, max_tokens, **opts):
     from kllm_amd.replay import Replayer
     options = EngineOptions(dtype=dtype, max_tokens=max_tokens, max_model_len=1 << 30,
                             poison_freed_pages=True, **opts)
-    rep = Replayer(model_dir, dtype, max_tokens, options=options)
+    rep = Replayer(model_dir, dtype, max_tokens or 0, options=options)
     outs = [rep.step(s["entries"], s["end"]) for s in steps]
     assert not rep.engine.cache.requests, "every request of the trace was ended"
     rep.engine.cache.check_invariants()
@@ -147,6 +147,32 @@ def test_every_choice_of_kernels_gives_the_same_logits(model_dirs, options):
     for steps in (traces.portions(reqs, 3), traces.mixed(reqs, seed=4)[0]):
         rows, _ = replay(d, "bfloat16", steps, traces.peak_tokens(steps), **options)
         compare(rows, want, "bfloat16", reqs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page_size", [4, 10, 12, 24, 48, 256])
+def test_page_sizes_that_are_no_multiple_of_16_and_large_ones(model_dirs, page_size, dtype):
+    """Pages of every size the engine accepts: those that only the kernel for every size
+    takes (10; in bfloat16 also 4, 12, 24), those the float32 matrix-core kernel takes (a
+    multiple of 4), and pages of 256 tokens.  Mixed steps, so that pages are used again."""
+    cfg, d = tiny.CONFIGS["A"], model_dirs("A")
+    reqs = make_requests(cfg, [70, 33, 120, 18, 64, 97], 6)
+    want = expected(d, cfg, reqs, dtype)
+    steps, peak = traces.mixed(reqs, seed=9)
+    held, most = {}, 0                  # exactly the pages the live requests hold at the worst step
+    for st in steps:
+        for e in st["entries"]:
+            held[e["id"]] = held.get(e["id"], 0) + len(e["tokens"])
+        most = max(most, sum(-(-n // page_size) for n in held.values()))
+        for rid in st["end"]:
+            del held[rid]
+    rows, rep = replay(d, dtype, steps, None, page_size=page_size, num_pages=most)
+    pool = rep.engine.cache.pools[0]
+    assert pool.high_water == most and (pool.total_allocs > most or page_size == 256)   # pages were used again
+    compare(rows, want, dtype, reqs)
+    steps = traces.bulk_then_tail(reqs, 32)
+    rows, _ = replay(d, dtype, steps, traces.peak_tokens(steps) + page_size, page_size=page_size)
+    compare(rows, want, dtype, reqs)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -319,3 +319,152 @@ def test_layers_with_a_window_have_pages_of_their_own(dtype, model_dirs, tmp_pat
         eng.cache.check_invariants()
     finally:
         unregister_architecture("ToyWindowForCausalLM")
+
+
+def test_pools_are_sized_per_group_and_from_a_byte_budget():
+    """A windowed group gets no more pages than its requests can hold; a byte budget
+    shrinks every pool; page sizes no kernel takes and portions larger than the engine
+    was sized for are refused when they are asked for, not at the first launch."""
+    from kllm_amd.cache.manager import window_pages
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry
+    from kllm_amd.engine.engine import StepError
+    register_architecture("ToyWindowForCausalLM", LlamaConfig, build_windowed)
+    try:
+        cfg = dict(tiny.CONFIGS["B"], architectures=["ToyWindowForCausalLM"])
+        base = dict(dtype="float32", num_pages=1000, max_requests=4, max_model_len=400, max_step_tokens=32)
+        eng = Engine.from_random(cfg, 1, EngineOptions(**base))
+        per_request = window_pages(400, 32, 16, WINDOW)
+        assert per_request == 5
+        assert [p.num_pages for p in eng.cache.pools] == [4 * per_request, 1000]
+        assert eng.kv[0].shape[1] == 20 and eng.kv[1].shape[1] == 1000
+        report = eng.capacity_report()
+        assert "window 20: 20 pages" in report and "asked for 1000 pages" in report and "1000 pages of 16" in report
+        with pytest.raises(StepError, match="sized for 32"):
+            eng.step([StepEntry("r", tiny.tokens(cfg, 33, 1), [32])])
+        assert eng.cache.pools[0].free_pages == 20 and "r" not in eng.cache
+        # a 200-token request in portions of 32 runs in the small windowed pool
+        ids = tiny.tokens(cfg, 200, 2)
+        for a in range(0, 200, 32):
+            eng.step([StepEntry("r", ids[a:a + 32], [])])
+        assert eng.cache.pools[0].high_water <= per_request
+        # a byte budget: one page of the windowed group (2 layers) and of the other (1 layer)
+        page_bytes = [2 * 2 * 1 * 16 * 32 * 4, 1 * 2 * 1 * 16 * 32 * 4]
+        full = 20 * page_bytes[0] + 1000 * page_bytes[1]
+        eng2 = Engine.from_random(cfg, 1, EngineOptions(**base, memory_bytes=full // 4))
+        pages = [p.num_pages for p in eng2.cache.pools]
+        assert pages == [5, 250] and eng2.cache_bytes() <= full // 4
+        assert "budget" in eng2.capacity_report()
+        with pytest.raises(ValueError, match="no room for a cache page"):
+            Engine.from_random(cfg, 1, EngineOptions(**base, memory_bytes=1000))
+        with pytest.raises(ValueError, match="pages of 512 tokens"):
+            Engine.from_random(cfg, 1, EngineOptions(dtype="float32", page_size=512))
+    finally:
+        unregister_architecture("ToyWindowForCausalLM")
+
+
+# ----------------------------------------------------------------------------- a mixer with its own tiling
+
+class ToyTiledMixer(Part):
+    """out_t = W x_t, computed tile by tile over tiles of at most TILE rows that never
+    cross a span: the tiling is this part's own, asked for through ``step_lists`` and
+    found on the device in ``ctx.lists``.  Rows that no tile covers stay NaN."""
+    step_lists_key = "toy.tiled"
+    TILE = 5
+    seen = []                                    # (starts, lens, tiles as the device held them)
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.hidden = self.param("hidden")
+
+    def weight_specs(self):
+        return [WeightSpec(self.tensor_name("weight"), (self.hidden, self.hidden))]
+
+    def bind(self, weights):
+        self.w = weights[self.tensor_name("weight")].float()
+
+    def step_lists(self, starts, lens):
+        tiles = []
+        for a, n in zip(starts, lens):
+            for t in range(a, a + n, self.TILE):
+                tiles += [t, min(self.TILE, a + n - t)]
+        return {"tiles": tiles}
+
+    def forward(self, ctx, xn, cache):
+        tiles = ctx.lists["toy.tiled.tiles"]
+        assert tiles.dtype == torch.int32 and tiles.is_cuda
+        host = tiles.tolist()
+        ToyTiledMixer.seen.append((list(ctx.h_span_start), list(ctx.h_span_len), host))
+        out = torch.full((ctx.n, self.hidden), float("nan"), dtype=torch.float32, device=xn.device)
+        for row, count in zip(host[0::2], host[1::2]):
+            out[row:row + count] = xn[row:row + count].float() @ self.w.t()
+        return out
+
+
+def build_tiled(cfg: LlamaConfig) -> ModelSpec:
+    """Layer 0: the tiled toy mixer and a feed-forward gated by the tanh approximation of
+    GELU; layer 1: attention (whose own span lists travel beside the toy's) and the
+    SiLU-gated feed-forward."""
+    from kllm_amd.models.llama import build_llama
+    spec = build_llama(cfg)
+    spec.layers[0].mixer = PartSpec("toy_tiled", "model.layers.0.mix", hidden=cfg.hidden_size)
+    spec.layers[0].feed_forward.params["activation"] = "gelu_tanh"
+    return spec
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_with_its_own_tiling_and_a_gelu_gated_feed_forward(dtype):
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry
+    register_part("mixer", "toy_tiled", ToyTiledMixer)
+    register_architecture("ToyTiledForCausalLM", LlamaConfig, build_tiled)
+    try:
+        cfg = dict(tiny.CONFIGS["A"], architectures=["ToyTiledForCausalLM"])
+        eng = Engine.from_random(cfg, 5, EngineOptions(dtype=dtype, max_tokens=256, max_requests=4),
+                                 std=0.08, norm_std=0.2)
+        assert sorted(eng.model.step_lists([0, 3, 4], [3, 1])) == ["attention.spans.blocks", "attention.spans.short",
+                                                                   "toy.tiled.tiles"]
+        w = engine_weights(eng)
+        r = (lambda t: t.to(torch.bfloat16).float()) if dtype == "bfloat16" else (lambda t: t)
+        c = P._cfg(cfg)
+
+        def reference(ids):
+            x = P.embedding(ids, w["model.embed_tokens.weight"])
+            xn = r(P.rmsnorm(x, w["model.layers.0.input_layernorm.weight"], c["eps"]))
+            x = x + P.linear(xn, w["model.layers.0.mix.weight"])
+            xn = r(P.rmsnorm(x, w["model.layers.0.post_attention_layernorm.weight"], c["eps"]))
+            h = P.gelu_tanh(P.linear(xn, w["model.layers.0.mlp.gate_proj.weight"])) * \
+                P.linear(xn, w["model.layers.0.mlp.up_proj.weight"])
+            x = x + P.linear(r(h), w["model.layers.0.mlp.down_proj.weight"])
+            x, _ = P.decoder_layer(w, 1, x, torch.arange(len(ids)), c, store=r if dtype == "bfloat16" else None)
+            return P.linear(r(P.rmsnorm(x, w["model.norm.weight"], c["eps"])), w["lm_head.weight"])
+
+        reqs = {"a": tiny.tokens(cfg, 45, 1), "b": tiny.tokens(cfg, 30, 2), "c": tiny.tokens(cfg, 22, 3)}
+        steps, _ = traces.mixed(reqs, seed=3, max_live=3, tail=6, max_portion=13)
+        ToyTiledMixer.seen.clear()
+        outs = []
+        for s in steps:
+            outs.append(eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]]).cpu().numpy())
+            for rid in s["end"]:
+                eng.release(rid)
+        rows = traces.collect(steps, outs)
+        for rid, toks in reqs.items():
+            want = reference(toks)
+            for p in range(len(toks)):
+                err = float((torch.from_numpy(rows[(rid, p)]) - want[p]).abs().max())
+                assert err < (2e-4 if dtype == "float32" else 8e-2), (rid, p, err)
+        # every step carried this part's tiling of exactly its spans
+        assert len(ToyTiledMixer.seen) == len(steps)
+        part = eng.model.blocks[0].mixer
+        for starts, lens, tiles in ToyTiledMixer.seen:
+            assert tiles == part.step_lists(starts, lens)["tiles"]
+            assert sum(tiles[1::2]) == sum(lens) and max(tiles[1::2]) <= ToyTiledMixer.TILE
+        assert any(len(l) > 1 and max(l) > ToyTiledMixer.TILE for _, l, _ in ToyTiledMixer.seen)
+        # the gate matters: SiLU instead of GELU moves the logits far beyond the tolerance
+        ids = reqs["a"]
+        x = P.embedding(ids, w["model.embed_tokens.weight"])
+        xn = P.rmsnorm(x + P.linear(P.rmsnorm(x, w["model.layers.0.input_layernorm.weight"], c["eps"]),
+                                    w["model.layers.0.mix.weight"]), w["model.layers.0.post_attention_layernorm.weight"], c["eps"])
+        g = P.linear(xn, w["model.layers.0.mlp.gate_proj.weight"])
+        assert float((P.gelu_tanh(g) - P.silu(g)).abs().max()) > 0.05
+    finally:
+        unregister_architecture("ToyTiledForCausalLM")
+        unregister_part("mixer", "toy_tiled")

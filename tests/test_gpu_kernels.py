@@ -184,6 +184,43 @@ def test_silu_mul(out_dtype, nsplit):
     assert (out.cpu().double() - want).abs().max() < bound
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_every_kernel_with_a_gate_takes_the_activation(dtype):
+    """The gate's activation is an argument: the tanh approximation of GELU through the
+    separate gate kernel, the two fused small-batch kernels and the tiled product's
+    epilogue, against the plain formula; and an activation nobody built is refused."""
+    k_ = K()
+    act = k_.ACT_GELU_TANH
+    f, k = 176, 264
+    w = rnd(2 * f, k, seed=2, dtype=dtype, scale=0.12)
+    wd = w.cpu().double()
+    tol = (lambda want: 1e-4) if dtype == torch.float32 else (lambda want: 0.01 * want.abs().max() + 1e-3)
+    for n in (3, 8, 20, 150):
+        x = rnd(n, k, seed=n, dtype=dtype, scale=0.7)
+        xd = x.cpu().double()
+        g, u = P.linear(xd, wd[:f]), P.linear(xd, wd[f:])
+        want = P.gelu_tanh(g) * u
+        assert (want - P.silu(g) * u).abs().max() > 0.05          # the two gates differ visibly
+        outs = {}
+        gu = torch.cat([g, u], dim=1).float().to(DEV).contiguous()
+        outs["gate kernel"] = torch.empty(n, f, dtype=dtype, device=DEV)
+        k_.silu_mul(gu.view(1, n, 2 * f), outs["gate kernel"], act)
+        if n <= 8:
+            outs["gemv"] = torch.empty(n, f, dtype=dtype, device=DEV)
+            k_.gemv_swiglu(x, w, outs["gemv"], act)
+        if dtype == torch.bfloat16 and n <= 32:
+            outs["fused_linear"] = torch.empty(n, f, dtype=dtype, device=DEV)
+            k_.fused_linear(w, outs["fused_linear"], k_.LINEAR_SWIGLU, x, act=act)
+        outs["tiles"] = torch.empty(n, f, dtype=dtype, device=DEV)
+        k_.gemm_swiglu(x, w, outs["tiles"], act)
+        for name, h in outs.items():
+            assert (h.cpu().double() - want).abs().max() < tol(want), (name, n)
+    with pytest.raises(k_.KernelError, match="unknown activation"):
+        k_.gemm_swiglu(x, w, outs["tiles"], 7)
+    with pytest.raises(k_.KernelError, match="unknown activation"):
+        k_.silu_mul(gu.view(1, n, 2 * f), outs["gate kernel"], -1)
+
+
 # ------------------------------------------------------------------ matrix products
 
 GEMM_SIZES = [(1, 64, 64), (2, 131, 88), (5, 100, 72), (8, 515, 2048), (3, 130, 5632), (8, 64, 20480),

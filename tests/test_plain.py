@@ -294,3 +294,10 @@ def test_storage_rounding_changes_little_and_nothing_when_it_is_the_identity():
     rounded = P.forward(w, cfg, ids, store=P.round_bfloat16)
     err = float((rounded - base).abs().max())
     assert 0 < err < 0.02 * float(base.abs().max())
+
+
+def test_gelu_tanh_is_the_library_routine():
+    x = torch.linspace(-8, 8, 4001, dtype=torch.float64)
+    want = torch.nn.functional.gelu(x, approximate="tanh")
+    assert (P.gelu_tanh(x) - want).abs().max() < 1e-12
+    assert abs(float(P.gelu_tanh(torch.tensor(1.0, dtype=torch.float64))) - 0.8411919906082768) < 1e-12

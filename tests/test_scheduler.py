@@ -136,6 +136,21 @@ def test_what_can_never_run_is_refused_at_submit():
     s.submit([1] * 10, 6)                            # 16 tokens fit exactly
 
 
+def test_a_long_request_fits_a_windowed_pool_when_its_portions_are_small():
+    """A windowed group holds the window and one portion, not the request: 200 tokens
+    run in a pool of 6 pages of 4 when no step brings more than 8, and are refused at
+    submit when a step may bring them all."""
+    p = prompts(3, 1, lo=150, hi=150)[0]
+    eng = StandIn(num_pages=6, page_size=4, window=9)
+    with pytest.raises(SchedulerError, match="could not run even alone"):
+        Scheduler(eng, max_batch=2, max_step_tokens=2048).submit(p, 50)
+    s = Scheduler(eng, max_batch=2, max_step_tokens=8)
+    i = s.submit(p, 50)
+    res = s.run_until_done()
+    assert res[i].tokens == alone(p, 50) and res[i].error is None
+    assert eng.cache.pools[0].high_water <= 6 and eng.cache.pools[0].free_pages == 6
+
+
 def test_long_prompt_is_cut_not_refused():
     # the reference refuses a prompt longer than the step budget (engine/scheduler.go:64-70)
     eng = StandIn(num_pages=100)

@@ -6,6 +6,18 @@ plus prefill of 2,048 tokens and decode at batch 1 and 64.
 
 Prints one JSON line.  A "step" is one decode step of the whole batch: the
 forward pass over the cache, sampling on the device, the tokens read back.
+
+Other workloads, each printing one JSON line of its own (``--model`` chooses the sizes):
+
+    --workload decode-run      prompts of 512 tokens decoded to 2,048: mean tok/s over the run
+                               and at context lengths 512, 1280 and 2047 (--batch)
+    --workload prefill-chunks  a 2,048-token prompt in portions of --chunk tokens
+    --workload mixed           --requests prompts of 128 to 2,048 tokens through the scheduler,
+                               prefilled in portions of --chunk tokens beside decode tokens
+    --kernel NAME --shape a,b,..   one kernel alone (gemm n,m,k; gemm_swiglu n,f,k; attn_prefill
+                               tokens,H,KV,hd; attn_decode batch,context,H,KV,hd; add_rmsnorm n,d;
+                               copy bytes), in microseconds and against nominal and measured peaks
+    --calibrate                the box's own copy bandwidth and MFMA rates
 """
 
 import argparse
@@ -32,6 +44,13 @@ def main(argv=None):
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--model", default="tinyllama-1.1b", choices=["tinyllama-1.1b", "llama2-7b", "llama3-8b"],
                     help="whose sizes to run (the default is the headline configuration)")
+    ap.add_argument("--workload", default="headline", choices=["headline", "decode-run", "prefill-chunks", "mixed"])
+    ap.add_argument("--chunk", type=int, default=512, help="tokens per prompt portion (prefill-chunks, mixed)")
+    ap.add_argument("--requests", type=int, default=32, help="requests of the mixed workload")
+    ap.add_argument("--new-tokens", type=int, default=64, help="tokens each request of the mixed workload generates")
+    ap.add_argument("--kernel", default=None, help="time one kernel alone (see the module's text)")
+    ap.add_argument("--shape", default="", help="comma-separated sizes for --kernel")
+    ap.add_argument("--calibrate", action="store_true", help="measure the box's copy bandwidth and MFMA rates")
     args = ap.parse_args(argv)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not built")
@@ -40,11 +59,24 @@ def main(argv=None):
     import torch
     from kllm_amd import benchmark as B
 
+    if args.calibrate:
+        print(json.dumps({"calibration": B.calibrate(), "peak_hbm_GBs": B.PEAK_HBM_GBS,
+                          "peak_TFLOPs": {k: v / 1e12 for k, v in B.PEAK_FLOPS.items()}}))
+        return 0
+    if args.kernel:
+        shape = [int(v) for v in args.shape.replace("x", ",").split(",") if v]
+        res = B.bench_kernel(args.kernel, shape, args.dtype, reps=max(1, args.steps), warmup=max(1, args.warmup))
+        res["calibration"] = B.calibrate()
+        print(json.dumps(res))
+        return 0
+
     cfg = dict(B.PRESETS[args.model])
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     elem = 2 if args.dtype == "bfloat16" else 4
+    if args.workload != "headline":
+        return other_workload(args, cfg, full_layers, B)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     eng = B.make_engine(cfg, args.dtype, max_tokens=max_batch * args.context + 4096,
                         max_model_len=args.context + 64, gemm=args.gemm, page_size=args.page_size)
@@ -77,12 +109,16 @@ def main(argv=None):
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": B.PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / B.PEAK_HBM_GBS, 4)},
     }
+    cal = B.calibrate()     # the box's own copy bandwidth and MFMA rate, beside the published peaks
+    out["roofline"]["measured_copy"] = cal["copy_GBs"]
+    out["roofline"]["frac_of_measured_copy"] = round(achieved / cal["copy_GBs"], 4)
     if not args.no_points:
         T = 2048
         pms = B.measure_prefill(eng, T)
         flops = B.prefill_flops(cfg, T)
         out["prefill"] = {"value": round(T * 1e3 / pms, 1), "tokens": T, "ms": round(pms, 3),
-                          "frac": round(flops / (pms * 1e-3) / B.PEAK_FLOPS[args.dtype], 4)}
+                          "frac": round(flops / (pms * 1e-3) / B.PEAK_FLOPS[args.dtype], 4),
+                          "frac_of_measured_mfma": round(flops / (pms * 1e-3) / 1e12 / cal[f"mfma_{args.dtype}_TFLOPs"], 4)}
         points = {}
         for b in (1, 64):
             k = max(16, args.steps // 2)
@@ -90,6 +126,41 @@ def main(argv=None):
             points[f"decode_b{b}"] = round(b * 1e3 / bms, 1)
         out["points"] = points
     print(json.dumps(out))
+    return 0
+
+
+def other_workload(args, cfg, full_layers, B):
+    import torch
+    elem = 2 if args.dtype == "bfloat16" else 4
+    base = {"workload": args.workload, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+            "model": args.model + "-sizes", "layers": cfg["num_hidden_layers"], "layers_full": full_layers,
+            "page_size": args.page_size, "gemm": args.gemm}
+    if args.workload == "decode-run":
+        eng = B.make_engine(cfg, args.dtype, max_tokens=args.batch * args.context + 4096,
+                            max_model_len=args.context + 64, gemm=args.gemm, page_size=args.page_size)
+        res = B.measure_decode_run(eng, args.batch, prompt_len=512, total_len=args.context)
+        base.update(batch=args.batch, prompt_len=512, total_len=args.context, unit="tok/s", **res)
+        worst = B.decode_step_bytes(cfg, args.batch, args.context - 1, elem)
+        base["frac_of_hbm_at_end"] = round(worst * res["at"][max(res["at"])] / args.batch / 1e9 / B.PEAK_HBM_GBS, 4)
+    elif args.workload == "prefill-chunks":
+        eng = B.make_engine(cfg, args.dtype, max_tokens=2 * 2048 + 4096, max_model_len=2048 + 64, gemm=args.gemm,
+                            page_size=args.page_size)
+        ms = B.measure_prefill_chunks(eng, 2048, args.chunk, reps=3, warmup=1)
+        whole = B.measure_prefill(eng, 2048)
+        flops = B.prefill_flops(cfg, 2048)
+        base.update(tokens=2048, chunk=args.chunk, ms=round(ms, 3), tok_s=round(2048e3 / ms, 1),
+                    frac=round(flops / (ms * 1e-3) / B.PEAK_FLOPS[args.dtype], 4),
+                    whole_prompt_ms=round(whole, 3))
+    else:
+        # room for every request's prompt and new tokens at once (no preemption in the timed run)
+        tokens = args.requests * (2048 + args.new_tokens + args.page_size)
+        eng = B.make_engine(cfg, args.dtype, max_tokens=tokens, max_model_len=2048 + args.new_tokens + 64,
+                            gemm=args.gemm, page_size=args.page_size, max_requests=max(64, args.requests))
+        res = B.measure_mixed(eng, args.requests, 128, 2048, args.new_tokens, args.chunk)
+        base.update(chunk=args.chunk, new_tokens=args.new_tokens, **res)
+        base["prefill_frac"] = round(res["prompt_tok_s"] * 2.0 * cfg["num_hidden_layers"] * B.layer_matrix_elements(cfg)
+                                     / B.PEAK_FLOPS[args.dtype], 4)
+    print(json.dumps(base))
     return 0
 
 

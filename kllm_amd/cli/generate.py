@@ -5,8 +5,13 @@ folder with config.json and safetensors), ``--device``, ``--ids``
 (space-separated prompt ids), ``--steps`` (most new tokens), ``--max-seq`` (KV
 capacity in tokens).  Its ``--backend`` named the CUDA library to load; here
 it may name a prebuilt kernel library and is otherwise not needed.  Added:
-``--dtype``, ``--temperature``, ``--seed``, and ``--random CONFIG.json`` for
-seeded random weights.  Output as the reference prints it:
+``--dtype``, ``--temperature``, ``--seed``, ``--sample-seed``, ``--random
+CONFIG.json`` for seeded random weights, ``--max-new-tokens`` (another name of
+``--steps``), and the engine's sizes: ``--page-size``, ``--num-pages``,
+``--max-step-tokens`` (the token budget of a step: longer prompts are cut
+into portions) and ``--memory-gib`` (a byte budget that the cache is fitted
+into).  What the cache was sized to is printed to standard error at start.
+Output as the reference prints it:
 
     prompt:    [1 17 42 100 7]
     generated: [...]
@@ -37,11 +42,17 @@ def build_parser():
                     help="use seeded random weights for this config.json instead of --model")
     ap.add_argument("--device", type=int, default=0, help="GPU index")
     ap.add_argument("--ids", default="1 17 42 100 7", help="space-separated prompt token ids")
-    ap.add_argument("--steps", type=int, default=16, help="max new tokens")
+    ap.add_argument("--steps", "--max-new-tokens", dest="steps", type=int, default=16, help="max new tokens")
     ap.add_argument("--max-seq", type=int, default=256, help="KV capacity in tokens")
+    ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page")
+    ap.add_argument("--num-pages", type=int, default=None, help="cache pages (default: --max-seq tokens' worth)")
+    ap.add_argument("--max-step-tokens", type=int, default=None,
+                    help="most tokens in one step; a longer prompt is cut into portions (default 2048)")
+    ap.add_argument("--memory-gib", type=float, default=None, help="fit the cache into this many GiB")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--temperature", type=float, default=0.0, help="0 = greedy")
     ap.add_argument("--seed", type=int, default=0, help="seed of sampling (and of --random weights)")
+    ap.add_argument("--sample-seed", type=int, default=None, help="seed of sampling alone (default: --seed)")
     return ap
 
 
@@ -52,7 +63,9 @@ def main(argv=None) -> int:
         import os
         os.environ["KLLM_AMD_LIBRARY"] = args.backend
     from ..engine import Engine, EngineOptions
-    opts = EngineOptions(device=args.device, dtype=args.dtype, max_tokens=args.max_seq,
+    opts = EngineOptions(device=args.device, dtype=args.dtype, page_size=args.page_size,
+                         max_tokens=args.max_seq, num_pages=args.num_pages,
+                         memory_bytes=None if args.memory_gib is None else int(args.memory_gib * 2**30),
                          max_model_len=args.max_seq, max_requests=4)
     try:
         if args.random:
@@ -60,7 +73,10 @@ def main(argv=None) -> int:
                 eng = Engine.from_random(json.load(f), args.seed, opts)
         else:
             eng = Engine.from_dir(args.model, opts)
-        out = eng.generate(prompt, args.steps, temperature=args.temperature, seed=args.seed)
+        print(eng.capacity_report(), file=sys.stderr)
+        out = eng.generate(prompt, args.steps, temperature=args.temperature,
+                           seed=args.seed if args.sample_seed is None else args.sample_seed,
+                           max_step_tokens=args.max_step_tokens)
     except Exception as e:  # the reference prints "error: ..." and exits 1
         print(f"error: {e}", file=sys.stderr)
         return 1

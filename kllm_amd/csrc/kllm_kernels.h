@@ -37,6 +37,13 @@ int kllm_abi_version(void);
 /* Compute units of the current device (the launch heuristics scale with it). */
 int kllm_device_cus(void);
 
+/* What the box reaches with nothing in the way, for quoting measured figures against: a
+ * plain copy of `bytes` (a multiple of 16) and a loop of `iters` rounds of four independent
+ * MFMAs per wave on every CU (bfloat16 32x32x16 or float32 32x32x2); *flops receives the
+ * floating-point operations of the launch.  The caller times them. */
+int kllm_calibrate_copy(void* dst, const void* src, long bytes, hipStream_t stream);
+int kllm_calibrate_mfma(int dtype, int iters, float* sink, double* flops, hipStream_t stream);
+
 /* out[t] = table[ids[t]]; with `from` (and `sampled`), token t whose from[t] >= 0 takes its id
  * from sampled[from[t]], a token id that an earlier launch left on the device. */
 int kllm_embed(float* out, const void* table, const int* ids, const int* from, const int* sampled,

@@ -30,7 +30,70 @@ int device_cus() {
   return cached[dev];
 }
 
+// ---- what the box reaches with nothing in the way (for quoting figures against) ----------
+__global__ __launch_bounds__(256) void calibrate_copy_kernel(floatx4* __restrict__ dst,
+                                                             const floatx4* __restrict__ src, long n16) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (long)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
+// Four independent accumulator tiles per wave, `iters` rounds of one MFMA each; the result is
+// written so that the loop cannot be dropped.
+template <bool F32>
+__global__ __launch_bounds__(256) void calibrate_mfma_kernel(float* __restrict__ sink, int iters) {
+  floatx16 acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+  const float v = 1.f + threadIdx.x * 1e-6f;
+  bf16x8 a8, b8;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    a8[e] = (bf16_t)v;
+    b8[e] = (bf16_t)(v * 0.5f);
+  }
+  for (int i = 0; i < iters; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (F32) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(v, v * 0.5f, acc[j], 0, 0, 0);
+      else acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a8, b8, acc[j], 0, 0, 0);
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s += acc[j][e];
+  if (s == 12345.678f) sink[threadIdx.x % 64] = s;   // never true; keeps the loop alive
+}
+
 }  // namespace kllm
+
+extern "C" int kllm_calibrate_copy(void* dst, const void* src, long bytes, hipStream_t stream) {
+  KLLM_REQUIRE(dst && src && bytes > 0 && bytes % 16 == 0 && ((uintptr_t)dst & 15) == 0 && ((uintptr_t)src & 15) == 0,
+               "calibrate_copy: %ld bytes must be a multiple of 16 and the buffers 16-byte aligned", bytes);
+  const int grid = kllm::device_cus() * 16;
+  hipLaunchKernelGGL(kllm::calibrate_copy_kernel, dim3(grid), dim3(256), 0, stream, (kllm::floatx4*)dst,
+                     (const kllm::floatx4*)src, bytes / 16);
+  KLLM_CHECK_LAUNCH("calibrate_copy");
+  return 0;
+}
+
+// Launches the MFMA loop; *flops receives the floating-point operations of the launch.
+extern "C" int kllm_calibrate_mfma(int dtype, int iters, float* sink, double* flops, hipStream_t stream) {
+  KLLM_REQUIRE(sink && flops && iters > 0 && iters <= (1 << 20), "calibrate_mfma: bad arguments");
+  KLLM_REQUIRE(dtype == kllm::DT_F32 || dtype == kllm::DT_BF16, "calibrate_mfma: unknown dtype %d", dtype);
+  const int grid = kllm::device_cus() * 8;          // eight workgroups of four waves per CU
+  const double per_mfma = dtype == kllm::DT_F32 ? 2.0 * 32 * 32 * 2 : 2.0 * 32 * 32 * 16;
+  *flops = per_mfma * 4.0 * iters * 4.0 * grid;
+  if (dtype == kllm::DT_F32)
+    hipLaunchKernelGGL(kllm::calibrate_mfma_kernel<true>, dim3(grid), dim3(256), 0, stream, sink, iters);
+  else
+    hipLaunchKernelGGL(kllm::calibrate_mfma_kernel<false>, dim3(grid), dim3(256), 0, stream, sink, iters);
+  KLLM_CHECK_LAUNCH("calibrate_mfma");
+  return 0;
+}
 
 extern "C" int kllm_device_cus(void) { return kllm::device_cus(); }
 

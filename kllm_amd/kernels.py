@@ -93,6 +93,8 @@ def _declare(lib):
         "kllm_sample": [P, P, P, P, I, I, P],
         "kllm_attn_decode_slices": [I, I, I, I],
         "kllm_device_cus": [],
+        "kllm_calibrate_copy": [P, P, L, P],
+        "kllm_calibrate_mfma": [I, I, P, P, P],
         "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, P],
         "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
     }
@@ -163,6 +165,22 @@ def device_info(device: int = 0) -> str:
 
 
 # ----------------------------------------------------------------------------- wrappers
+
+def calibrate_copy(dst, src):
+    """dst = src with a plain copy kernel (for measuring the box's copy bandwidth)."""
+    if dst.numel() * dst.element_size() != src.numel() * src.element_size():
+        raise KernelError("calibrate_copy: sizes differ")
+    _check(library().kllm_calibrate_copy(_ptr(dst, "copy dst"), _ptr(src, "copy src"),
+                                         src.numel() * src.element_size(), _stream()), "calibrate_copy")
+
+
+def calibrate_mfma(dtype_code_, iters, sink) -> float:
+    """Launch the MFMA loop; returns the floating-point operations of the launch."""
+    flops = c_double(0.0)
+    _check(library().kllm_calibrate_mfma(int(dtype_code_), int(iters), _ptr(sink, "mfma sink", torch.float32),
+                                         ctypes.byref(flops), _stream()), "calibrate_mfma")
+    return flops.value
+
 
 def embed(out, table, ids, from_sampled=None, sampled=None):
     """out [n, d] = table[ids]; where ``from_sampled[t] >= 0`` the id is

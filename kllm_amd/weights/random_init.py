@@ -1,11 +1,20 @@
-"""Random-weights mode: a model folder from a configuration and a seed.
+"""Random-weights mode: a model folder, or tensors in memory, from a
+configuration and a seed.
 
 Distributions follow the reference's test-model generator
 (tools/make_test_model.py:59-80): matrices and embedding tables are
-``std * N(0, 1)``, norm weights ``1 + norm_std * N(0, 1)``.  Each tensor is
-drawn from a generator seeded by (seed, tensor name), so a tensor's values do
-not depend on which other tensors the model has or in which order they are
-made.
+``std * z``, norm weights ``1 + norm_std * z`` with z of mean 0 and variance 1.
+
+The generator is counter-based: element i of a tensor is a function of (seed,
+tensor name, i) alone, made of 32-bit integer mixing and one exact
+integer-to-float conversion, with no transcendental function.  A tensor's
+values therefore do not depend on which other tensors the model has, on the
+order in which they are made, on how the work is cut into pieces, or on
+whether the CPU or the GPU computes them: the engine draws a model of any
+size directly in device memory, and a test can draw the same tensors on the
+CPU for the plain implementation.  z is the sum of eight uniform 16-bit
+numbers, centred and scaled to variance 1 (within 4.9 standard deviations;
+close to normal, which is all that random test weights need).
 """
 
 from __future__ import annotations
@@ -22,25 +31,64 @@ from ..parts.spec import WeightSpec
 from .loader import merge_specs, target_dtype
 from .safetensors_io import write_safetensors
 
+_M32 = 0xFFFFFFFF
+_CHUNK = 1 << 22        # elements drawn at a time (bounds the temporaries)
 
-def _tensor_seed(seed: int, name: str) -> int:
+
+def _tensor_key(seed: int, name: str):
+    """Two 32-bit words that stand for (seed, tensor name)."""
     h = hashlib.sha256(f"{seed}:{name}".encode("utf-8")).digest()
-    return int.from_bytes(h[:8], "little") & ((1 << 63) - 1)
+    return int.from_bytes(h[:4], "little"), int.from_bytes(h[4:8], "little")
+
+
+def _mul32(x: torch.Tensor, c: int) -> torch.Tensor:
+    """(x * c) mod 2^32 for int64 tensors holding 32-bit values, without ever
+    leaving 63 bits (so that no device's overflow behaviour matters)."""
+    lo = (x & 0xFFFF) * c
+    hi = (((x >> 16) * c) & 0xFFFF) << 16
+    return (lo + hi) & _M32
+
+
+def _mix32(x: torch.Tensor) -> torch.Tensor:
+    """A 32-bit finalizer of the multiply-xorshift kind (two multiplications,
+    three shifts): every input bit reaches every output bit."""
+    x = x ^ (x >> 16)
+    x = _mul32(x, 0x7FEB352D)
+    x = x ^ (x >> 15)
+    x = _mul32(x, 0x846CA68B)
+    return x ^ (x >> 16)
+
+
+def unit_variates(seed: int, name: str, start: int, count: int, device="cpu") -> torch.Tensor:
+    """z[start : start + count] of the tensor ``name`` as float32 on ``device``."""
+    k0, k1 = _tensor_key(seed, name)
+    i = torch.arange(start, start + count, dtype=torch.int64, device=device)
+    state = _mix32((i & _M32) ^ k0)
+    state = _mix32(state ^ k1 ^ _mul32((i >> 32) & _M32, 0x9E3779B1))
+    total = torch.zeros_like(state)
+    for j in range(4):
+        u = _mix32((state + ((j + 1) * 0x9E3779B9 & _M32)) & _M32)
+        total += (u & 0xFFFF) + (u >> 16)
+    # eight uniforms on {0..65535}: mean 8 * 32767.5, variance 8 * (65536^2 - 1) / 12
+    z = (total - 262140).to(torch.float32)
+    return z * (1.0 / 53509.61)             # sqrt(8 * (65536^2 - 1) / 12) = 53509.61...
 
 
 def random_tensor(spec: WeightSpec, seed: int, dtype: torch.dtype, std=0.02, norm_std=0.02,
                   device="cpu") -> torch.Tensor:
-    """The seeded value of one tensor.  Values are drawn in float32 on the CPU
-    (so they are the same everywhere) and then rounded to ``dtype``."""
-    g = torch.Generator(device="cpu").manual_seed(_tensor_seed(seed, spec.name))
+    """The seeded value of one tensor, computed on ``device`` in float32 and
+    rounded to ``dtype`` there."""
     if spec.role == "table":
         return torch.zeros(spec.shape, dtype=torch.int32, device=device)
-    r = torch.randn(spec.shape, generator=g, dtype=torch.float32)
-    if spec.role == "vector":
-        r = 1.0 + norm_std * r
-    else:
-        r = std * r
-    return r.to(device).to(dtype)
+    numel = 1
+    for d in spec.shape:
+        numel *= int(d)
+    out = torch.empty(numel, dtype=dtype, device=device)
+    for a in range(0, numel, _CHUNK):
+        n = min(_CHUNK, numel - a)
+        z = unit_variates(seed, spec.name, a, n, device)
+        out[a:a + n] = (1.0 + norm_std * z if spec.role == "vector" else std * z).to(dtype)
+    return out.view(*spec.shape)
 
 
 def random_weights(specs: Iterable[WeightSpec], seed: int, compute_dtype: torch.dtype,

@@ -414,3 +414,38 @@ def test_command_line_generate(model_dirs):
     assert lines[0] == "prompt:    [1 17 42 100 7]"
     want = P.generate_greedy(tiny.read_weights(d), cfg, [1, 17, 42, 100, 7], 16, eos={2})
     assert lines[1] == "generated: [" + " ".join(map(str, want)) + "]"
+
+
+def test_command_line_options_of_the_engine_sizes(model_dirs):
+    """--page-size, --num-pages, --max-step-tokens, --max-new-tokens and --sample-seed: a
+    prompt longer than the step's budget is cut into portions, the tokens stay the same,
+    and what the cache was sized to is printed at start."""
+    cfg, d = tiny.CONFIGS["R"], model_dirs("R")
+    prompt = tiny.tokens(cfg, 45, 8)
+    base = [sys.executable, os.path.join(ROOT, "bin", "generate"), "--model", d, "--ids", " ".join(map(str, prompt)),
+            "--dtype", "float32", "--max-seq", "256"]
+    out = subprocess.run(base + ["--max-new-tokens", "12", "--page-size", "8", "--num-pages", "9", "--max-step-tokens", "7",
+                                 "--sample-seed", "3"], capture_output=True, text=True, timeout=120, cwd="/")
+    assert out.returncode == 0, out.stderr
+    want = P.generate_greedy(tiny.read_weights(d), cfg, prompt, 12, eos={2})
+    assert out.stdout.strip().splitlines()[1] == "generated: [" + " ".join(map(str, want)) + "]"
+    assert "9 pages of 8 tokens" in out.stderr
+    small = subprocess.run(base + ["--steps", "12", "--page-size", "8", "--num-pages", "3"],
+                           capture_output=True, text=True, timeout=120, cwd="/")
+    assert small.returncode == 1 and "could not run even alone" in small.stderr
+
+
+def test_command_line_bench_one_kernel_and_a_sweep_of_batches(model_dirs):
+    d = model_dirs("A")
+    bench = [sys.executable, os.path.join(ROOT, "bin", "bench"), "--json", "--dtype", "bfloat16"]
+    out = subprocess.run(bench + ["--kernel", "gemm", "--shape", "200,256,512", "--steps", "5"],
+                         capture_output=True, text=True, timeout=120, cwd="/")
+    assert out.returncode == 0, out.stderr
+    res = json.loads(out.stdout.strip().splitlines()[-1])
+    assert res["kernel"] == "gemm" and res["us"] > 0 and 0 < res["frac_of_peak"] < 1 and res["frac_of_measured"] > 0
+    out = subprocess.run(bench + ["--model", d, "--prompt", "16", "--steps", "8", "--reps", "1", "--max-seq", "64",
+                                  "--batch", "1,3"], capture_output=True, text=True, timeout=120, cwd="/")
+    assert out.returncode == 0, out.stderr
+    rows = [json.loads(l) for l in out.stdout.strip().splitlines()]
+    assert [r["batch"] for r in rows] == [1, 3] and all(r["decode_tok_s"] > 0 and r["ttft_ms"] > 0 for r in rows)
+    assert "pages of 16 tokens" in out.stderr

@@ -216,3 +216,19 @@ def test_unknown_part_kind_names_the_registered_ones():
     rt = T.runtime(torch.float32)
     with pytest.raises(ValueError, match="rmsnorm"):
         make_part("norm", PartSpec("layernorm", size=8, eps=1e-5), rt)
+
+
+def test_weights_drawn_on_the_gpu_equal_those_drawn_on_the_cpu():
+    """The seeded generator is integer mixing and one exact conversion: bit for bit the
+    same on both devices, in any piece, for every role and dtype."""
+    from kllm_amd.parts import WeightSpec
+    from kllm_amd.weights import random_tensor
+    from kllm_amd.weights.random_init import unit_variates
+    for spec, dtype in [(WeightSpec("a.weight", (300, 257)), torch.float32), (WeightSpec("a.weight", (300, 257)), torch.bfloat16),
+                        (WeightSpec("n.weight", (1000,), "vector"), torch.float32)]:
+        cpu = random_tensor(spec, 9, dtype, 0.05, 0.1, "cpu")
+        gpu = random_tensor(spec, 9, dtype, 0.05, 0.1, "cuda")
+        assert torch.equal(cpu, gpu.cpu()) and gpu.dtype == dtype
+    far = (1 << 33) + 12345                              # beyond 32 bits of element index
+    assert torch.equal(unit_variates(9, "t", far, 1000, "cpu"), unit_variates(9, "t", far, 1000, "cuda").cpu())
+    assert not torch.equal(unit_variates(9, "t", far, 1000, "cpu"), unit_variates(9, "t", far - (1 << 32), 1000, "cpu"))

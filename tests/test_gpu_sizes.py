@@ -50,15 +50,18 @@ _weights, _expected = {}, {}
 
 
 def weights(name):
-    """name -> float32 CPU tensor, from the package's seeded generator; the engine is
-    given exactly these (rounded to bfloat16 for a bfloat16 engine, as the loader would)."""
+    """name -> float32 CPU tensor, from the package's seeded generator (drawn on the GPU,
+    whose values equal the CPU's: test_weights_drawn_on_the_gpu_equal_those_drawn_on_the_cpu);
+    the engine is given exactly these (rounded to bfloat16 for a bfloat16 engine, as the
+    loader would)."""
     if name not in _weights:
         from kllm_amd.config import config_from_dict, resolve_architecture
         from kllm_amd.engine.model import collect_weight_specs
         from kllm_amd.weights import random_weights
         raw = SIZES[name]
         spec = resolve_architecture(raw).build(config_from_dict(raw, where=name))
-        _weights[name] = random_weights(collect_weight_specs(spec), SEED, torch.float32, "cpu")
+        _weights[name] = {k: v.cpu() for k, v in
+                          random_weights(collect_weight_specs(spec), SEED, torch.float32, "cuda").items()}
     return _weights[name]
 
 

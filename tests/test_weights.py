@@ -196,3 +196,20 @@ def test_random_model_folder(tmp_path, name, store):
     # the loader reads what the writer wrote
     got = load_weights(out, llama_specs(name), torch.float32, "cpu")
     assert torch.equal(got["model.embed_tokens.weight"], emb)
+
+
+KNOWN_VARIATES = [-0.207383, 0.869825, 1.187076]
+
+
+def test_the_seeded_generator_depends_on_seed_name_and_index_only():
+    from kllm_amd.weights.random_init import unit_variates
+    z = unit_variates(3, "a.weight", 0, 200000)
+    pieces = torch.cat([unit_variates(3, "a.weight", 0, 777), unit_variates(3, "a.weight", 777, 200000 - 777)])
+    assert torch.equal(z, pieces)
+    assert abs(float(z.mean())) < 0.01 and abs(float(z.std()) - 1.0) < 0.01 and float(z.abs().max()) < 4.9
+    assert abs(float((z[:-1] * z[1:]).mean())) < 0.01                 # neighbours are uncorrelated
+    other = unit_variates(3, "b.weight", 0, 200000)
+    assert abs(float((z * other).mean())) < 0.01 and not torch.equal(z, other)
+    assert not torch.equal(z, unit_variates(4, "a.weight", 0, 200000))
+    # three known values pin the function itself (computed once with this definition)
+    assert [round(float(v), 6) for v in unit_variates(1, "w", 5, 3)] == KNOWN_VARIATES

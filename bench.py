@@ -44,6 +44,7 @@ def main(argv=None):
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--model", default="tinyllama-1.1b", choices=["tinyllama-1.1b", "llama2-7b", "llama3-8b"],
                     help="whose sizes to run (the default is the headline configuration)")
+    ap.add_argument("--extra", default="", help="engine options for experiments: key=value,key=value (ints or words)")
     ap.add_argument("--workload", default="headline", choices=["headline", "decode-run", "prefill-chunks", "mixed"])
     ap.add_argument("--chunk", type=int, default=512, help="tokens per prompt portion (prefill-chunks, mixed)")
     ap.add_argument("--requests", type=int, default=32, help="requests of the mixed workload")
@@ -78,8 +79,12 @@ def main(argv=None):
     if args.workload != "headline":
         return other_workload(args, cfg, full_layers, B)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
+    extra = {}
+    for item in filter(None, args.extra.split(",")):
+        key, _, val = item.partition("=")
+        extra[key] = int(val) if val.lstrip("-").isdigit() else (val or True)
     eng = B.make_engine(cfg, args.dtype, max_tokens=max_batch * args.context + 4096,
-                        max_model_len=args.context + 64, gemm=args.gemm, page_size=args.page_size)
+                        max_model_len=args.context + 64, gemm=args.gemm, page_size=args.page_size, extra=extra)
 
     if args.prefill_only:
         pms = B.measure_prefill(eng, 2048, reps=max(1, args.steps), warmup=args.warmup)

@@ -96,16 +96,32 @@ int kllm_gemm_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f
  *   swiglu:      h[n][f] = act(x . w[0:f]^T) * (x . w[f:2f]^T), h in dtype
  *   rope_append: w = [q; k; v] rows (only q when cache is null); rotates q and k
  *                with cos/sin [n][hd/2] (if given), writes q_out [n][H*hd] and
- *                puts k, v into the pages of `cache` */
+ *                puts k, v into the pages of `cache`
+ * With `normed` (may be null) x is not read (it may be null): the kernel stages
+ * normed->x * rsqrt(sum of normed->ss[row][:] / k + eps) * normed->weight, rounded to dtype,
+ * the RMS norm of the residual stream that a resid product (kllm_gemv_resid) has just
+ * updated, without a launch of its own; built for up to 4 rows. */
+typedef struct {
+  const float* x;      /* the residual stream [n][k], float32 */
+  const float* weight; /* the norm's weight [k] */
+  const float* ss;     /* [n][parts rounded up to 4] partial sums of squares of x's rows */
+  int parts;           /* at most 512 */
+  float eps;
+} KllmNormedInput;     /* all three 16-byte aligned */
 int kllm_gemv_plain(const void* x, const void* w, float* y, int n, int m, int k, int dtype,
-                    hipStream_t stream);
+                    const KllmNormedInput* normed, hipStream_t stream);
 int kllm_gemv_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f, int k, int dtype,
-                     int act, hipStream_t stream);
+                     int act, const KllmNormedInput* normed, hipStream_t stream);
+/* resid [n][m] float32 += x . w^T in place; ss_out [n][P rounded up to 4] = the
+ * workgroups' partial sums of squares of resid's new rows, P = kllm_gemv_resid_parts(m). */
+int kllm_gemv_resid(const void* x, const void* w, float* resid, float* ss_out, int n, int m, int k,
+                    int dtype, hipStream_t stream);
+int kllm_gemv_resid_parts(int m);
 int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_out, const float* cos_t,
                           const float* sin_t, void* cache, const int* positions,
                           const int* span_of_token, const int* block_table, int max_pages,
                           int page_size, int n, int H, int KV, int hd, int k, int dtype,
-                          hipStream_t stream);
+                          const KllmNormedInput* normed, hipStream_t stream);
 
 /* Products of a decode batch (bfloat16, up to KLLM_FUSED_LINEAR_MAX_ROWS rows)
  * on the matrix cores, fused with the step after them.  x is [n][k] with a row

@@ -157,7 +157,14 @@ class Model:
             ctx.taps.append(x.clone())
         pending = None
         for i, run in enumerate(self.schedule):
-            x, pending = self.blocks[run.layer].forward(ctx, x, pending, cache_views[i])
+            block = self.blocks[run.layer]
+            if getattr(block, "takes_next_norm", False) and i + 1 < len(self.schedule):
+                # the norm that will take this layer's output, if the next layer names one
+                nxt = self.blocks[self.schedule[i + 1].layer]
+                first = nxt.first_norm() if hasattr(nxt, "first_norm") else None
+                x, pending = block.forward(ctx, x, pending, cache_views[i], next_norm=first)
+            else:
+                x, pending = block.forward(ctx, x, pending, cache_views[i])
             if ctx.taps is not None:
                 if pending is not None:
                     self.final_norm.add(ctx, x, pending)

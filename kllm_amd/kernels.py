@@ -85,9 +85,11 @@ def _declare(lib):
         "kllm_gemm": [P, P, P, I, I, I, I, I, I, I, P],
         "kllm_sum_splits": [P, I, L, P, I, P],
         "kllm_gemm_swiglu": [P, P, P, I, I, I, I, I, P],
-        "kllm_gemv_plain": [P, P, P, I, I, I, I, P],
-        "kllm_gemv_swiglu": [P, P, P, I, I, I, I, I, P],
-        "kllm_gemv_rope_append": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
+        "kllm_gemv_plain": [P, P, P, I, I, I, I, P, P],
+        "kllm_gemv_swiglu": [P, P, P, I, I, I, I, I, P, P],
+        "kllm_gemv_rope_append": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P],
+        "kllm_gemv_resid": [P, P, P, P, I, I, I, I, P],
+        "kllm_gemv_resid_parts": [I],
         "kllm_fused_linear": [P, I, P, P, I, I, I, I, P],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
@@ -283,6 +285,76 @@ def silu_mul(gu, out, act=ACT_SILU):
         dtype_code(out.dtype), n, f, int(act), _stream()), "silu_mul")
 
 
+class _NormedInput(ctypes.Structure):
+    _fields_ = [("x", c_void_p), ("weight", c_void_p), ("ss", c_void_p), ("parts", c_int), ("eps", c_float)]
+
+
+class NormedInput:
+    """The input of a product as the RMS norm of a residual stream, made by the product's
+    kernel while it stages X: ``x`` [n, k] float32 (the stream, already holding what was
+    added), the norm's ``weight`` [k] and ``eps``, and ``ss`` [n, parts rounded up to 4]
+    float32, the partial sums of squares of x's rows that a residual product left."""
+    MAX_PARTS = 512
+
+    def __init__(self, x, weight, ss, parts, eps):
+        self.x, self.weight, self.ss, self.parts, self.eps = x, weight, ss, int(parts), float(eps)
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+    def struct(self, n, k):
+        stride = -(-self.parts // 4) * 4
+        if (tuple(self.x.shape) != (n, k) or self.weight.numel() != k or tuple(self.ss.shape) != (n, stride)
+                or not 1 <= self.parts <= self.MAX_PARTS):
+            raise KernelError(f"normed input: stream {tuple(self.x.shape)}, weight {tuple(self.weight.shape)}, sums of "
+                              f"squares {tuple(self.ss.shape)} do not fit {n} x {k} with {self.parts} parts")
+        return _NormedInput(_ptr(self.x, "normed x", torch.float32), _ptr(self.weight, "normed weight", torch.float32),
+                            _ptr(self.ss, "normed ss", torch.float32), self.parts, self.eps)
+
+
+def _x_and_norm(x, dtype):
+    """(pointer of x or None, struct or None, n, k) for an input that is a tensor or a NormedInput."""
+    if isinstance(x, NormedInput):
+        n, k = x.shape
+        st = x.struct(n, k)
+        return None, st, n, k
+    n, k = x.shape
+    if x.dtype != dtype:
+        raise KernelError(f"input dtype {x.dtype}, weights {dtype}")
+    return _ptr(x, "x"), None, n, k
+
+
+NORMED_MAX_ROWS = 4    # rows that the small-batch kernels normalise while they stage their input
+
+
+def resid_parts(n, m, k, dtype):
+    """Partial sums of squares per row that a residual product of these sizes
+    leaves (one per workgroup of eight rows of W), or 0 if the small-batch
+    kernel with that epilogue does not take them."""
+    if not (gemv_fits(n, m, k, dtype) and n <= NORMED_MAX_ROWS):
+        return 0
+    parts = library().kllm_gemv_resid_parts(m)
+    return parts if parts <= NormedInput.MAX_PARTS else 0
+
+
+def linear_resid(x, w, resid, ss):
+    """resid [n, m] float32 += x . w^T in place; ss [n, parts rounded up to 4] receives the
+    partial sums of squares of resid's new rows (parts = resid_parts(...), returned)."""
+    n, k = x.shape
+    m = w.shape[0]
+    parts = resid_parts(n, m, k, x.dtype)
+    stride = -(-parts // 4) * 4
+    if (parts == 0 or tuple(resid.shape) != (n, m) or tuple(ss.shape) != (n, stride) or w.shape[1] != k
+            or w.dtype != x.dtype):
+        raise KernelError(f"linear_resid: x {tuple(x.shape)}, w {tuple(w.shape)}, resid {tuple(resid.shape)}, "
+                          f"ss {tuple(ss.shape)} do not fit ({parts} parts)")
+    _check(library().kllm_gemv_resid(
+        _ptr(x, "resid x"), _ptr(w, "resid w"), _ptr(resid, "resid", torch.float32),
+        _ptr(ss, "resid ss", torch.float32), n, m, k, dtype_code(x.dtype), _stream()), "gemv_resid")
+    return parts
+
+
 def gemm(x, w, y, algo, nsplit=1):
     """y [nsplit, n, m] (or [n, m]) = x [n, k] . w [m, k]^T."""
     n, k = x.shape
@@ -297,7 +369,7 @@ def gemm(x, w, y, algo, nsplit=1):
             raise KernelError("gemm: the LDS gemv does not split K")
         _check(library().kllm_gemv_plain(
             _ptr(x, "gemv x"), _ptr(w, "gemv w"), _ptr(y, "gemv y", torch.float32), n, m, k,
-            dtype_code(x.dtype), _stream()), "gemv_plain")
+            dtype_code(x.dtype), None, _stream()), "gemv_plain")
         return
     _check(library().kllm_gemm(
         _ptr(x, "gemm x"), _ptr(w, "gemm w"), _ptr(y, "gemm y"), n, m, k, dtype_code(x.dtype),
@@ -324,26 +396,29 @@ def gemm_swiglu(x, w_gate_up, h, act=ACT_SILU):
 
 
 def gemv_swiglu(x, w_gate_up, h, act=ACT_SILU):
-    """h [n, f] = silu(x . gate^T) * (x . up^T); w_gate_up is [2f, k], gate rows first."""
-    n, k = x.shape
+    """h [n, f] = act(x . gate^T) * (x . up^T); w_gate_up is [2f, k], gate rows first.  x
+    is a tensor or a NormedInput."""
+    xp, st, n, k = _x_and_norm(x, w_gate_up.dtype)
     f = h.shape[1]
-    if tuple(w_gate_up.shape) != (2 * f, k) or h.shape[0] != n or x.dtype != w_gate_up.dtype or h.dtype != x.dtype:
+    if tuple(w_gate_up.shape) != (2 * f, k) or h.shape[0] != n or h.dtype != w_gate_up.dtype:
         raise KernelError("gemv_swiglu: shapes or dtypes do not fit")
-    _check(library().kllm_gemv_swiglu(_ptr(x, "gemv x"), _ptr(w_gate_up, "gemv w"), _ptr(h, "gemv h"), n, f, k,
-                                      dtype_code(x.dtype), int(act), _stream()), "gemv_swiglu")
+    _check(library().kllm_gemv_swiglu(xp, _ptr(w_gate_up, "gemv w"), _ptr(h, "gemv h"), n, f, k,
+                                      dtype_code(w_gate_up.dtype), int(act), ctypes.byref(st) if st else None, _stream()),
+           "gemv_swiglu")
 
 
 def gemv_rope_append(x, w_qkv, q_out, cos, sin, cache, positions, span_of_token, block_table, page_size,
                      n_heads, n_kv_heads, head_dim):
-    """q, k, v projections of up to 8 rows, rotation, q_out and the cache append in one launch."""
-    n, k = x.shape
+    """q, k, v projections of up to 8 rows (x a tensor or a NormedInput), rotation, q_out and
+    the cache append in one launch."""
+    xp, st, n, k = _x_and_norm(x, w_qkv.dtype)
     rows = n_heads * head_dim + (2 * n_kv_heads * head_dim if cache is not None else 0)
     if (tuple(w_qkv.shape) != (rows, k) or tuple(q_out.shape) != (n, n_heads * head_dim)
-            or x.dtype != w_qkv.dtype or q_out.dtype != x.dtype):
+            or q_out.dtype != w_qkv.dtype):
         raise KernelError("gemv_rope_append: shapes or dtypes do not fit")
     max_pages = 0
     if cache is not None:
-        if tuple(cache.shape[1:]) != (2, n_kv_heads, page_size * head_dim) or cache.dtype != x.dtype:
+        if tuple(cache.shape[1:]) != (2, n_kv_heads, page_size * head_dim) or cache.dtype != w_qkv.dtype:
             raise KernelError(f"gemv_rope_append: cache {tuple(cache.shape)} {cache.dtype} does not fit")
         max_pages = block_table.shape[1]
         if positions.numel() < n or span_of_token.numel() < n:
@@ -351,12 +426,13 @@ def gemv_rope_append(x, w_qkv, q_out, cos, sin, cache, positions, span_of_token,
     if cos is not None and (tuple(cos.shape) != (n, head_dim // 2) or tuple(sin.shape) != tuple(cos.shape)):
         raise KernelError("gemv_rope_append: cos/sin shapes do not fit")
     _check(library().kllm_gemv_rope_append(
-        _ptr(x, "gemv x"), _ptr(w_qkv, "gemv w"), _ptr(q_out, "gemv q_out"),
+        xp, _ptr(w_qkv, "gemv w"), _ptr(q_out, "gemv q_out"),
         _ptr(cos, "gemv cos", torch.float32, True), _ptr(sin, "gemv sin", torch.float32, True),
         _ptr(cache, "gemv cache", None, True), _ptr(positions, "gemv positions", torch.int32, True),
         _ptr(span_of_token, "gemv span_of_token", torch.int32, True),
         _ptr(block_table, "gemv block_table", torch.int32, True), max_pages, page_size, n, n_heads,
-        n_kv_heads, head_dim, k, dtype_code(x.dtype), _stream()), "gemv_rope_append")
+        n_kv_heads, head_dim, k, dtype_code(w_qkv.dtype), ctypes.byref(st) if st else None, _stream()),
+        "gemv_rope_append")
 
 
 class _LinearOut(ctypes.Structure):
@@ -408,10 +484,10 @@ def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None, act=ACT_SIL
     if w.dtype != torch.bfloat16:
         raise KernelError("fused_linear: bfloat16 weights only")
     n = x.shape[0]
+    lo.kind, lo.nsplit, lo.act = kind, nsplit, int(act)
     if x.dim() != 2 or x.shape[1] != k or x.dtype != torch.bfloat16 or x.stride(1) != 1 or not x.is_cuda:
         raise KernelError(f"fused_linear: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)}")
-    x_stride = x.stride(0) if n > 1 else k
-    lo.kind, lo.nsplit, lo.act = kind, nsplit, int(act)
+    x_ptr, x_stride = x.data_ptr(), (x.stride(0) if n > 1 else k)
     if kind == LINEAR_PARTS:
         want, dt = (nsplit, n, m), torch.float32
     elif kind == LINEAR_SWIGLU:
@@ -442,7 +518,7 @@ def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None, act=ACT_SIL
     if tuple(y.shape) != want or y.dtype != dt:
         raise KernelError(f"fused_linear: output {tuple(y.shape)} {y.dtype}, expected {want} {dt}")
     lo.y = _ptr(y, "fused_linear y")
-    _check(library().kllm_fused_linear(x.data_ptr(), x_stride, ctypes.byref(lo), _ptr(w, "fused_linear w"), n, m, k,
+    _check(library().kllm_fused_linear(x_ptr, x_stride, ctypes.byref(lo), _ptr(w, "fused_linear w"), n, m, k,
                                        tiles_per_wg, _stream()), "fused_linear")
 
 

@@ -20,14 +20,16 @@ import math
 import torch
 
 from .. import kernels as K
-from .base import Part, register_part
-from .linear import linear
+from .base import Normed, Part, register_part
+from .linear import linear, linear_into
 from .spec import CacheNeed, WeightSpec
 
 
 @register_part("mixer", "attention")
 class CausalSelfAttention(Part):
     graph_safe = True
+    takes_normed = True     # the q, k, v product of a decode batch applies the norm's row scale itself
+    fills_sink = True       # the output projection of a decode batch adds itself to the residual stream
     # How the attention kernels want a step's spans listed: the tokens of spans of at most
     # SHORT_SPAN tokens one by one (for the kernel that cuts a token's keys into slices),
     # longer spans in blocks of QUERY_BLOCK tokens (for the prompt kernel).
@@ -90,7 +92,14 @@ class CausalSelfAttention(Part):
             raise ValueError(f"attention: pages of {page_size} tokens are not built "
                              f"(1 to {K.GENERIC_MAX_PAGE_SIZE})")
 
-    def forward(self, ctx, xn, cache):
+    def forward(self, ctx, xn, cache, sink=None):
+        if isinstance(xn, Normed):
+            n = xn.rows
+            opts = self.runtime.options
+            gemv = (K.gemv_fits(n, self.w_in.shape[0], self.hidden, self.runtime.dtype) and n <= K.NORMED_MAX_ROWS
+                    and not opts.get("no_fused_gemv"))
+            # the small-batch kernel below normalises while it stages its input
+            xn = xn.kernel_input() if gemv else xn.materialize(ctx)
         n = xn.shape[0]
         dtype = self.runtime.dtype
         writes = self.own_kv
@@ -120,6 +129,10 @@ class CausalSelfAttention(Part):
                           self.head_dim)
         out = ctx.buf("attn.out", (n, self.q_dim), dtype)
         self.attend(ctx, q, out, cache)
+        if sink is not None:
+            normed = linear_into(ctx, out, self.w_o, sink, "attn.proj")
+            if normed is not None:
+                return normed
         return linear(ctx, out, self.w_o, "attn.proj")
 
     def attend(self, ctx, q, out, cache):

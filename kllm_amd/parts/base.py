@@ -156,6 +156,41 @@ class StateCacheView:
 
 
 @dataclass
+class ResidualSink:
+    """An offer to a sub-layer that ends in a matrix product: add your output to the
+    residual stream ``x`` yourself, in the product's epilogue, and leave what the norm
+    behind the addition needs (``norm`` has ``weight`` and ``eps`` of an RMS norm).  A part
+    that takes the offer (it declares ``fills_sink = True`` and gets ``sink=`` in forward)
+    returns a ``Normed`` instead of its output; it may decline and return its output."""
+    x: torch.Tensor
+    norm: "Part"
+
+
+@dataclass
+class Normed:
+    """An RMS norm that its consumer performs, as a residual product leaves it: ``x`` is
+    the residual stream [n, d] (it already holds the sub-layer's output), ``ss`` [n, parts
+    rounded up to 4] the partial sums of squares of its rows, ``norm`` the norm part it
+    stands for (weight and eps).  A consumer whose kernel normalises while it stages its
+    input takes ``kernel_input()``; any other calls ``materialize``, which runs the norm."""
+    x: torch.Tensor
+    ss: torch.Tensor
+    parts: int
+    norm: "Part"
+
+    @property
+    def rows(self) -> int:
+        return self.x.shape[0]
+
+    def kernel_input(self):
+        from .. import kernels as K
+        return K.NormedInput(self.x, self.norm.weight, self.ss, self.parts, self.norm.eps)
+
+    def materialize(self, ctx):
+        return self.norm.forward(ctx, self.x, delta=self)
+
+
+@dataclass
 class StepContext:
     """One step's batch as the parts see it.  All index tensors are int32 on
     the device; the ``h_`` lists are their host copies.
@@ -210,6 +245,14 @@ class Part:
     # ``ctx.lists["<key>.<name>"]``.  Parts with the same key share one set of lists.  The
     # lists may depend on nothing but ``starts`` and ``lens`` (a recorded step replays them).
     step_lists_key: Optional[str] = None
+    # A mixer or feed-forward whose first product can normalise its input while staging it
+    # declares ``takes_normed`` and may then get a ``Normed`` as its input; one whose
+    # last product can add itself to the residual stream declares ``fills_sink`` and then
+    # gets ``sink=ResidualSink`` (see those classes).  A norm that others may fuse this way
+    # declares ``fusable`` (it has ``weight`` and ``eps`` of an RMS norm).
+    takes_normed = False
+    fills_sink = False
+    fusable = False
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
         self.spec = spec

@@ -4,12 +4,15 @@
 (backend/model.cu:1083-1117).  As in the reference, a sub-layer's output is
 not added to the residual stream by a pass of its own: it travels as
 ``pending`` into the next norm, which adds it while it normalises (:1084,
-:1105, :1117).
+:1105, :1117).  For decode batches even that launch goes: where the parts
+allow it, a sub-layer's last product adds its sums to the stream in its
+epilogue (``ResidualSink``) and the next sub-layer's first product applies the
+norm's row scale to its own sums (``Normed``).
 """
 
 from __future__ import annotations
 
-from .base import Part, make_part, register_part
+from .base import Part, ResidualSink, make_part, register_part
 
 
 @register_part("block", "pre_norm")
@@ -42,9 +45,28 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
-    def forward(self, ctx, x, pending, cache):
-        xn = self.norm_mixer.forward(ctx, x, delta=pending)
-        delta = self.mixer.forward(ctx, xn, cache)
-        xn = self.norm_ff.forward(ctx, x, delta=delta)
-        pending = self.feed_forward.forward(ctx, xn)
+    takes_next_norm = True
+
+    def first_norm(self):
+        """The norm that takes what the layer before this one leaves pending."""
+        return self.norm_mixer
+
+    @staticmethod
+    def _normed_ok(ctx, norm, consumer):
+        return {"normed_ok": True} if (norm.fusable and consumer.takes_normed and ctx.taps is None) else {}
+
+    @staticmethod
+    def _sink(ctx, x, producer, norm):
+        if norm is None or not (producer.fills_sink and norm.fusable) or ctx.taps is not None:
+            return {}
+        return {"sink": ResidualSink(x, norm)}
+
+    def forward(self, ctx, x, pending, cache, next_norm=None):
+        """``next_norm``: the norm that will take this layer's pending output
+        (the next layer's first norm), if the caller knows it; the feed-forward
+        may then add its output to x itself."""
+        xn = self.norm_mixer.forward(ctx, x, delta=pending, **self._normed_ok(ctx, self.norm_mixer, self.mixer))
+        delta = self.mixer.forward(ctx, xn, cache, **self._sink(ctx, x, self.mixer, self.norm_ff))
+        xn = self.norm_ff.forward(ctx, x, delta=delta, **self._normed_ok(ctx, self.norm_ff, self.feed_forward))
+        pending = self.feed_forward.forward(ctx, xn, **self._sink(ctx, x, self.feed_forward, next_norm))
         return x, pending

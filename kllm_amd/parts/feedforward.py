@@ -12,14 +12,16 @@ from __future__ import annotations
 import torch
 
 from .. import kernels as K
-from .base import Part, register_part
-from .linear import linear
+from .base import Normed, Part, register_part
+from .linear import linear, linear_into
 from .spec import WeightSpec
 
 
 @register_part("feed_forward", "gated_mlp")
 class GatedFeedForward(Part):
     graph_safe = True
+    takes_normed = True     # the gate and up products of a decode batch apply the norm's row scale
+    fills_sink = True       # the down projection of a decode batch adds itself to the residual stream
 
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)
@@ -42,16 +44,19 @@ class GatedFeedForward(Part):
                                weights[self.tensor_name("up_proj.weight")]], dim=0).contiguous()
         self.w_down = weights[self.tensor_name("down_proj.weight")]
 
-    def forward(self, ctx, xn):
-        n = xn.shape[0]
-        h = ctx.buf("ffn.h", (n, self.intermediate), self.runtime.dtype)
-        if (K.gemv_fits(n, 2 * self.intermediate, self.hidden, xn.dtype)
-                and not self.runtime.options.get("no_fused_gemv")):
-            K.gemv_swiglu(xn, self.w_gu, h, self.act)          # few tokens: both products and the gate in one launch
-        elif (xn.dtype == torch.bfloat16 and n <= K.FUSED_SWIGLU_BEST_ROWS
-              and K.fused_linear_fits(n, self.hidden)
-              and not self.runtime.options.get("no_fused_linear")):
-            K.fused_linear(self.w_gu, h, K.LINEAR_SWIGLU, x=xn, act=self.act)    # a decode batch: the same on the matrix cores
+    def forward(self, ctx, xn, sink=None):
+        dtype, opts = self.runtime.dtype, self.runtime.options
+        n = xn.rows if isinstance(xn, Normed) else xn.shape[0]
+        gemv = K.gemv_fits(n, 2 * self.intermediate, self.hidden, dtype) and not opts.get("no_fused_gemv")
+        fused = (not gemv and dtype == torch.bfloat16 and n <= K.FUSED_SWIGLU_BEST_ROWS
+                 and K.fused_linear_fits(n, self.hidden) and not opts.get("no_fused_linear"))
+        if isinstance(xn, Normed):     # the small-batch kernel below normalises while it stages its input
+            xn = xn.kernel_input() if gemv and n <= K.NORMED_MAX_ROWS else xn.materialize(ctx)
+        h = ctx.buf("ffn.h", (n, self.intermediate), dtype)
+        if gemv:
+            K.gemv_swiglu(xn, self.w_gu, h, self.act)   # few tokens: both products and the gate in one launch
+        elif fused:
+            K.fused_linear(self.w_gu, h, K.LINEAR_SWIGLU, x=xn, act=self.act)   # a decode batch: the same on the matrix cores
         elif (n > 128 and self.runtime.options.get("gemm") != "library"
               and self.hidden % (8 if xn.dtype == torch.bfloat16 else 4) == 0):
             # prompts: the gate in the product's epilogue (up to 128 rows the product with K
@@ -60,4 +65,8 @@ class GatedFeedForward(Part):
         else:
             gu = linear(ctx, xn, self.w_gu, "ffn.gu")
             K.silu_mul(gu, h, self.act)
+        if sink is not None:
+            normed = linear_into(ctx, h, self.w_down, sink, "ffn.down")
+            if normed is not None:
+                return normed
         return linear(ctx, h, self.w_down, "ffn.down")

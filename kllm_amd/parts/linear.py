@@ -108,6 +108,34 @@ def choose(dtype, n, m, k, options=None):
     return K.GEMM_MFMA_BF16, _mfma_split(n, m, k)
 
 
+def linear_into(ctx, x, w, sink, tag):
+    """x . w^T added to the residual stream of ``sink`` in the product's own
+    epilogue, for up to four tokens: returns the ``Normed`` that stands for the
+    norm behind the addition, or None if the kernel with that epilogue does
+    not take these sizes (the caller then returns the product and the norm
+    adds it).  Measured at width 2048: 4 % of a decode step at one token; for
+    decode batches on the matrix cores the same was built and lost 4 % at
+    eight tokens (every workgroup of the consuming product then stages 72 KB
+    of float32 rows where it staged 32 KB of bfloat16), so it stops at four."""
+    from .base import Normed
+    n, k = x.shape
+    m = w.shape[0]
+    rt = ctx.runtime
+    if rt.options.get("no_fused_norm") or rt.options.get("gemm_algo") is not None:
+        return None
+    if rt.options.get("no_fused_gemv"):
+        return None
+    norm = sink.norm
+    if tuple(sink.x.shape) != (n, m) or norm.weight is None or norm.weight.numel() != m:
+        return None
+    parts = K.resid_parts(n, m, k, x.dtype)
+    if parts == 0:
+        return None
+    ss = ctx.buf(tag + ".ss", (n, -(-parts // 4) * 4), torch.float32)
+    K.linear_resid(x, w, sink.x, ss)
+    return Normed(sink.x, ss, parts, norm)
+
+
 def linear(ctx, x, w, tag, out_dtype=torch.float32, split=True):
     """x [n, k] . w [m, k]^T.  With a float32 result and ``split``: partial
     sums [nsplit, n, m] for a consumer that adds them; otherwise one [n, m]

@@ -134,6 +134,7 @@ def test_all_families_agree_with_each_other(model_dirs, dtype):
 @pytest.mark.parametrize("options", [
     {"extra": {"no_fused_gemv": True}},                              # few tokens through the split-K kernels
     {"extra": {"no_fused_gemv": True, "no_fused_linear": True}},     # and without the decode-batch kernel
+    {"extra": {"no_fused_norm": True}},                              # every norm as a launch of its own
     {"attention": "generic"},                                        # the attention kernel that takes every size
     {"gemm": "library"},                                             # prompt-sized products from the vendor library
     {"graphs": False},

@@ -492,6 +492,68 @@ def test_fused_linear_rope_append(H, KV, hd, ps, d):
     assert (q2.cpu().double() - want2).abs().max() < 0.01 * want2.abs().max() + 1e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n", [1, 2, 3, 4])
+@pytest.mark.parametrize("d,kin,f", [(64, 48, 88), (2048, 2048, 5632), (2048, 5632, 256), (104, 264, 72), (4096, 512, 64)])
+def test_a_product_adds_itself_to_the_stream_and_its_consumer_normalises(dtype, n, d, kin, f):
+    """The residual product (x += a . w^T in the epilogue, partial sums of squares left
+    behind) and the consumers that normalise the stream while they stage their input,
+    against the plain add, RMS norm and products, and against the norm kernel's own bits."""
+    k_ = K()
+    parts = k_.resid_parts(n, d, kin, dtype)
+    if parts == 0:
+        pytest.skip("no kernel with a residual epilogue takes these sizes")
+    eps = 1e-5
+    a, w = rnd(n, kin, seed=1, dtype=dtype, scale=0.5), rnd(d, kin, seed=2, dtype=dtype, scale=0.05)
+    x0 = rnd(n, d, seed=3)
+    nw = (1 + 0.2 * rnd(d, seed=4)).contiguous()
+    x = x0.clone()
+    ss = torch.full((n, -(-parts // 4) * 4), float("nan"), device=DEV)
+    assert k_.linear_resid(a, w, x, ss) == parts
+    want_x = x0.cpu().double() + P.linear(a.cpu().double(), w.cpu().double())
+    tol_x = 1e-5 * kin ** 0.5 if dtype == torch.float32 else 1e-4 * kin ** 0.5
+    assert (x.cpu().double() - want_x).abs().max() < tol_x
+    got_ss = ss.cpu().double()[:, :parts].sum(1)
+    assert ((got_ss - (x.cpu().double() ** 2).sum(1)).abs() / got_ss).max() < 1e-5
+    normed = k_.NormedInput(x, nw, ss, parts, eps)
+    xn_kernel = torch.empty(n, d, dtype=dtype, device=DEV)            # the norm kernel on the same stream
+    k_.add_rmsnorm(x.clone(), weight=nw, out=xn_kernel, eps=eps)
+    xn = P.rmsnorm(want_x, nw.cpu().double(), eps)
+    rel = 1e-4 if dtype == torch.float32 else 2e-2
+    # gate + up with the activation
+    wgu = rnd(2 * f, d, seed=5, dtype=dtype, scale=0.1)
+    want_h = P.silu(P.linear(xn, wgu.cpu().double()[:f])) * P.linear(xn, wgu.cpu().double()[f:])
+    h, h2 = (torch.full((n, f), float("nan"), dtype=dtype, device=DEV) for _ in range(2))
+    if k_.gemv_fits(n, 2 * f, d, dtype):
+        k_.gemv_swiglu(normed, wgu, h)
+        k_.gemv_swiglu(xn_kernel, wgu, h2)
+    if not torch.isnan(h).all():
+        assert (h.cpu().double() - want_h).abs().max() < rel * want_h.abs().max() + 1e-4
+        # normalising while staging gives what the norm kernel gives, up to the last bit of the row's scale
+        assert (h.float() - h2.float()).abs().max() <= (1e-5 if dtype == torch.float32 else 0.008) * want_h.abs().max()
+    # q, k, v with rotation and append
+    H, KV, hd, ps = 2, 1, 16, 16
+    wq = rnd((H + 2 * KV) * hd, d, seed=6, dtype=dtype, scale=0.1)
+    pos = torch.arange(3, 3 + n, dtype=torch.int32, device=DEV)
+    sot = torch.zeros(n, dtype=torch.int32, device=DEV)
+    bt = torch.tensor([[1, 0, 2]], dtype=torch.int32, device=DEV)
+    cos, sin = torch.empty(n, hd // 2, device=DEV), torch.empty(n, hd // 2, device=DEV)
+    k_.rope_tables(cos, sin, pos, hd, 10000.0)
+    cache = torch.full((3, 2, KV, ps * hd), float("nan"), dtype=dtype, device=DEV)
+    q = torch.full((n, H * hd), float("nan"), dtype=dtype, device=DEV)
+    k_.gemv_rope_append(normed, wq, q, cos, sin, cache, pos, sot, bt, ps, H, KV, hd)
+    full = P.linear(xn, wq.cpu().double())
+    want_q = P.rope(full[:, :H * hd], pos.cpu().tolist(), H, hd, 10000.0)
+    assert (q.cpu().double() - want_q).abs().max() < rel * full.abs().max() + 1e-4
+    kk, vv = read_cache(cache, [1, 0, 2], 3 + n, KV, hd, ps)
+    want_k = P.rope(full[:, H * hd:(H + KV) * hd], pos.cpu().tolist(), KV, hd, 10000.0)
+    assert (kk[3:].double() - want_k).abs().max() < rel * full.abs().max() + 1e-4
+    assert (vv[3:].double() - full[:, (H + KV) * hd:]).abs().max() < rel * full.abs().max() + 1e-4
+    with pytest.raises(k_.KernelError, match="up to 4 rows"):
+        five = k_.NormedInput(torch.zeros(5, d, device=DEV), nw, torch.zeros(5, ss.shape[1], device=DEV), parts, eps)
+        k_.gemv_swiglu(five, rnd(2 * f, d, seed=5, dtype=torch.float32, scale=0.1), torch.empty(5, f, device=DEV))
+
+
 def test_fused_linear_refuses_what_it_does_not_take():
     k_ = K()
     w = _bf(32, 64, seed=1, scale=0.1)

@@ -8,7 +8,8 @@
 // other path.  Running maximum and sum per query (online softmax), no score
 // matrix in memory, context bounded by pages only.  Formulas as in the generic
 // kernel (reference: backend/model.cu:343-408, window :224-225), in 32-bit;
-// probabilities are rounded to bfloat16 for the product with the values.
+// probabilities are rounded to bfloat16 for the product with the values and
+// their sum is taken over the rounded numbers, as in the decode kernel.
 //
 // The first kernel (attn_prefill_mfma_kernel): a workgroup takes up to 128
 // consecutive tokens of one request (a query block) and one head; each wave of
@@ -256,8 +257,9 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const float p = __builtin_amdgcn_exp2f(fmaf(s[b][i], c2, -mc));   // exp2(-inf) = 0
-        pb[b][i / 8][i % 8] = (bf16_t)p;
-        psum[i % 4] += p;
+        const bf16_t pr = (bf16_t)p;
+        pb[b][i / 8][i % 8] = pr;
+        psum[i % 4] += (float)pr;                                         // the sum of what the values are multiplied with
       }
     l = l * alpha + ((psum[0] + psum[1]) + (psum[2] + psum[3]));
     m = m_new;
@@ -505,8 +507,9 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const float p = __builtin_amdgcn_exp2f(fmaf(s[i], c2, -mc));   // exp2(-inf) = 0
-      pb[i / 8][i % 8] = (bf16_t)p;
-      psum += p;
+      const bf16_t pr = (bf16_t)p;
+      pb[i / 8][i % 8] = pr;
+      psum += (float)pr;                                             // the sum of what the values are multiplied with
     }
     l = l * alpha + psum;
     m = m_new;

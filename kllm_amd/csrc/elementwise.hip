@@ -168,6 +168,11 @@ __global__ void rope_tables_kernel(float* __restrict__ cos_t, float* __restrict_
 // Rotate q and k (pairs (j, j + hd/2), reference: backend/model.cu:170-184),
 // store q, and put k and v into the token's page (reference: :187-201).
 // Page layout, per page and KV head: keys [slot][hd], values [hd][slot].
+// How a head is rotated is data: the first `rot` elements of a head are rotated
+// (the rest pass through), in pairs (j, j + rot/2) or, `interleaved`, (2j, 2j+1);
+// cos and sin are [n][rot/2].  The reference's rotation is rot = hd, not
+// interleaved, which is also what the vector kernel below and the fused
+// epilogues of the small-batch products take.
 template <typename TIN, typename T>
 __global__ void rope_append_kernel(const TIN* __restrict__ qkv, int nsplit, long split_stride,
                                    T* __restrict__ q_out, const float* __restrict__ cos_t,
@@ -175,14 +180,14 @@ __global__ void rope_append_kernel(const TIN* __restrict__ qkv, int nsplit, long
                                    const int* __restrict__ positions,
                                    const int* __restrict__ span_of_token,
                                    const int* __restrict__ block_table, int max_pages,
-                                   int page_size, int H, int KV, int hd) {
+                                   int page_size, int H, int KV, int hd, int rot, int interleaved) {
   const long t = blockIdx.x;
-  const int half = hd / 2;
+  const int half = hd / 2, rhalf = rot / 2;
   const int qd = H * hd, kvd = cache ? KV * hd : 0;
   const long row = qd + 2 * kvd;
   const TIN* in = qkv + t * row;
-  const float* c = cos_t ? cos_t + t * half : nullptr;
-  const float* s = sin_t ? sin_t + t * half : nullptr;
+  const float* c = cos_t ? cos_t + t * rhalf : nullptr;
+  const float* s = sin_t ? sin_t + t * rhalf : nullptr;
   // Items of a token: H*half query pairs, KV*half key pairs, KV*hd values.
   const int q_items = H * half, k_items = cache ? KV * half : 0;
   const int items = q_items + k_items + kvd;
@@ -198,14 +203,18 @@ __global__ void rope_append_kernel(const TIN* __restrict__ qkv, int nsplit, long
       const bool is_q = item < q_items;
       const int idx = is_q ? item : item - q_items;
       const int h = idx / half, j = idx % half;
-      const TIN* src = in + (is_q ? 0 : qd) + h * hd + j;
-      const float a = sum_splits(src, nsplit, split_stride);
-      const float b = sum_splits(src + half, nsplit, split_stride);
-      const float cc = c ? c[j] : 1.f, sn = s ? s[j] : 0.f;
+      // the two elements of this item: a rotated pair, or two that pass through
+      const bool turns = j < rhalf;
+      const int ea = turns ? (interleaved ? 2 * j : j) : rot + 2 * (j - rhalf);
+      const int eb = turns ? (interleaved ? 2 * j + 1 : j + rhalf) : ea + 1;
+      const TIN* src = in + (is_q ? 0 : qd) + h * hd;
+      const float a = sum_splits(src + ea, nsplit, split_stride);
+      const float b = sum_splits(src + eb, nsplit, split_stride);
+      const float cc = (c && turns) ? c[j] : 1.f, sn = (s && turns) ? s[j] : 0.f;
       T* o = is_q ? q_out + t * qd + h * hd
                   : cache + (((long)page * 2 + 0) * KV + h) * block + (long)slot * hd;
-      o[j] = from_f32<T>(a * cc - b * sn);
-      o[j + half] = from_f32<T>(b * cc + a * sn);
+      o[ea] = from_f32<T>(a * cc - b * sn);
+      o[eb] = from_f32<T>(b * cc + a * sn);
     } else {
       const int idx = item - q_items - k_items;
       const int h = idx / hd, j = idx % hd;
@@ -403,11 +412,11 @@ static int launch_rope_append(const void* qkv, int nsplit, long split_stride, vo
                               const float* cos_t, const float* sin_t, void* cache,
                               const int* positions, const int* span_of_token,
                               const int* block_table, int max_pages, int page_size, int n, int H,
-                              int KV, int hd, hipStream_t stream) {
+                              int KV, int hd, int rot, int interleaved, hipStream_t stream) {
   const int items = H * (hd / 2) + (cache ? KV * (hd / 2) + KV * hd : 0);
   int chunks = ceil_div(items, kThreads);
   if ((long)n * chunks > 16384) chunks = ceil_div(16384, n);   // many tokens: fewer, longer workgroups
-  if (sizeof(TIN) == 4 && nsplit == 1 && hd % 8 == 0 && ((uintptr_t)qkv & 15) == 0 &&
+  if (rot == hd && !interleaved && sizeof(TIN) == 4 && nsplit == 1 && hd % 8 == 0 && ((uintptr_t)qkv & 15) == 0 &&
       ((uintptr_t)q_out & 15) == 0 && (!cache || ((uintptr_t)cache & 15) == 0) &&
       (!cos_t || (((uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0)) {
     hipLaunchKernelGGL((rope_append_vec_kernel<T>), dim3(n, ceil_div(items, 4 * kThreads)), dim3(kThreads), 0,
@@ -418,7 +427,7 @@ static int launch_rope_append(const void* qkv, int nsplit, long split_stride, vo
   }
   hipLaunchKernelGGL((rope_append_kernel<TIN, T>), dim3(n, chunks), dim3(kThreads), 0, stream,
                      (const TIN*)qkv, nsplit, split_stride, (T*)q_out, cos_t, sin_t, (T*)cache,
-                     positions, span_of_token, block_table, max_pages, page_size, H, KV, hd);
+                     positions, span_of_token, block_table, max_pages, page_size, H, KV, hd, rot, interleaved);
   KLLM_CHECK_LAUNCH("rope_append");
   return 0;
 }
@@ -427,8 +436,11 @@ extern "C" int kllm_rope_append(const void* qkv, int in_dtype, int nsplit, long 
                                 void* q_out, const float* cos_t, const float* sin_t, void* cache,
                                 const int* positions, const int* span_of_token,
                                 const int* block_table, int max_pages, int page_size, int n, int H,
-                                int KV, int hd, int dtype, hipStream_t stream) {
+                                int KV, int hd, int rot, int interleaved, int dtype, hipStream_t stream) {
   KLLM_REQUIRE(qkv && q_out, "rope_append: null pointer");
+  KLLM_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0 && (interleaved == 0 || interleaved == 1),
+               "rope_append: rotary dimension %d of a head of %d (even, at most the head), interleaved %d", rot, hd,
+               interleaved);
   KLLM_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "rope_append: cos and sin go together");
   KLLM_REQUIRE(n > 0 && H > 0 && hd > 0 && hd % 2 == 0, "rope_append: bad sizes n=%d H=%d hd=%d", n,
                H, hd);
@@ -444,7 +456,7 @@ extern "C" int kllm_rope_append(const void* qkv, int in_dtype, int nsplit, long 
 #define KLLM_RA(TIN, T)                                                                         \
   return launch_rope_append<TIN, T>(qkv, nsplit, split_stride, q_out, cos_t, sin_t, cache,      \
                                     positions, span_of_token, block_table, max_pages, page_size, \
-                                    n, H, KV, hd, stream)
+                                    n, H, KV, hd, rot, interleaved, stream)
   if (in_dtype == DT_F32 && dtype == DT_F32) KLLM_RA(float, float);
   if (in_dtype == DT_F32 && dtype == DT_BF16) KLLM_RA(float, bf16_t);
   if (in_dtype == DT_BF16 && dtype == DT_BF16) KLLM_RA(bf16_t, bf16_t);

@@ -61,13 +61,16 @@ int kllm_rope_tables(float* cos_t, float* sin_t, const int* positions, int n, in
                      double theta, hipStream_t stream);
 
 /* qkv: [nsplit][n][H*hd + 2*KV*hd] (only [n][H*hd] when cache is null).
- * Rotates q and k when cos/sin are given, writes q_out [n][H*hd] and puts k, v
- * into the pages of `cache` ([pages][2][KV][page_size*hd]; keys [slot][hd],
- * values [hd][slot]). */
+ * Rotates q and k when cos/sin ([n][rot/2]) are given, writes q_out [n][H*hd]
+ * and puts k, v into the pages of `cache` ([pages][2][KV][page_size*hd]; keys
+ * [slot][hd], values [hd][slot]).  The first `rot` elements of a head are
+ * rotated (rot even, at most hd; the rest pass through), in pairs (j, j + rot/2)
+ * or, `interleaved`, (2j, 2j + 1). */
 int kllm_rope_append(const void* qkv, int in_dtype, int nsplit, long split_stride, void* q_out,
                      const float* cos_t, const float* sin_t, void* cache, const int* positions,
                      const int* span_of_token, const int* block_table, int max_pages,
-                     int page_size, int n, int H, int KV, int hd, int dtype, hipStream_t stream);
+                     int page_size, int n, int H, int KV, int hd, int rot, int interleaved, int dtype,
+                     hipStream_t stream);
 
 /* The gate's activation of a gated feed-forward (`act` below). */
 #define KLLM_ACT_SILU 0

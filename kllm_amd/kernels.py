@@ -80,7 +80,7 @@ def _declare(lib):
         "kllm_embed": [P, P, P, P, P, I, I, I, I, P],
         "kllm_add_rmsnorm": [P, P, I, I, L, P, P, I, P, I, I, F, I, P],
         "kllm_rope_tables": [P, P, P, I, I, D, P],
-        "kllm_rope_append": [P, I, I, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "kllm_rope_append": [P, I, I, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P],
         "kllm_silu_mul": [P, I, I, L, P, I, I, I, I, P],
         "kllm_gemm": [P, P, P, I, I, I, I, I, I, I, P],
         "kllm_sum_splits": [P, I, L, P, I, P],
@@ -240,8 +240,11 @@ def rope_tables(cos, sin, positions, head_dim, theta):
 
 
 def rope_append(qkv, q_out, cos, sin, cache, positions, span_of_token, block_table, page_size,
-                n_heads, n_kv_heads, head_dim):
-    """qkv [nsplit, n, cols] or [n, cols]; cache [pages, 2, KV, page_size*hd] or None."""
+                n_heads, n_kv_heads, head_dim, rotary_dim=None, interleaved=False):
+    """qkv [nsplit, n, cols] or [n, cols]; cache [pages, 2, KV, page_size*hd] or None.
+    ``rotary_dim`` (default: the head) elements of every head are rotated, in pairs
+    (j, j + rotary_dim/2) or, ``interleaved``, (2j, 2j + 1); cos and sin are [n, rotary_dim/2]."""
+    rot = head_dim if rotary_dim is None else int(rotary_dim)
     n = q_out.shape[0]
     nsplit, stride = 1, 0
     if qkv.dim() == 3:
@@ -256,7 +259,7 @@ def rope_append(qkv, q_out, cos, sin, cache, positions, span_of_token, block_tab
         max_pages = block_table.shape[1]
         if positions.numel() < n or span_of_token.numel() < n:
             raise KernelError("rope_append: index arrays are too short")
-    if cos is not None and (tuple(cos.shape) != (n, head_dim // 2) or tuple(sin.shape) != tuple(cos.shape)):
+    if cos is not None and (tuple(cos.shape) != (n, rot // 2) or tuple(sin.shape) != tuple(cos.shape)):
         raise KernelError("rope_append: cos/sin shapes do not fit")
     _check(library().kllm_rope_append(
         _ptr(qkv, "rope_append qkv"), dtype_code(qkv.dtype), nsplit, stride,
@@ -265,7 +268,8 @@ def rope_append(qkv, q_out, cos, sin, cache, positions, span_of_token, block_tab
         _ptr(positions, "rope_append positions", torch.int32, True),
         _ptr(span_of_token, "rope_append span_of_token", torch.int32, True),
         _ptr(block_table, "rope_append block_table", torch.int32, True), max_pages, page_size, n,
-        n_heads, n_kv_heads, head_dim, dtype_code(q_out.dtype), _stream()), "rope_append")
+        n_heads, n_kv_heads, head_dim, rot, int(bool(interleaved)), dtype_code(q_out.dtype), _stream()),
+        "rope_append")
 
 
 ACT_SILU, ACT_GELU_TANH = 0, 1

@@ -62,6 +62,15 @@ class CausalSelfAttention(Part):
             raise ValueError(f"attention: head_dim {self.head_dim} must be even and at most 256")
         pos = self.param("position", None)
         self.position = runtime.shared_part("position", pos) if pos is not None else None
+        # How the position part wants a head rotated (default: the whole head, halves paired, which
+        # is what the fused epilogues of the small-batch products do; anything else goes through
+        # the separate rotate-and-append kernel, which takes the pairing as arguments).
+        rotates = self.position is not None and hasattr(self.position, "tables")
+        self.rotary_dim = int(getattr(self.position, "rotary_dim", self.head_dim)) if rotates else self.head_dim
+        self.interleaved = bool(getattr(self.position, "interleaved", False)) if rotates else False
+        if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.head_dim:
+            raise ValueError(f"attention: rotary dimension {self.rotary_dim} of a head of {self.head_dim}")
+        self.plain_rotation = self.rotary_dim == self.head_dim and not self.interleaved
         self.scale = 1.0 / math.sqrt(self.head_dim)
         self.q_dim = self.heads * self.head_dim
         self.kv_dim = self.kv_heads * self.head_dim
@@ -97,7 +106,7 @@ class CausalSelfAttention(Part):
             n = xn.rows
             opts = self.runtime.options
             gemv = (K.gemv_fits(n, self.w_in.shape[0], self.hidden, self.runtime.dtype) and n <= K.NORMED_MAX_ROWS
-                    and not opts.get("no_fused_gemv"))
+                    and not opts.get("no_fused_gemv") and self.plain_rotation)
             # the small-batch kernel below normalises while it stages its input
             xn = xn.kernel_input() if gemv else xn.materialize(ctx)
         n = xn.shape[0]
@@ -109,15 +118,16 @@ class CausalSelfAttention(Part):
         cos = sin = None
         if self.position is not None and hasattr(self.position, "tables"):
             cos, sin = self.position.tables(ctx)
+        plain_rotation = self.plain_rotation
         pages = cache.pages if writes else None
         opts = self.runtime.options
-        if K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype) and not opts.get("no_fused_gemv"):
+        if K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype) and not opts.get("no_fused_gemv") and plain_rotation:
             # few tokens: projections, rotation and append in one launch
             K.gemv_rope_append(xn, self.w_in, q, cos, sin, pages, ctx.positions, ctx.span_of_token,
                                cache.block_table, cache.page_size, self.heads, self.kv_heads,
                                self.head_dim)
         elif (dtype == torch.bfloat16 and n <= K.FUSED_ROPE_BEST_ROWS and K.fused_linear_fits(n, self.hidden)
-              and not opts.get("no_fused_linear")):
+              and not opts.get("no_fused_linear") and plain_rotation):
             # a decode batch: the same on the matrix cores
             K.fused_linear(self.w_in, q, K.LINEAR_ROPE, x=xn,
                            rope=K.Rope(cos, sin, pages, ctx.positions, ctx.span_of_token, cache.block_table,
@@ -126,7 +136,7 @@ class CausalSelfAttention(Part):
             qkv = linear(ctx, xn, self.w_in, "attn.qkv")
             K.rope_append(qkv, q, cos, sin, pages, ctx.positions, ctx.span_of_token,
                           cache.block_table, cache.page_size, self.heads, self.kv_heads,
-                          self.head_dim)
+                          self.head_dim, self.rotary_dim, self.interleaved)
         out = ctx.buf("attn.out", (n, self.q_dim), dtype)
         self.attend(ctx, q, out, cache)
         if sink is not None:

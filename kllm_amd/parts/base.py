@@ -21,8 +21,12 @@ sums to be added to x):
                 on_embedding(ctx, x)          optional: acts on the embedded
                                               tokens (additive encodings)
                 tables(ctx) -> (cos, sin)     optional: rotation tables
-                                              [n, head_dim/2] that a mixer
-                                              applies to queries and keys
+                                              [n, rotary_dim/2] that a mixer
+                                              applies to queries and keys;
+                                              ``rotary_dim`` (default: the
+                                              head) and ``interleaved`` (pairs
+                                              (2j, 2j+1) instead of
+                                              (j, j + rotary_dim/2)) say how
   mixer         cache_need() -> CacheNeed | None
                 forward(ctx, xn, cache) -> delta
                   ``cache`` is a PagedCacheView or StateCacheView (or None)

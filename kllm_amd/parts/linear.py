@@ -153,12 +153,14 @@ def linear(ctx, x, w, tag, out_dtype=torch.float32, split=True):
         K.fused_linear(w, y, K.LINEAR_PARTS, x=x, tiles_per_wg=4 if m >= 16384 else 1)
         return y[0]
     if algo == "library":
+        if out_dtype == torch.float32:
+            # float32 sums straight from the library's accumulators: a result that the caller
+            # wants in 32-bit (a residual delta, logits) is never rounded to bfloat16 on the way
+            y32 = ctx.buf(tag + ".f32", (1, n, m), torch.float32)
+            torch.mm(x, w.t(), out_dtype=torch.float32, out=y32[0])
+            return y32[0] if whole else y32
         y = ctx.buf(tag, (n, m), x.dtype)
         torch.matmul(x, w.t(), out=y)
-        if out_dtype == torch.float32:
-            y32 = ctx.buf(tag + ".f32", (1, n, m), torch.float32)
-            y32[0].copy_(y)
-            return y32[0] if whole else y32
         return y
     if (algo == K.GEMM_MFMA_BF16 or algo == K.GEMM_PLAIN
             or (algo == K.GEMM_MFMA_F32 and (nsplit == 1 or not whole))):   # write either dtype themselves

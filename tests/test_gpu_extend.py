@@ -180,10 +180,14 @@ def toy_registered():
         unregister_part(cat, kind)
 
 
-def engine_weights(eng):
+def engine_weights_seed(eng, seed):
     """name -> float32 CPU tensor of what the engine's parts were given."""
     from kllm_amd.weights import random_weights
-    return {k: v.float().cpu() for k, v in random_weights(eng.model.weight_specs(), 5, eng.dtype, "cpu", 0.08, 0.2).items()}
+    return {k: v.float().cpu() for k, v in random_weights(eng.model.weight_specs(), seed, eng.dtype, "cpu", 0.08, 0.2).items()}
+
+
+def engine_weights(eng):
+    return engine_weights_seed(eng, 5)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -468,3 +472,105 @@ def test_a_mixer_with_its_own_tiling_and_a_gelu_gated_feed_forward(dtype):
     finally:
         unregister_architecture("ToyTiledForCausalLM")
         unregister_part("mixer", "toy_tiled")
+
+
+# ----------------------------------------------------------------------------- another rotation
+
+class ToyPartialInterleavedRotary(Part):
+    """Rotates only the first ``rotary_dim`` elements of a head, in neighbouring pairs
+    (2j, 2j + 1), with angles position * base^(-j / pairs): neither the pairing nor the
+    extent of the built-in rotary part.  The tables are made with torch in the test."""
+    interleaved = True
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.rotary_dim, self.base = int(self.param("rotary_dim")), float(self.param("base"))
+
+    @staticmethod
+    def angles(positions, rotary_dim, base):
+        pairs = rotary_dim // 2
+        freq = base ** (-torch.arange(pairs, dtype=torch.float64) / pairs)
+        return positions.double()[:, None] * freq[None, :]
+
+    def prepare(self, ctx):
+        ang = self.angles(ctx.positions[:ctx.n].cpu(), self.rotary_dim, self.base)
+        ctx.scratch[("toy_rot", id(self))] = (torch.cos(ang).float().to(ctx.positions.device).contiguous(),
+                                              torch.sin(ang).float().to(ctx.positions.device).contiguous())
+
+    def tables(self, ctx):
+        return ctx.scratch[("toy_rot", id(self))]
+
+
+ROT_DIM, ROT_BASE = 8, 50.0
+
+
+def build_other_rotation(cfg: LlamaConfig) -> ModelSpec:
+    from kllm_amd.models.llama import build_llama
+    spec = build_llama(cfg)
+    pos = PartSpec("toy_partial_interleaved", rotary_dim=ROT_DIM, base=ROT_BASE)
+    for layer in spec.layers:
+        layer.mixer.params["position"] = pos
+    return spec
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_rotation_with_another_pairing_and_extent(dtype):
+    """A position part that rotates half of each head in neighbouring pairs is registered
+    and used without a change to the package: the attention part reads the pairing from the
+    position part and the rotate-and-append kernel takes it as arguments."""
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry
+    register_part("position", "toy_partial_interleaved", ToyPartialInterleavedRotary)
+    register_architecture("ToyRotationForCausalLM", LlamaConfig, build_other_rotation)
+    try:
+        cfg = dict(tiny.CONFIGS["A"], architectures=["ToyRotationForCausalLM"])
+        eng = Engine.from_random(cfg, 7, EngineOptions(dtype=dtype, max_tokens=256, max_requests=4), std=0.08, norm_std=0.2)
+        w = engine_weights_seed(eng, 7)
+        c = P._cfg(cfg)
+        r = (lambda t: t.to(torch.bfloat16).float()) if dtype == "bfloat16" else (lambda t: t)
+
+        def rotate(x, positions, heads):
+            ang = ToyPartialInterleavedRotary.angles(positions, ROT_DIM, ROT_BASE).float()
+            cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            x = x.view(len(positions), heads, c["hd"]).clone()
+            a, b = x[..., 0:ROT_DIM:2].clone(), x[..., 1:ROT_DIM:2].clone()
+            x[..., 0:ROT_DIM:2] = a * cos - b * sin
+            x[..., 1:ROT_DIM:2] = b * cos + a * sin
+            return x.reshape(len(positions), heads * c["hd"])
+
+        def reference(ids):
+            T = len(ids)
+            pos = torch.arange(T)
+            x = P.embedding(ids, w["model.embed_tokens.weight"])
+            for l in range(c["L"]):
+                p = f"model.layers.{l}."
+                xn = r(P.rmsnorm(x, w[p + "input_layernorm.weight"], c["eps"]))
+                q = r(rotate(P.linear(xn, w[p + "self_attn.q_proj.weight"]), pos, c["H"]))
+                k = r(rotate(P.linear(xn, w[p + "self_attn.k_proj.weight"]), pos, c["KV"]))
+                v = r(P.linear(xn, w[p + "self_attn.v_proj.weight"]))
+                a = r(P.attention(q, k, v, pos, c["H"], c["KV"], c["hd"], store=r if dtype == "bfloat16" else None))
+                x = x + P.linear(a, w[p + "self_attn.o_proj.weight"])
+                xn = r(P.rmsnorm(x, w[p + "post_attention_layernorm.weight"], c["eps"]))
+                x = x + P.swiglu(xn, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
+                                 w[p + "mlp.down_proj.weight"], r if dtype == "bfloat16" else None)
+            return P.linear(r(P.rmsnorm(x, w["model.norm.weight"], c["eps"])), w["lm_head.weight"])
+
+        reqs = {"a": tiny.tokens(cfg, 45, 1), "b": tiny.tokens(cfg, 30, 2), "c": tiny.tokens(cfg, 22, 3)}
+        steps, _ = traces.mixed(reqs, seed=5, max_live=3, tail=6, max_portion=13)
+        outs = []
+        for s in steps:
+            outs.append(eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]]).cpu().numpy())
+            for rid in s["end"]:
+                eng.release(rid)
+        rows = traces.collect(steps, outs)
+        for rid, toks in reqs.items():
+            want = reference(toks)
+            for p in range(len(toks)):
+                err = float((torch.from_numpy(rows[(rid, p)]) - want[p]).abs().max())
+                assert err < (2e-4 if dtype == "float32" else 8e-2), (rid, p, err)
+        # the rotation matters, and so do its pairing and extent: the built-in rotation over the
+        # same weights gives other logits
+        plain = P.forward(w, cfg, reqs["a"])
+        assert float((plain - reference(reqs["a"])).abs().max()) > 0.05
+    finally:
+        unregister_architecture("ToyRotationForCausalLM")
+        unregister_part("position", "toy_partial_interleaved")

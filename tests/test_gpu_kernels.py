@@ -169,6 +169,50 @@ def test_rope_append(dtype, H, KV, hd, ps, nsplit):
 
 # ------------------------------------------------------------------ silu gate
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hd,rot,interleaved", [(16, 16, True), (32, 8, False), (48, 24, True), (64, 0, False), (80, 80, True)])
+def test_rope_append_with_another_pairing_and_extent(dtype, hd, rot, interleaved):
+    """The rotation's pairing and extent are arguments: neighbouring pairs, a part of the
+    head, no rotation at all; what is not rotated passes through."""
+    k_ = K()
+    H, KV, ps, n = 3, 2, 16, 7
+    pos = torch.tensor([5, 6, 7, 0, 40, 41, 15], dtype=torch.int32, device=DEV)
+    sot = torch.tensor([0, 0, 0, 1, 2, 2, 3], dtype=torch.int32, device=DEV)
+    tables = [[3, -1, -1], [5, -1, -1], [1, 0, 4], [2, -1, -1]]
+    bt = torch.tensor(tables, dtype=torch.int32, device=DEV)
+    qd, kvd = H * hd, KV * hd
+    qkv = rnd(2, n, qd + 2 * kvd, seed=4)
+    g = torch.Generator().manual_seed(3)
+    ang = torch.rand(n, rot // 2, generator=g, dtype=torch.float64) * 6.0
+    cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    cache = torch.full((6, 2, KV, ps * hd), float("nan"), dtype=dtype, device=DEV)
+    q_out = torch.full((n, qd), float("nan"), dtype=dtype, device=DEV)
+    k_.rope_append(qkv, q_out, cos if rot else None, sin if rot else None, cache, pos, sot, bt, ps, H, KV, hd, rot, interleaved)
+    full = qkv.cpu().double().sum(0)
+
+    def rotate(x, heads):
+        x = x.reshape(n, heads, hd).clone()
+        ia = torch.arange(0, rot, 2) if interleaved else torch.arange(rot // 2)
+        ib = ia + 1 if interleaved else ia + rot // 2
+        a, b = x[..., ia].clone(), x[..., ib].clone()
+        x[..., ia] = a * torch.cos(ang)[:, None, :] - b * torch.sin(ang)[:, None, :]
+        x[..., ib] = b * torch.cos(ang)[:, None, :] + a * torch.sin(ang)[:, None, :]
+        return x.reshape(n, heads * hd)
+
+    want_q, want_k, want_v = rotate(full[:, :qd], H), rotate(full[:, qd:qd + kvd], KV), full[:, qd + kvd:]
+    t = 1e-5 if dtype == torch.float32 else 0.01 * full.abs().max()
+    assert (q_out.cpu().double() - want_q).abs().max() < t
+    for i in range(n):
+        page, slot = tables[int(sot[i])][int(pos[i]) // ps], int(pos[i]) % ps
+        for h in range(KV):
+            got_k = cache[page, 0, h].view(ps, hd)[slot].cpu().double()
+            got_v = cache[page, 1, h].view(hd, ps)[:, slot].cpu().double()
+            assert (got_k - want_k[i, h * hd:(h + 1) * hd]).abs().max() < t
+            assert (got_v - want_v[i, h * hd:(h + 1) * hd]).abs().max() < t
+    with pytest.raises(k_.KernelError, match="rotary dimension"):
+        k_.rope_append(qkv, q_out, None, None, cache, pos, sot, bt, ps, H, KV, hd, hd + 2, False)
+
+
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nsplit", [1, 2, 4, 7, 8, 11, 16])
 def test_silu_mul(out_dtype, nsplit):

@@ -39,6 +39,8 @@
 // keys [64][hd + 8], values [hd][64 + 4] (tiles of 32 keys for head sizes above 128).
 #include <math.h>
 
+#include <type_traits>
+
 #include "attention_f32.hpp"
 #include "common.hpp"
 #include "kllm_kernels.h"
@@ -47,6 +49,9 @@ namespace kllm {
 
 constexpr int kPrefillWaves = 4;
 constexpr int kQueryBlock = 32 * kPrefillWaves;   // queries of a workgroup
+// Limits of the division-free page arithmetic (page_magic in the first kernel).
+constexpr int kPrefillMaxPage = 2048;
+constexpr int kPrefillMaxKeys = 1 << 24;
 
 template <int HDT>
 struct PrefillShape {
@@ -67,7 +72,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ query_tiles, int n_tiles, const int* __restrict__ span_start,
     const int* __restrict__ span_pos, const int* __restrict__ block_table, int max_pages,
-    int page_size, int H, int KV, int window, float scale) {
+    int page_size, unsigned page_magic, int H, int KV, int window, float scale) {
   typedef PrefillShape<HDT> S;
   constexpr int hd = S::hd, KS = S::KS, NB = S::NB, KT = S::KT, KLD = S::KLD, VLD = S::VLD, CPT = S::CPT;
   extern __shared__ __attribute__((aligned(16))) bf16_t tiles_lds[];   // [PAR][2][kBuf]
@@ -125,9 +130,9 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
   const int ntiles = (ntiles_all + PAR - 1) / PAR;          // steps of the loop: the same for both groups
   auto tile_key = [&](int t) { return kb0 + KT * (PAR * t + par); };   // first key of this group's t-th tile
   // page and slot of a key: a shift and a mask when the page size is a power of two
-  const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
-  auto page_index = [&](int key) { return page_shift >= 0 ? key >> page_shift : key / page_size; };
-  auto page_slot = [&](int key) { return page_shift >= 0 ? key & (page_size - 1) : key % page_size; };
+  // Page of a key without a division: page_magic = ceil(2^35 / page_size) from the host, exact
+  // for keys below 2^24 and pages of up to 2,048 tokens (kPrefillMaxKeys, checked at the launch).
+  auto page_index = [&](int key) { return (int)(__umulhi((unsigned)key, page_magic) >> 3); };
   const int first_page_key = page_index(lowest) * page_size;   // pages before this may be gone
 
   // ---- a tile's way from memory to LDS.  Thread tid moves the same pieces of every tile:
@@ -144,8 +149,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     half_of[j] = __builtin_amdgcn_readfirstlane(i / (2 * hd));
     const int krow = i / (hd / 8), kcol = i % (hd / 8) * 8;
     const int rest = i % (2 * hd), d = rest / 2, part = rest % 2;
-    k_off[j] = (krow % 16) * hd + kcol;                     // from the half's first key row in its page
-    v_off[j] = d * page_size + 8 * part;                    // from the half's first slot of the page's values
+    k_off[j] = ((krow % 16) * hd + kcol) * (int)sizeof(bf16_t);   // bytes from the half's first key row in its page
+    v_off[j] = (d * page_size + 8 * part) * (int)sizeof(bf16_t);  // bytes from the half's first slot of the page's values
     k_lds[j] = krow * KLD + kcol;
     v_lds[j] = KT * KLD + d * VLD + 16 * half_of[j] + 8 * part;
     v_key[j] = 16 * half_of[j] + 8 * part;                  // first key of the values piece, from the tile's
@@ -171,16 +176,25 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     }
     return P;
   };
+  // A page's bytes are addressed from its first: one 64-bit product per page, the rest in 32 bits
+  // (a page of all heads' keys and values is far below 4 GB), so that the scalar unit has little
+  // to do per tile.
+  const unsigned page_bytes = (unsigned)(2 * KV * block * sizeof(bf16_t));
+  const unsigned k_head = (unsigned)(kvh * block * sizeof(bf16_t));
+  const unsigned v_head = (unsigned)((KV + kvh) * block * sizeof(bf16_t));
+  const char* const cache_bytes = reinterpret_cast<const char*>(cache);
   auto fetch = [&](int t, const Pages& P) -> Stage {
     Stage T;
 #pragma unroll
     for (int j = 0; j < CPT; ++j) {
-      const int slot0 = page_slot(tile_key(t) + 16 * half_of[j]);
-      const int page = max(__builtin_amdgcn_readfirstlane(P.page[j]), 0);
-      const bf16_t* kbase = cache + (((long)page * 2 + 0) * KV + kvh) * block + (long)slot0 * hd;
-      const bf16_t* vbase = cache + (((long)page * 2 + 1) * KV + kvh) * block + slot0;
-      T.k[j] = *reinterpret_cast<const bf16x8*>(kbase + k_off[j]);
-      T.v[j] = *reinterpret_cast<const bf16x8*>(vbase + v_off[j]);
+      const int key0 = tile_key(t) + 16 * half_of[j];
+      const unsigned slot0 = (unsigned)(key0 - page_index(key0) * page_size);
+      const unsigned page = (unsigned)max(__builtin_amdgcn_readfirstlane(P.page[j]), 0);
+      const char* pbase = cache_bytes + (unsigned long)page * page_bytes;
+      const unsigned kb_off = k_head + slot0 * (unsigned)(hd * sizeof(bf16_t));
+      const unsigned vb_off = v_head + slot0 * (unsigned)sizeof(bf16_t);
+      T.k[j] = *reinterpret_cast<const bf16x8*>(pbase + (kb_off + (unsigned)k_off[j]));
+      T.v[j] = *reinterpret_cast<const bf16x8*>(pbase + (vb_off + (unsigned)v_off[j]));
     }
     return T;
   };
@@ -211,69 +225,78 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     asm volatile("" ::: "memory");
   };
 
-  auto compute = [&](int t, const bf16_t* buf) {
-    const int kb = tile_key(t);
-    if (!active || kb > w_qmax || kb + KT <= w_lowest) return;   // nothing here for this wave's queries
-    const bool two = NB == 2 && kb + 32 <= w_qmax;            // the second block of 32 keys has keys to read
+  // One tile's arithmetic for this wave's 32 queries.  `masked` is a type (a constant of the
+  // code): tiles whose every key is read by every query of the wave, the bulk, carry no mask.
+  // The vector unit's share is kept small, it bounds the kernel: one multiply-add, one exp2 and
+  // half a conversion per score, a sixth of a three-way maximum; the sum of the probabilities is
+  // a matrix product with ones (of the rounded probabilities, as they multiply the values), and
+  // the output is brought to a new maximum only when the maximum has grown by more than
+  // kGrow binary orders (probabilities then stay below 2^kGrow instead of 1; the quotient at
+  // the end is the same).
+  constexpr float kGrow = 8.f;
+  const bf16_t one = (bf16_t)1.f;
+  const bf16x8 ones = {one, one, one, one, one, one, one, one};
+  const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const float grow_raw = kGrow / c2;                        // kGrow in units of raw scores
+  float mc = 0.f;                                           // m * c2, 0 while m is -inf
+  float m_limit = -INFINITY;                                // m + grow_raw
+  auto tile_math = [&](auto masked, int kb, const bf16_t* buf) {
     // ---- scores: this lane's key rows are kb + c and kb + 32 + c
     floatx16 s[NB];
 #pragma unroll
-    for (int b = 0; b < NB; ++b)
+    for (int kk = 0; kk < KS; ++kk)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s[b][i] = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < KS; ++kk) {
-      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(&buf[c * KLD + 16 * kk + 8 * g]);
-      s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qb[kk], s[0], 0, 0, 0);
-      if (two) {
-        const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(&buf[(32 + c) * KLD + 16 * kk + 8 * g]);
-        s[NB - 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qb[kk], s[NB - 1], 0, 0, 0);
+      for (int b = 0; b < NB; ++b) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&buf[(32 * b + c) * KLD + 16 * kk + 8 * g]);
+        s[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qb[kk], kk == 0 ? zero16 : s[b], 0, 0, 0);
       }
-    }
-    // ---- mask (only where a tile touches an edge), maximum, probabilities.
-    // exp(x) is taken as exp2(x * log2 e) with the hardware's exp2.
-    const bool inner = kb >= my_start && kb + KT - 1 <= qpos && kb + KT <= kv_len;   // no mask needed
-    if (__any(!inner)) {
+    if constexpr (decltype(masked)::value) {
+      const int hi = min(qpos, kv_len - 1) - kb - 4 * g, lo = my_start - kb - 4 * g;   // offsets in the tile this lane's query reads
 #pragma unroll
       for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const int key = kb + 32 * b + 8 * (i / 4) + 4 * g + i % 4;
-          const bool ok = inner || (key <= qpos && key >= my_start);
+          const int e = 32 * b + 8 * (i / 4) + i % 4;
+          const bool ok = (e <= hi) & (e >= lo);
           s[b][i] = ok ? s[b][i] : -INFINITY;
         }
     }
-    float tmax = fmaxf(s[0][0], s[NB - 1][0]);
+    // ---- maximum; exp(x) is taken as exp2(x * log2 e) with the hardware's exp2
+    float tmax = s[0][0];
 #pragma unroll
-    for (int i = 1; i < 16; ++i) tmax = fmaxf(tmax, fmaxf(s[0][i], s[NB - 1][i]));
+    for (int e = 1; e < 16 * NB; ++e) tmax = fmaxf(tmax, s[e / 16][e % 16]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-    const float m_new = fmaxf(m, tmax);                       // in units of raw scores
-    const float mc = (m_new == -INFINITY) ? 0.f : m_new * c2;
-    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m * c2 - mc);
-    bf16x8 pb[NB][2];
-    float psum[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int b = 0; b < NB; ++b)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float p = __builtin_amdgcn_exp2f(fmaf(s[b][i], c2, -mc));   // exp2(-inf) = 0
-        const bf16_t pr = (bf16_t)p;
-        pb[b][i / 8][i % 8] = pr;
-        psum[i % 4] += (float)pr;                                         // the sum of what the values are multiplied with
-      }
-    l = l * alpha + ((psum[0] + psum[1]) + (psum[2] + psum[3]));
-    m = m_new;
-    if (__any(alpha != 1.f)) {
+    const bool grow = tmax > m_limit;                         // never for a maximum of -inf
+    if (__any(grow)) {
+      const float m_new = grow ? tmax : m;
+      const float alpha = grow ? __builtin_amdgcn_exp2f(mc - m_new * c2) : 1.f;   // m = -inf: what was accumulated is 0 anyway
+      const float a0 = (m == -INFINITY) ? 0.f : alpha;
+      l *= a0;
 #pragma unroll
       for (int r = 0; r < HDT; ++r)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[r][i] *= alpha;
+        for (int i = 0; i < 16; ++i) acc[r][i] *= a0;
+      m = m_new;
+      mc = (m == -INFINITY) ? 0.f : m * c2;
+      m_limit = m + grow_raw;
+    }
+    // ---- probabilities, rounded, and their sum
+    bf16x8 pb[NB][2];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        pb[b][i / 8][i % 8] = (bf16_t)__builtin_amdgcn_exp2f(fmaf(s[b][i], c2, -mc));   // exp2(-inf) = 0
+    floatx16 ls = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[0][0], zero16, 0, 0, 0);
+    ls = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[0][1], ls, 0, 0, 0);
+    if (NB == 2) {
+      ls = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[NB - 1][0], ls, 0, 0, 0);
+      ls = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[NB - 1][1], ls, 0, 0, 0);
     }
     // ---- values: half u of block b holds keys kb + 32b + 16u .. + 15
     const bf16_t* vt = buf + KT * KLD;
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      if (b == 1 && !two) break;
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
       for (int r = 0; r < HDT; ++r)
 #pragma unroll
@@ -284,7 +307,16 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
           const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[b][u], acc[r], 0, 0, 0);
         }
-    }
+    l += ls[0];                                               // every row of ls is the sum over the tile's keys
+  };
+  const int w_highstart = (window > 0) ? max(0, w_qmax - window + 1) : 0;   // from here on no query of the wave masks a key below it
+  auto compute = [&](int t, const bf16_t* buf) {
+    const int kb = tile_key(t);
+    if (!active || kb > w_qmax || kb + KT <= w_lowest) return;   // nothing here for this wave's queries
+    if (kb >= w_highstart && kb + KT - 1 <= w_qmin)             // every key for every query of the wave
+      tile_math(std::false_type(), kb, buf);
+    else
+      tile_math(std::true_type(), kb, buf);
   };
 
   constexpr int kAhead = HDT <= 3 ? 2 : 1;                  // large heads leave registers for one
@@ -347,7 +379,6 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
       for (int i = 0; i < 16; ++i) acc[r][i] = acc[r][i] * w0 + mine[(16 * r + i) * kWave] * w1;
   }
   if (!active || c >= nq) return;
-  l += __shfl_xor(l, 32, kWave);
   const float inv = 1.f / l;                                  // finite: a query reads its own key
   bf16_t* orow = out + ((long)tq * H + h) * hd;
 #pragma unroll
@@ -632,9 +663,10 @@ static void launch_prefill_par(int grid, hipStream_t stream, const void* q, void
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     raised = 1;
   }
+  const unsigned page_magic = (unsigned)(((1UL << 35) + page_size - 1) / page_size);   // ceil(2^35 / page_size)
   hipLaunchKernelGGL((attn_prefill_mfma_kernel<HDT, PAR>), dim3(grid), dim3(64 * kPrefillWaves * PAR), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, query_tiles, n_tiles,
-                     span_start, span_pos, block_table, max_pages, page_size, H, KV, window, scale);
+                     span_start, span_pos, block_table, max_pages, page_size, page_magic, H, KV, window, scale);
 }
 
 template <int HDT>
@@ -705,6 +737,9 @@ extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, co
   KLLM_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_prefill: page_size %d must be a multiple of 16",
                page_size);
   KLLM_REQUIRE(max_pages > 0 && window >= 0, "attn_prefill: bad table width or window");
+  KLLM_REQUIRE(page_size <= kPrefillMaxPage && (long)max_pages * page_size <= kPrefillMaxKeys,
+               "attn_prefill: page_size %d x table width %d beyond %d tokens per page or %d per request", page_size,
+               max_pages, kPrefillMaxPage, kPrefillMaxKeys);
   const long items = (long)n_tiles * H;
   KLLM_REQUIRE(items < (1L << 31), "attn_prefill: too many tiles");
   const int grid = (int)items;

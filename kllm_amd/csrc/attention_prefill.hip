@@ -226,7 +226,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
   };
 
   // One tile's arithmetic for this wave's 32 queries.  `masked` is a type (a constant of the
-  // code): tiles whose every key is read by every query of the wave, the bulk, carry no mask.
+  // code): tiles whose every key is read by every query of the wave, the bulk, carry no mask
+  // (head sizes up to 128; for larger ones, where the matrix unit bounds the time, one code).
   // The vector unit's share is kept small, it bounds the kernel: one multiply-add, one exp2 and
   // half a conversion per score, a sixth of a three-way maximum; the sum of the probabilities is
   // a matrix product with ones (of the rounded probabilities, as they multiply the values), and
@@ -267,15 +268,13 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     for (int e = 1; e < 16 * NB; ++e) tmax = fmaxf(tmax, s[e / 16][e % 16]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
     const bool grow = tmax > m_limit;                         // never for a maximum of -inf
-    if (__any(grow)) {
+    const bool any_grow = __any(grow);
+    float a0 = 1.f;
+    if (any_grow) {
       const float m_new = grow ? tmax : m;
       const float alpha = grow ? __builtin_amdgcn_exp2f(mc - m_new * c2) : 1.f;   // m = -inf: what was accumulated is 0 anyway
-      const float a0 = (m == -INFINITY) ? 0.f : alpha;
+      a0 = (m == -INFINITY) ? 0.f : alpha;
       l *= a0;
-#pragma unroll
-      for (int r = 0; r < HDT; ++r)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[r][i] *= a0;
       m = m_new;
       mc = (m == -INFINITY) ? 0.f : m * c2;
       m_limit = m + grow_raw;
@@ -293,27 +292,49 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
       ls = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[NB - 1][0], ls, 0, 0, 0);
       ls = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[NB - 1][1], ls, 0, 0, 0);
     }
-    // ---- values: half u of block b holds keys kb + 32b + 16u .. + 15
+    // ---- values: half u of block b holds keys kb + 32b + 16u .. + 15.  For head sizes up to
+    // 128 the products follow the rescaling inside each branch, not behind their join: the
+    // accumulators then stay where they are on the common path (behind the join the compiler
+    // copies all of them every tile).
     const bf16_t* vt = buf + KT * KLD;
+    auto values = [&]() {
 #pragma unroll
-    for (int b = 0; b < NB; ++b)
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int r = 0; r < HDT; ++r)
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const bf16_t* vrow = vt + (32 * r + c) * VLD + 32 * b + 16 * u + 4 * g;
+            const bf16x4 lo = *reinterpret_cast<const bf16x4*>(vrow);
+            const bf16x4 hi = *reinterpret_cast<const bf16x4*>(vrow + 8);
+            const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[b][u], acc[r], 0, 0, 0);
+          }
+    };
+    auto rescale = [&]() {
 #pragma unroll
       for (int r = 0; r < HDT; ++r)
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const bf16_t* vrow = vt + (32 * r + c) * VLD + 32 * b + 16 * u + 4 * g;
-          const bf16x4 lo = *reinterpret_cast<const bf16x4*>(vrow);
-          const bf16x4 hi = *reinterpret_cast<const bf16x4*>(vrow + 8);
-          const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[b][u], acc[r], 0, 0, 0);
-        }
+        for (int i = 0; i < 16; ++i) acc[r][i] *= a0;
+    };
+    if constexpr (HDT <= 4) {
+      if (any_grow) {
+        rescale();
+        values();
+      } else {
+        values();
+      }
+    } else {                                                  // large heads: their code is long as it is
+      if (any_grow) rescale();
+      values();
+    }
     l += ls[0];                                               // every row of ls is the sum over the tile's keys
   };
   const int w_highstart = (window > 0) ? max(0, w_qmax - window + 1) : 0;   // from here on no query of the wave masks a key below it
   auto compute = [&](int t, const bf16_t* buf) {
     const int kb = tile_key(t);
     if (!active || kb > w_qmax || kb + KT <= w_lowest) return;   // nothing here for this wave's queries
-    if (kb >= w_highstart && kb + KT - 1 <= w_qmin)             // every key for every query of the wave
+    if (HDT <= 4 && kb >= w_highstart && kb + KT - 1 <= w_qmin)   // every key for every query of the wave
       tile_math(std::false_type(), kb, buf);
     else
       tile_math(std::true_type(), kb, buf);

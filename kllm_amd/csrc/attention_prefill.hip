@@ -68,7 +68,7 @@ struct PrefillShape {
 };
 
 template <int HDT, int PAR>  // head_dim = 32 * HDT; PAR groups of four waves
-__global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_waves_per_eu(HDT <= 4 ? 2 : 1))) void attn_prefill_mfma_kernel(
+__global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_waves_per_eu(HDT <= 2 && PAR == 1 ? 3 : (HDT <= 4 ? 2 : 1)))) void attn_prefill_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ query_tiles, int n_tiles, const int* __restrict__ span_start,
     const int* __restrict__ span_pos, const int* __restrict__ block_table, int max_pages,
@@ -340,7 +340,10 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
       tile_math(std::true_type(), kb, buf);
   };
 
-  constexpr int kAhead = HDT <= 3 ? 2 : 1;                  // large heads leave registers for one
+  // Tiles in registers on their way to LDS: two for head size 96; one for the small heads, whose
+  // registers buy a third wave per SIMD instead (8,192 tokens x 32 heads of 64: 469 -> 411 us),
+  // and for the large ones, which have none to spare.
+  constexpr int kAhead = HDT == 3 ? 2 : 1;
   constexpr int kRound = kAhead > 2 ? kAhead : 2;            // steps of a round: even, so that buffers alternate
   bf16_t* const bufs[2] = {tiles_lds + (2 * par) * S::kBuf, tiles_lds + (2 * par + 1) * S::kBuf};
   Pages pg[2];                                              // pg[x % 2]: the pages of tile x, then of x + 2

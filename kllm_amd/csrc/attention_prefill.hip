@@ -531,22 +531,31 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
     return T;
   };
 
+  // The vector unit's share per score as in the first kernel: the sum of the rounded
+  // probabilities is a product with ones, and the output is brought to a new maximum only when
+  // the maximum has grown by more than kGrow binary orders.
+  constexpr float kGrow = 8.f;
+  const bf16_t one = (bf16_t)1.f;
+  const bf16x8 ones = {one, one, one, one, one, one, one, one};
+  const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const float grow_raw = kGrow / c2;                        // kGrow in units of raw scores
+  float mc = 0.f;                                           // m * c2, 0 while m is -inf
+  float m_limit = -INFINITY;                                // m + grow_raw
   auto compute = [&](const Tile& cur, int kb) {
     // ---- scores: this lane's key row is kb + c
     floatx16 s;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) s[i] = 0.f;
-#pragma unroll
     for (int kk = 0; kk < KS; ++kk)
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur.k[kk], qb[kk], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur.k[kk], qb[kk], kk == 0 ? zero16 : s, 0, 0, 0);
     // ---- mask (only where a tile touches an edge), maximum, probabilities.
     // exp(x) is taken as exp2(x * log2 e) with the hardware's exp2.
     const bool inner = kb >= my_start && kb + 31 <= qpos && kb + 32 <= kv_len;   // no mask needed
     if (__any(!inner)) {
+      const int hi = min(qpos, kv_len - 1) - kb - 4 * g, lo = my_start - kb - 4 * g;   // offsets in the tile this lane's query reads
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int key = kb + 8 * (i / 4) + 4 * g + i % 4;
-        const bool ok = inner || (key <= qpos && key >= my_start);
+        const int e = 8 * (i / 4) + i % 4;
+        const bool ok = (e <= hi) & (e >= lo);
         s[i] = ok ? s[i] : -INFINITY;
       }
     }
@@ -554,26 +563,26 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
 #pragma unroll
     for (int i = 1; i < 16; ++i) tmax = fmaxf(tmax, s[i]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-    const float m_new = fmaxf(m, tmax);                       // in units of raw scores
-    const float mc = (m_new == -INFINITY) ? 0.f : m_new * c2;
-    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m * c2 - mc);
-    bf16x8 pb[2];
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float p = __builtin_amdgcn_exp2f(fmaf(s[i], c2, -mc));   // exp2(-inf) = 0
-      const bf16_t pr = (bf16_t)p;
-      pb[i / 8][i % 8] = pr;
-      psum += (float)pr;                                             // the sum of what the values are multiplied with
-    }
-    l = l * alpha + psum;
-    m = m_new;
-    if (__any(alpha != 1.f)) {
+    const bool grow = tmax > m_limit;                         // never for a maximum of -inf
+    if (__any(grow)) {
+      const float m_new = grow ? tmax : m;
+      const float alpha = grow ? __builtin_amdgcn_exp2f(mc - m_new * c2) : 1.f;   // m = -inf: what was accumulated is 0 anyway
+      const float a0 = (m == -INFINITY) ? 0.f : alpha;
+      l *= a0;
 #pragma unroll
       for (int r = 0; r < HDT; ++r)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[r][i] *= alpha;
+        for (int i = 0; i < 16; ++i) acc[r][i] *= a0;
+      m = m_new;
+      mc = (m == -INFINITY) ? 0.f : m * c2;
+      m_limit = m + grow_raw;
     }
+    bf16x8 pb[2];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      pb[i / 8][i % 8] = (bf16_t)__builtin_amdgcn_exp2f(fmaf(s[i], c2, -mc));   // exp2(-inf) = 0
+    floatx16 ls = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[0], zero16, 0, 0, 0);
+    ls = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[1], ls, 0, 0, 0);
     // ---- values: page u of this tile holds keys kb + 16u .. kb + 16u + 15
     const bool v_edge = kb < lowest || kb + 32 > kv_len;     // slots that may hold anything
     if (!v_edge) {
@@ -605,6 +614,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
           acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[u], acc[r], 0, 0, 0);
         }
     }
+    l += ls[0];                                               // every row of ls is the sum over the tile's keys
   };
 
   // A and B take turns, so that no tile is copied from register to register.
@@ -622,8 +632,6 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
     P = pages_of(kb + 3 * kStride);
     compute(B, kb + kStride);
   }
-
-  l += __shfl_xor(l, 32, kWave);
 
   // ---- the waves meet: waves 1..3 leave maximum, sum and output in LDS (lane-contiguous),
   // wave 0 adds them in a fixed order with weights exp(m_w - max m) and writes the tile.

@@ -798,6 +798,24 @@ def test_attention_prefill(H, KV, hd, ps, window, dtype):
     assert torch.isnan(out2.cpu()[~rows2]).all() and torch.equal(out2.cpu()[rows2], out.cpu()[rows2])
 
 
+def test_attention_prefill_refuses_tables_beyond_its_page_arithmetic():
+    """The prompt kernel finds a key's page with a multiplication that is exact for
+    requests of up to 2^24 tokens and pages of up to 2,048: a wider block table or a
+    larger page is refused, not computed wrongly."""
+    k_ = K()
+    c = attention_case(4, 2, 64, 16, torch.bfloat16, 0, [(0, 40)], seed=1)
+    qt = torch.tensor([(0, 0)], dtype=torch.int32, device=DEV)
+    out = torch.empty_like(c["q"])
+    wide = torch.zeros((1, (1 << 24) // 16 + 1), dtype=torch.int32, device=DEV)
+    wide[:, :c["bt"].shape[1]] = c["bt"]
+    with pytest.raises(k_.KernelError, match="per request"):
+        k_.attn_prefill(c["q"], out, c["cache"], qt, 1, c["span_start"], c["span_pos"], wide, c["ps"], c["H"],
+                        c["KV"], c["hd"], 0, c["scale"])
+    k_.attn_prefill(c["q"], out, c["cache"], qt, 1, c["span_start"], c["span_pos"], wide[:, :(1 << 24) // 16],
+                    c["ps"], c["H"], c["KV"], c["hd"], 0, c["scale"])
+    assert (out.cpu().double() - c["want"]).abs().max() < attn_tol(torch.bfloat16)
+
+
 @pytest.mark.parametrize("H,KV,hd,ps", [(24, 4, 32, 16), (24, 3, 64, 16), (22, 2, 96, 32), (22, 11, 128, 16),
                                         (24, 6, 64, 48)])
 @pytest.mark.parametrize("window", [0, 150])

@@ -274,17 +274,22 @@ static void launch_decode(dim3 grid, hipStream_t stream, const void* q, float* p
 
 using namespace kllm;
 
-extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int dtype) {
+extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int dtype, int max_keys) {
   if (KV <= 0 || H <= 0 || n <= 0) return 1;
   if (dtype == DT_F32) return attn_f32_slices(n, KV, H);
   // About eight waves per CU across the chip, shared out over tokens x KV heads x head tiles;
-  // a workgroup is four waves and leaves one partial result.
+  // a workgroup is four waves and leaves one partial result.  A wave should have two tiles of
+  // 16 keys at least: 16 workgroups to a token at contexts of 2,048, more where the caller
+  // says that requests may be longer (one token at 32,768 keys: 37 us with 16, 4 x 128
+  // workgroups otherwise).
   const int head_tiles = (H / KV + 15) / 16;
   long groups = (long)n * KV * head_tiles;
   long want = 8L * device_cus() / (groups > 0 ? groups : 1);
   int wg = (int)((want + kDecodeWaves - 1) / kDecodeWaves);
+  int most = max_keys > 2048 ? max_keys / (32 * kDecodeWaves) : 16;
+  if (most > 256) most = 256;
+  if (wg > most) wg = most;
   if (wg < 1) wg = 1;
-  if (wg > 16) wg = 16;
   return wg;
 }
 

@@ -8,7 +8,8 @@
 namespace kllm {
 
 // out[t, h, :] = sum_s w_s o_s / sum_s w_s l_s with w_s = exp(m_s - max m).
-// One wave per (token, head); eight slices are read at a time.
+// One wave per (token, head); sixteen slices are read at a time (a token's slices are
+// many where contexts are long, and a round of reads costs a trip to memory).
 template <typename T>
 __global__ __launch_bounds__(64) void attn_merge_kernel(T* __restrict__ out,
                                                         const float* __restrict__ part, int H, int hd,
@@ -28,16 +29,16 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(T* __restrict__ out,
   denom = wave_sum(denom);
   for (int d = lane; d < hd; d += kWave) {
     float o = 0.f;
-    for (int s0 = 0; s0 < nslices; s0 += 8) {
-      float ms[8], os[8];
+    for (int s0 = 0; s0 < nslices; s0 += 16) {
+      float ms[16], os[16];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < 16; ++j) {
         const bool ok = s0 + j < nslices;
         ms[j] = ok ? p[(long)(s0 + j) * stride + hd] : -INFINITY;
         os[j] = ok ? p[(long)(s0 + j) * stride + d] : 0.f;
       }
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
+      for (int j = 0; j < 16; ++j)
         if (ms[j] != -INFINITY) o += expf(ms[j] - M) * os[j];
     }
     out[((long)t * H + h) * hd + d] = from_f32<T>(o / denom);

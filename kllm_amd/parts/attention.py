@@ -180,7 +180,12 @@ class CausalSelfAttention(Part):
 
     def _decode(self, ctx, q, out, cache, token_list, count):
         n = q.shape[0]
-        nslices = K.attn_decode_slices(count, self.kv_heads, self.heads, q.dtype)
+        # the block table's width bounds the keys of the step's longest request (a recorded step
+        # is replayed only with tables of its own width)
+        max_keys = cache.block_table.shape[1] * cache.page_size
+        if self.window:
+            max_keys = min(max_keys, self.window + cache.page_size)
+        nslices = K.attn_decode_slices(count, self.kv_heads, self.heads, q.dtype, max_keys)
         part = ctx.buf("attn.part", (n * self.heads * nslices * (self.head_dim + 2),), torch.float32)
         K.attn_decode(q, out, part, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                       cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,

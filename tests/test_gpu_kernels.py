@@ -871,6 +871,22 @@ def test_attention_decode_many_heads_and_slices(H, KV, hd, ps, nslices, dtype):
     assert (out.cpu().double() - c["want"]).abs().max() < attn_tol(dtype)
 
 
+def test_attention_decode_takes_more_slices_for_longer_contexts():
+    """The proposed number of slices grows with the longest context the caller
+    announces (one token over 20,000 keys would otherwise run on 64 workgroups),
+    and the many partial results merge to the same output."""
+    k_ = K()
+    H, KV, hd, ps, dtype = 8, 2, 64, 16, torch.bfloat16
+    few = k_.attn_decode_slices(1, KV, H, dtype, 2048)
+    assert few == k_.attn_decode_slices(1, KV, H, dtype) == 16
+    c = attention_case(H, KV, hd, ps, dtype, 0, [(20000, 1), (37, 1)], seed=9)
+    many = k_.attn_decode_slices(2, KV, H, dtype, c["bt"].shape[1] * ps)
+    assert 100 <= many <= 256
+    for ns in (few, many, 256):
+        out = run_attention("decode", c["q"], c["cache"], c["pos"], c["sot"], c["bt"], ps, H, KV, hd, 0, c["scale"], ns)
+        assert (out.cpu().double() - c["want"]).abs().max() < attn_tol(dtype), ns
+
+
 def standout_case(H, KV, hd, key_pos, ctx_len):
     """One decode token whose query matches exactly one key, far stronger than
     all others (score 40 against about 0): the output must be that key's

@@ -169,23 +169,25 @@ __device__ __forceinline__ floatx16 mfma_tile_step(floatx4 a, floatx4 b, floatx1
 // different slots, so that the 16-byte reads of 16 lanes spread over all 64 banks.
 __device__ __forceinline__ int mfma_swz(int row) { return (row >> 1) & 7; }
 
-template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES>   // WR: rows of waves (1, 2 or 4), two waves a row
-__global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) void gemm_mfma_kernel(const T* __restrict__ X,
+// WR x WC waves, each with WTM x 2 MFMA tiles of 32 x 32: a workgroup's tile is 32 WTM WR rows
+// of X by 64 WC rows of W (128 x 128 with four waves, 256 x 128 and 256 x 256 with eight).
+template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES, int WC = 2, int WTM = 2>
+__global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2))) void gemm_mfma_kernel(const T* __restrict__ X,
                                                              const T* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
                                                              int k, int tiles_x, int tiles_y, int kslice, int act) {
   typedef typename MfmaOperand<T>::type op_t;   // 16 bytes of a row
   constexpr int EPC = 16 / sizeof(T);           // elements of a 16-byte chunk
   constexpr int MBK = MROW / sizeof(T);         // elements of K per stage
-  constexpr int WTM = 2;                        // 32-row MFMA tiles per wave, each way
-  constexpr int BM = 64 * WR;                   // rows of X per workgroup
-  constexpr int NW = 2 * WR;                    // waves
+  constexpr int BM = 32 * WTM * WR;             // rows of X per workgroup
+  constexpr int BN = 64 * WC;                   // rows of W per workgroup
+  constexpr int NW = WR * WC;                   // waves
   constexpr int XI = BM / 8 / NW;               // load instructions of X per wave and stage (8 rows each)
-  constexpr int WI = MBN / 8 / NW;
-  constexpr int XBYTES = BM * MROW, WBYTES = MBN * MROW;
+  constexpr int WI = BN / 8 / NW;
+  constexpr int XBYTES = BM * MROW, WBYTES = BN * MROW;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];   // [MSTAGES][X tile | W tile]
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const int wr = wave / 2, wc = wave % 2;
+  const int wr = wave / WC, wc = wave % WC;
   const long total = (long)tiles_x * tiles_y;
   const long per_xcd = (total + 7) / 8;
   const long id = (long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
   const bool x_major = tiles_x >= tiles_y;
   const long trow = x_major ? id % tiles_y : id / tiles_x;
   const long tcol = x_major ? id / tiles_y : id % tiles_x;
-  const long row0 = trow * BM, col0 = tcol * (DUAL ? MBN / 2 : MBN);
+  const long row0 = trow * BM, col0 = tcol * (DUAL ? BN / 2 : BN);
 
   // Wave w loads rows [8 XI w, 8 XI (w+1)) of the X tile and [8 WI w, 8 WI (w+1)) of the W
   // tile.  In one instruction lane l serves row l / 8 (of 8), slot l % 8.
@@ -210,10 +212,10 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
   }
 #pragma unroll
   for (int i = 0; i < WI; ++i) {
-    const int r = 8 * (WI * wave + i) + lane / 8;             // DUAL: rows 0..63 gate, 64..127 up
+    const int r = 8 * (WI * wave + i) + lane / 8;             // DUAL: the first half of the rows gate, the second up
     wchunk[i] = ((lane % 8) ^ mfma_swz(r)) * EPC;
-    const long col = DUAL ? col0 + r % 64 : col0 + r;
-    const long wrow = min(col, (long)m - 1) + (DUAL && r >= 64 ? m : 0);
+    const long col = DUAL ? col0 + r % (BN / 2) : col0 + r;
+    const long wrow = min(col, (long)m - 1) + (DUAL && r >= BN / 2 ? m : 0);
     wsrc[i] = W + wrow * k + wchunk[i];
   }
   // blockIdx.y: a slice of K (kslice a multiple of a stage); its sums go to Y[blockIdx.y]
@@ -274,7 +276,7 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
       }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const int r = (DUAL ? j * 64 + wc * 32 : wc * 64 + j * 32) + lane % 32;
+        const int r = (DUAL ? j * (BN / 2) + wc * 32 : wc * 64 + j * 32) + lane % 32;
         br[j] = *reinterpret_cast<const op_t*>(ws + r * MROW + (chunk ^ mfma_swz(r)) * 16);
       }
     };
@@ -317,28 +319,30 @@ __global__ __launch_bounds__(128 * WR) __attribute__((amdgpu_waves_per_eu(2))) v
     }
 }
 
-template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES>
+template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES, int WC = 2, int WTM = 2>
 static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, int act,
                             hipStream_t stream) {
   constexpr int MBK = MROW / sizeof(T);
-  const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN), ty = ceil_div(n, 64 * WR);
+  constexpr int BM = 32 * WTM * WR, BN = 64 * WC;
+  const int tx = ceil_div(m, DUAL ? BN / 2 : BN), ty = ceil_div(n, BM);
   const int kslice = ceil_div(ceil_div(k, nsplit), MBK) * MBK;
   const dim3 grid(ceil_div((long)tx * ty, 8) * 8, nsplit);   // padded so that every XCD gets as many
-  const size_t lds = (size_t)MSTAGES * (64 * WR + MBN) * MROW;
+  const size_t lds = (size_t)MSTAGES * (BM + BN) * MROW;
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES, WC, WTM>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) KLLM_FAIL((int)e, "gemm mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = 1;
   }
-  hipLaunchKernelGGL((gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES>), grid, dim3(128 * WR), lds, stream,
+  hipLaunchKernelGGL((gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES, WC, WTM>), grid, dim3(64 * WR * WC), lds, stream,
                      (const T*)x, (const T*)w, (TOUT*)y, n, m, k, tx, ty, kslice, act);
   return 0;
 }
 
 // Tiles of 256 rows of X (eight waves) fetch a quarter less per flop than two tiles of 128;
-// they are taken when they still give every CU two rounds of work.  The thresholds follow
+// they are taken when they still give every CU two rounds of work and the last round is not
+// mostly idle (8,192 x 2,560 x 2,048, two and a half rounds: 113 us against 101 us with 128 rows).  The thresholds follow
 // the chip's number of CUs.
 template <typename T, typename TOUT, bool DUAL>
 static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, int act,
@@ -347,7 +351,19 @@ static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int 
   const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN);
   if (sizeof(T) == 4 && n <= 64)   // a decode batch in float32: tiles of 64 rows, half the products of 128
     return launch_mfma_tile<T, TOUT, DUAL, 1, 2>(x, w, y, n, m, k, nsplit, act, stream);
-  if ((long)ceil_div(n, 256) * tx * nsplit >= 2L * cus)
+  // 256 x 256 tiles (eight waves of 128 x 64, one workgroup a CU) fetch a third less again and
+  // are 10-27 % faster (2,048 x 28,672 x 4,096: 499 us against 561 us) where their rounds fill
+  // the chip: three quarters of the CUs busy on average, counting the last round.  With 80, 128,
+  // 320 or 352 such tiles on 256 CUs they lose by as much.  bfloat16 only: float32 is bound by
+  // its products, not its loads.
+  if constexpr (sizeof(T) == 2) {
+    const long big = (long)ceil_div(n, 256) * ceil_div(m, DUAL ? 128 : 256) * nsplit;
+    const long rounds = ceil_div(big, (long)cus);
+    if (4 * big >= 3 * rounds * cus)
+      return launch_mfma_tile<T, TOUT, DUAL, 2, 2, 4, 4>(x, w, y, n, m, k, nsplit, act, stream);
+  }
+  const long tall = (long)ceil_div(n, 256) * tx * nsplit;
+  if (tall >= 2L * cus && 10 * tall >= 9L * ceil_div(tall, (long)cus) * cus)   // two rounds at least, nine tenths full
     return launch_mfma_tile<T, TOUT, DUAL, 4, 2>(x, w, y, n, m, k, nsplit, act, stream);
   const long tiles = (long)ceil_div(n, 128) * tx * nsplit;
   if (tiles <= cus) return launch_mfma_tile<T, TOUT, DUAL, 2, 3>(x, w, y, n, m, k, nsplit, act, stream);   // one per CU at most

@@ -326,7 +326,9 @@ def _gpu_reference(x, w):
     (1000, 5000, 2056, 3),
     (700, 2100, 264, 1),        # two stages, ragged
     (4096, 4096, 4096, 1),
-    (2048, 32000, 2048, 1),     # the logits of a whole prompt
+    (2048, 32000, 2048, 1),     # the logits of a whole prompt: 256 x 256 tiles (two rounds of them per CU)
+    (1000, 16284, 264, 1),      # 256 x 256 tiles (one full round of them), ragged in every direction
+    (1000, 8100, 520, 2),       # ... in two slices of K
 ])
 @pytest.mark.parametrize("dtype,out_dtype", [(torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16),
                                              (torch.float32, torch.float32)])
@@ -354,7 +356,8 @@ def test_gemm_mfma_at_prompt_sizes(n, m, k, nsplit, dtype, out_dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("n,f,k", [(2048, 5632, 2048), (1000, 2500, 2056), (2048, 14336, 4096), (300, 5632, 2048)])
+@pytest.mark.parametrize("n,f,k", [(2048, 5632, 2048), (1000, 2500, 2056), (2048, 14336, 4096), (300, 5632, 2048),
+                                   (1000, 8100, 264)])    # (2048, 14336, 4096) and the last: 256 x 256 tiles, whole and ragged
 def test_gemm_swiglu_at_prompt_sizes(n, f, k, dtype):
     x, w = rnd(n, k, seed=1, dtype=dtype, scale=0.5), rnd(2 * f, k, seed=2, dtype=dtype, scale=0.05)
     h = torch.full((n, f), float("nan"), dtype=dtype, device=DEV)

@@ -198,7 +198,8 @@ int kllm_attn_decode_static(const void* q, void* out, const void* cache, const i
 
 /* Prompt attention on the matrix cores (bfloat16, or float32 with 32-bit MFMA).
  * query_tiles holds (first token row, span) pairs: up to 128 consecutive tokens
- * of one span. */
+ * of one span.  bfloat16: head sizes 32, 64, 96, 128, 192, 256, pages a multiple
+ * of 16 and of at most 2,048 tokens, max_pages * page_size at most 2^24. */
 int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                       int n_tiles, const int* span_start, const int* span_pos,
                       const int* block_table, int max_pages, int page_size, int H, int KV, int hd,

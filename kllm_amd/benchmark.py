@@ -226,7 +226,7 @@ def measure_prefill_chunks(engine: Engine, tokens: int, chunk: int, reps: int = 
 
 def measure_mixed(engine: Engine, requests: int = 32, min_prompt: int = 128, max_prompt: int = 2048,
                   new_tokens: int = 64, chunk: int = 512, seed: int = 0):
-    """The serving workload the survey names for the 7B sizes: ``requests``
+    """A serving workload for the 7B sizes: ``requests``
     prompts with lengths uniform in [min_prompt, max_prompt] (seeded, ids
     uniform in the vocabulary, as the reference's load generator draws them:
     cmd/loadgen/main.go:98-103), all submitted at once to the scheduler, which

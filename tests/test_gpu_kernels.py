@@ -855,6 +855,49 @@ def test_attention_float32_takes_head_sizes_in_steps_of_8(H, KV, hd, ps, window)
         assert (out.cpu().double() - c["want"]).abs().max() < 2e-5, nslices
 
 
+@pytest.mark.parametrize("H,KV,ps,news", [(66, 2, 16, (260, 200, 129)), (6, 2, 48, (140, 1, 70))])
+def test_attention_prefill_far_into_long_contexts(H, KV, ps, news):
+    """Portions of prompts behind 70,000 cached keys: the page of a key is found by a
+    multiplication instead of a division, and addresses inside a page are 32-bit; both are
+    shown here at large key numbers, for both prompt kernels (many query blocks, few),
+    against the decode kernel, which divides."""
+    k_ = K()
+    hd, dtype = 64, torch.bfloat16
+    spans = list(zip((70000, 65003, 100), news))
+    lens = [a + b for a, b in spans]
+    counts = [-(-L // ps) for L in lens]
+    maxp, num_pages = max(counts), sum(counts) + 2
+    g = torch.Generator(device=DEV).manual_seed(11)
+    cache = torch.full((num_pages, 2, KV, ps * hd), float("nan"), dtype=dtype, device=DEV)
+    tables, used = [], 1
+    for L, cnt in zip(lens, counts):
+        ids = list(range(used + cnt - 1, used - 1, -1))          # a request's pages in falling order
+        used += cnt
+        tables.append(ids + [-1] * (maxp - cnt))
+        kv = torch.randn(2, cnt * ps, KV, hd, generator=g, device=DEV).to(dtype)
+        idx = torch.tensor(ids, device=DEV)
+        cache[idx, 0] = kv[0].view(cnt, ps, KV, hd).permute(0, 2, 1, 3).reshape(cnt, KV, ps * hd)
+        cache[idx, 1] = kv[1].view(cnt, ps, KV, hd).permute(0, 2, 3, 1).reshape(cnt, KV, hd * ps)
+    n = sum(news)
+    q = (torch.randn(n, H * hd, generator=g, device=DEV) * 2).to(dtype)
+    pos = torch.tensor([a + i for a, b in spans for i in range(b)], dtype=torch.int32, device=DEV)
+    sot = torch.tensor([s_ for s_, (_, b) in enumerate(spans) for _ in range(b)], dtype=torch.int32, device=DEV)
+    bt = torch.tensor(tables, dtype=torch.int32, device=DEV)
+    starts = [0]
+    for b in news:
+        starts.append(starts[-1] + b)
+    scale = 1.0 / math.sqrt(hd)
+    want = run_attention("decode", q, cache, pos, sot, bt, ps, H, KV, hd, 0, scale)
+    tiles = [(t, s_) for s_, b in enumerate(news) for t in range(starts[s_], starts[s_] + b, k_.PREFILL_QUERY_BLOCK)]
+    assert (len(tiles) * H > 256) == (H > 6)
+    out = torch.full_like(q, float("nan"))
+    k_.attn_prefill(q, out, cache, torch.tensor(tiles, dtype=torch.int32, device=DEV), len(tiles),
+                    torch.tensor(starts, dtype=torch.int32, device=DEV),
+                    torch.tensor([a for a, _ in spans], dtype=torch.int32, device=DEV), bt, ps, H, KV, hd, 0, scale)
+    assert torch.isfinite(out).all()
+    assert (out.float() - want.float()).abs().max() < attn_tol(dtype)
+
+
 def test_attention_prefill_refuses_what_it_does_not_take():
     k_ = K()
     c = attention_case(2, 1, 48, 16, torch.bfloat16, 0, [(0, 40)])

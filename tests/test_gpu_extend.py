@@ -574,3 +574,145 @@ def test_a_rotation_with_another_pairing_and_extent(dtype):
     finally:
         unregister_architecture("ToyRotationForCausalLM")
         unregister_part("position", "toy_partial_interleaved")
+
+
+# ----------------------------------------------------------------------------- another norm, another arrangement
+
+class ToyCenteredNorm(Part):
+    """y = (x - mean(x)) / sqrt(var(x) + eps) * w + b, written with torch operations.  It
+    takes what every norm takes: a ``delta`` (one tensor or a stack of partial sums over
+    slices of K) that is added into the float32 stream first, or ``rows`` to read."""
+    graph_safe = False
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.size, self.eps = int(self.param("size")), float(self.param("eps"))
+
+    def weight_specs(self):
+        return [WeightSpec(self.tensor_name("weight"), (self.size,), "vector"),
+                WeightSpec(self.tensor_name("bias"), (self.size,), "vector")]
+
+    def bind(self, weights):
+        self.weight, self.bias = weights[self.tensor_name("weight")], weights[self.tensor_name("bias")]
+
+    def add(self, ctx, x, delta):
+        x += delta.sum(0) if delta.dim() == 3 else delta
+        return x
+
+    def normalise(self, x):
+        mu = x.mean(-1, keepdim=True)
+        var = ((x - mu) ** 2).mean(-1, keepdim=True)
+        return (x - mu) / torch.sqrt(var + self.eps) * self.weight + self.bias
+
+    def forward(self, ctx, x, delta=None, rows=None, tag="xn", normed_ok=False):
+        if delta is not None and rows is None:
+            self.add(ctx, x, delta)
+        src = x if rows is None else x[rows.long()]
+        return self.normalise(src).to(self.runtime.dtype)
+
+
+class ToyPostNormBlock(Part):
+    """h = Norm1(h + Mixer(h)); h' = Norm2(h + FeedForward(h)): the norms stand behind the
+    additions and their result is the stream.  Built from the same kinds of parts as the
+    arrangement the package has; leaves nothing pending."""
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        from kllm_amd.parts import make_part
+        layer = self.param("layer")
+        self.norm_mixer = make_part("norm", layer.norm_mixer, runtime)
+        self.mixer = make_part("mixer", layer.mixer, runtime)
+        self.norm_ff = make_part("norm", layer.norm_feed_forward, runtime)
+        self.feed_forward = make_part("feed_forward", layer.feed_forward, runtime)
+
+    graph_safe = False
+
+    def children(self):
+        return [self.norm_mixer, self.mixer, self.norm_ff, self.feed_forward]
+
+    def weight_specs(self):
+        return [s for p in self.children() for s in p.weight_specs()]
+
+    def bind(self, weights):
+        for p in self.children():
+            p.bind(weights)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, ctx, x, pending, cache, next_norm=None):
+        assert pending is None                         # no layer before this kind leaves anything pending
+        dtype = self.runtime.dtype
+        a = self.mixer.forward(ctx, x.to(dtype), cache)
+        x.copy_(self.norm_mixer.forward(ctx, x, delta=a).float())
+        f = self.feed_forward.forward(ctx, x.to(dtype))
+        x.copy_(self.norm_ff.forward(ctx, x, delta=f).float())
+        return x, None
+
+
+def build_post_norm(cfg: LlamaConfig) -> ModelSpec:
+    from kllm_amd.models.llama import build_llama
+    spec = build_llama(cfg)
+    for i, layer in enumerate(spec.layers):
+        layer.block = "toy_post_norm"
+        layer.norm_mixer = PartSpec("toy_centered", f"model.layers.{i}.norm_a", size=cfg.hidden_size, eps=1e-3)
+        layer.norm_feed_forward = PartSpec("toy_centered", f"model.layers.{i}.norm_b", size=cfg.hidden_size, eps=1e-3)
+    spec.final_norm = PartSpec("toy_centered", "model.final", size=cfg.hidden_size, eps=1e-3)
+    return spec
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_norm_with_a_bias_and_an_arrangement_with_the_norms_behind_the_additions(dtype):
+    """Another norm (centred, with a bias) and another arrangement of a layer (post-norm) are
+    registered from here and run with the package's attention and feed-forward: mixed
+    steps with page reuse against a plain computation of the same formulas."""
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry
+    register_part("norm", "toy_centered", ToyCenteredNorm)
+    register_part("block", "toy_post_norm", ToyPostNormBlock)
+    register_architecture("ToyPostNormForCausalLM", LlamaConfig, build_post_norm)
+    try:
+        cfg = dict(tiny.CONFIGS["B"], architectures=["ToyPostNormForCausalLM"])
+        eng = Engine.from_random(cfg, 5, EngineOptions(dtype=dtype, max_tokens=192, max_requests=4),
+                                 std=0.08, norm_std=0.2)
+        w = engine_weights(eng)
+        assert "model.layers.0.norm_a.bias" in w and "model.final.weight" in w
+        r = (lambda t: t.to(torch.bfloat16).float()) if dtype == "bfloat16" else (lambda t: t)
+        c = P._cfg(cfg)
+
+        def centred(x, name):
+            mu = x.mean(-1, keepdim=True)
+            var = ((x - mu) ** 2).mean(-1, keepdim=True)
+            return (x - mu) / torch.sqrt(var + 1e-3) * w[name + ".weight"] + w[name + ".bias"]
+
+        def reference(ids):
+            x = P.embedding(ids, w["model.embed_tokens.weight"])
+            pos = torch.arange(len(ids))
+            for i in range(c["L"]):
+                p = f"model.layers.{i}."
+                a, _ = P.attention_sublayer(w, p, r(x), pos, c, store=r if dtype == "bfloat16" else None)
+                x = r(centred(x + a, p + "norm_a"))
+                f = P.swiglu(r(x), w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
+                             w[p + "mlp.down_proj.weight"], r if dtype == "bfloat16" else None)
+                x = r(centred(x + f, p + "norm_b"))
+            head = w["model.embed_tokens.weight"] if c["tied"] else w["lm_head.weight"]
+            return P.linear(r(centred(x, "model.final")), head)
+
+        reqs = {"a": tiny.tokens(cfg, 45, 1), "b": tiny.tokens(cfg, 30, 2), "c": tiny.tokens(cfg, 22, 3),
+                "d": tiny.tokens(cfg, 37, 4)}
+        steps, _ = traces.mixed(reqs, seed=5, max_live=3, tail=6, max_portion=11)
+        outs = []
+        for s in steps:
+            outs.append(eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]]).cpu().numpy())
+            for rid in s["end"]:
+                eng.release(rid)
+        rows = traces.collect(steps, outs)
+        for rid, toks in reqs.items():
+            want = reference(toks)
+            for p in range(len(toks)):
+                err = float((torch.from_numpy(rows[(rid, p)]) - want[p]).abs().max())
+                assert err < (2e-4 if dtype == "float32" else 8e-2), (rid, p, err)
+        assert not eng.cache.requests
+    finally:
+        unregister_architecture("ToyPostNormForCausalLM")
+        unregister_part("block", "toy_post_norm")
+        unregister_part("norm", "toy_centered")

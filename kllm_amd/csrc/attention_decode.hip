@@ -276,7 +276,7 @@ using namespace kllm;
 
 extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int dtype, int max_keys) {
   if (KV <= 0 || H <= 0 || n <= 0) return 1;
-  if (dtype == DT_F32) return attn_f32_slices(n, KV, H);
+  if (dtype == DT_F32) return attn_f32_slices(n, KV, H, max_keys);
   // About eight waves per CU across the chip, shared out over tokens x KV heads x head tiles;
   // a workgroup is four waves and leaves one partial result.  A wave should have two tiles of
   // 16 keys at least: 16 workgroups to a token at contexts of 2,048, more where the caller

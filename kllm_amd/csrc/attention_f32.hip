@@ -357,14 +357,20 @@ bool attn_f32_fits(int hd, int page_size) {
   return hd >= 8 && hd <= 256 && hd % 8 == 0 && page_size > 0 && page_size % 4 == 0;
 }
 
-int attn_f32_slices(int n, int KV, int H) {
-  // About four waves per CU across the chip, shared out over tokens x KV heads x blocks of 32
-  // heads; a slice is one wave.
+int attn_f32_slices(int n, int KV, int H, int max_keys) {
+  // About four waves per CU across the chip (eight from one group per CU on, where partial
+  // results cost little beside the keys), shared out over tokens x KV heads x blocks of 32
+  // heads; a slice is one wave and should have 32 keys at least (measured: 64 tokens at 2,048
+  // keys 61 us with 8 slices against 68 with 4; one token at 32,768 keys 47 us with 256 against
+  // 69 with 64; 8 tokens at 512 keys 13 us with 16 against 15 with 32).
   const int col_blocks = (H / KV + 31) / 32;
   const long groups = (long)n * KV * col_blocks;
-  long want = 4L * device_cus() / (groups > 0 ? groups : 1);
+  const int cus = device_cus();
+  long want = (groups >= cus ? 8L : 4L) * cus / (groups > 0 ? groups : 1);
+  long most = max_keys > 0 ? max_keys / 32 : 64;
+  if (most > kAttnF32MaxSlices) most = kAttnF32MaxSlices;
+  if (want > most) want = most;
   if (want < 1) want = 1;
-  if (want > 64) want = 64;
   return (int)want;
 }
 

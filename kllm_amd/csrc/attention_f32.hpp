@@ -27,7 +27,8 @@ int attn_f32_prefill(const float* q, float* out, const float* cache, const int* 
                      const int* span_start, const int* span_pos, const int* block_table, int max_pages,
                      int page_size, int H, int KV, int hd, int window, float scale, hipStream_t stream);
 
-// Slices proposed for a decode batch of n tokens.
-int attn_f32_slices(int n, int KV, int H);
+// Slices proposed for a decode batch of n tokens whose longest request has at most max_keys
+// keys (0: unknown).
+int attn_f32_slices(int n, int KV, int H, int max_keys);
 
 }  // namespace kllm

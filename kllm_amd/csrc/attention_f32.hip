@@ -62,6 +62,7 @@ struct AttnF32Args {
   int max_pages, page_size, H, KV, hd, window;
   float scale;
   int nslices, col_blocks;     // decode: slices of the keys, blocks of 32 heads per group
+  int wg_merge;                // decode: a workgroup's four slices leave one partial result
 };
 
 template <int HDT, bool DECODE>   // head_dim <= 32 * HDT
@@ -289,6 +290,52 @@ __global__ __launch_bounds__(64 * kF32Waves) void attn_f32_mfma_kernel(const Att
     }
   }
   l += __shfl_xor(l, 32, kWave);
+  if (DECODE && a.wg_merge) {
+    // The four waves of a workgroup hold four neighbouring slices of the same token and heads
+    // (the number of slices is a multiple of four): they meet in LDS, each in the place of its
+    // queries, and leave one partial result, so that the second kernel reads a quarter.
+    if (col_ok) {
+#pragma unroll
+      for (int r = 0; r < HDT; ++r)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const int d = 32 * r + 8 * b + 4 * g;
+          if (d < hd) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) qs[c * QLD + d + j] = acc[r][4 * b + j];
+          }
+        }
+      if (g == 0) {
+        qs[c * QLD + hd] = m;                                // -inf and 0 for a slice without keys
+        qs[c * QLD + hd + 1] = l;
+      }
+    }
+    __syncthreads();
+    const int nout = nslices / kF32Waves, sout = slice / kF32Waves;
+    for (int idx = threadIdx.x; idx < ncol * hd; idx += 64 * kF32Waves) {
+      const int col = idx / hd, d = idx % hd;
+      float mw[kF32Waves], M = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < kF32Waves; ++w) {
+        mw[w] = q_lds[(w * 32 + col) * QLD + hd];
+        M = fmaxf(M, mw[w]);
+      }
+      float o = 0.f, L = 0.f;
+#pragma unroll
+      for (int w = 0; w < kF32Waves; ++w) {
+        const float wt = mw[w] == -INFINITY ? 0.f : expf(mw[w] - M);
+        o += wt * q_lds[(w * 32 + col) * QLD + d];
+        L += wt * q_lds[(w * 32 + col) * QLD + hd + 1];
+      }
+      float* prow = a.part + (((long)t_base * H + h_base + col) * nout + sout) * (hd + 2);
+      prow[d] = o;
+      if (d == 0) {
+        prow[hd] = M;
+        prow[hd + 1] = L;
+      }
+    }
+    return;
+  }
   if (!col_ok) return;
 
   // acc[r][i] is output element 32r + 8(i/4) + 4g + i%4 of this lane's column
@@ -389,12 +436,13 @@ int attn_f32_decode(const float* q, float* out, float* part, const float* cache,
   a.block_table = block_table; a.count = count;
   a.max_pages = max_pages; a.page_size = page_size; a.H = H; a.KV = KV; a.hd = hd; a.window = window;
   a.scale = scale; a.nslices = nslices; a.col_blocks = (H / KV + 31) / 32;
+  a.wg_merge = nslices % kF32Waves == 0;
   const long items = (long)count * KV * a.col_blocks * nslices;
   if (int rc = dispatch_f32<true>(a, items, stream)) return rc;
   KLLM_CHECK_LAUNCH("attn_decode float32");
   if (nslices > 1) {
-    hipLaunchKernelGGL(attn_merge_kernel<float>, dim3(count, H), dim3(64), 0, stream, out, part, H, hd, nslices,
-                       token_list);
+    hipLaunchKernelGGL(attn_merge_kernel<float>, dim3(count, H), dim3(64), 0, stream, out, part, H, hd,
+                       a.wg_merge ? nslices / kF32Waves : nslices, token_list);
     KLLM_CHECK_LAUNCH("attn_merge float32");
   }
   return 0;

@@ -180,9 +180,14 @@ class CausalSelfAttention(Part):
 
     def _decode(self, ctx, q, out, cache, token_list, count):
         n = q.shape[0]
-        # the block table's width bounds the keys of the step's longest request (a recorded step
-        # is replayed only with tables of its own width)
-        max_keys = cache.block_table.shape[1] * cache.page_size
+        # The block table's width bounds the keys of the step's longest request.  It is rounded up
+        # to a power of two of pages (from 8), as recorded steps round theirs: a step then cuts
+        # the keys alike, and gives the same sums bit for bit, whether it runs directly or as
+        # a replayed recording with a wider table.
+        pages = 8
+        while pages < cache.block_table.shape[1]:
+            pages *= 2
+        max_keys = pages * cache.page_size
         if self.window:
             max_keys = min(max_keys, self.window + cache.page_size)
         nslices = K.attn_decode_slices(count, self.kv_heads, self.heads, q.dtype, max_keys)

@@ -25,6 +25,7 @@ recording clears memory with a memset node.
 
 from __future__ import annotations
 
+import gc
 from collections import OrderedDict
 from typing import List, Sequence
 
@@ -156,8 +157,17 @@ class DecodeGraphs:
                 out = self._read_back(batch, rec.logits)
                 out.tokens()                            # before the capture's second run of the kernels
                 graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph, capture_error_mode="thread_local"):
-                    self._run(rec, lens, pos0)          # recorded, not executed
+                # No collection of garbage while recording: it may destroy the recordings of an
+                # engine that is no longer used, which HIP refuses on a thread that records, and
+                # the error leaves a destructor and ends the process.
+                collecting = gc.isenabled()
+                gc.disable()
+                try:
+                    with torch.cuda.graph(graph, capture_error_mode="thread_local"):
+                        self._run(rec, lens, pos0)      # recorded, not executed
+                finally:
+                    if collecting:
+                        gc.enable()
                 rec.graph = graph
                 self.captures += 1
             else:

@@ -216,6 +216,39 @@ def test_a_step_queued_ahead_takes_its_ids_from_the_device(model_dirs, dtype):
         assert [[step[i] for step in runs[1]] for i in range(3)] == want
 
 
+def test_no_collection_of_garbage_falls_into_a_recording(model_dirs):
+    """An engine that is dropped is garbage in a reference cycle, its recorded steps with
+    it.  HIP refuses to destroy a graph on a thread that records one, and the error would
+    leave a destructor and end the process, so a collection must not start while a later
+    engine records: with the collector set to run at every allocation, none does."""
+    import gc
+    from kllm_amd.engine import Engine, EngineOptions
+    cfg, d = tiny.CONFIGS["A"], model_dirs("A")
+    prompt = tiny.tokens(cfg, 9, 3)
+    started = []
+
+    def watch(phase, info):
+        if phase == "start":
+            started.append(torch.cuda.is_current_stream_capturing())
+
+    before = gc.get_threshold()
+    outs = []
+    gc.callbacks.append(watch)
+    try:
+        for _ in range(2):
+            eng = Engine.from_dir(d, EngineOptions(dtype="float32", max_tokens=128))
+            gc.set_threshold(1, 1, 1)
+            outs.append(eng.generate(prompt, 6))
+            gc.set_threshold(*before)
+            assert eng._graphs.captures > 0
+            del eng
+    finally:
+        gc.set_threshold(*before)
+        gc.callbacks.remove(watch)
+    assert len(started) > 10 and not any(started)
+    assert outs[0] == outs[1] == P.generate_greedy(tiny.read_weights(d), cfg, prompt, 6)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(model_dirs, dtype):
     """One token per step for 400 steps, past several pages and past the

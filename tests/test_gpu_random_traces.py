@@ -3,7 +3,8 @@ configuration, the page size, the number and lengths of requests and the way of
 cutting them (whole, a bulk and single tokens, portions of random sizes, mixed
 with up to four live requests on a pool that just holds them) are all drawn
 from a seed.  The fixed traces of the other tests hold the cases that were
-thought of; these hold the ones that were not."""
+thought of; these hold the ones that were not.  A second test draws the
+configuration itself, every size of it."""
 
 import random
 
@@ -82,3 +83,59 @@ def test_random_traces_match_the_plain_implementation(tmp_path, dtype):
                 assert err < TOL_RANDOM[dtype], f"{case}: {rid} position {p} off by {err}"
         seen.add((name, family))
     assert len({n for n, _ in seen}) == 5 and len({f for _, f in seen}) == 4
+
+
+def draw_configuration(seed):
+    """Every size of the architecture drawn: heads and groups, head sizes in
+    steps of 16, widths and vocabularies that are no multiple of anything."""
+    rng = random.Random(seed)
+    heads = rng.randint(1, 12)
+    groups = rng.choice([g for g in range(1, heads + 1) if heads % g == 0])
+    hidden = rng.choice([rng.randint(16, 400), 8 * rng.randint(2, 50), 64 * rng.randint(1, 8)])
+    cfg = tiny._cfg(
+        num_hidden_layers=rng.randint(1, 3), hidden_size=hidden, num_attention_heads=heads,
+        num_key_value_heads=groups,
+        head_dim=rng.choice([16, 32, 48, 64, 64, 80, 96, 112, 128, 128, 144, 160, 192, 256]),
+        intermediate_size=rng.choice([rng.randint(8, 700), 8 * rng.randint(1, 90), 128 * rng.randint(1, 6)]),
+        vocab_size=rng.choice([rng.randint(20, 3000), 64 * rng.randint(1, 40)]),
+        rope_theta=rng.choice([1000.0, 10000.0, 500000.0]), max_position_embeddings=4096,
+        rms_norm_eps=rng.choice([1e-6, 1e-5, 1e-3]), tie_word_embeddings=rng.random() < 0.4)
+    page = rng.choice([16, 16, 32, 64, 128, 8, 20])
+    lengths = [rng.randint(1, rng.choice([30, 120, 300])) for _ in range(rng.randint(1, 4))]
+    requests = {f"r{i}": tiny.tokens(cfg, n, seed * 100 + i) for i, n in enumerate(lengths)}
+    steps, peak = traces.mixed(requests, seed=seed, max_live=rng.randint(1, 4),
+                               tail=rng.choice([0, 3, 12]), max_portion=rng.choice([5, 24, 70, 200]))
+    return cfg, page, requests, steps, peak
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_random_configurations_match_the_plain_implementation(tmp_path, dtype):
+    """Weights of deviation 0.4 / sqrt(width), so that logits are of size 1 to 2
+    at every width; the bound counts in units of the largest logit.  Over 6,500
+    such configurations the worst was 2.2e-6 in float32 and, from a width of 16
+    on, 1.3e-2 in bfloat16."""
+    from kllm_amd.engine import EngineOptions
+    from kllm_amd.replay import Replayer
+    for seed in range(64):
+        cfg, page, requests, steps, peak = draw_configuration(seed)
+        case = f"seed {seed}: pages of {page}, {[len(t) for t in requests.values()]}, {cfg}"
+        print(case, flush=True)
+        folder = tiny.write_model(str(tmp_path / str(seed)), cfg, seed,
+                                  std=0.4 / cfg["hidden_size"] ** 0.5)
+        pool = peak + page * 4
+        options = EngineOptions(dtype=dtype, max_tokens=pool, max_model_len=1 << 30,
+                                poison_freed_pages=True, page_size=page)
+        rep = Replayer(folder, dtype, pool, options=options)
+        outs = [rep.step(s["entries"], s["end"]) for s in steps]
+        rep.engine.cache.check_invariants()
+        assert not rep.engine.cache.requests, case
+        rows = traces.collect(steps, outs)
+        weights = tiny.read_weights(folder, as_stored_in=dtype)
+        for rid, toks in requests.items():
+            want = P.forward(weights, cfg, toks).numpy()
+            bound = TOL_RANDOM[dtype] * max(1.0, float(np.abs(want).max()))
+            for p in range(len(toks)):
+                got = rows[(rid, p)]
+                assert np.isfinite(got).all(), f"{case}: {rid} position {p}"
+                err = float(np.abs(got - want[p]).max())
+                assert err < bound, f"{case}: {rid} position {p} off by {err}"

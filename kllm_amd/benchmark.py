@@ -370,7 +370,7 @@ def bench_kernel(name: str, shape, dtype: str = "bfloat16", reps: int = 50, warm
             nbytes = (2 * tokens * H * hd + 2 * tokens * KV * hd) * elem
         else:
             posn, sot = i32([ctx - 1] * batch), i32(list(range(batch)))
-            ns = K.attn_decode_slices(batch, KV, H, td, ctx)
+            ns = K.attn_decode_slices(batch, KV, H, hd, td, ctx)
             part = torch.empty(batch * H * ns * (hd + 2), dtype=torch.float32, device=dev)
             fn = lambda: K.attn_decode(q, out, part, cache, posn, sot, bt, ps, H, KV, hd, 0, scale, ns)
             flops = 4.0 * batch * H * hd * ctx

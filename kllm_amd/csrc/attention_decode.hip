@@ -2,10 +2,12 @@
 //
 // One wave takes one token, one KV head with up to 16 of its query heads, and
 // one slice of the token's keys; it streams that slice's pages from memory
-// once, for all heads of the group.  The four waves of a workgroup merge their
-// results in LDS and leave one partial result (running maximum, sum,
-// unnormalised output); a second kernel merges the workgroups' partials.  The
-// launch does not depend on any context length, so a recorded step can be
+// once, for all heads of the group.  The waves of a workgroup (sixteen for
+// heads up to 64, fewer where a wave needs more registers) merge their results
+// in LDS.  Where one workgroup covers all keys of its token it writes the
+// output itself; otherwise it leaves one partial result (running maximum, sum,
+// unnormalised output) and a second kernel merges the workgroups' partials.
+// The launch does not depend on any context length, so a recorded step can be
 // replayed as contexts grow.
 //
 // Formulas as in the generic kernel (reference: backend/model.cu:343-408):
@@ -30,7 +32,14 @@
 
 namespace kllm {
 
-constexpr int kDecodeWaves = 4;
+// Waves of a workgroup: four where a token's keys are shared out over several workgroups
+// (small batches: many small workgroups start sooner than few large ones; 8 tokens at 2,048
+// keys: 6.4 us with 16 workgroups of 4 waves to a token and KV head, 9.7 us with 4 of 16),
+// and as many as the registers of a wave allow (a workgroup of 1,024 threads leaves each 128)
+// where one workgroup takes all keys of its token and writes the output itself (64 tokens:
+// 26.1 us against 25.6 + 5.6 us for two workgroups and their merge).
+constexpr int kDecodeWavesShared = 4;
+constexpr int decode_waves_whole(int hdt) { return hdt <= 4 ? 16 : (hdt <= 8 ? 8 : 4); }
 // Tiles of 32 keys in a group; two groups are in registers.
 constexpr int decode_ahead(int hdt) { return 1; }
 
@@ -43,9 +52,10 @@ __device__ __forceinline__ float group4_sum(float v) {
   return v + __shfl_xor(v, 32, kWave);
 }
 
-template <int HDT>  // head_dim = 16 * HDT
+template <int HDT, int kDecodeWaves>  // head_dim = 16 * HDT
 __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
-    const bf16_t* __restrict__ q, float* __restrict__ part, const bf16_t* __restrict__ cache,
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ final_out, float* __restrict__ part,
+    const bf16_t* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token,
     const int* __restrict__ block_table, int max_pages, int page_size, int H, int KV, int window,
     float scale, int head_tiles, const int* __restrict__ token_list) {
@@ -213,80 +223,99 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
 
   l = group4_sum(l);
 
-  // ---- the four waves' results meet in LDS; wave 0 merges them in a fixed order and
-  // writes the workgroup's partial result
-  __shared__ float red[(kDecodeWaves - 1) * 16 * (hd + 2)];
-  if (wave > 0) {
-    float* mine = red + ((wave - 1) * 16 + c) * (hd + 2);
+  // ---- the waves' results meet in LDS; then a thread merges, in the order of the waves,
+  // four elements of one head and writes them: the output itself where this workgroup had
+  // all the keys, else the workgroup's partial result
+  extern __shared__ __attribute__((aligned(16))) float red[];   // [waves][heads of the tile][hd + 4]
+  constexpr int RS = hd + 4;                                 // row stride: 16-byte rows
+  const int heads_here = min(16, G - ht * 16);
+  if (head_ok) {
+    float* mine = red + (wave * heads_here + c) * RS;
 #pragma unroll
-    for (int r = 0; r < HDT; ++r)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) mine[16 * r + 4 * g + i] = acc[r][i];
+    for (int r = 0; r < HDT; ++r) *reinterpret_cast<floatx4*>(mine + 16 * r + 4 * g) = acc[r];
     if (g == 0) {
       mine[hd] = m;
       mine[hd + 1] = l;
     }
   }
   __syncthreads();
-  if (wave > 0 || !head_ok) return;
-  float mj[kDecodeWaves - 1], M = m;
+  const bool whole = gridDim.z == 1;
+  constexpr int CH = hd / 4;                                 // pieces of four elements in a head
+  for (int idx = threadIdx.x; idx < heads_here * CH; idx += 64 * kDecodeWaves) {
+    const int hc = idx / CH, d4 = (idx % CH) * 4;
+    const float* col = red + hc * RS;
+    float mj[kDecodeWaves], M = -INFINITY;
 #pragma unroll
-  for (int j = 0; j < kDecodeWaves - 1; ++j) {
-    mj[j] = red[(j * 16 + c) * (hd + 2) + hd];
-    M = fmaxf(M, mj[j]);
-  }
-  const bool any = M != -INFINITY;                          // a workgroup beyond the last key has nothing
-  const float w0 = any ? expf(m - M) : 0.f;
-  float wj[kDecodeWaves - 1];
-  l *= w0;
-#pragma unroll
-  for (int j = 0; j < kDecodeWaves - 1; ++j) {
-    wj[j] = any ? expf(mj[j] - M) : 0.f;
-    l += wj[j] * red[(j * 16 + c) * (hd + 2) + hd + 1];
-  }
-  float* out = part + (((long)t * H + head) * gridDim.z + blockIdx.z) * (hd + 2);
-#pragma unroll
-  for (int r = 0; r < HDT; ++r)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float v = acc[r][i] * w0;
-#pragma unroll
-      for (int j = 0; j < kDecodeWaves - 1; ++j) v += wj[j] * red[(j * 16 + c) * (hd + 2) + 16 * r + 4 * g + i];
-      out[16 * r + 4 * g + i] = v;
+    for (int j = 0; j < kDecodeWaves; ++j) {
+      mj[j] = col[j * heads_here * RS + hd];
+      M = fmaxf(M, mj[j]);
     }
-  if (g == 0) {
-    out[hd] = M;
-    out[hd + 1] = l;
+    const bool any = M != -INFINITY;                         // a workgroup beyond the last key has nothing
+    floatx4 v = {0.f, 0.f, 0.f, 0.f};
+    float L = 0.f;
+#pragma unroll
+    for (int j = 0; j < kDecodeWaves; ++j) {
+      const float* w = col + j * heads_here * RS;
+      const float wj = any ? expf(mj[j] - M) : 0.f;
+      L += wj * w[hd + 1];
+      v += wj * *reinterpret_cast<const floatx4*>(w + d4);
+    }
+    const int head_o = kvh * G + ht * 16 + hc;
+    if (whole) {
+      const float inv = 1.f / L;
+      bf16x4 o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = (bf16_t)(v[i] * inv);
+      *reinterpret_cast<bf16x4*>(final_out + ((long)t * H + head_o) * hd + d4) = o;
+    } else {
+      float* out = part + (((long)t * H + head_o) * gridDim.z + blockIdx.z) * (hd + 2);   // 8-byte rows
+      *reinterpret_cast<floatx2*>(out + d4) = floatx2{v[0], v[1]};
+      *reinterpret_cast<floatx2*>(out + d4 + 2) = floatx2{v[2], v[3]};
+      if (d4 == 0) *reinterpret_cast<floatx2*>(out + hd) = floatx2{M, L};
+    }
   }
 }
 
-template <int HDT>
-static void launch_decode(dim3 grid, hipStream_t stream, const void* q, float* part, const void* cache,
-                          const int* positions, const int* span_of_token, const int* block_table,
-                          int max_pages, int page_size, int H, int KV, int window, float scale,
-                          int head_tiles, const int* token_list) {
-  hipLaunchKernelGGL(attn_decode_mfma_kernel<HDT>, grid, dim3(64 * kDecodeWaves), 0, stream,
-                     (const bf16_t*)q, part, (const bf16_t*)cache, positions, span_of_token,
+template <int HDT, int W>
+static int launch_decode(dim3 grid, hipStream_t stream, const void* q, void* out, float* part,
+                         const void* cache, const int* positions, const int* span_of_token,
+                         const int* block_table, int max_pages, int page_size, int H, int KV, int window,
+                         float scale, int head_tiles, const int* token_list) {
+  const int heads = H / KV < 16 ? H / KV : 16;
+  const size_t lds = (size_t)W * heads * (16 * HDT + 4) * sizeof(float);
+  static int raised = 0;
+  if (lds > 64 * 1024 && !raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<HDT, W>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       W * 16 * (16 * HDT + 4) * (int)sizeof(float));
+    if (e != hipSuccess) KLLM_FAIL((int)e, "attn_decode: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = 1;
+  }
+  hipLaunchKernelGGL((attn_decode_mfma_kernel<HDT, W>), grid, dim3(64 * W), lds, stream,
+                     (const bf16_t*)q, (bf16_t*)out, part, (const bf16_t*)cache, positions, span_of_token,
                      block_table, max_pages, page_size, H, KV, window, scale, head_tiles, token_list);
+  return 0;
 }
 
 }  // namespace kllm
 
 using namespace kllm;
 
-extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int dtype, int max_keys) {
-  if (KV <= 0 || H <= 0 || n <= 0) return 1;
+extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, int max_keys) {
+  if (KV <= 0 || H <= 0 || n <= 0 || hd <= 0) return 1;
   if (dtype == DT_F32) return attn_f32_slices(n, KV, H, max_keys);
-  // About eight waves per CU across the chip, shared out over tokens x KV heads x head tiles;
-  // a workgroup is four waves and leaves one partial result.  A wave should have two tiles of
-  // 16 keys at least: 16 workgroups to a token at contexts of 2,048, more where the caller
-  // says that requests may be longer (one token at 32,768 keys: 37 us with 16, 4 x 128
-  // workgroups otherwise).
+  // As many token x KV head x head tile groups as CUs: one workgroup takes all keys of its
+  // group and writes the output.  Otherwise about eight waves per CU across the chip, shared
+  // out over the groups in workgroups of four waves that each leave a partial result.  A wave
+  // should have two tiles of 16 keys at least: 16 workgroups to a group at contexts of 2,048,
+  // more where the caller says that requests may be longer (one token at 32,768 keys: 37 us
+  // with 16, 27 us with the 128 that it gets).
   const int head_tiles = (H / KV + 15) / 16;
   long groups = (long)n * KV * head_tiles;
+  if (decode_waves_whole((hd + 15) / 16) > kDecodeWavesShared && groups >= device_cus()) return 1;
   long want = 8L * device_cus() / (groups > 0 ? groups : 1);
-  int wg = (int)((want + kDecodeWaves - 1) / kDecodeWaves);
-  int most = max_keys > 2048 ? max_keys / (32 * kDecodeWaves) : 16;
+  int wg = (int)((want + kDecodeWavesShared - 1) / kDecodeWavesShared);
+  int most = max_keys > 2048 ? max_keys / (32 * kDecodeWavesShared) : 16;
   if (most > 256) most = 256;
   if (wg > most) wg = most;
   if (wg < 1) wg = 1;
@@ -320,6 +349,9 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
                "%s: page_size %d must be a multiple of 16", who, page_size);
   KLLM_REQUIRE(nslices >= 1 && nslices <= 256, "%s: nslices %d is outside [1, 256]", who, nslices);
   KLLM_REQUIRE(window >= 0, "%s: negative window", who);
+  KLLM_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)cache & 15) == 0 &&
+                   ((uintptr_t)part & 15) == 0,
+               "%s: q, out, cache and part must be 16-byte aligned", who);
   KLLM_REQUIRE(part_floats >= (long)n * H * nslices * (hd + 2),
                "%s: the partial results of n=%d H=%d nslices=%d head_dim=%d need %ld floats, the workspace has %ld",
                who, n, H, nslices, hd, (long)n * H * nslices * (hd + 2), part_floats);
@@ -330,8 +362,16 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
   const dim3 grid(count, KV * head_tiles, nslices);
 #define KLLM_DEC(HDT)                                                                             \
   case HDT:                                                                                       \
-    launch_decode<HDT>(grid, stream, q, part, cache, positions, span_of_token, block_table,       \
-                       max_pages, page_size, H, KV, window, scale, head_tiles, token_list);       \
+    if (int rc = nslices == 1                                                                     \
+                     ? launch_decode<HDT, decode_waves_whole(HDT)>(                               \
+                           grid, stream, q, out, part, cache, positions, span_of_token,           \
+                           block_table, max_pages, page_size, H, KV, window, scale, head_tiles,   \
+                           token_list)                                                            \
+                     : launch_decode<HDT, kDecodeWavesShared>(                                    \
+                           grid, stream, q, out, part, cache, positions, span_of_token,           \
+                           block_table, max_pages, page_size, H, KV, window, scale, head_tiles,   \
+                           token_list))                                                           \
+      return rc;                                                                                  \
     break
   switch (hd / 16) {
     KLLM_DEC(1); KLLM_DEC(2); KLLM_DEC(3); KLLM_DEC(4); KLLM_DEC(5); KLLM_DEC(6); KLLM_DEC(7);
@@ -340,6 +380,7 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
   }
 #undef KLLM_DEC
   KLLM_CHECK_LAUNCH(who);
+  if (nslices == 1) return 0;                      // the one workgroup of a token has written the output
   hipLaunchKernelGGL(attn_merge_kernel<bf16_t>, dim3(count, H), dim3(64), 0, stream, (bf16_t*)out, part,
                      H, hd, nslices, token_list);
   KLLM_CHECK_LAUNCH("attn_merge");

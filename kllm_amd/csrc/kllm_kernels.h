@@ -164,15 +164,16 @@ int kllm_attn_generic(const void* q, void* out, const void* cache, const int* po
                       int dtype, hipStream_t stream);
 
 /* Decode attention on the matrix cores: every token's keys are cut into
- * `nslices` slices (1..256) that run side by side (bfloat16: four waves to a
- * slice, head sizes 16..128 in steps of 16, 192, 256, pages a multiple of 16;
- * float32: one wave to a slice, 32-bit MFMA, head sizes in steps of 8, pages a
- * multiple of 4); `part` is float32 scratch of n*H*nslices*(hd+2) elements.
- * kllm_attn_decode_slices proposes nslices for a batch whose longest request has
- * at most max_keys keys (0: unknown, as for contexts of 2,048).  With token_list only
- * the n_listed tokens it names are computed (q, out and part stay indexed by
- * token row). */
-int kllm_attn_decode_slices(int n, int KV, int H, int dtype, int max_keys);
+ * `nslices` slices (1..256) that run side by side (bfloat16: a workgroup of 16,
+ * 8 or 4 waves to a slice, by head size; head sizes 16..128 in steps of 16, 192,
+ * 256, pages a multiple of 16; float32: one wave to a slice, 32-bit MFMA, head
+ * sizes in steps of 8, pages a multiple of 4); `part` is float32 scratch of
+ * n*H*nslices*(hd+2) elements (bfloat16 with one slice writes the output at once
+ * and leaves it untouched).  kllm_attn_decode_slices proposes nslices for a batch
+ * whose longest request has at most max_keys keys (0: unknown, as for contexts
+ * of 2,048).  With token_list only the n_listed tokens it names are computed (q,
+ * out and part stay indexed by token row). */
+int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, int max_keys);
 int kllm_attn_decode(const void* q, void* out, float* part, long part_floats, const void* cache,
                      const int* positions, const int* span_of_token, const int* block_table,
                      int max_pages, int page_size, int n, int H, int KV, int hd, int window,

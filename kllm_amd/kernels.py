@@ -20,7 +20,7 @@ DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
 GEMV_MAX_ROWS = 8          # what the fused kernels take
 GEMV_BEST_ROWS = 4         # up to here they beat the MFMA kernel with split K
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class KernelError(RuntimeError):
@@ -93,7 +93,7 @@ def _declare(lib):
         "kllm_fused_linear": [P, I, P, P, I, I, I, I, P],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
-        "kllm_attn_decode_slices": [I, I, I, I, I],
+        "kllm_attn_decode_slices": [I, I, I, I, I, I],
         "kllm_device_cus": [],
         "kllm_calibrate_copy": [P, P, L, P],
         "kllm_calibrate_mfma": [I, I, P, P, P],
@@ -559,10 +559,11 @@ GENERIC_MAX_PAGE_SIZE = 256     # pages of the kernel that takes every size
 DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
 
 
-def attn_decode_slices(n, n_kv_heads, n_heads, dtype=torch.bfloat16, max_keys=0) -> int:
+def attn_decode_slices(n, n_kv_heads, n_heads, head_dim, dtype=torch.bfloat16, max_keys=0) -> int:
     """Slices of keys for a decode batch of n tokens; ``max_keys`` bounds the keys of the
     longest request (block-table width x page size, or the window), 0 if unknown."""
-    return library().kllm_attn_decode_slices(n, n_kv_heads, n_heads, dtype_code(dtype), int(max_keys))
+    return library().kllm_attn_decode_slices(n, n_kv_heads, n_heads, int(head_dim), dtype_code(dtype),
+                                             int(max_keys))
 
 
 def attn_f32_fits(head_dim, page_size) -> bool:

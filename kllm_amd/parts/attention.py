@@ -190,7 +190,7 @@ class CausalSelfAttention(Part):
         max_keys = pages * cache.page_size
         if self.window:
             max_keys = min(max_keys, self.window + cache.page_size)
-        nslices = K.attn_decode_slices(count, self.kv_heads, self.heads, q.dtype, max_keys)
+        nslices = K.attn_decode_slices(count, self.kv_heads, self.heads, self.head_dim, q.dtype, max_keys)
         part = ctx.buf("attn.part", (n * self.heads * nslices * (self.head_dim + 2),), torch.float32)
         K.attn_decode(q, out, part, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                       cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,

@@ -750,7 +750,7 @@ def run_attention(kernel, q, cache, pos, sot, bt, ps, H, KV, hd, window, scale, 
         K().attn_generic(q, out, cache, pos, sot, bt, ps, H, KV, hd, window, scale)
     else:
         n = q.shape[0]
-        ns = nslices or K().attn_decode_slices(n, KV, H, q.dtype)
+        ns = nslices or K().attn_decode_slices(n, KV, H, hd, q.dtype)
         part = torch.full((n * H * ns * (hd + 2),), float("nan"), device=DEV)
         K().attn_decode(q, out, part, cache, pos, sot, bt, ps, H, KV, hd, window, scale, ns)
     return out
@@ -919,16 +919,18 @@ def test_attention_decode_many_heads_and_slices(H, KV, hd, ps, nslices, dtype):
 
 def test_attention_decode_takes_more_slices_for_longer_contexts():
     """The proposed number of slices grows with the longest context the caller
-    announces (one token over 20,000 keys would otherwise run on 64 workgroups),
-    and the many partial results merge to the same output."""
+    announces (one token over 20,000 keys would otherwise run on 64 waves),
+    and the many partial results merge to the same output; one slice writes
+    the output without a merge."""
     k_ = K()
     H, KV, hd, ps, dtype = 8, 2, 64, 16, torch.bfloat16
-    few = k_.attn_decode_slices(1, KV, H, dtype, 2048)
-    assert few == k_.attn_decode_slices(1, KV, H, dtype) == 16
+    few = k_.attn_decode_slices(1, KV, H, hd, dtype, 2048)
+    assert few == k_.attn_decode_slices(1, KV, H, hd, dtype) == 16
+    assert k_.attn_decode_slices(k_.device_cus(), 1, 8, hd, dtype) == 1     # a workgroup to a token
     c = attention_case(H, KV, hd, ps, dtype, 0, [(20000, 1), (37, 1)], seed=9)
-    many = k_.attn_decode_slices(2, KV, H, dtype, c["bt"].shape[1] * ps)
+    many = k_.attn_decode_slices(2, KV, H, hd, dtype, c["bt"].shape[1] * ps)
     assert 100 <= many <= 256
-    for ns in (few, many, 256):
+    for ns in (1, few, many, 256):
         out = run_attention("decode", c["q"], c["cache"], c["pos"], c["sot"], c["bt"], ps, H, KV, hd, 0, c["scale"], ns)
         assert (out.cpu().double() - c["want"]).abs().max() < attn_tol(dtype), ns
 

@@ -46,7 +46,7 @@ def test_two_calls_in_a_row_equal_the_entry_point_with_a_workspace():
     assert cases[1]["q"].numel() < cases[0]["q"].numel()
     for c in cases:
         n = c["q"].shape[0]
-        ns = k_.attn_decode_slices(n, c["KV"], c["H"])
+        ns = k_.attn_decode_slices(n, c["KV"], c["H"], c["hd"])
         want = torch.full_like(c["q"], float("nan"))
         part = torch.full((n * c["H"] * ns * (c["hd"] + 2),), float("nan"), device=DEV)
         k_.attn_decode(c["q"], want, part, c["cache"], c["pos"], c["sot"], c["bt"], c["ps"], c["H"], c["KV"],

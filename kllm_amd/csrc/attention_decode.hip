@@ -2,9 +2,8 @@
 //
 // One wave takes one token, one KV head with up to 16 of its query heads, and
 // one slice of the token's keys; it streams that slice's pages from memory
-// once, for all heads of the group.  The waves of a workgroup (sixteen for
-// heads up to 64, fewer where a wave needs more registers) merge their results
-// in LDS.  Where one workgroup covers all keys of its token it writes the
+// once, for all heads of the group.  The waves of a workgroup (four or eight)
+// merge their results in LDS.  Where one workgroup covers all keys of its token it writes the
 // output itself; otherwise it leaves one partial result (running maximum, sum,
 // unnormalised output) and a second kernel merges the workgroups' partials.
 // The launch does not depend on any context length, so a recorded step can be
@@ -34,12 +33,14 @@ namespace kllm {
 
 // Waves of a workgroup: four where a token's keys are shared out over several workgroups
 // (small batches: many small workgroups start sooner than few large ones; 8 tokens at 2,048
-// keys: 6.4 us with 16 workgroups of 4 waves to a token and KV head, 9.7 us with 4 of 16),
-// and as many as the registers of a wave allow (a workgroup of 1,024 threads leaves each 128)
-// where one workgroup takes all keys of its token and writes the output itself (64 tokens:
-// 26.1 us against 25.6 + 5.6 us for two workgroups and their merge).
+// keys: 6.1 us with 16 workgroups of 4 waves to a token and KV head, 9.7 us with 4 of 16),
+// and eight, where the registers of the head size allow them, where one workgroup takes all
+// keys of its token and writes the output itself.  Measured with 4 / 8 / 16 waves, in us:
+// 64 tokens x 4 KV heads of 64 at 2,048 keys 37.1 / 25.8 / 25.9 (two workgroups of four waves
+// and their merge: 29.9); 128 such tokens 44.0 / 44.7 / 48.9; 64 tokens x 8 KV heads of 128 at
+// 4,096 keys 220 / 195; 32 tokens x 32 KV heads of 128 at 2,048 keys 221 / 208.
 constexpr int kDecodeWavesShared = 4;
-constexpr int decode_waves_whole(int hdt) { return hdt <= 4 ? 16 : (hdt <= 8 ? 8 : 4); }
+constexpr int decode_waves_whole(int hdt) { return hdt <= 8 ? 8 : 4; }
 // Tiles of 32 keys in a group; two groups are in registers.
 constexpr int decode_ahead(int hdt) { return 1; }
 
@@ -304,15 +305,17 @@ using namespace kllm;
 extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, int max_keys) {
   if (KV <= 0 || H <= 0 || n <= 0 || hd <= 0) return 1;
   if (dtype == DT_F32) return attn_f32_slices(n, KV, H, max_keys);
-  // As many token x KV head x head tile groups as CUs: one workgroup takes all keys of its
-  // group and writes the output.  Otherwise about eight waves per CU across the chip, shared
-  // out over the groups in workgroups of four waves that each leave a partial result.  A wave
-  // should have two tiles of 16 keys at least: 16 workgroups to a group at contexts of 2,048,
-  // more where the caller says that requests may be longer (one token at 32,768 keys: 37 us
-  // with 16, 27 us with the 128 that it gets).
+  // Three quarters as many token x KV head x head tile groups as CUs, or more: one workgroup
+  // takes all keys of its group and writes the output.  Otherwise about eight waves per CU
+  // across the chip, shared out over the groups in workgroups of four waves that each leave
+  // a partial result.  A wave should have two tiles of 16 keys at least: 16 workgroups to a
+  // group at contexts of 2,048, more where the caller says that requests may be longer (one
+  // token at 32,768 keys: 37 us with 16, 27 us with the 128 that it gets).
   const int head_tiles = (H / KV + 15) / 16;
   long groups = (long)n * KV * head_tiles;
-  if (decode_waves_whole((hd + 15) / 16) > kDecodeWavesShared && groups >= device_cus()) return 1;
+  // (measured at 2,048 keys, one workgroup against the rule below: 192 groups 23.4 against
+  // 28.7 us, 128 groups 22.6 against 20.0 us)
+  if (decode_waves_whole((hd + 15) / 16) > kDecodeWavesShared && 4 * groups >= 3L * device_cus()) return 1;
   long want = 8L * device_cus() / (groups > 0 ? groups : 1);
   int wg = (int)((want + kDecodeWavesShared - 1) / kDecodeWavesShared);
   int most = max_keys > 2048 ? max_keys / (32 * kDecodeWavesShared) : 16;

@@ -164,8 +164,8 @@ int kllm_attn_generic(const void* q, void* out, const void* cache, const int* po
                       int dtype, hipStream_t stream);
 
 /* Decode attention on the matrix cores: every token's keys are cut into
- * `nslices` slices (1..256) that run side by side (bfloat16: a workgroup of 16,
- * 8 or 4 waves to a slice, by head size; head sizes 16..128 in steps of 16, 192,
+ * `nslices` slices (1..256) that run side by side (bfloat16: a workgroup of 4
+ * or 8 waves to a slice; head sizes 16..128 in steps of 16, 192,
  * 256, pages a multiple of 16; float32: one wave to a slice, 32-bit MFMA, head
  * sizes in steps of 8, pages a multiple of 4); `part` is float32 scratch of
  * n*H*nslices*(hd+2) elements (bfloat16 with one slice writes the output at once

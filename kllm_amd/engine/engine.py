@@ -18,6 +18,7 @@ from typing import Dict, Hashable, List, Optional, Sequence
 import numpy as np
 import torch
 
+from .. import kernels as K
 from ..cache import CacheManager, GroupSpec, OutOfPages
 from ..cache.manager import window_pages
 from ..config import ModelConfig, config_from_dict, load_config, resolve_architecture
@@ -111,6 +112,9 @@ class Engine:
         self.steps_run = 0
         self.tokens_run = 0
         self._graphs = DecodeGraphs(self)
+        # What a scheduler should know of the kernels: a step's tokens are the rows of every
+        # product, and those work on tiles of this many rows.
+        self.step_row_multiple = K.GEMM_TILE_ROWS
 
     # ------------------------------------------------------------------ construction
     @classmethod

@@ -103,7 +103,8 @@ class Scheduler:
     ``eos_token_ids`` and ``max_model_len``."""
 
     def __init__(self, engine, max_batch: Optional[int] = None,
-                 max_step_tokens: Optional[int] = None, chunk_size: Optional[int] = None):
+                 max_step_tokens: Optional[int] = None, chunk_size: Optional[int] = None,
+                 row_multiple: Optional[int] = None):
         self.engine = engine
         # The reference's default batch is 8 (engine/scheduler.go:44-46).
         self.max_batch = int(max_batch) if max_batch else 8
@@ -112,7 +113,12 @@ class Scheduler:
         sized_for = getattr(getattr(engine, "options", None), "max_step_tokens", None)
         if sized_for:                        # the engine takes no larger portion of one request
             self.chunk_size = min(self.chunk_size, int(sized_for))
-        if self.max_batch <= 0 or self.max_step_tokens <= 0 or self.chunk_size <= 0:
+        # Rows of the tiles that the engine's products work on (0: none known).  A step a few
+        # tokens above a multiple pays for a whole further tile of every product.
+        if row_multiple is None:
+            row_multiple = getattr(engine, "step_row_multiple", 0)
+        self.row_multiple = int(row_multiple or 0)
+        if self.max_batch <= 0 or self.max_step_tokens <= 0 or self.chunk_size <= 0 or self.row_multiple < 0:
             raise SchedulerError("batch, token budget and chunk size must be positive")
         self.waiting: deque = deque()
         self.running: List[Request] = []
@@ -217,7 +223,32 @@ class Scheduler:
             entries.append(PlannedEntry(r, r.cursor, count, count == r.pending()))
         if not entries and self.running:
             return [], min(self.running, key=lambda q: q.admitted_at)
+        self._trim_to_tiles(entries)
         return entries, None
+
+    def _trim_to_tiles(self, entries: List[PlannedEntry]) -> None:
+        """A step of more than one tile of rows that ends less than half a tile
+        above a multiple gives the excess back from its last prompt portions:
+        the tokens go into the next step, and this one does not pay a further tile
+        of every product for them (512 + 31 tokens on tiles of 128: five tiles
+        for 4.2 tiles' worth)."""
+        m = self.row_multiple
+        if not m or not entries:
+            return
+        total = sum(e.count for e in entries)
+        excess = total % m
+        if total <= m or 2 * excess >= m:
+            return
+        while excess and entries:
+            last = entries[-1]
+            if last.count == 1 and last.request.generated:
+                return                                   # decoding requests are never put off
+            if last.count > excess:
+                last.count -= excess
+                last.wants_logits = False
+                return
+            excess -= last.count                         # a portion smaller than the excess waits whole
+            entries.pop()
 
     def plan(self) -> StepPlan:
         """Decide the next step.  Changes the queues (admission, preemption)

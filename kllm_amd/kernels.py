@@ -584,6 +584,7 @@ def device_cus() -> int:
     return _cus
 
 
+GEMM_TILE_ROWS = 128           # rows of X in a tile of the prompt products (256 where those fill the chip)
 PREFILL_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
 PREFILL_QUERY_BLOCK = 128      # tokens of one request that a workgroup of the prompt kernel takes
 

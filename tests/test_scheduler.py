@@ -107,6 +107,33 @@ def test_token_budget_and_portions():
     assert s.stats["decode_tokens"] == 4 * len(ps)
 
 
+def test_steps_end_on_whole_tiles_of_rows():
+    """With an engine whose products work on tiles of 8 rows, a step of more
+    than one tile that ends less than half a tile above a multiple gives the
+    excess of its last prompt portion back; everything else stays as planned,
+    and every request still gets its tokens."""
+    ps = prompts(5, 6, lo=30, hi=90)
+    plain, trimmed = StandIn(num_pages=400), StandIn(num_pages=400)
+    trimmed.step_row_multiple = 8
+    outs = []
+    for eng in (plain, trimmed):
+        s = Scheduler(eng, max_batch=4, max_step_tokens=35, chunk_size=32)
+        assert s.row_multiple == (8 if eng is trimmed else 0)
+        ids = [s.submit(p, 6) for p in ps]
+        res = s.run_until_done()
+        outs.append([res[i].tokens for i in ids])
+        assert s.stats["prefill_tokens"] == sum(len(p) for p in ps)
+    assert outs[0] == outs[1] == [alone(p, 6) for p in ps]
+    sizes = [sum(c for _, c in step) for step in plain.steps]
+    assert any(t > 8 and 0 < t % 8 < 4 for t in sizes)              # the plain plan has such steps
+    for step in trimmed.steps:
+        total = sum(c for _, c in step)
+        last_is_prompt = step[-1][1] > 1
+        if total > 8 and last_is_prompt:
+            assert not 0 < total % 8 < 4, step
+    assert Scheduler(plain, row_multiple=16).row_multiple == 16     # the caller may say it
+
+
 def test_stops_at_eos_and_at_the_limit():
     p = [3, 1, 4, 1, 5]
     free_run = alone(p, 30)

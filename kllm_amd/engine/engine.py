@@ -281,15 +281,27 @@ class Engine:
         ev.record()
         self._pinned_events[self._staging_index] = ev
 
-    def _validate(self, entries: Sequence[StepEntry]):
+    def _validate(self, entries: Sequence[StepEntry], allow_refs: bool = True):
+        """Checks the entries and returns each one's token ids as an array (a
+        TokenRef stands as 0).  Plain ids are converted once, here, and the
+        arrays go on into the control buffer."""
         if not entries:
             raise StepError("a step needs at least one entry")
         seen = set()
+        arrays = []
         for e in entries:
             if e.request_id in seen:
                 raise StepError(f"request {e.request_id!r} appears twice in one step")
             seen.add(e.request_id)
-            toks = np.asarray([0 if isinstance(t, TokenRef) else t for t in e.tokens], dtype=np.int64)
+            try:
+                toks = np.asarray(e.tokens, dtype=np.int64)          # plain ids: one pass
+            except (TypeError, ValueError):
+                if not all(isinstance(t, (int, np.integer, TokenRef)) for t in e.tokens):
+                    raise StepError(f"request {e.request_id!r}: token ids must be integers") from None
+                if not allow_refs:
+                    raise StepError("a TokenRef can only stand in a batch of single decode tokens "
+                                    "that is sampled") from None
+                toks = np.asarray([0 if isinstance(t, TokenRef) else t for t in e.tokens], dtype=np.int64)
             if toks.ndim != 1 or toks.size == 0:
                 raise StepError(f"request {e.request_id!r}: a step needs at least one token")
             if toks.min() < 0 or toks.max() >= self.vocab_size:
@@ -300,6 +312,8 @@ class Engine:
                 if not 0 <= int(w) < toks.size:
                     raise StepError(f"request {e.request_id!r}: wanted place {w} is outside its "
                                     f"{toks.size} tokens")
+            arrays.append(toks)
+        return arrays
 
     def _reserve(self, entries: Sequence[StepEntry]):
         """Room for every entry's tokens, or nothing taken.  Returns what to
@@ -363,9 +377,7 @@ class Engine:
         device, in the order of the entries and of their ``want`` lists, or
         None if nothing is wanted.  Raises OutOfPages (and changes nothing) if
         the cache cannot hold the step's tokens."""
-        if any(isinstance(t, TokenRef) for e in entries for t in e.tokens):
-            raise StepError("a TokenRef can only stand in a batch of single decode tokens that is sampled")
-        self._validate(entries)
+        arrays = self._validate(entries, allow_refs=False)
         opened, reserved = self._reserve(entries)
         try:
             rcs, lens, rows, tables = self._describe(entries)
@@ -378,7 +390,7 @@ class Engine:
             total = layout.total
             host = self._staging(total)
             pos0 = [rc.length for rc in rcs]
-            starts = control.fill(host.numpy(), layout, [e.tokens for e in entries], pos0,
+            starts = control.fill(host.numpy(), layout, arrays, pos0,
                                   [rc.slot for rc in rcs], rows, tables, lists=lists)
             if self._control is None or self._control.numel() < total:
                 self._control = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)

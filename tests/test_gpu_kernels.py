@@ -750,14 +750,16 @@ def run_attention(kernel, q, cache, pos, sot, bt, ps, H, KV, hd, window, scale, 
         K().attn_generic(q, out, cache, pos, sot, bt, ps, H, KV, hd, window, scale)
     else:
         n = q.shape[0]
-        ns = nslices or K().attn_decode_slices(n, KV, H, hd, q.dtype)
+        ns = 1 if kernel == "decode_whole" else nslices or K().attn_decode_slices(n, KV, H, hd, q.dtype)
         part = torch.full((n * H * ns * (hd + 2),), float("nan"), device=DEV)
         K().attn_decode(q, out, part, cache, pos, sot, bt, ps, H, KV, hd, window, scale, ns)
     return out
 
 
 def kernels_for(dtype):
-    return ["generic", "decode"]
+    # "decode_whole": one slice, so that one workgroup takes all keys of a token and writes
+    # the output without a merge (what large batches run)
+    return ["generic", "decode", "decode_whole"]
 
 
 def attn_tol(dtype):

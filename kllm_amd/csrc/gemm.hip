@@ -349,8 +349,13 @@ static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int 
                        hipStream_t stream) {
   const int cus = device_cus();
   const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN);
-  if (sizeof(T) == 4 && n <= 64)   // a decode batch in float32: tiles of 64 rows, half the products of 128
+  // A decode batch: tiles of 64 rows, half the products and half the loads of X of 128.  In
+  // bfloat16 a product of few tiles keeps three stages of loads in flight (one workgroup a CU).
+  if (n <= 64) {
+    if (sizeof(T) == 2 && (long)tx * nsplit <= cus)
+      return launch_mfma_tile<T, TOUT, DUAL, 1, 3>(x, w, y, n, m, k, nsplit, act, stream);
     return launch_mfma_tile<T, TOUT, DUAL, 1, 2>(x, w, y, n, m, k, nsplit, act, stream);
+  }
   // 256 x 256 tiles (eight waves of 128 x 64, one workgroup a CU) fetch a third less again and
   // are 10-27 % faster (2,048 x 28,672 x 4,096: 499 us against 561 us) where their rounds fill
   // the chip: three quarters of the CUs busy on average, counting the last round.  With 80, 128,

@@ -57,10 +57,15 @@ class GatedFeedForward(Part):
             K.gemv_swiglu(xn, self.w_gu, h, self.act)   # few tokens: both products and the gate in one launch
         elif fused:
             K.fused_linear(self.w_gu, h, K.LINEAR_SWIGLU, x=xn, act=self.act)   # a decode batch: the same on the matrix cores
-        elif (n > 128 and self.runtime.options.get("gemm") != "library"
+        elif ((n > 128 or (n > 32 and dtype == torch.bfloat16 and 5 * -(-self.intermediate // 64) >= 3 * K.device_cus()))
+              and self.runtime.options.get("gemm") != "library"
               and self.hidden % (8 if xn.dtype == torch.bfloat16 else 4) == 0):
             # prompts: the gate in the product's epilogue (up to 128 rows the product with K
-            # in slices and a separate gate is faster: the epilogue cannot split K)
+            # in slices and a separate gate is faster: the epilogue cannot split K), and decode
+            # batches of more than 32 rows where the tiles of 64 gate columns alone give most
+            # CUs a workgroup (64 rows, intermediate 14,336 x 4,096: 59 us against 83 us for
+            # the product in slices and the gate; 11,008: 56 against 68; 5,632 x 2,048: 30
+            # against 23)
             K.gemm_swiglu(xn, self.w_gu, h, self.act)
         else:
             gu = linear(ctx, xn, self.w_gu, "ffn.gu")

@@ -13,7 +13,8 @@ rotary + append, SiLU gate); with the compute dtype as result it returns
             few rows, where one wave's chain of products bounds the time), or
             tiled FMA where K is no multiple of 4
   bfloat16  n <= 64: MFMA skinny (n <= 16 and one float32 result wanted: the
-            decode-batch kernel with all of K in a workgroup)
+            decode-batch kernel with all of K in a workgroup; more than 32 rows
+            against large weights: MFMA tiles of 64 rows)
             else: MFMA tiles (K in slices where the tiles alone do not fill the chip),
             or the vendor library (torch.matmul) when the engine option
             ``gemm`` is "library" -- the reference uses its vendor library for
@@ -85,6 +86,19 @@ def _mfma_f32_split(n, m, k):
     return int(nsplit)
 
 
+def _tiles_beat_skinny(n, m, k):
+    """Decode batches of more than 32 rows against large weights: the tiled kernel (tiles of 64
+    rows, both operands through LDS in whole cache lines, K in up to 8 slices) streams them
+    faster than the skinny one, whose workgroups each stage all rows of X for 512 of K and
+    leave up to 28 partial sums.  Measured at 64 rows, tiled against skinny in us: 11,264 x
+    2,048: 15.7 / 19.6; 4,096 x 14,336: 28.5 / 41.3; 6,144 x 4,096: 16.5 / 20.6; 4,096 x 4,096:
+    11.8 / 14.9; 28,672 x 4,096: 58.0 / 72.7; 2,048 x 5,632: 13.2 / 13.0; 2,048 x 2,048: 8.2 /
+    6.9.  At 32 rows only the largest gain (4,096 x 14,336: 25.1 / 32.4; 6,144 x 4,096: 14.9 /
+    15.4; 11,264 x 2,048: 13.8 / 14.2)."""
+    weights = m * k
+    return (n > 32 and weights >= 12_000_000) or (n > 16 and weights >= 50_000_000)
+
+
 def choose(dtype, n, m, k, options=None):
     """(algorithm, nsplit) for a product of these sizes."""
     options = options or {}
@@ -102,6 +116,8 @@ def choose(dtype, n, m, k, options=None):
     if k % 8 != 0:
         return (K.GEMM_GEMV, 1) if n <= 8 else (K.GEMM_PLAIN, 1)
     if n <= 64:
+        if _tiles_beat_skinny(n, m, k) and options.get("gemm") != "library":
+            return K.GEMM_MFMA_BF16, _mfma_split(n, m, k)
         return K.GEMM_SKINNY_BF16, _skinny_split(n, m, k)
     if options.get("gemm") == "library":
         return "library", 1

@@ -329,6 +329,9 @@ def _gpu_reference(x, w):
     (2048, 32000, 2048, 1),     # the logits of a whole prompt: 256 x 256 tiles (two rounds of them per CU)
     (1000, 16284, 264, 1),      # 256 x 256 tiles (one full round of them), ragged in every direction
     (1000, 8100, 520, 2),       # ... in two slices of K
+    (64, 11264, 2048, 4),       # a decode batch on tiles of 64 rows, more tiles than CUs: two stages
+    (40, 4096, 14336, 8),       # ... few tiles: three stages
+    (33, 28700, 264, 1),        # ... ragged
 ])
 @pytest.mark.parametrize("dtype,out_dtype", [(torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16),
                                              (torch.float32, torch.float32)])
@@ -357,7 +360,8 @@ def test_gemm_mfma_at_prompt_sizes(n, m, k, nsplit, dtype, out_dtype):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("n,f,k", [(2048, 5632, 2048), (1000, 2500, 2056), (2048, 14336, 4096), (300, 5632, 2048),
-                                   (1000, 8100, 264)])    # (2048, 14336, 4096) and the last: 256 x 256 tiles, whole and ragged
+                                   (1000, 8100, 264),     # (2048, 14336, 4096) and this one: 256 x 256 tiles, whole and ragged
+                                   (64, 14336, 4096), (40, 20000, 264)])   # decode batches: tiles of 64 rows, three and two stages
 def test_gemm_swiglu_at_prompt_sizes(n, f, k, dtype):
     x, w = rnd(n, k, seed=1, dtype=dtype, scale=0.5), rnd(2 * f, k, seed=2, dtype=dtype, scale=0.05)
     h = torch.full((n, f), float("nan"), dtype=dtype, device=DEV)
@@ -371,12 +375,15 @@ def test_gemm_swiglu_at_prompt_sizes(n, f, k, dtype):
 @pytest.mark.parametrize("n", [5, 8, 16, 33, 64])
 @pytest.mark.parametrize("m,k", [(2048, 2048), (2048, 5632), (4096, 14336), (2560, 2048)])
 def test_split_product_into_its_consumers(n, m, k):
-    """A decode batch's product with K in as many slices as the engine chooses at these sizes
-    (8 at K = 2048, 11 at 5632), consumed by the norm and by the sum kernel."""
+    """A decode batch's product with the kernel and with K in as many slices as the engine
+    chooses at these sizes (skinny: 8 at K = 2048, 11 at 5632, 28 at 14,336; from 17 rows
+    against the largest weights the tiles of 64 rows, 8 slices), consumed by the norm and
+    by the sum kernel."""
     from kllm_amd.parts.linear import choose
     k_ = K()
     algo, nsplit = choose(torch.bfloat16, n, m, k)
-    assert algo == k_.GEMM_SKINNY_BF16 and nsplit >= 4
+    tiled = n > 16 and m * k >= 50_000_000
+    assert algo == (k_.GEMM_MFMA_BF16 if tiled else k_.GEMM_SKINNY_BF16) and nsplit >= 4
     x, w = rnd(n, k, seed=1, dtype=torch.bfloat16, scale=0.5), rnd(m, k, seed=2, dtype=torch.bfloat16, scale=0.05)
     parts = torch.full((nsplit, n, m), float("nan"), device=DEV)
     k_.gemm(x, w, parts, algo, nsplit)
@@ -663,6 +670,10 @@ def test_linear_chooses_a_kernel_for_every_size():
     assert choose(torch.bfloat16, 40, 64, 64)[0] == k_.GEMM_SKINNY_BF16
     assert choose(torch.bfloat16, 40, 64, 60)[0] == k_.GEMM_PLAIN          # K not a multiple of 8
     assert choose(torch.bfloat16, 64, 2048, 5632) == (k_.GEMM_SKINNY_BF16, 11)
+    assert choose(torch.bfloat16, 64, 11264, 2048) == (k_.GEMM_MFMA_BF16, 4)   # many rows, large weights: tiles of 64 rows
+    assert choose(torch.bfloat16, 32, 11264, 2048)[0] == k_.GEMM_SKINNY_BF16
+    assert choose(torch.bfloat16, 24, 4096, 14336) == (k_.GEMM_MFMA_BF16, 8)
+    assert choose(torch.bfloat16, 64, 11264, 2048, {"gemm": "library"})[0] == k_.GEMM_SKINNY_BF16
     assert choose(torch.bfloat16, 3, 32001, 2048) == (k_.GEMM_GEMV, 1)
     for n, m, k in [(5, 100, 72), (64, 2048, 5632), (33, 96, 176), (9, 320, 520), (20, 64, 4104)]:
         ns = choose(torch.bfloat16, n, m, k)[1]

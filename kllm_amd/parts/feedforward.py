@@ -44,6 +44,17 @@ class GatedFeedForward(Part):
                                weights[self.tensor_name("up_proj.weight")]], dim=0).contiguous()
         self.w_down = weights[self.tensor_name("down_proj.weight")]
 
+    def _gate_in_tiles(self, n, dtype):
+        """Decode batches whose gate runs in the tiled product's epilogue: more than 32 rows
+        where the tiles of 64 gate columns give three fifths of the CUs a workgroup, more
+        than 16 where they give seven eighths (measured against the product in slices of K and
+        a separate gate, in us: 64 rows, intermediate 14,336 x 4,096: 59 / 83; 11,008: 56 / 68;
+        5,632 x 2,048: 30 / 23; 32 rows: 58 / 66; 54 / 53; 17 rows, 14,336: 57 / 61)."""
+        if dtype != torch.bfloat16 or n <= 16:
+            return False
+        tiles, cus = -(-self.intermediate // 64), K.device_cus()
+        return (n > 32 and 5 * tiles >= 3 * cus) or 8 * tiles >= 7 * cus
+
     def forward(self, ctx, xn, sink=None):
         dtype, opts = self.runtime.dtype, self.runtime.options
         n = xn.rows if isinstance(xn, Normed) else xn.shape[0]
@@ -57,15 +68,12 @@ class GatedFeedForward(Part):
             K.gemv_swiglu(xn, self.w_gu, h, self.act)   # few tokens: both products and the gate in one launch
         elif fused:
             K.fused_linear(self.w_gu, h, K.LINEAR_SWIGLU, x=xn, act=self.act)   # a decode batch: the same on the matrix cores
-        elif ((n > 128 or (n > 32 and dtype == torch.bfloat16 and 5 * -(-self.intermediate // 64) >= 3 * K.device_cus()))
+        elif ((n > 128 or self._gate_in_tiles(n, dtype))
               and self.runtime.options.get("gemm") != "library"
               and self.hidden % (8 if xn.dtype == torch.bfloat16 else 4) == 0):
             # prompts: the gate in the product's epilogue (up to 128 rows the product with K
             # in slices and a separate gate is faster: the epilogue cannot split K), and decode
-            # batches of more than 32 rows where the tiles of 64 gate columns alone give most
-            # CUs a workgroup (64 rows, intermediate 14,336 x 4,096: 59 us against 83 us for
-            # the product in slices and the gate; 11,008: 56 against 68; 5,632 x 2,048: 30
-            # against 23)
+            # batches against wide feed-forwards
             K.gemm_swiglu(xn, self.w_gu, h, self.act)
         else:
             gu = linear(ctx, xn, self.w_gu, "ffn.gu")

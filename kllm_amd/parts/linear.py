@@ -87,16 +87,19 @@ def _mfma_f32_split(n, m, k):
 
 
 def _tiles_beat_skinny(n, m, k):
-    """Decode batches of more than 32 rows against large weights: the tiled kernel (tiles of 64
-    rows, both operands through LDS in whole cache lines, K in up to 8 slices) streams them
-    faster than the skinny one, whose workgroups each stage all rows of X for 512 of K and
-    leave up to 28 partial sums.  Measured at 64 rows, tiled against skinny in us: 11,264 x
-    2,048: 15.7 / 19.6; 4,096 x 14,336: 28.5 / 41.3; 6,144 x 4,096: 16.5 / 20.6; 4,096 x 4,096:
-    11.8 / 14.9; 28,672 x 4,096: 58.0 / 72.7; 2,048 x 5,632: 13.2 / 13.0; 2,048 x 2,048: 8.2 /
-    6.9.  At 32 rows only the largest gain (4,096 x 14,336: 25.1 / 32.4; 6,144 x 4,096: 14.9 /
-    15.4; 11,264 x 2,048: 13.8 / 14.2)."""
+    """Decode batches against large weights: the tiled kernel (tiles of 64 rows, both operands
+    through LDS in whole cache lines, K in up to 8 slices) takes the same time from 8 to 64
+    rows, the time of its weights; the skinny one, whose workgroups each stage all rows of X
+    for 512 of K and leave up to 28 partial sums, grows with the rows.  Measured, tiled
+    against skinny in us, at 64 rows: 11,264 x 2,048: 15.7 / 19.6; 4,096 x 14,336: 28.5 /
+    41.3; 6,144 x 4,096: 16.5 / 20.6; 4,096 x 4,096: 11.8 / 14.9; 28,672 x 4,096: 58.0 / 72.7;
+    2,048 x 5,632: 13.2 / 13.0; 2,048 x 2,048: 8.2 / 6.9.  At 24 rows: 4,096 x 14,336: 27.1 /
+    31.3; 4,096 x 11,008: 22.8 / 27.3; 12,288 x 4,096: 24.1 / 27.4; 6,144 x 4,096: 15.2 / 14.7;
+    11,264 x 2,048: 14.0 / 13.4.  At 16 rows: 4,096 x 14,336: 26.9 / 28.2; 12,288 x 4,096:
+    23.1 / 25.3, but no gain in a whole step (8B sizes: 2,745 against 2,731 tok/s at 16 rows,
+    4,053 against 3,761 at 24, 6,296 against 5,414 at 48)."""
     weights = m * k
-    return (n > 32 and weights >= 12_000_000) or (n > 16 and weights >= 50_000_000)
+    return (n > 32 and weights >= 12_000_000) or (n > 16 and weights >= 40_000_000)
 
 
 def choose(dtype, n, m, k, options=None):

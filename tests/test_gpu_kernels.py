@@ -382,7 +382,7 @@ def test_split_product_into_its_consumers(n, m, k):
     from kllm_amd.parts.linear import choose
     k_ = K()
     algo, nsplit = choose(torch.bfloat16, n, m, k)
-    tiled = n > 16 and m * k >= 50_000_000
+    tiled = n > 16 and m * k >= 40_000_000
     assert algo == (k_.GEMM_MFMA_BF16 if tiled else k_.GEMM_SKINNY_BF16) and nsplit >= 4
     x, w = rnd(n, k, seed=1, dtype=torch.bfloat16, scale=0.5), rnd(m, k, seed=2, dtype=torch.bfloat16, scale=0.05)
     parts = torch.full((nsplit, n, m), float("nan"), device=DEV)

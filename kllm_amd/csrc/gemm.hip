@@ -344,6 +344,8 @@ static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m,
 // they are taken when they still give every CU two rounds of work and the last round is not
 // mostly idle (8,192 x 2,560 x 2,048, two and a half rounds: 113 us against 101 us with 128 rows).  The thresholds follow
 // the chip's number of CUs.
+constexpr long kNarrowBelow = 40000000;   // weights (elements) below which a decode batch gets tiles of 64 columns
+
 template <typename T, typename TOUT, bool DUAL>
 static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, int act,
                        hipStream_t stream) {
@@ -352,6 +354,17 @@ static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int 
   // A decode batch: tiles of 64 rows, half the products and half the loads of X of 128.  In
   // bfloat16 a product of few tiles keeps three stages of loads in flight (one workgroup a CU).
   if (n <= 64) {
+    // ... and against weights below 40 M elements tiles of 64 columns (two waves of 32 x 64):
+    // twice the workgroups, which is what a product of few column tiles lacks (64 rows, 2,048
+    // x 5,632 in 8 slices: 9.8 us against 13.2 us; 11,264 x 2,048 in 4: 14.3 against 16.2; 4,096
+    // x 14,336 in 8: 32.9 against 28.7).
+    if constexpr (sizeof(T) == 2 && !DUAL) {
+      if ((long)m * k < kNarrowBelow) {
+        if ((long)ceil_div(m, 64) * nsplit <= cus)
+          return launch_mfma_tile<T, TOUT, DUAL, 2, 3, 1, 1>(x, w, y, n, m, k, nsplit, act, stream);
+        return launch_mfma_tile<T, TOUT, DUAL, 2, 2, 1, 1>(x, w, y, n, m, k, nsplit, act, stream);
+      }
+    }
     if (sizeof(T) == 2 && (long)tx * nsplit <= cus)
       return launch_mfma_tile<T, TOUT, DUAL, 1, 3>(x, w, y, n, m, k, nsplit, act, stream);
     return launch_mfma_tile<T, TOUT, DUAL, 1, 2>(x, w, y, n, m, k, nsplit, act, stream);

@@ -13,8 +13,8 @@ rotary + append, SiLU gate); with the compute dtype as result it returns
             few rows, where one wave's chain of products bounds the time), or
             tiled FMA where K is no multiple of 4
   bfloat16  n <= 64: MFMA skinny (n <= 16 and one float32 result wanted: the
-            decode-batch kernel with all of K in a workgroup; more than 32 rows
-            against large weights: MFMA tiles of 64 rows)
+            decode-batch kernel with all of K in a workgroup; from 24 rows on, and
+            from 17 against the largest weights: MFMA tiles of 64 rows)
             else: MFMA tiles (K in slices where the tiles alone do not fill the chip),
             or the vendor library (torch.matmul) when the engine option
             ``gemm`` is "library" -- the reference uses its vendor library for
@@ -86,20 +86,38 @@ def _mfma_f32_split(n, m, k):
     return int(nsplit)
 
 
+NARROW_BELOW = 40_000_000     # weights (elements) below which the library gives a decode batch tiles of 64 columns
+
+
 def _tiles_beat_skinny(n, m, k):
-    """Decode batches against large weights: the tiled kernel (tiles of 64 rows, both operands
-    through LDS in whole cache lines, K in up to 8 slices) takes the same time from 8 to 64
-    rows, the time of its weights; the skinny one, whose workgroups each stage all rows of X
-    for 512 of K and leave up to 28 partial sums, grows with the rows.  Measured, tiled
-    against skinny in us, at 64 rows: 11,264 x 2,048: 15.7 / 19.6; 4,096 x 14,336: 28.5 /
-    41.3; 6,144 x 4,096: 16.5 / 20.6; 4,096 x 4,096: 11.8 / 14.9; 28,672 x 4,096: 58.0 / 72.7;
-    2,048 x 5,632: 13.2 / 13.0; 2,048 x 2,048: 8.2 / 6.9.  At 24 rows: 4,096 x 14,336: 27.1 /
-    31.3; 4,096 x 11,008: 22.8 / 27.3; 12,288 x 4,096: 24.1 / 27.4; 6,144 x 4,096: 15.2 / 14.7;
-    11,264 x 2,048: 14.0 / 13.4.  At 16 rows: 4,096 x 14,336: 26.9 / 28.2; 12,288 x 4,096:
-    23.1 / 25.3, but no gain in a whole step (8B sizes: 2,745 against 2,731 tok/s at 16 rows,
-    4,053 against 3,761 at 24, 6,296 against 5,414 at 48)."""
-    weights = m * k
-    return (n > 32 and weights >= 12_000_000) or (n > 16 and weights >= 40_000_000)
+    """Decode batches from 24 rows on, and from 17 against the largest weights: the tiled
+    kernel (tiles of 64 rows, both operands through LDS in whole cache lines) takes nearly
+    the same time from 24 to 64 rows, the time of its weights; the skinny one, whose
+    workgroups each stage all rows of X for 512 of K and leave up to 28 partial sums, grows
+    with the rows.  Measured, tiled against skinny in us (tiles of 64 columns below 40 M
+    weights, of 128 above), at 64 rows: 2,048 x 5,632: 9.8 / 13.5; 2,560 x 2,048: 7.0 / 8.6;
+    2,048 x 2,048: 6.1 / 6.9; 11,264 x 2,048: 14.3 / 19.7; 4,096 x 4,096: 10.3 / 15.1; 4,096 x
+    14,336: 28.7 / 41.1; 28,672 x 4,096: 58.0 / 72.7.  At 24 rows: 8.6 / 9.5; 6.4 / 6.4; 5.6 /
+    5.4; 12.3 / 13.5; 9.3 / 10.8; 27.8 / 30.5.  At 16 rows the largest gain 4,096 x 14,336: 26.9
+    / 28.2, but none in a whole step (8B sizes: 2,745 against 2,731 tok/s)."""
+    return n >= 24 or (n > 16 and m * k >= NARROW_BELOW)
+
+
+def _decode_tile_split(n, m, k):
+    """Slices of K for a decode batch on the tiled kernel.  Against the largest weights: as
+    for prompts.  Below (tiles of 64 columns): slices of at least 256 of K until every CU
+    has a workgroup, then further ones of at least 512, up to 16 (measured at 64 rows, in us
+    by slices: 2,048 x 5,632: 14.9 with 4, 9.8 with 8; 11,264 x 2,048: 17.3 with 2, 14.3 with 4,
+    17.7 with 8; 4,096 x 4,096: 12.2 with 4, 10.3 with 8, 11.2 with 16)."""
+    if m * k >= NARROW_BELOW:
+        return _mfma_split(n, m, k)
+    tiles, cus = -(-m // 64), K.device_cus()
+    nsplit = 1
+    while nsplit < 16 and ((tiles * nsplit < cus and k // (2 * nsplit) >= 256) or k // (2 * nsplit) >= 512):
+        nsplit *= 2
+    while nsplit > 1 and (-(-(-(-k // nsplit)) // 64) * 64) * (nsplit - 1) >= k:   # no empty slice
+        nsplit -= 1
+    return nsplit
 
 
 def choose(dtype, n, m, k, options=None):
@@ -120,7 +138,7 @@ def choose(dtype, n, m, k, options=None):
         return (K.GEMM_GEMV, 1) if n <= 8 else (K.GEMM_PLAIN, 1)
     if n <= 64:
         if _tiles_beat_skinny(n, m, k) and options.get("gemm") != "library":
-            return K.GEMM_MFMA_BF16, _mfma_split(n, m, k)
+            return K.GEMM_MFMA_BF16, _decode_tile_split(n, m, k)
         return K.GEMM_SKINNY_BF16, _skinny_split(n, m, k)
     if options.get("gemm") == "library":
         return "library", 1

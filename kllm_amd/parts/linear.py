@@ -58,13 +58,17 @@ def _mfma_split(n, m, k):
     """Slices of K for the tiled MFMA kernel.  A product with fewer 128 x 128
     tiles than the chip has room for workgroups (a portion of a prompt, a
     projection to a narrow output) is bound by how many workgroups stream the
-    weights: up to 8 slices of at least 256 of K bring it to about 512
+    weights: up to 8 slices of at least 512 of K bring it to about 512
     workgroups (measured, 72 rows: 2048 -> 2560 in 9 us instead of 26 us,
     5632 -> 2048 in 13 us instead of 62 us; 2048 rows, 5632 -> 2048: 57 us
     instead of 68 us with two slices, the second sum's traffic included)."""
     tiles = -(-n // 128) * -(-m // 128)
     nsplit = 1
-    while nsplit * 2 <= min(8, 2 * K.device_cus() // tiles, k // 256):
+    # slices of at least 512 of K (512 rows, 2,048 -> 2,048 with the norm behind it: 22.1 us in
+    # 4 slices, 23.5 in 8); a deep K bears twice the workgroups if the tiles alone leave CUs idle (1,024 rows, 14,336 -> 4,096:
+    # 136 us in 4 slices, 160 in 2; 512 rows: 83 us in 8, 94 in 4)
+    reach = (4 if k >= 8192 and tiles <= K.device_cus() else 2) * K.device_cus()
+    while nsplit * 2 <= min(8, reach // tiles, k // 512):
         nsplit *= 2
     while nsplit > 1 and (-(-(-(-k // nsplit)) // 64) * 64) * (nsplit - 1) >= k:   # no empty slice
         nsplit -= 1

@@ -340,12 +340,12 @@ static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m,
   return 0;
 }
 
+constexpr long kNarrowBelow = 40000000;   // weights (elements) below which a decode batch gets tiles of 64 columns
+
 // Tiles of 256 rows of X (eight waves) fetch a quarter less per flop than two tiles of 128;
 // they are taken when they still give every CU two rounds of work and the last round is not
 // mostly idle (8,192 x 2,560 x 2,048, two and a half rounds: 113 us against 101 us with 128 rows).  The thresholds follow
 // the chip's number of CUs.
-constexpr long kNarrowBelow = 40000000;   // weights (elements) below which a decode batch gets tiles of 64 columns
-
 template <typename T, typename TOUT, bool DUAL>
 static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, int act,
                        hipStream_t stream) {
@@ -357,8 +357,10 @@ static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int 
     // ... and against weights below 40 M elements tiles of 64 columns (two waves of 32 x 64):
     // twice the workgroups, which is what a product of few column tiles lacks (64 rows, 2,048
     // x 5,632 in 8 slices: 9.8 us against 13.2 us; 11,264 x 2,048 in 4: 14.3 against 16.2; 4,096
-    // x 14,336 in 8: 32.9 against 28.7).
-    if constexpr (sizeof(T) == 2 && !DUAL) {
+    // x 14,336 in 8: 32.9 against 28.7).  In float32, where a wave's chain of products bounds
+    // the time, the same halves the chain (a decode step of 64 tokens at 1.1B sizes: 4.75 ->
+    // 4.30 ms).
+    if constexpr (!DUAL) {
       if ((long)m * k < kNarrowBelow) {
         if ((long)ceil_div(m, 64) * nsplit <= cus)
           return launch_mfma_tile<T, TOUT, DUAL, 2, 3, 1, 1>(x, w, y, n, m, k, nsplit, act, stream);

@@ -13,8 +13,8 @@ rotary + append, SiLU gate); with the compute dtype as result it returns
             few rows, where one wave's chain of products bounds the time), or
             tiled FMA where K is no multiple of 4
   bfloat16  n <= 64: MFMA skinny (n <= 16 and one float32 result wanted: the
-            decode-batch kernel with all of K in a workgroup; from 24 rows on, and
-            from 17 against the largest weights: MFMA tiles of 64 rows)
+            decode-batch kernel with all of K in a workgroup; from 17 rows on: MFMA
+            tiles of 64 rows)
             else: MFMA tiles (K in slices where the tiles alone do not fill the chip),
             or the vendor library (torch.matmul) when the engine option
             ``gemm`` is "library" -- the reference uses its vendor library for
@@ -94,8 +94,8 @@ NARROW_BELOW = 40_000_000     # weights (elements) below which the library gives
 
 
 def _tiles_beat_skinny(n, m, k):
-    """Decode batches from 24 rows on, and from 17 against the largest weights: the tiled
-    kernel (tiles of 64 rows, both operands through LDS in whole cache lines) takes nearly
+    """Decode batches of more than 16 rows (two or more of the skinny kernel's 16-row
+    tiles): the tiled kernel (tiles of 64 rows, both operands through LDS in whole cache lines) takes nearly
     the same time from 24 to 64 rows, the time of its weights; the skinny one, whose
     workgroups each stage all rows of X for 512 of K and leave up to 28 partial sums, grows
     with the rows.  Measured, tiled against skinny in us (tiles of 64 columns below 40 M
@@ -103,8 +103,9 @@ def _tiles_beat_skinny(n, m, k):
     2,048 x 2,048: 6.1 / 6.9; 11,264 x 2,048: 14.3 / 19.7; 4,096 x 4,096: 10.3 / 15.1; 4,096 x
     14,336: 28.7 / 41.1; 28,672 x 4,096: 58.0 / 72.7.  At 24 rows: 8.6 / 9.5; 6.4 / 6.4; 5.6 /
     5.4; 12.3 / 13.5; 9.3 / 10.8; 27.8 / 30.5.  At 16 rows the largest gain 4,096 x 14,336: 26.9
-    / 28.2, but none in a whole step (8B sizes: 2,745 against 2,731 tok/s)."""
-    return n >= 24 or (n > 16 and m * k >= NARROW_BELOW)
+    / 28.2, but none in a whole step (8B sizes: 2,745 against 2,731 tok/s).  At 20 rows:
+    8.6 / 9.4; 6.2 / 6.4; 5.6 / 5.4; 12.3 / 13.4; 9.4 / 10.6; 26.1 / 30.0."""
+    return n > 16
 
 
 def _decode_tile_split(n, m, k):

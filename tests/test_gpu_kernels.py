@@ -378,13 +378,13 @@ def test_gemm_swiglu_at_prompt_sizes(n, f, k, dtype):
 @pytest.mark.parametrize("m,k", [(2048, 2048), (2048, 5632), (4096, 14336), (2560, 2048)])
 def test_split_product_into_its_consumers(n, m, k):
     """A decode batch's product with the kernel and with K in as many slices as the engine
-    chooses at these sizes (skinny: 8 at K = 2048, 11 at 5632, 28 at 14,336; from 24 rows on,
-    and from 17 against the largest weights, the tiles of 64 rows, 8 slices), consumed by the norm and
+    chooses at these sizes (skinny: 8 at K = 2048, 11 at 5632, 28 at 14,336; from 17 rows on
+    the tiles of 64 rows, 8 slices), consumed by the norm and
     by the sum kernel."""
     from kllm_amd.parts.linear import choose
     k_ = K()
     algo, nsplit = choose(torch.bfloat16, n, m, k)
-    tiled = n >= 24 or (n > 16 and m * k >= 40_000_000)
+    tiled = n > 16
     assert algo == (k_.GEMM_MFMA_BF16 if tiled else k_.GEMM_SKINNY_BF16) and nsplit >= 4
     x, w = rnd(n, k, seed=1, dtype=torch.bfloat16, scale=0.5), rnd(m, k, seed=2, dtype=torch.bfloat16, scale=0.05)
     parts = torch.full((nsplit, n, m), float("nan"), device=DEV)
@@ -669,17 +669,17 @@ def test_linear_chooses_a_kernel_for_every_size():
     for n, m, k in [(9, 100, 72), (64, 2048, 5632), (300, 257, 520), (70, 64, 4104), (2048, 2048, 5632)]:
         ns = choose(torch.float32, n, m, k)[1]
         assert 1 <= ns <= 16 and (-(-(-(-k // ns)) // 32) * 32) * (ns - 1) < k, (n, m, k, ns)
-    assert choose(torch.bfloat16, 20, 64, 64)[0] == k_.GEMM_SKINNY_BF16
+    assert choose(torch.bfloat16, 16, 64, 64)[0] == k_.GEMM_SKINNY_BF16
     assert choose(torch.bfloat16, 40, 64, 60)[0] == k_.GEMM_PLAIN          # K not a multiple of 8
-    assert choose(torch.bfloat16, 20, 2048, 5632) == (k_.GEMM_SKINNY_BF16, 11)
-    assert choose(torch.bfloat16, 40, 64, 64) == (k_.GEMM_MFMA_BF16, 1)          # from 24 rows: tiles of 64 rows
+    assert choose(torch.bfloat16, 16, 2048, 5632) == (k_.GEMM_SKINNY_BF16, 11)
+    assert choose(torch.bfloat16, 40, 64, 64) == (k_.GEMM_MFMA_BF16, 1)          # from 17 rows: tiles of 64 rows
     assert choose(torch.bfloat16, 64, 2048, 5632) == (k_.GEMM_MFMA_BF16, 8)
     assert choose(torch.bfloat16, 64, 11264, 2048) == (k_.GEMM_MFMA_BF16, 4)
-    assert choose(torch.bfloat16, 23, 11264, 2048)[0] == k_.GEMM_SKINNY_BF16
-    assert choose(torch.bfloat16, 17, 4096, 14336) == (k_.GEMM_MFMA_BF16, 8)     # from 17 against the largest weights
+    assert choose(torch.bfloat16, 17, 11264, 2048) == (k_.GEMM_MFMA_BF16, 4)
+    assert choose(torch.bfloat16, 17, 4096, 14336) == (k_.GEMM_MFMA_BF16, 8)
     assert choose(torch.bfloat16, 64, 11264, 2048, {"gemm": "library"})[0] == k_.GEMM_SKINNY_BF16
     assert choose(torch.bfloat16, 3, 32001, 2048) == (k_.GEMM_GEMV, 1)
-    for n, m, k in [(5, 100, 72), (23, 2048, 5632), (17, 96, 176), (9, 320, 520), (20, 64, 4104)]:
+    for n, m, k in [(5, 100, 72), (16, 2048, 5632), (13, 96, 176), (9, 320, 520), (12, 64, 4104)]:
         ns = choose(torch.bfloat16, n, m, k)[1]
         kslice = -(-(-(-k // ns)) // 32) * 32
         assert kslice <= 512 and kslice * (ns - 1) < k, (n, m, k, ns)

@@ -170,7 +170,8 @@ __device__ __forceinline__ floatx16 mfma_tile_step(floatx4 a, floatx4 b, floatx1
 __device__ __forceinline__ int mfma_swz(int row) { return (row >> 1) & 7; }
 
 // WR x WC waves, each with WTM x 2 MFMA tiles of 32 x 32: a workgroup's tile is 32 WTM WR rows
-// of X by 64 WC rows of W (128 x 128 with four waves, 256 x 128 and 256 x 256 with eight).
+// of X by 64 WC rows of W (128 x 128 with four waves, 256 x 128 and 256 x 256 with eight; for
+// decode batches 64 x 128 and 64 x 64 with two).
 template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES, int WC = 2, int WTM = 2>
 __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2))) void gemm_mfma_kernel(const T* __restrict__ X,
                                                              const T* __restrict__ W,

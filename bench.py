@@ -83,7 +83,7 @@ def main(argv=None):
     for item in filter(None, args.extra.split(",")):
         key, _, val = item.partition("=")
         extra[key] = int(val) if val.lstrip("-").isdigit() else (val or True)
-    eng = B.make_engine(cfg, args.dtype, max_tokens=max_batch * args.context + 4096,
+    eng = B.make_engine(cfg, args.dtype, max_tokens=max_batch * args.context + 4096, max_requests=max_batch,
                         max_model_len=args.context + 64, gemm=args.gemm, page_size=args.page_size, extra=extra)
 
     if args.prefill_only:
@@ -141,7 +141,7 @@ def other_workload(args, cfg, full_layers, B):
             "model": args.model + "-sizes", "layers": cfg["num_hidden_layers"], "layers_full": full_layers,
             "page_size": args.page_size, "gemm": args.gemm}
     if args.workload == "decode-run":
-        eng = B.make_engine(cfg, args.dtype, max_tokens=args.batch * args.context + 4096,
+        eng = B.make_engine(cfg, args.dtype, max_tokens=args.batch * args.context + 4096, max_requests=args.batch,
                             max_model_len=args.context + 64, gemm=args.gemm, page_size=args.page_size)
         res = B.measure_decode_run(eng, args.batch, prompt_len=512, total_len=args.context)
         base.update(batch=args.batch, prompt_len=512, total_len=args.context, unit="tok/s", **res)

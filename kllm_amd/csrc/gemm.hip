@@ -172,7 +172,7 @@ __device__ __forceinline__ int mfma_swz(int row) { return (row >> 1) & 7; }
 // WR x WC waves, each with WTM x 2 MFMA tiles of 32 x 32: a workgroup's tile is 32 WTM WR rows
 // of X by 64 WC rows of W (128 x 128 with four waves, 256 x 128 and 256 x 256 with eight; for
 // decode batches 64 x 128 and 64 x 64 with two).
-template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES, int WC = 2, int WTM = 2>
+template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES, int WC = 2, int WTM = 2, int WTN = 2>
 __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2))) void gemm_mfma_kernel(const T* __restrict__ X,
                                                              const T* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
@@ -181,8 +181,12 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
   constexpr int EPC = 16 / sizeof(T);           // elements of a 16-byte chunk
   constexpr int MBK = MROW / sizeof(T);         // elements of K per stage
   constexpr int BM = 32 * WTM * WR;             // rows of X per workgroup
-  constexpr int BN = 64 * WC;                   // rows of W per workgroup
+  constexpr int BN = 32 * WTN * WC;             // rows of W per workgroup
   constexpr int NW = WR * WC;                   // waves
+  // DUAL with an odd number of column tiles a wave: gate and up rows share every tile of 32
+  // columns, 16 each (see the epilogue); with an even number they have tiles of their own.
+  constexpr bool PAIRED = DUAL && WTN % 2 == 1;
+  static_assert(!DUAL || PAIRED || WTN == 2, "DUAL: two column tiles a wave (gate, up) or an odd number of shared ones");
   constexpr int XI = BM / 8 / NW;               // load instructions of X per wave and stage (8 rows each)
   constexpr int WI = BN / 8 / NW;
   constexpr int XBYTES = BM * MROW, WBYTES = BN * MROW;
@@ -215,8 +219,15 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
   for (int i = 0; i < WI; ++i) {
     const int r = 8 * (WI * wave + i) + lane / 8;             // DUAL: the first half of the rows gate, the second up
     wchunk[i] = ((lane % 8) ^ mfma_swz(r)) * EPC;
-    const long col = DUAL ? col0 + r % (BN / 2) : col0 + r;
-    const long wrow = min(col, (long)m - 1) + (DUAL && r >= BN / 2 ? m : 0);
+    long col, up;
+    if (PAIRED) {                                              // ... or 16 gate rows and their 16 up rows in turn
+      col = col0 + 16 * (r / 32) + r % 16;
+      up = r % 32 >= 16;
+    } else {
+      col = DUAL ? col0 + r % (BN / 2) : col0 + r;
+      up = DUAL && r >= BN / 2;
+    }
+    const long wrow = min(col, (long)m - 1) + (up ? m : 0);
     wsrc[i] = W + wrow * k + wchunk[i];
   }
   // blockIdx.y: a slice of K (kslice a multiple of a stage); its sums go to Y[blockIdx.y]
@@ -241,11 +252,11 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
     }
   };
 
-  floatx16 acc[WTM][2];
+  floatx16 acc[WTM][WTN];
 #pragma unroll
   for (int i = 0; i < WTM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WTN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
@@ -267,8 +278,8 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
     const unsigned char* ws = xs + XBYTES;
     // The operands of step ks + 1 are asked for before the MFMAs of step ks are issued, so
     // that LDS answers while the matrix unit works.
-    op_t a[2][WTM], b[2][2];
-    auto read_step = [&](int ks, op_t (&ar)[WTM], op_t (&br)[2]) {
+    op_t a[2][WTM], b[2][WTN];
+    auto read_step = [&](int ks, op_t (&ar)[WTM], op_t (&br)[WTN]) {
       const int chunk = ks * 2 + lane / 32;
 #pragma unroll
       for (int i = 0; i < WTM; ++i) {
@@ -276,8 +287,8 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
         ar[i] = *reinterpret_cast<const op_t*>(xs + r * MROW + (chunk ^ mfma_swz(r)) * 16);
       }
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int r = (DUAL ? j * (BN / 2) + wc * 32 : wc * 64 + j * 32) + lane % 32;
+      for (int j = 0; j < WTN; ++j) {
+        const int r = (DUAL && !PAIRED ? j * (BN / 2) + wc * 32 : wc * 32 * WTN + j * 32) + lane % 32;
         br[j] = *reinterpret_cast<const op_t*>(ws + r * MROW + (chunk ^ mfma_swz(r)) * 16);
       }
     };
@@ -288,11 +299,35 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
       for (int i = 0; i < WTM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < WTN; ++j)
           acc[i][j] = mfma_tile_step(a[ks & 1][i], b[ks & 1][j], acc[i][j]);
     }
   }
 
+  if (PAIRED) {
+    // Lanes c and c + 16 of a tile of 32 columns hold the gate and the up sum of one output
+    // column, for 16 rows each.  They share the rows out: the lane with the gates takes the
+    // first eight and is sent their up sums, the lane with the up sums the other eight and is
+    // sent their gates; every lane then has eight outputs to gate and to store.
+    const int cl = lane % 32;
+    const bool has_gate = cl < 16;
+#pragma unroll
+    for (int j = 0; j < WTN; ++j) {
+      const long c = col0 + 16 * (wc * WTN + j) + cl % 16;
+#pragma unroll
+      for (int i = 0; i < WTM; ++i)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          const float lo = acc[i][j][t], hi = acc[i][j][8 + t];
+          const float got = __shfl_xor(has_gate ? hi : lo, 16, kWave);
+          const float gate = has_gate ? lo : got, up = has_gate ? got : hi;
+          const int e = has_gate ? t : 8 + t;
+          const long r = row0 + wr * 32 * WTM + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+          if (c < m && r < n) Y[r * m + c] = from_f32<TOUT>(gate_act(gate, act) * up);
+        }
+    }
+    return;
+  }
   if (DUAL) {
     const long c = col0 + wc * 32 + lane % 32;
     if (c >= m) return;
@@ -309,8 +344,8 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
   for (int i = 0; i < WTM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const long c = col0 + wc * 64 + j * 32 + lane % 32;
+    for (int j = 0; j < WTN; ++j) {
+      const long c = col0 + wc * 32 * WTN + j * 32 + lane % 32;
       if (c >= m) continue;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
@@ -320,23 +355,23 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
     }
 }
 
-template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES, int WC = 2, int WTM = 2>
+template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES, int WC = 2, int WTM = 2, int WTN = 2>
 static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, int act,
                             hipStream_t stream) {
   constexpr int MBK = MROW / sizeof(T);
-  constexpr int BM = 32 * WTM * WR, BN = 64 * WC;
+  constexpr int BM = 32 * WTM * WR, BN = 32 * WTN * WC;
   const int tx = ceil_div(m, DUAL ? BN / 2 : BN), ty = ceil_div(n, BM);
   const int kslice = ceil_div(ceil_div(k, nsplit), MBK) * MBK;
   const dim3 grid(ceil_div((long)tx * ty, 8) * 8, nsplit);   // padded so that every XCD gets as many
   const size_t lds = (size_t)MSTAGES * (BM + BN) * MROW;
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES, WC, WTM>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES, WC, WTM, WTN>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) KLLM_FAIL((int)e, "gemm mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = 1;
   }
-  hipLaunchKernelGGL((gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES, WC, WTM>), grid, dim3(64 * WR * WC), lds, stream,
+  hipLaunchKernelGGL((gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES, WC, WTM, WTN>), grid, dim3(64 * WR * WC), lds, stream,
                      (const T*)x, (const T*)w, (TOUT*)y, n, m, k, tx, ty, kslice, act);
   return 0;
 }
@@ -380,7 +415,18 @@ static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int 
   if constexpr (sizeof(T) == 2) {
     const long big = (long)ceil_div(n, 256) * ceil_div(m, DUAL ? 128 : 256) * nsplit;
     const long rounds = ceil_div(big, (long)cus);
-    if (4 * big >= 3 * rounds * cus)
+    const bool big_fits = 4 * big >= 3 * rounds * cus;
+    // 256 x 192 tiles (eight waves of 64 x 96; with the gate, 96 output columns whose gate and
+    // up rows share the column tiles): the fastest tile here where its rounds fill the chip
+    // (2,048 x 11,264 x 2,048: 103 us against 123 us with 256 x 128; 2,048 x 12,288 x 4,096: 195
+    // against 227 us with 128 x 128 and 241 us with 256 x 256; 512 x 22,016 x 4,096: 93 against
+    // 113 us with 256 x 256), taken when its last round is at least 85 % full and it does not
+    // need more time than 256 x 256 by their tiles' sizes and rounds.
+    const long mid = (long)ceil_div(n, 256) * ceil_div(m, DUAL ? 96 : 192) * nsplit;
+    const long mid_rounds = ceil_div(mid, (long)cus);
+    if (100 * mid >= 85 * mid_rounds * cus && (!big_fits || 3 * mid_rounds <= 4 * rounds))
+      return launch_mfma_tile<T, TOUT, DUAL, 4, 2, 2, 2, 3>(x, w, y, n, m, k, nsplit, act, stream);
+    if (big_fits)
       return launch_mfma_tile<T, TOUT, DUAL, 2, 2, 4, 4>(x, w, y, n, m, k, nsplit, act, stream);
   }
   const long tall = (long)ceil_div(n, 256) * tx * nsplit;

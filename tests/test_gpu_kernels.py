@@ -329,6 +329,8 @@ def _gpu_reference(x, w):
     (2048, 32000, 2048, 1),     # the logits of a whole prompt: 256 x 256 tiles (two rounds of them per CU)
     (1000, 16284, 264, 1),      # 256 x 256 tiles (one full round of them), ragged in every direction
     (1000, 8100, 520, 2),       # ... in two slices of K
+    (1000, 11000, 264, 1),      # 256 x 192 tiles (2,048 x 11,264 x 2,048 above takes them too), ragged
+    (1000, 5600, 520, 2),       # ... in two slices of K
     (64, 11264, 2048, 4),       # a decode batch on tiles of 64 rows and 64 columns, more tiles than CUs: two stages
     (40, 2048, 5632, 8),        # ... as many tiles as CUs: three stages
     (33, 1000, 264, 1),         # ... ragged
@@ -363,7 +365,8 @@ def test_gemm_mfma_at_prompt_sizes(n, m, k, nsplit, dtype, out_dtype):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("n,f,k", [(2048, 5632, 2048), (1000, 2500, 2056), (2048, 14336, 4096), (300, 5632, 2048),
                                    (1000, 8100, 264),     # (2048, 14336, 4096) and this one: 256 x 256 tiles, whole and ragged
-                                   (64, 14336, 4096), (40, 20000, 264)])   # decode batches: tiles of 64 rows, three and two stages
+                                   (64, 14336, 4096), (40, 20000, 264),    # decode batches: tiles of 64 rows, three and two stages
+                                   (1000, 5500, 264)])    # 256 x 192 tiles whose column tiles gate and up share (the first case too), ragged
 def test_gemm_swiglu_at_prompt_sizes(n, f, k, dtype):
     x, w = rnd(n, k, seed=1, dtype=dtype, scale=0.5), rnd(2 * f, k, seed=2, dtype=dtype, scale=0.05)
     h = torch.full((n, f), float("nan"), dtype=dtype, device=DEV)

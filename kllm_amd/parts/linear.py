@@ -70,6 +70,16 @@ def _mfma_split(n, m, k):
     reach = (4 if k >= 8192 and tiles <= K.device_cus() else 2) * K.device_cus()
     while nsplit * 2 <= min(8, reach // tiles, k // 512):
         nsplit *= 2
+    if nsplit == 1 and n > 64:
+        # More 128 x 128 tiles than workgroups fit, but few 256 x 256 ones: slices of at least
+        # 2,048 of K that make those one full round of the chip (2,048 rows, 4,096 wide, with the
+        # norm behind: K = 4,096 114 us in 2 slices against 126 us; 11,008: 208 against 246;
+        # 14,336: 263 against 305)
+        big, cus = -(-n // 256) * -(-m // 256), K.device_cus()
+        for slices in (2, 3, 4):
+            if k // slices >= 2048 and 4 * slices * big >= 3 * cus and slices * big <= cus:
+                nsplit = slices
+                break
     while nsplit > 1 and (-(-(-(-k // nsplit)) // 64) * 64) * (nsplit - 1) >= k:   # no empty slice
         nsplit -= 1
     return nsplit

@@ -82,11 +82,13 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave) % kPrefillWaves;
   const int g = lane / 32, c = lane % 32;
   const long item = blockIdx.x;                               // (block, head), head fastest
-  // Later blocks read more keys.  The later half of the list is started first, longest block
-  // first, then the earlier half, shortest first: a CU that holds one workgroup of each half
-  // gets a long and a short one, and all CUs about the same number of keys.
+  // Later blocks read more keys.  With three workgroups a CU (one group of waves) the later
+  // half of the list is started first, longest block first, then the earlier half, shortest
+  // first: a CU that holds one workgroup of each half gets a long and a short one, and all CUs
+  // about the same number of keys.  With one workgroup a CU (two groups) a CU takes the next
+  // block when it is done with one: longest first throughout.
   const int place = (int)(item / H), h = item % H, n_late = (n_tiles + 1) / 2;
-  const int blk = place < n_late ? n_tiles - 1 - place : place - n_late;
+  const int blk = (PAR == 2 || place < n_late) ? n_tiles - 1 - place : place - n_late;
   const int kvh = h / (H / KV);
   // The same for every lane: said so explicitly, which keeps the loop's address arithmetic on
   // the scalar unit.
@@ -719,31 +721,32 @@ static void launch_prefill_split(int n_tiles, hipStream_t stream, const void* q,
                      span_start, span_pos, block_table, max_pages, page_size, H, KV, window, scale);
 }
 
-// Which kernel: with more than one query block per CU the CUs are full either way and the
-// traffic decides (keys through LDS, one group of waves); with fewer the chain of tiles
-// decides (keys shared out over the waves of small workgroups; for head sizes from 128 on,
-// whose tiles are heavy, through LDS with two groups of waves).
+// Which kernel.  One group of waves with the keys through LDS (three workgroups a CU) when
+// there are more than two query blocks per CU: the CUs are full and the traffic decides.  With
+// fewer, the longest block's chain of tiles decides, and two groups of waves that take its
+// tiles in turn halve it (one workgroup a CU, longest blocks first); measured, 32 heads, one
+// prompt, us with one group -> two: head 64, 2,048 tokens 47.7 -> 42.9, 1,500 tokens
+// 36.3 -> 27.9; 24 heads of 96, 2,048 tokens 60.7 -> 46.8; head 128, 2,048 tokens 74.4 -> 69.6;
+// 40 heads of 64 (2.5 blocks per CU) 53.5 -> 59.2.  For heads below 128 and no more blocks than
+// three quarters of the CUs, the keys are shared out over the waves of small workgroups instead
+// (512 tokens: 11.2 us against 12.4 with two groups; 8 heads, 2,048 tokens: 28.4 against 31.8;
+// 1,024 tokens of 32 heads, one block per CU: 22.6 against 20.0).
 template <int HDT>
 static void launch_prefill(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
                            const int* query_tiles, int n_tiles, const int* span_start,
                            const int* span_pos, const int* block_table, int max_pages, int page_size,
                            int H, int KV, int window, float scale) {
-  if constexpr (HDT >= 4) {
-    if (grid > device_cus() || PrefillShape<HDT>::kMaxPar == 1)
-      launch_prefill_par<HDT, 1>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,
-                                 block_table, max_pages, page_size, H, KV, window, scale);
-    else
-      launch_prefill_par<HDT, PrefillShape<HDT>::kMaxPar>(grid, stream, q, out, cache, query_tiles, n_tiles,
-                                                          span_start, span_pos, block_table, max_pages, page_size,
-                                                          H, KV, window, scale);
-  } else {
-    if (grid > device_cus())
-      launch_prefill_par<HDT, 1>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,
-                                 block_table, max_pages, page_size, H, KV, window, scale);
-    else
-      launch_prefill_split<HDT>(n_tiles, stream, q, out, cache, query_tiles, span_start, span_pos, block_table,
-                                max_pages, page_size, H, KV, window, scale);
-  }
+  const int cus = device_cus();
+  if (grid > 2 * cus || PrefillShape<HDT>::kMaxPar == 1)
+    launch_prefill_par<HDT, 1>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,
+                               block_table, max_pages, page_size, H, KV, window, scale);
+  else if (HDT >= 4 || 4 * grid > 3 * cus)
+    launch_prefill_par<HDT, PrefillShape<HDT>::kMaxPar>(grid, stream, q, out, cache, query_tiles, n_tiles,
+                                                        span_start, span_pos, block_table, max_pages, page_size,
+                                                        H, KV, window, scale);
+  else
+    launch_prefill_split<HDT>(n_tiles, stream, q, out, cache, query_tiles, span_start, span_pos, block_table,
+                              max_pages, page_size, H, KV, window, scale);
 }
 
 }  // namespace kllm

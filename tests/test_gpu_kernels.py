@@ -816,9 +816,10 @@ def test_attention_prefill(H, KV, hd, ps, window, dtype):
     assert rows.all() and torch.isfinite(out).all()
     err = (out.cpu().double() - c["want"]).abs().max()
     assert err < attn_tol(dtype), float(err)
-    # only the listed spans are touched
+    # only the listed spans are touched (fewer query blocks: possibly another of the kernels)
     out2, rows2 = run_prefill(c, min_len=33)
-    assert torch.isnan(out2.cpu()[~rows2]).all() and torch.equal(out2.cpu()[rows2], out.cpu()[rows2])
+    assert torch.isnan(out2.cpu()[~rows2]).all() and torch.isfinite(out2.cpu()[rows2]).all()
+    assert (out2.cpu().double() - c["want"])[rows2].abs().max() < attn_tol(dtype)
 
 
 def test_attention_prefill_refuses_tables_beyond_its_page_arithmetic():
@@ -843,14 +844,16 @@ def test_attention_prefill_refuses_tables_beyond_its_page_arithmetic():
                                         (24, 6, 64, 48)])
 @pytest.mark.parametrize("window", [0, 150])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-def test_attention_prefill_many_blocks(H, KV, hd, ps, window, dtype):
-    """More query blocks than CUs: the kernel that passes the keys through LDS,
-    with blocks of 128 queries that end inside a tile, long chains of tiles,
-    portions behind cached keys, and a window that ends inside a block."""
-    spans = [(0, 300), (500, 260), (100, 129), (37, 70), (5, 1), (16, 32), (31, 33)]
+@pytest.mark.parametrize("twice", [False, True])
+def test_attention_prefill_many_blocks(H, KV, hd, ps, window, dtype, twice):
+    """More query blocks than CUs: the kernel that passes the keys through LDS, with two
+    groups of waves that take the tiles in turn (up to two blocks per CU) and with one (more:
+    the list of spans twice), with blocks of 128 queries that end inside a tile, long chains of
+    tiles, portions behind cached keys, and a window that ends inside a block."""
+    spans = [(0, 300), (500, 260), (100, 129), (37, 70), (5, 1), (16, 32), (31, 33)] * (2 if twice else 1)
     c = attention_case(H, KV, hd, ps, dtype, window, spans, seed=6)
     blocks = sum(-(-b // K().PREFILL_QUERY_BLOCK) for _, b in spans)
-    assert blocks * H > 256
+    assert (blocks * H > 512) == twice and blocks * H > 256
     out, rows = run_prefill(c)
     assert rows.all() and torch.isfinite(out).all()
     err = (out.cpu().double() - c["want"]).abs().max()
@@ -875,11 +878,12 @@ def test_attention_float32_takes_head_sizes_in_steps_of_8(H, KV, hd, ps, window)
         assert (out.cpu().double() - c["want"]).abs().max() < 2e-5, nslices
 
 
-@pytest.mark.parametrize("H,KV,ps,news", [(66, 2, 16, (260, 200, 129)), (6, 2, 48, (140, 1, 70))])
+@pytest.mark.parametrize("H,KV,ps,news", [(80, 2, 16, (260, 200, 129)), (66, 2, 16, (260, 200, 129)),
+                                          (6, 2, 48, (140, 1, 70))])
 def test_attention_prefill_far_into_long_contexts(H, KV, ps, news):
     """Portions of prompts behind 70,000 cached keys: the page of a key is found by a
     multiplication instead of a division, and addresses inside a page are 32-bit; both are
-    shown here at large key numbers, for both prompt kernels (many query blocks, few),
+    shown here at large key numbers, for the prompt kernels (many query blocks, some, few),
     against the decode kernel, which divides."""
     k_ = K()
     hd, dtype = 64, torch.bfloat16

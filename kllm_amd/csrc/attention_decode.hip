@@ -309,8 +309,11 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, 
   // takes all keys of its group and writes the output.  Otherwise about eight waves per CU
   // across the chip, shared out over the groups in workgroups of four waves that each leave
   // a partial result.  A wave should have two tiles of 16 keys at least: 16 workgroups to a
-  // group at contexts of 2,048, more where the caller says that requests may be longer (one
-  // token at 32,768 keys: 37 us with 16, 27 us with the 128 that it gets).
+  // group at contexts of 2,048, more where the caller says that requests may be longer, up to
+  // 32 and, beyond 16,384 keys, 64: every workgroup more is a partial result more to merge
+  // (one token, 4 KV heads of 64, attention and merge in us with 16 / 32 / 64 / 128 workgroups
+  // to a group: 8,192 keys 14.3 / 12.5 / 13.4 / 19.4, 16,384 keys 22.7 / 15.9 / 15.9 / 21.0,
+  // 32,768 keys 37.0 / 25.3 / 20.0 / 26.0, 131,072 keys 129 / 70.6 / 44.7 / 47.1).
   const int head_tiles = (H / KV + 15) / 16;
   long groups = (long)n * KV * head_tiles;
   // (measured at 2,048 keys, one workgroup against the rule below: 192 groups 23.4 against
@@ -319,7 +322,8 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, 
   long want = 8L * device_cus() / (groups > 0 ? groups : 1);
   int wg = (int)((want + kDecodeWavesShared - 1) / kDecodeWavesShared);
   int most = max_keys > 2048 ? max_keys / (32 * kDecodeWavesShared) : 16;
-  if (most > 256) most = 256;
+  const int cap = max_keys > 16384 ? 64 : 32;
+  if (most > cap) most = cap;
   if (wg > most) wg = most;
   if (wg < 1) wg = 1;
   return wg;

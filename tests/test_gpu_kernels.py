@@ -953,7 +953,7 @@ def test_attention_decode_takes_more_slices_for_longer_contexts():
     assert k_.attn_decode_slices(k_.device_cus(), 1, 8, hd, dtype) == 1     # a workgroup to a token
     c = attention_case(H, KV, hd, ps, dtype, 0, [(20000, 1), (37, 1)], seed=9)
     many = k_.attn_decode_slices(2, KV, H, hd, dtype, c["bt"].shape[1] * ps)
-    assert 100 <= many <= 256
+    assert few < many <= 64
     for ns in (1, few, many, 256):
         out = run_attention("decode", c["q"], c["cache"], c["pos"], c["sot"], c["bt"], ps, H, KV, hd, 0, c["scale"], ns)
         assert (out.cpu().double() - c["want"]).abs().max() < attn_tol(dtype), ns

@@ -464,13 +464,17 @@ class Engine:
                  max_step_tokens: Optional[int] = None, max_batch: Optional[int] = None):
         """Generate for each prompt (a list of token ids) up to
         ``max_new_tokens`` tokens, stopping at an end-of-sequence id; all
-        prompts are scheduled together.  Returns one list of ids per prompt.
+        prompts are scheduled together, as many at a time as ``max_batch``
+        says (default: all of them, up to the engine's number of requests).
+        Returns one list of ids per prompt.
         The reference's Generate runs one prompt, greedily
         (engine/engine.go:192-213)."""
         from .scheduler import Scheduler
         single = bool(prompts) and isinstance(prompts[0], int)
         if single:
             prompts = [prompts]
+        if max_batch is None:
+            max_batch = max(1, min(len(prompts), self.options.max_requests))
         sched = Scheduler(self, max_batch=max_batch, max_step_tokens=max_step_tokens)
         ids = [sched.submit(list(p), max_new_tokens, temperature=temperature, seed=seed + i)
                for i, p in enumerate(prompts)]

@@ -326,6 +326,7 @@ def _gpu_reference(x, w):
     (1000, 5000, 2056, 3),
     (700, 2100, 264, 1),        # two stages, ragged
     (4096, 4096, 4096, 1),
+    (2048, 4096, 4096, 2),      # what the engine takes here: 256 x 256 tiles, one round of the chip in two slices of K
     (2048, 32000, 2048, 1),     # the logits of a whole prompt: 256 x 256 tiles (two rounds of them per CU)
     (1000, 16284, 264, 1),      # 256 x 256 tiles (one full round of them), ragged in every direction
     (1000, 8100, 520, 2),       # ... in two slices of K

@@ -723,21 +723,31 @@ static void launch_prefill_split(int n_tiles, hipStream_t stream, const void* q,
 
 // Which kernel.  One group of waves with the keys through LDS (three workgroups a CU) when
 // there are more than two query blocks per CU: the CUs are full and the traffic decides.  With
-// fewer, the longest block's chain of tiles decides, and two groups of waves that take its
-// tiles in turn halve it (one workgroup a CU, longest blocks first); measured, 32 heads, one
-// prompt, us with one group -> two: head 64, 2,048 tokens 47.7 -> 42.9, 1,500 tokens
-// 36.3 -> 27.9; 24 heads of 96, 2,048 tokens 60.7 -> 46.8; head 128, 2,048 tokens 74.4 -> 69.6;
-// 40 heads of 64 (2.5 blocks per CU) 53.5 -> 59.2.  For heads below 128 and no more blocks than
-// three quarters of the CUs, the keys are shared out over the waves of small workgroups instead
-// (512 tokens: 11.2 us against 12.4 with two groups; 8 heads, 2,048 tokens: 28.4 against 31.8;
-// 1,024 tokens of 32 heads, one block per CU: 22.6 against 20.0).
+// fewer, a block's chain of tiles takes about 2,700 cycles a tile whatever else the CU holds;
+// two groups of waves that take the tiles in turn (one workgroup a CU, longest blocks first)
+// bring a pair of tiles to 3,900 cycles.  That pays when the longest chain bounds the time:
+// whole prompts, whose later blocks read more keys (32 heads, one prompt, us with one group ->
+// two: head 64, 2,048 tokens 47.7 -> 42.9, 1,500 tokens 36.3 -> 27.9; 24 heads of 96, 2,048
+// tokens 60.7 -> 46.8; head 128, 2,048 tokens 74.4 -> 69.6), or one block per CU.  It does not
+// when every block has a long chain and a CU holds two of them, a portion of a prompt far into
+// its context: then the CU's tiles bound the time, and one group with its blocks side by side
+// takes fewer cycles a tile (32,768 tokens in portions of 2,048: 237 ms against 252).  The
+// caller says how many keys the blocks read together and the longest block alone
+// (`keys_total`, `keys_longest`; 0: not known, the prompt is taken to start at its beginning).
+// For heads below 128 and no more blocks than three quarters of the CUs, the keys are shared
+// out over the waves of small workgroups instead (512 tokens: 11.2 us against 12.4 with two
+// groups; 8 heads, 2,048 tokens: 28.4 against 31.8; 1,024 tokens of 32 heads, one block per CU:
+// 22.6 against 20.0).
 template <int HDT>
 static void launch_prefill(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
                            const int* query_tiles, int n_tiles, const int* span_start,
                            const int* span_pos, const int* block_table, int max_pages, int page_size,
-                           int H, int KV, int window, float scale) {
+                           int H, int KV, int window, float scale, long keys_total, int keys_longest) {
   const int cus = device_cus();
-  if (grid > 2 * cus || PrefillShape<HDT>::kMaxPar == 1)
+  bool chain_bound = true;
+  if (keys_total > 0 && keys_longest > 0)   // tiles of a CU's share of all blocks against the longest block's
+    chain_bound = 5 * (keys_total * H / cus) < 6 * (long)keys_longest;
+  if (grid > 2 * cus || PrefillShape<HDT>::kMaxPar == 1 || (grid > cus && !chain_bound))
     launch_prefill_par<HDT, 1>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,
                                block_table, max_pages, page_size, H, KV, window, scale);
   else if (HDT >= 4 || 4 * grid > 3 * cus)
@@ -756,9 +766,11 @@ using namespace kllm;
 extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                                  int n_tiles, const int* span_start, const int* span_pos,
                                  const int* block_table, int max_pages, int page_size, int H, int KV,
-                                 int hd, int window, float scale, int dtype, hipStream_t stream) {
+                                 int hd, int window, float scale, long keys_total, int keys_longest, int dtype,
+                                 hipStream_t stream) {
   KLLM_REQUIRE(q && out && cache && query_tiles && span_start && span_pos && block_table,
                "attn_prefill: null pointer");
+  KLLM_REQUIRE(keys_total >= 0 && keys_longest >= 0, "attn_prefill: negative numbers of keys");
   KLLM_REQUIRE(dtype == DT_BF16 || dtype == DT_F32, "attn_prefill: unknown dtype %d", dtype);
   KLLM_REQUIRE(n_tiles > 0 && H > 0 && KV > 0 && H % KV == 0, "attn_prefill: bad sizes tiles=%d H=%d KV=%d",
                n_tiles, H, KV);
@@ -781,7 +793,8 @@ extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, co
 #define KLLM_PF(HDT)                                                                              \
   case HDT:                                                                                       \
     launch_prefill<HDT>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,  \
-                        block_table, max_pages, page_size, H, KV, window, scale);                 \
+                        block_table, max_pages, page_size, H, KV, window, scale, keys_total,      \
+                        keys_longest);                                                            \
     break
   switch (hd / 32) {
     KLLM_PF(1); KLLM_PF(2); KLLM_PF(3); KLLM_PF(4); KLLM_PF(6); KLLM_PF(8);

@@ -200,11 +200,14 @@ int kllm_attn_decode_static(const void* q, void* out, const void* cache, const i
 /* Prompt attention on the matrix cores (bfloat16, or float32 with 32-bit MFMA).
  * query_tiles holds (first token row, span) pairs: up to 128 consecutive tokens
  * of one span.  bfloat16: head sizes 32, 64, 96, 128, 192, 256, pages a multiple
- * of 16 and of at most 2,048 tokens, max_pages * page_size at most 2^24. */
+ * of 16 and of at most 2,048 tokens, max_pages * page_size at most 2^24.
+ * keys_total / keys_longest: the keys that the blocks read, all together and the
+ * longest block alone, for the choice of the kernel (0: not known). */
 int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                       int n_tiles, const int* span_start, const int* span_pos,
                       const int* block_table, int max_pages, int page_size, int H, int KV, int hd,
-                      int window, float scale, int dtype, hipStream_t stream);
+                      int window, float scale, long keys_total, int keys_longest, int dtype,
+                      hipStream_t stream);
 
 /* out[r] = sampled index of logits[r][:]; temperature/uniform null: greedy. */
 int kllm_sample(int* out, const float* logits, const float* temperature, const float* uniform,

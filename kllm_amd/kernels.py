@@ -20,7 +20,7 @@ DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
 GEMV_MAX_ROWS = 8          # what the fused kernels take
 GEMV_BEST_ROWS = 4         # up to here they beat the MFMA kernel with split K
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class KernelError(RuntimeError):
@@ -98,7 +98,7 @@ def _declare(lib):
         "kllm_calibrate_copy": [P, P, L, P],
         "kllm_calibrate_mfma": [I, I, P, P, P],
         "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, P],
-        "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
+        "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, L, I, I, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -590,9 +590,11 @@ PREFILL_QUERY_BLOCK = 128      # tokens of one request that a workgroup of the p
 
 
 def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, block_table, page_size,
-                 n_heads, n_kv_heads, head_dim, window, scale):
+                 n_heads, n_kv_heads, head_dim, window, scale, keys_total=0, keys_longest=0):
     """query_tiles [n_tiles, 2] int32: (first token row, span) of each block of up to
-    PREFILL_QUERY_BLOCK consecutive tokens of one span."""
+    PREFILL_QUERY_BLOCK consecutive tokens of one span.  ``keys_total`` and
+    ``keys_longest``: how many keys the blocks read, all together and the longest block
+    alone, if the caller knows (the kernel is chosen by them)."""
     n = q.shape[0]
     if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape)
             or q.dtype != cache.dtype or out.dtype != q.dtype):
@@ -606,7 +608,8 @@ def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, bloc
         _ptr(query_tiles, "attn query_tiles", torch.int32), n_tiles,
         _ptr(span_start, "attn span_start", torch.int32), _ptr(span_pos, "attn span_pos", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size,
-        n_heads, n_kv_heads, head_dim, int(window), float(scale), dtype_code(q.dtype), _stream()),
+        n_heads, n_kv_heads, head_dim, int(window), float(scale), int(keys_total), int(keys_longest),
+        dtype_code(q.dtype), _stream()),
         "attn_prefill")
 
 

@@ -174,9 +174,26 @@ class CausalSelfAttention(Part):
         if n_short:
             self._decode(ctx, q, out, cache, None if n_short == n else short, n_short)
         if n_blocks:
+            total, longest = self._keys_read(ctx)
             K.attn_prefill(q, out, cache.pages, blocks, n_blocks, ctx.span_start,
                            ctx.span_pos, cache.block_table, cache.page_size, self.heads,
-                           self.kv_heads, self.head_dim, self.window, self.scale)
+                           self.kv_heads, self.head_dim, self.window, self.scale, total, longest)
+
+    def _keys_read(self, ctx):
+        """How many keys the step's query blocks read, all together and the
+        longest block alone (from the host's copies of the spans): a whole
+        prompt's blocks read more and more, a portion far into its context
+        reads many in every block, and the prompt kernel is chosen by that."""
+        total = longest = 0
+        for pos, n in zip(ctx.h_span_pos, ctx.h_span_len):
+            if n <= self.SHORT_SPAN:
+                continue
+            for first in range(0, n, self.QUERY_BLOCK):
+                last = pos + min(first + self.QUERY_BLOCK, n)          # keys [0, last) are before the block's end
+                keys = min(last, self.window + self.QUERY_BLOCK) if self.window else last
+                total += keys
+                longest = max(longest, keys)
+        return total, longest
 
     def _decode(self, ctx, q, out, cache, token_list, count):
         n = q.shape[0]

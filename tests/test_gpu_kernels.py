@@ -746,9 +746,10 @@ def attention_case(H, KV, hd, ps, dtype, window, spans, seed=0):
                 span_pos=torch.tensor([a for a, _ in spans], dtype=torch.int32, device=DEV))
 
 
-def run_prefill(c, min_len=1):
+def run_prefill(c, min_len=1, keys=(0, 0)):
     """The prompt kernel over the spans of at least min_len tokens; returns
-    (output, mask of the rows it computed)."""
+    (output, mask of the rows it computed).  ``keys``: what the caller says
+    about the keys that the blocks read (all together, the longest block)."""
     tiles, rows = [], torch.zeros(c["q"].shape[0], dtype=torch.bool)
     start = 0
     for s, (_, b) in enumerate(c["spans"]):
@@ -759,7 +760,7 @@ def run_prefill(c, min_len=1):
     qt = torch.tensor(tiles, dtype=torch.int32, device=DEV)
     out = torch.full_like(c["q"], float("nan"))
     K().attn_prefill(c["q"], out, c["cache"], qt, len(tiles), c["span_start"], c["span_pos"], c["bt"],
-                     c["ps"], c["H"], c["KV"], c["hd"], c["window"], c["scale"])
+                     c["ps"], c["H"], c["KV"], c["hd"], c["window"], c["scale"], *keys)
     return out, rows
 
 
@@ -859,6 +860,12 @@ def test_attention_prefill_many_blocks(H, KV, hd, ps, window, dtype, twice):
     assert rows.all() and torch.isfinite(out).all()
     err = (out.cpu().double() - c["want"]).abs().max()
     assert err < attn_tol(dtype), float(err)
+    # told that every block reads many keys (a portion far into its context), the launch
+    # takes one group of waves also for few blocks per CU; told that one block reads nearly
+    # all of them, two groups
+    for keys in ((10 ** 9, 1000), (1000, 1000)):
+        out2, _ = run_prefill(c, keys=keys)
+        assert (out2.cpu().double() - c["want"]).abs().max() < attn_tol(dtype), keys
 
 
 @pytest.mark.parametrize("H,KV,hd,ps", [(5, 5, 48, 16), (6, 3, 80, 32), (3, 1, 40, 12), (2, 1, 8, 4), (2, 2, 136, 20),

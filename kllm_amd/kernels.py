@@ -454,7 +454,16 @@ LINEAR_PARTS, LINEAR_SWIGLU, LINEAR_ROPE = 0, 2, 3
 # Rows up to which the decode-batch kernel beats the split-K kernel plus a separate
 # elementwise launch (measured at widths 2048 -> 2560 and 2048 -> 11264).
 FUSED_ROPE_BEST_ROWS = 16
-FUSED_SWIGLU_BEST_ROWS = 8
+FUSED_SWIGLU_BEST_ROWS = 16
+
+
+def fused_tiles_per_wg(n, m, k) -> int:
+    """Tiles of 16 rows of W that one workgroup of the decode-batch kernel takes, one after
+    the other, with the rows of X staged once: two from 9 rows of X on against large weights
+    (16 rows, 4,096 -> 2 x 14,336 with the gate: 58.8 us against 66.1; 4,096 -> 6,144 with the
+    rotation: 18.1 against 22.4), one otherwise (2,048 -> 2 x 5,632: 15.6 either way at 16
+    rows, 13.5 against 14.6 at 10)."""
+    return 2 if n > 8 and m * k >= 20_000_000 else 1
 
 
 def fused_linear_fits(n, k, nsplit=1) -> bool:

@@ -130,6 +130,7 @@ class CausalSelfAttention(Part):
               and not opts.get("no_fused_linear") and plain_rotation):
             # a decode batch: the same on the matrix cores
             K.fused_linear(self.w_in, q, K.LINEAR_ROPE, x=xn,
+                           tiles_per_wg=K.fused_tiles_per_wg(n, self.w_in.shape[0], self.hidden),
                            rope=K.Rope(cos, sin, pages, ctx.positions, ctx.span_of_token, cache.block_table,
                                        cache.page_size, self.heads, self.kv_heads, self.head_dim))
         else:

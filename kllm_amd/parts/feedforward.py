@@ -67,7 +67,9 @@ class GatedFeedForward(Part):
         if gemv:
             K.gemv_swiglu(xn, self.w_gu, h, self.act)   # few tokens: both products and the gate in one launch
         elif fused:
-            K.fused_linear(self.w_gu, h, K.LINEAR_SWIGLU, x=xn, act=self.act)   # a decode batch: the same on the matrix cores
+            # a decode batch: the same on the matrix cores
+            K.fused_linear(self.w_gu, h, K.LINEAR_SWIGLU, x=xn, act=self.act,
+                           tiles_per_wg=K.fused_tiles_per_wg(n, 2 * self.intermediate, self.hidden))
         elif ((n > 128 or self._gate_in_tiles(n, dtype))
               and self.runtime.options.get("gemm") != "library"
               and self.hidden % (8 if xn.dtype == torch.bfloat16 else 4) == 0):

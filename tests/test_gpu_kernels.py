@@ -511,8 +511,10 @@ def test_fused_linear_swiglu(n, f, k, tpw):
 
 @pytest.mark.parametrize("H,KV,hd,ps,d", [(4, 2, 16, 16, 64), (3, 1, 32, 16, 96), (5, 5, 48, 32, 88),
                                           (32, 4, 64, 16, 2048), (3, 3, 80, 16, 104)])
-def test_fused_linear_rope_append(H, KV, hd, ps, d):
-    """Projections, rotation and append in one launch, against the plain functions."""
+@pytest.mark.parametrize("tpw", [1, 2])
+def test_fused_linear_rope_append(H, KV, hd, ps, d, tpw):
+    """Projections, rotation and append in one launch, against the plain functions; a
+    workgroup takes one tile of 16 rows of W, or two in turn."""
     k_ = K()
     theta = 10000.0
     spans = [(37, 3), (0, 2), (ps - 1, 1), (5, 11)]       # seventeen tokens of four requests
@@ -529,7 +531,8 @@ def test_fused_linear_rope_append(H, KV, hd, ps, d):
     k_.rope_tables(cos, sin, pos, hd, theta)
     cache = torch.full((12, 2, KV, ps * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
     q_out = torch.full((n, qd), float("nan"), dtype=torch.bfloat16, device=DEV)
-    k_.fused_linear(w, q_out, k_.LINEAR_ROPE, x, rope=k_.Rope(cos, sin, cache, pos, sot, bt, ps, H, KV, hd))
+    k_.fused_linear(w, q_out, k_.LINEAR_ROPE, x, tiles_per_wg=tpw,
+                    rope=k_.Rope(cos, sin, cache, pos, sot, bt, ps, H, KV, hd))
     full = P.linear(x.cpu().double(), w.cpu().double())
     want_q = P.rope(full[:, :qd], pos.cpu().tolist(), H, hd, theta)
     want_k = P.rope(full[:, qd:qd + kvd], pos.cpu().tolist(), KV, hd, theta)

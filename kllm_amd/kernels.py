@@ -19,7 +19,7 @@ import torch
 DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
 GEMV_MAX_ROWS = 8          # what the fused kernels take
-GEMV_BEST_ROWS = 4         # up to here they beat the MFMA kernel with split K
+GEMV_BEST_ROWS = 2         # up to here they beat the MFMA kernels in bfloat16 (3 rows: 1.29 against 1.21 ms a step at 1.1B sizes)
 ABI_VERSION = 6
 
 
@@ -332,11 +332,12 @@ def _x_and_norm(x, dtype):
 NORMED_MAX_ROWS = 4    # rows that the small-batch kernels normalise while they stage their input
 
 
-def resid_parts(n, m, k, dtype):
+def resid_parts(n, m, k, dtype, best=True):
     """Partial sums of squares per row that a residual product of these sizes
     leaves (one per workgroup of eight rows of W), or 0 if the small-batch
-    kernel with that epilogue does not take them."""
-    if not (gemv_fits(n, m, k, dtype) and n <= NORMED_MAX_ROWS):
+    kernel with that epilogue does not take them (``best``: or is not the
+    faster choice)."""
+    if not (gemv_fits(n, m, k, dtype, best) and n <= NORMED_MAX_ROWS):
         return 0
     parts = library().kllm_gemv_resid_parts(m)
     return parts if parts <= NormedInput.MAX_PARTS else 0
@@ -347,7 +348,7 @@ def linear_resid(x, w, resid, ss):
     partial sums of squares of resid's new rows (parts = resid_parts(...), returned)."""
     n, k = x.shape
     m = w.shape[0]
-    parts = resid_parts(n, m, k, x.dtype)
+    parts = resid_parts(n, m, k, x.dtype, best=False)
     stride = -(-parts // 4) * 4
     if (parts == 0 or tuple(resid.shape) != (n, m) or tuple(ss.shape) != (n, stride) or w.shape[1] != k
             or w.dtype != x.dtype):
@@ -380,12 +381,12 @@ def gemm(x, w, y, algo, nsplit=1):
         dtype_code(y.dtype), algo, nsplit, _stream()), "gemm")
 
 
-def gemv_fits(n, m, k, dtype) -> bool:
-    """Whether the fused small-batch products take these sizes and are the
-    faster choice: always in float32 (which has no MFMA kernel), up to
-    GEMV_BEST_ROWS rows in bfloat16."""
+def gemv_fits(n, m, k, dtype, best=True) -> bool:
+    """Whether the fused small-batch products take these sizes and, with
+    ``best``, are the faster choice: always in float32 (which has no MFMA
+    kernel for decode batches), up to GEMV_BEST_ROWS rows in bfloat16."""
     v = 4 if dtype == torch.float32 else 8
-    most = GEMV_MAX_ROWS if dtype == torch.float32 else GEMV_BEST_ROWS
+    most = GEMV_MAX_ROWS if dtype == torch.float32 or not best else GEMV_BEST_ROWS
     return n <= most and m % 2 == 0 and k % v == 0
 
 

@@ -298,6 +298,42 @@ static int launch_decode(dim3 grid, hipStream_t stream, const void* q, void* out
   return 0;
 }
 
+// Workgroups of four waves of the shared variant that one CU holds at a time (registers and
+// LDS decide: four for heads of 64, two for heads of 128), asked of the runtime once per head
+// size; `heads` as in launch_decode.
+template <int HDT>
+static int decode_resident_of(int heads) {
+  int blocks = 0;
+  const size_t lds = (size_t)kDecodeWavesShared * heads * (16 * HDT + 4) * sizeof(float);
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, attn_decode_mfma_kernel<HDT, kDecodeWavesShared>,
+                                                   64 * kDecodeWavesShared, lds) != hipSuccess || blocks < 1) {
+    (void)hipGetLastError();
+    blocks = 2;
+  }
+  return blocks;
+}
+
+static int decode_resident(int hdt, int heads) {
+  static int known[17][17];                       // by head size / 16 and heads of a group (up to 16); 0: not asked yet
+  if (hdt < 1 || hdt > 16 || heads < 1 || heads > 16) return 2;
+  int& r = known[hdt][heads];
+  if (r) return r;
+  switch (hdt) {
+    case 1: r = decode_resident_of<1>(heads); break;
+    case 2: r = decode_resident_of<2>(heads); break;
+    case 3: r = decode_resident_of<3>(heads); break;
+    case 4: r = decode_resident_of<4>(heads); break;
+    case 5: r = decode_resident_of<5>(heads); break;
+    case 6: r = decode_resident_of<6>(heads); break;
+    case 7: r = decode_resident_of<7>(heads); break;
+    case 8: r = decode_resident_of<8>(heads); break;
+    case 12: r = decode_resident_of<12>(heads); break;
+    case 16: r = decode_resident_of<16>(heads); break;
+    default: r = 2;
+  }
+  return r;
+}
+
 }  // namespace kllm
 
 using namespace kllm;
@@ -306,21 +342,30 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, 
   if (KV <= 0 || H <= 0 || n <= 0 || hd <= 0) return 1;
   if (dtype == DT_F32) return attn_f32_slices(n, KV, H, max_keys);
   // Three quarters as many token x KV head x head tile groups as CUs, or more: one workgroup
-  // takes all keys of its group and writes the output.  Otherwise about eight waves per CU
-  // across the chip, shared out over the groups in workgroups of four waves that each leave
-  // a partial result.  A wave should have two tiles of 16 keys at least: 16 workgroups to a
-  // group at contexts of 2,048, more where the caller says that requests may be longer, up to
-  // 32 and, beyond 16,384 keys, 64: every workgroup more is a partial result more to merge
-  // (one token, 4 KV heads of 64, attention and merge in us with 16 / 32 / 64 / 128 workgroups
-  // to a group: 8,192 keys 14.3 / 12.5 / 13.4 / 19.4, 16,384 keys 22.7 / 15.9 / 15.9 / 21.0,
+  // takes all keys of its group and writes the output.  Otherwise workgroups of four waves
+  // that each leave a partial result: about two per CU across the chip, their number per
+  // group rounded up to a power of two (the keys of a context then go evenly to slices and
+  // waves: 10 tokens x 4 KV heads of 64 at 2,048 keys, attention and merge: 11.7 us with 16,
+  // 12.6 us with 13), but no more than the chip holds at a time (10 tokens x 8 KV heads of
+  // 128 at 4,096 keys, two workgroups a CU: 35.5 us with 6, 41.1 us with 8, which is 640
+  // workgroups).  A wave should have two tiles of 16 keys at least: 16 workgroups to a group
+  // at contexts of 2,048, more where the caller says that requests may be longer, up to 32
+  // and, beyond 16,384 keys, 64: every workgroup more is a partial result more to merge (one
+  // token, 4 KV heads of 64, attention and merge in us with 16 / 32 / 64 / 128 workgroups to
+  // a group: 8,192 keys 14.3 / 12.5 / 13.4 / 19.4, 16,384 keys 22.7 / 15.9 / 15.9 / 21.0,
   // 32,768 keys 37.0 / 25.3 / 20.0 / 26.0, 131,072 keys 129 / 70.6 / 44.7 / 47.1).
   const int head_tiles = (H / KV + 15) / 16;
   long groups = (long)n * KV * head_tiles;
+  const int hdt = (hd + 15) / 16;
   // (measured at 2,048 keys, one workgroup against the rule below: 192 groups 23.4 against
   // 28.7 us, 128 groups 22.6 against 20.0 us)
-  if (decode_waves_whole((hd + 15) / 16) > kDecodeWavesShared && 4 * groups >= 3L * device_cus()) return 1;
-  long want = 8L * device_cus() / (groups > 0 ? groups : 1);
-  int wg = (int)((want + kDecodeWavesShared - 1) / kDecodeWavesShared);
+  if (decode_waves_whole(hdt) > kDecodeWavesShared && 4 * groups >= 3L * device_cus()) return 1;
+  if (groups < 1) groups = 1;
+  int wg = 1;
+  while ((long)wg * groups < 2L * device_cus()) wg *= 2;
+  const int heads = H / KV < 16 ? H / KV : 16;
+  const long fit = (long)decode_resident(hdt, heads) * device_cus() / groups;   // what the chip holds at a time
+  if (wg > fit) wg = (int)fit;
   int most = max_keys > 2048 ? max_keys / (32 * kDecodeWavesShared) : 16;
   const int cap = max_keys > 16384 ? 64 : 32;
   if (most > cap) most = cap;

@@ -454,7 +454,7 @@ LINEAR_PARTS, LINEAR_SWIGLU, LINEAR_ROPE = 0, 2, 3
 
 # Rows up to which the decode-batch kernel beats the split-K kernel plus a separate
 # elementwise launch (measured at widths 2048 -> 2560 and 2048 -> 11264).
-FUSED_ROPE_BEST_ROWS = 16
+FUSED_ROPE_BEST_ROWS = 32      # (17 tokens at 1.1B sizes: 1.59 -> 1.55 ms a step against the tiled product and a rotation kernel)
 FUSED_SWIGLU_BEST_ROWS = 16
 
 

@@ -298,39 +298,37 @@ static int launch_decode(dim3 grid, hipStream_t stream, const void* q, void* out
   return 0;
 }
 
-// Workgroups of four waves of the shared variant that one CU holds at a time (registers and
-// LDS decide: four for heads of 64, two for heads of 128), asked of the runtime once per head
-// size; `heads` as in launch_decode.
-template <int HDT>
+// Workgroups that one CU holds at a time (registers and LDS decide: four of the shared
+// variant's for heads of 64, two for heads of 128; of the variant that takes all keys, two and
+// one), asked of the runtime once per head size; `heads` as in launch_decode.
+template <int HDT, int W>
 static int decode_resident_of(int heads) {
   int blocks = 0;
-  const size_t lds = (size_t)kDecodeWavesShared * heads * (16 * HDT + 4) * sizeof(float);
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, attn_decode_mfma_kernel<HDT, kDecodeWavesShared>,
-                                                   64 * kDecodeWavesShared, lds) != hipSuccess || blocks < 1) {
+  const size_t lds = (size_t)W * heads * (16 * HDT + 4) * sizeof(float);
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, attn_decode_mfma_kernel<HDT, W>, 64 * W, lds) !=
+          hipSuccess || blocks < 1) {
     (void)hipGetLastError();
-    blocks = 2;
+    blocks = W > kDecodeWavesShared ? 1 : 2;
   }
   return blocks;
 }
 
-static int decode_resident(int hdt, int heads) {
-  static int known[17][17];                       // by head size / 16 and heads of a group (up to 16); 0: not asked yet
-  if (hdt < 1 || hdt > 16 || heads < 1 || heads > 16) return 2;
-  int& r = known[hdt][heads];
+static int decode_resident(int hdt, int heads, bool whole) {
+  static int known[2][17][17];                    // by variant, head size / 16 and heads of a group; 0: not asked yet
+  if (hdt < 1 || hdt > 16 || heads < 1 || heads > 16) return whole ? 1 : 2;
+  int& r = known[whole][hdt][heads];
   if (r) return r;
+#define KLLM_RES(HDT)                                                                          \
+  case HDT:                                                                                    \
+    r = whole ? decode_resident_of<HDT, decode_waves_whole(HDT)>(heads)                        \
+              : decode_resident_of<HDT, kDecodeWavesShared>(heads);                            \
+    break
   switch (hdt) {
-    case 1: r = decode_resident_of<1>(heads); break;
-    case 2: r = decode_resident_of<2>(heads); break;
-    case 3: r = decode_resident_of<3>(heads); break;
-    case 4: r = decode_resident_of<4>(heads); break;
-    case 5: r = decode_resident_of<5>(heads); break;
-    case 6: r = decode_resident_of<6>(heads); break;
-    case 7: r = decode_resident_of<7>(heads); break;
-    case 8: r = decode_resident_of<8>(heads); break;
-    case 12: r = decode_resident_of<12>(heads); break;
-    case 16: r = decode_resident_of<16>(heads); break;
-    default: r = 2;
+    KLLM_RES(1); KLLM_RES(2); KLLM_RES(3); KLLM_RES(4); KLLM_RES(5); KLLM_RES(6); KLLM_RES(7);
+    KLLM_RES(8); KLLM_RES(12); KLLM_RES(16);
+    default: r = whole ? 1 : 2;
   }
+#undef KLLM_RES
   return r;
 }
 
@@ -359,12 +357,21 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, 
   const int hdt = (hd + 15) / 16;
   // (measured at 2,048 keys, one workgroup against the rule below: 192 groups 23.4 against
   // 28.7 us, 128 groups 22.6 against 20.0 us)
-  if (decode_waves_whole(hdt) > kDecodeWavesShared && 4 * groups >= 3L * device_cus()) return 1;
+  const int heads = H / KV < 16 ? H / KV : 16;
+  if (decode_waves_whole(hdt) > kDecodeWavesShared && 4 * groups >= 3L * device_cus()) {
+    // ... unless the groups are a few more than the chip holds of such workgroups at a time:
+    // the CUs that get a second one take twice as long as the others, and four workgroups
+    // to a group spread the keys evenly (33 tokens x 8 KV heads of 128 at 2,048 keys, one
+    // workgroup a CU: 71.2 us with one, 57.9 us with four and the merge; 40 tokens: 83.7 and
+    // 75.7; 48 tokens: the same; 9 tokens x 32 KV heads: 78.4 and 62.4)
+    const long held = (long)decode_resident(hdt, heads, true) * device_cus();
+    if (groups <= held || 5 * groups >= 8 * held) return 1;
+    return 4;
+  }
   if (groups < 1) groups = 1;
   int wg = 1;
   while ((long)wg * groups < 2L * device_cus()) wg *= 2;
-  const int heads = H / KV < 16 ? H / KV : 16;
-  const long fit = (long)decode_resident(hdt, heads) * device_cus() / groups;   // what the chip holds at a time
+  const long fit = (long)decode_resident(hdt, heads, false) * device_cus() / groups;   // what the chip holds at a time
   if (wg > fit) wg = (int)fit;
   int most = max_keys > 2048 ? max_keys / (32 * kDecodeWavesShared) : 16;
   const int cap = max_keys > 16384 ? 64 : 32;

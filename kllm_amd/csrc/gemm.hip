@@ -411,8 +411,10 @@ static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int 
   // are 10-27 % faster (2,048 x 28,672 x 4,096: 499 us against 561 us) where their rounds fill
   // the chip: three quarters of the CUs busy on average, counting the last round.  With 80, 128,
   // 320 or 352 such tiles on 256 CUs they lose by as much.  bfloat16 only: float32 is bound by
-  // its products, not its loads.
-  if constexpr (sizeof(T) == 2) {
+  // its products, not its loads.  Tiles of 256 rows are for more than 128 rows: below, half of
+  // every tile's products would be of rows that are not there (a decode step of 72 tokens at
+  // 1.1B sizes: 2.60 -> 2.54 ms, of 128 at Llama-3-8B sizes: 11.98 -> 11.84 ms).
+  if (sizeof(T) == 2 && n > 128) {
     const long big = (long)ceil_div(n, 256) * ceil_div(m, DUAL ? 128 : 256) * nsplit;
     const long rounds = ceil_div(big, (long)cus);
     const bool big_fits = 4 * big >= 3 * rounds * cus;

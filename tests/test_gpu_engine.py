@@ -383,6 +383,32 @@ def test_greedy_generation_through_the_entry_point(model_dirs, name, dtype):
     assert not eng.cache.requests
 
 
+def test_generate_takes_all_its_prompts_together(model_dirs):
+    """Twelve prompts and no batch size given: they decode together (more than the
+    scheduler's own default of eight), and each gets the plain implementation's tokens."""
+    from kllm_amd.engine import Engine, EngineOptions
+    from kllm_amd.engine import scheduler as S
+    cfg, d = tiny.CONFIGS["A"], model_dirs("A")
+    eng = Engine.from_dir(d, EngineOptions(dtype="float32", max_tokens=1024))
+    prompts = [tiny.tokens(cfg, 3 + 2 * i, 70 + i) for i in range(12)]
+    seen = []
+    run = S.Scheduler.run_until_done
+    def watched(self, *a, **k):
+        out = run(self, *a, **k)
+        seen.append(self.stats["max_batch_seen"])
+        return out
+    S.Scheduler.run_until_done = watched
+    try:
+        got = eng.generate(prompts, 12)
+    finally:
+        S.Scheduler.run_until_done = run
+    assert seen == [12]
+    w = tiny.read_weights(d, as_stored_in="float32")
+    for p, g in zip(prompts, got):
+        assert g == P.generate_greedy(w, cfg, p, 12, eos={cfg["eos_token_id"]} if "eos_token_id" in cfg else None)
+    assert not eng.cache.requests
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_generation_when_pages_run_out(model_dirs, dtype):
     """A pool too small for the requests together: the scheduler gives the youngest one's

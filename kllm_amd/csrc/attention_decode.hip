@@ -364,8 +364,12 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, 
     // to a group spread the keys evenly (33 tokens x 8 KV heads of 128 at 2,048 keys, one
     // workgroup a CU: 71.2 us with one, 57.9 us with four and the merge; 40 tokens: 83.7 and
     // 75.7; 48 tokens: the same; 9 tokens x 32 KV heads: 78.4 and 62.4)
-    const long held = (long)decode_resident(hdt, heads, true) * device_cus();
-    if (groups <= held || 5 * groups >= 8 * held) return 1;
+    // Where a CU holds two such workgroups (heads of 64) the second one shares the CU's
+    // bandwidth with the first and nothing is gained (160 tokens x 4 KV heads of 64: 67.1 us
+    // with one, 77.0 us with four).
+    const int resident = decode_resident(hdt, heads, true);
+    const long held = (long)resident * device_cus();
+    if (resident > 1 || groups <= held || 5 * groups >= 8 * held) return 1;
     return 4;
   }
   if (groups < 1) groups = 1;

@@ -426,7 +426,15 @@ static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int 
     // need more time than 256 x 256 by their tiles' sizes and rounds.
     const long mid = (long)ceil_div(n, 256) * ceil_div(m, DUAL ? 96 : 192) * nsplit;
     const long mid_rounds = ceil_div(mid, (long)cus);
-    if (100 * mid >= 85 * mid_rounds * cus && (!big_fits || 3 * mid_rounds <= 4 * rounds))
+    // (a single round of them from three fifths of the CUs on: 768 x 11,264 x 2,048 on 177 tiles 50 us
+    // against 63 us, 1,536 x 6,144 x 4,096 on 192 tiles 92 against 115; on 118 tiles, 512 rows,
+    // 50 against 39)
+    // for a product that is not cut along K, counting only the rows that are there (640 rows
+    // in three tiles of 256: slower, 3.34 -> 3.63 ms for the whole step at 1.1B sizes)
+    const bool one_round = mid_rounds == 1 && nsplit == 1 &&
+                           5L * mid * n >= 3L * cus * 256 * ceil_div(n, 256);
+    const bool mid_fits = 100 * mid >= 85 * mid_rounds * cus || one_round;
+    if (mid_fits && (!big_fits || 3 * mid_rounds <= 4 * rounds))
       return launch_mfma_tile<T, TOUT, DUAL, 4, 2, 2, 2, 3>(x, w, y, n, m, k, nsplit, act, stream);
     if (big_fits)
       return launch_mfma_tile<T, TOUT, DUAL, 2, 2, 4, 4>(x, w, y, n, m, k, nsplit, act, stream);

@@ -168,7 +168,10 @@ def linear_into(ctx, x, w, sink, tag):
     adds it).  Measured at width 2048: 4 % of a decode step at one token; for
     decode batches on the matrix cores the same was built and lost 4 % at
     eight tokens (every workgroup of the consuming product then stages 72 KB
-    of float32 rows where it staged 32 KB of bfloat16), so it stops at four."""
+    of float32 rows where it staged 32 KB of bfloat16), so it stops at four; in
+    float32, where rows are staged in 32 bits either way, the kernels for eight
+    rows with these epilogues are the slower ones (2.53 against 2.27 ms a step
+    at five to eight tokens)."""
     from .base import Normed
     n, k = x.shape
     m = w.shape[0]

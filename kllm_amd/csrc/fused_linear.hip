@@ -2,14 +2,26 @@
 // the step after the product done in the same launch.  Y = X . W^T, then
 //
 //   PARTS    float32 sums [nsplit, n, m] (only this one may split K);
+//   RESID    the sums are added to the float32 residual stream in place; the
+//            new rows times the weight of the RMS norm behind the addition go
+//            out in bfloat16, and each workgroup leaves the sums of squares of
+//            its columns of the new rows (reference: the fused add + norm,
+//            backend/model.cu:144-165, here without a launch of its own);
 //   SWIGLU   silu(gate) * up in bfloat16 (reference backend/model.cu:477-483);
 //   ROPE     rotated queries and keys, and values, written to q_out and to
 //            the tokens' pages (reference backend/model.cu:170-201).
 //
+// The consumer of a RESID product (SWIGLU or ROPE, `SCALED`) reads those
+// bfloat16 rows x * w as its X and multiplies its float32 sums by the row's
+// rsqrt(sum of squares / K + eps): the RMS norm without a kernel of its own
+// and with 16-bit staging.  Against the norm kernel the rounding to bfloat16
+// happens before the row scale instead of after it; both round every element
+// of the normalised row once.
+//
 // A workgroup owns tiles of 16 rows of W and one slice of K (all of K unless
 // the caller splits).  It puts its slice of X, all rows, into LDS once.  Each
 // of its four waves takes a quarter of the slice: it streams its part of the 16
-// rows of W straight from memory, sixteen 16-byte loads per lane in flight, the
+// rows of W straight from memory, eight 16-byte loads per lane in flight, the
 // first of them before X is staged, and multiplies with X from LDS
 // (MFMA 16x16x32: A = W tile, B = X^T, D[w row][x row]).  The four partial
 // tiles meet in LDS, are added in a fixed order, and the epilogue runs on the
@@ -31,12 +43,21 @@
 
 namespace kllm {
 
-constexpr int FL_AHEAD = 8;        // W loads per lane in one of the two buffers
-constexpr int FL_PAD = 136;        // LDS row padding (elements): 128 of zeros behind K, 8 to shift banks
+// W loads per lane in one of the two buffers.  Four, not more: in a decode step the kernel runs
+// with a cold instruction cache, and its time follows its code size (8 ahead: 2,000 instructions
+// and 6.7 us for 2,048 x 2,048 weights at 8 rows; 4 ahead: 1,660 and 6.0 us; more waves to a
+// workgroup or more of X in registers measured slower for the same reason).
+constexpr int FL_AHEAD = 4;
+constexpr int XB = 8;              // 16-byte loads of X per lane that are in flight together
+// LDS row padding (elements): zeros behind K as far as the waves' slices reach beyond it
+// (less than 32 per wave), 8 to shift banks
+constexpr int fl_pad(int nw) { return 32 * nw + 8; }
+constexpr int FL_SS_LOADS = 4;     // 16-byte loads per lane of a row's partial sums of squares: 16 lanes a row
+constexpr int FL_SS_MAX = 16 * 4 * FL_SS_LOADS;   // partial sums of squares per row at most
 constexpr int FL_LDS_MAX = 160 * 1024;
 constexpr int FL_TILE = 16 * 17;    // floats of one wave's partial tile in LDS: [x row][w row], padded
 
-enum : int { FL_PARTS = 0, FL_SWIGLU = 2, FL_ROPE = 3 };
+enum : int { FL_PARTS = 0, FL_RESID = 1, FL_SWIGLU = 2, FL_ROPE = 3 };
 
 struct FlOut {
   void* y;
@@ -48,12 +69,18 @@ struct FlOut {
   const int* block_table;
   int max_pages, page_size, H, KV, hd;
   int act;                      // the gate's activation (FL_SWIGLU)
+  float* resid;                 // FL_RESID: the residual stream [n][m]; y receives bfloat16 resid * norm_w
+  const float* norm_w;          // FL_RESID: weight [m] of the norm behind the addition
+  float* ss_out;                // FL_RESID: [n][workgroups rounded up to 4] sums of squares of the new rows
+  const float* ss_in;           // SCALED: [n][ss_parts rounded up to 4], what a FL_RESID product left
+  int ss_parts;
+  float eps;
 };
 
 // Row of W behind MFMA row c of a tile, or -1.  Pair epilogues: unit = pair.
 template <int EP>
 __device__ __forceinline__ long fl_row(int tile, int c, int m, const FlOut& o) {
-  if (EP == FL_PARTS) {
+  if (EP == FL_PARTS || EP == FL_RESID) {
     const long r = (long)tile * 16 + c;
     return r < m ? r : -1;
   }
@@ -81,21 +108,23 @@ __device__ __forceinline__ void fl_lds_barrier() {
   asm volatile("" ::: "memory");
 }
 
-template <int NT, int EP>
-__global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restrict__ X, FlOut out,
+// NW waves share a tile's K; SCALED: the sums are multiplied by a row scale made from out.ss_in.
+template <int NT, int EP, int NW, bool SCALED>
+__global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __restrict__ X, FlOut out,
                                                            const bf16_t* __restrict__ W, int n, int m,
                                                            int k, int kslice, int tiles, int tiles_per_wg,
                                                            int x_stride) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  const int ld = kslice + FL_PAD;
+  const int ld = kslice + fl_pad(NW);
   bf16_t* xs = reinterpret_cast<bf16_t*>(lds_raw);                            // [n][ld]
-  float* part = reinterpret_cast<float*>(lds_raw + (size_t)n * ld * sizeof(bf16_t));   // [2][4][NT][x row 16][17]
+  float* part = reinterpret_cast<float*>(lds_raw + (size_t)n * ld * sizeof(bf16_t));   // [2][NW][NT][x row 16][17]
+  float* row_scale = part + 2 * NW * NT * FL_TILE;                            // [32]
 
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int g = lane / 16, c = lane % 16;
   const int kbeg = blockIdx.y * kslice;
   const int klen = min(k, kbeg + kslice) - kbeg;            // a multiple of 8
-  const int kw = ((klen + 3) / 4 + 31) / 32 * 32;           // K of one wave
+  const int kw = ((klen + NW - 1) / NW + 31) / 32 * 32;     // K of one wave
   const int wk0 = wave * kw;                                // this wave's offset in the slice
   const int wlen = max(0, min(klen, wk0 + kw) - wk0);
   const int steps = kw / 32;
@@ -119,40 +148,75 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
     }
   }
 
-  // ---- X: wave w stages rows w, w + 4, ... of the slice, eight 16-byte loads a lane at a
+  // ---- X: wave w stages rows w, w + NW, ... of the slice, eight 16-byte loads a lane at a
   // time.  Loads return in order, so the last batch goes out before the weights: X is
   // then in LDS and the workgroup past its barrier while the weights are still arriving.
   // No load carries a branch (an index beyond the wave's share reads its last item again), so
   // that the compiler can count what is in flight and wait for X alone.
   const int chunks = klen / 8;
-  const int mine = (n - wave + 3) / 4;                    // rows of this wave
+  const int mine = (n - wave + NW - 1) / NW;              // rows of this wave
   const int items = mine * chunks;
-  auto x_load = [&](int base, bf16x8 (&v)[8]) {
+  auto x_load = [&](int base, bf16x8 (&v)[XB]) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < XB; ++j) {
       const int idx = min(base + j * kWave, max(items - 1, 0));
       const int ri = idx / chunks, ch = idx - ri * chunks;
-      const int row = min(wave + 4 * ri, n - 1);          // a wave without rows reads the last row
+      const int row = min(wave + NW * ri, n - 1);         // a wave without rows reads the last row
       v[j] = *reinterpret_cast<const bf16x8*>(X + (long)row * x_stride + kbeg + ch * 8);
     }
   };
-  auto x_store = [&](int base, const bf16x8 (&v)[8]) {
+  auto x_store = [&](int base, const bf16x8 (&v)[XB]) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < XB; ++j) {
       const int idx = base + j * kWave;
       if (idx < items) {
         const int ri = idx / chunks, ch = idx - ri * chunks;
-        *reinterpret_cast<bf16x8*>(&xs[(wave + 4 * ri) * ld + ch * 8]) = v[j];
+        *reinterpret_cast<bf16x8*>(&xs[(wave + NW * ri) * ld + ch * 8]) = v[j];
       }
     }
   };
-  bf16x8 xv0[8];
+  bf16x8 xv0[XB];
   int xbase = lane;
-  for (; xbase + kWave * 8 < items; xbase += kWave * 8) {   // all but the last batch (more than eight rows)
+  for (; xbase + kWave * XB < items; xbase += kWave * XB) {   // all but the last batch (more than eight rows)
     x_load(xbase, xv0);
     x_store(xbase, xv0);
   }
   x_load(xbase, xv0);
+
+  // ---- SCALED: a row's partial sums of squares, sixteen lanes to a row, asked for behind X
+  // and before the weights (loads return in order)
+  floatx4 ssv[SCALED ? NT : 1][FL_SS_LOADS];
+  if (SCALED) {
+    const int stride = (out.ss_parts + 3) / 4 * 4;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int i = 0; i < FL_SS_LOADS; ++i) {
+        const int at = 4 * (tid % 16 + 16 * i);
+        ssv[t][i] = *reinterpret_cast<const floatx4*>(out.ss_in + (long)min(t * 16 + (tid / 16) % 16, n - 1) * stride +
+                                                      (at < stride ? at : 0));
+      }
+  }
+  // ---- FL_RESID: thread (w row tid % 16, x row tid / 16) adds to resid[x row][w row]; the old
+  // value and the norm's weight are asked for now and needed in the epilogue
+  float res_old[EP == FL_RESID ? NT : 1], res_w = 0.f;
+  float ss_acc[EP == FL_RESID ? NT : 1];
+  auto resid_load = [&](int tile_index) {
+    if (EP != FL_RESID) return;
+    const long row = (long)(tile0 + tile_index) * 16 + tid % 16;
+    const bool live = tid < 256 && row < m && tile_index < my_tiles;
+    res_w = out.norm_w[live ? row : 0];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int xr = t * 16 + tid / 16;
+      res_old[t] = out.resid[live && xr < n ? (long)xr * m + row : 0];
+    }
+  };
+  if (EP == FL_RESID) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) ss_acc[t] = 0.f;
+    resid_load(0);
+  }
 
   // ---- W: two buffers of FL_AHEAD loads each, used in turn: while one is multiplied the
   // other is on its way, and it is asked for again as soon as it has been used.  No register
@@ -189,10 +253,24 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
   // ---- X into LDS: what was asked for before the weights has arrived first
   x_store(xbase, xv0);
   {   // zeros in X's columns [klen, klen + 128): what the waves' slices of K reach beyond klen
-    const int r = tid / 16, ch = tid % 16;
+    constexpr int per_row = 4 * NW;                         // threads to a row's 32 * NW zeros: 16 rows a pass
+    const int r = tid / per_row, ch = tid % per_row;
 #pragma unroll
     for (int t = 0; t < NT; ++t)
       if (t * 16 + r < n) *reinterpret_cast<bf16x8*>(&xs[(t * 16 + r) * ld + klen + 8 * ch]) = zero;
+  }
+  if (SCALED) {   // the rows' scales: sums in a fixed order, then across the row's sixteen lanes
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      float v = 0.f;
+#pragma unroll
+      for (int i = 0; i < FL_SS_LOADS; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v += 4 * (tid % 16 + 16 * i) + e < out.ss_parts ? ssv[t][i][e] : 0.f;
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+      if (tid % 16 == 0 && tid < 256) row_scale[t * 16 + tid / 16] = rsqrtf(v / (float)k + out.eps);
+    }
   }
   int ep_page[NT], ep_slot[NT];
   float ep_cos[NT], ep_sin[NT];
@@ -251,7 +329,7 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
       fill(bufb);
     }
     // ---- the tile is complete in this wave: meet the other waves in LDS
-    float* pb = part + (tile & 1) * 4 * NT * FL_TILE;
+    float* pb = part + (tile & 1) * NW * NT * FL_TILE;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
@@ -269,9 +347,28 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
         const int xr = t * 16 + xc;
         float v = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) v += pb[(w * NT + t) * FL_TILE + xc * 17 + r16];
+        for (int w = 0; w < NW; ++w) v += pb[(w * NT + t) * FL_TILE + xc * 17 + r16];
         if (row < m && xr < n) reinterpret_cast<float*>(out.y)[((long)blockIdx.y * n + xr) * m + row] = v;
       }
+    } else if (EP == FL_RESID) {
+      if (tid < 256) {
+        const int r16 = tid % 16, xc = tid / 16;
+        const long row = (long)tl * 16 + r16;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          const int xr = t * 16 + xc;
+          float v = 0.f;
+#pragma unroll
+          for (int w = 0; w < NW; ++w) v += pb[(w * NT + t) * FL_TILE + xc * 17 + r16];
+          if (row < m && xr < n) {
+            const float x = res_old[t] + v;
+            out.resid[(long)xr * m + row] = x;
+            reinterpret_cast<bf16_t*>(out.y)[(long)xr * m + row] = from_f32<bf16_t>(x * res_w);
+            ss_acc[t] += x * x;
+          }
+        }
+      }
+      resid_load(tile + 1);
     } else if (tid < 128) {
       const int p8 = tid % 8, xc = tid / 8;
       const int pair = tl * 8 + p8, pairs = m / 2;
@@ -280,11 +377,16 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
         const int xr = t * 16 + xc;
         float a = 0.f, b = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 0; w < NW; ++w) {
           a += pb[(w * NT + t) * FL_TILE + xc * 17 + p8];
           b += pb[(w * NT + t) * FL_TILE + xc * 17 + p8 + 8];
         }
         if (pair >= pairs || xr >= n) continue;
+        if (SCALED) {
+          const float rs = row_scale[xr];
+          a *= rs;
+          b *= rs;
+        }
         if (EP == FL_SWIGLU) {
           bf16_t* h = reinterpret_cast<bf16_t*>(out.y);
           h[(long)xr * pairs + pair] = from_f32<bf16_t>(gate_act(a, out.act) * b);
@@ -317,36 +419,52 @@ __global__ __launch_bounds__(256) void fused_linear_kernel(const bf16_t* __restr
     }
     rope_angles(tile + 1);
   }
+  if (EP == FL_RESID && tid < 256) {   // the workgroup's sums of squares, one per row of X
+    const int stride = ((int)gridDim.x + 3) / 4 * 4;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      float v = ss_acc[t];
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+      const int xr = t * 16 + tid / 16;
+      if (tid % 16 == 0 && xr < n) out.ss_out[(long)xr * stride + blockIdx.x] = v;
+    }
+  }
 }
 
-static size_t fl_lds_bytes(int n, int nt, int kslice) {
-  return (size_t)n * (kslice + FL_PAD) * sizeof(bf16_t) + (size_t)(2 * 4 * nt * FL_TILE) * sizeof(float);
+static size_t fl_lds_bytes(int n, int nt, int kslice, int nw = 4) {
+  return (size_t)n * (kslice + fl_pad(nw)) * sizeof(bf16_t) + (size_t)(2 * nw * nt * FL_TILE + 32) * sizeof(float);
 }
 
-template <int NT, int EP>
+template <int NT, int EP, int NW, bool SCALED>
 static int fl_launch(const void* x, const FlOut& out, const void* w, int n, int m, int k, int kslice,
                      int nsplit, int tiles, int tiles_per_wg, int x_stride, hipStream_t stream) {
-  const size_t lds = fl_lds_bytes(n, NT, kslice);
-  static size_t allowed = 64 * 1024;
+  const size_t lds = fl_lds_bytes(n, NT, kslice, NW);
+  static size_t allowed = 64 * 1024;          // one per instantiation
   if (lds > allowed) {
-    hipError_t e = hipFuncSetAttribute((const void*)fused_linear_kernel<NT, EP>,
+    hipError_t e = hipFuncSetAttribute((const void*)fused_linear_kernel<NT, EP, NW, SCALED>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, FL_LDS_MAX);
     if (e != hipSuccess) KLLM_FAIL((int)e, "fused_linear: cannot raise the LDS limit: %s", hipGetErrorString(e));
     allowed = FL_LDS_MAX;
   }
   const dim3 grid(ceil_div(tiles, tiles_per_wg), nsplit);
-  hipLaunchKernelGGL((fused_linear_kernel<NT, EP>), grid, dim3(256), lds, stream, (const bf16_t*)x, out,
-                     (const bf16_t*)w, n, m, k, kslice, tiles, tiles_per_wg, x_stride);
+  hipLaunchKernelGGL((fused_linear_kernel<NT, EP, NW, SCALED>), grid, dim3(64 * NW), lds, stream, (const bf16_t*)x,
+                     out, (const bf16_t*)w, n, m, k, kslice, tiles, tiles_per_wg, x_stride);
   return 0;
 }
 
 template <int NT>
-static int fl_launch_ep(int ep, const void* x, const FlOut& out, const void* w, int n, int m, int k,
+static int fl_launch_ep(int ep, bool scaled, const void* x, const FlOut& out, const void* w, int n, int m, int k,
                         int kslice, int nsplit, int tiles, int tpw, int xs, hipStream_t st) {
   switch (ep) {
-    case FL_PARTS: return fl_launch<NT, FL_PARTS>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
-    case FL_SWIGLU: return fl_launch<NT, FL_SWIGLU>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
-    default: return fl_launch<NT, FL_ROPE>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+    case FL_PARTS: return fl_launch<NT, FL_PARTS, 4, false>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+    case FL_RESID: return fl_launch<NT, FL_RESID, 4, false>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+    case FL_SWIGLU:
+      return scaled ? fl_launch<NT, FL_SWIGLU, 4, true>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st)
+                    : fl_launch<NT, FL_SWIGLU, 4, false>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+    default:
+      return scaled ? fl_launch<NT, FL_ROPE, 4, true>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st)
+                    : fl_launch<NT, FL_ROPE, 4, false>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
   }
 }
 
@@ -362,6 +480,13 @@ extern "C" long kllm_fused_linear_lds_bytes(int n, int k, int nsplit) {
   return (long)fl_lds_bytes(n, ceil_div(n, 16), kslice);
 }
 
+extern "C" int kllm_fused_linear_resid_parts(int m, int tiles_per_wg) {
+  if (m <= 0 || tiles_per_wg <= 0) return -1;
+  return ceil_div(ceil_div(m, 16), tiles_per_wg);
+}
+
+extern "C" int kllm_fused_linear_max_parts(void) { return FL_SS_MAX; }
+
 extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOut* yout, const void* w,
                                  int n, int m, int k, int tiles_per_wg, hipStream_t stream) {
   KLLM_REQUIRE(x && yout && w && yout->y, "fused_linear: null pointer");
@@ -372,7 +497,8 @@ extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOu
   KLLM_REQUIRE(fl_aligned16(w) && fl_aligned16(x), "fused_linear: operands must be 16-byte aligned");
   KLLM_REQUIRE(tiles_per_wg >= 1 && tiles_per_wg <= 64, "fused_linear: %d tiles per workgroup", tiles_per_wg);
   const int ep = yout->kind;
-  KLLM_REQUIRE(ep == FL_PARTS || ep == FL_SWIGLU || ep == FL_ROPE, "fused_linear: unknown output kind %d", ep);
+  KLLM_REQUIRE(ep == FL_PARTS || ep == FL_RESID || ep == FL_SWIGLU || ep == FL_ROPE,
+               "fused_linear: unknown output kind %d", ep);
   const int nsplit = yout->nsplit;
   KLLM_REQUIRE(nsplit >= 1 && nsplit <= 64, "fused_linear: nsplit %d is outside [1, 64]", nsplit);
   KLLM_REQUIRE(nsplit == 1 || ep == FL_PARTS, "fused_linear: K is split only for partial sums");
@@ -390,6 +516,25 @@ extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOu
   out.act = yout->act;
   KLLM_REQUIRE(ep != FL_SWIGLU || (out.act >= 0 && out.act < ACT_COUNT), "fused_linear: unknown activation %d", out.act);
   int tiles = ceil_div(m, 16);
+  const bool scaled = yout->ss_in != nullptr;
+  if (scaled) {
+    KLLM_REQUIRE(ep == FL_SWIGLU || ep == FL_ROPE, "fused_linear: only the gate and the rotation epilogues scale their rows");
+    KLLM_REQUIRE(yout->ss_parts >= 1 && yout->ss_parts <= FL_SS_MAX && fl_aligned16(yout->ss_in) && yout->eps >= 0.f,
+                 "fused_linear: %d partial sums of squares per row are outside [1, %d], or they are not 16-byte aligned",
+                 yout->ss_parts, FL_SS_MAX);
+    out.ss_in = yout->ss_in;
+    out.ss_parts = yout->ss_parts;
+    out.eps = yout->eps;
+  }
+  if (ep == FL_RESID) {
+    KLLM_REQUIRE(yout->resid && yout->norm_w && yout->ss_out, "fused_linear: the residual epilogue needs the stream, "
+                 "the norm's weight and room for the sums of squares");
+    KLLM_REQUIRE(ceil_div(tiles, tiles_per_wg) <= FL_SS_MAX, "fused_linear: %d workgroups leave more than %d sums of "
+                 "squares per row (take more tiles per workgroup)", ceil_div(tiles, tiles_per_wg), FL_SS_MAX);
+    out.resid = yout->resid;
+    out.norm_w = yout->norm_w;
+    out.ss_out = yout->ss_out;
+  }
   if (ep == FL_SWIGLU || ep == FL_ROPE) {
     KLLM_REQUIRE(m % 2 == 0, "fused_linear: m=%d must be even for a pair epilogue", m);
     tiles = ceil_div(m / 2, 8);
@@ -415,8 +560,8 @@ extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOu
     out.KV = KV;
     out.hd = hd;
   }
-  const int rc = nt == 1 ? fl_launch_ep<1>(ep, x, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream)
-                         : fl_launch_ep<2>(ep, x, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream);
+  const int rc = nt == 1 ? fl_launch_ep<1>(ep, scaled, x, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream)
+                         : fl_launch_ep<2>(ep, scaled, x, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream);
   if (rc) return rc;
   KLLM_CHECK_LAUNCH("fused_linear");
   return 0;

@@ -130,14 +130,23 @@ int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_out, const f
  * on the matrix cores, fused with the step after them.  x is [n][k] with a row
  * stride of x_stride elements (0 = k), w is [m][k].  Output:
  *   PARTS   y float32 [nsplit][n][m]; only this one may split K
+ *   RESID   resid float32 [n][m] += x . w^T in place; y bfloat16 [n][m] = the new rows times
+ *           norm_w [m] (the weight of the RMS norm behind the addition); ss_out
+ *           [n][P rounded up to 4] = the workgroups' sums of squares of the new rows,
+ *           P = kllm_fused_linear_resid_parts(m, tiles_per_wg), at most
+ *           kllm_fused_linear_max_parts()
  *   SWIGLU  y bfloat16 [n][m/2] = act(x . w[0:m/2]^T) * (x . w[m/2:m]^T)
  *   ROPE    w = [q; k; v] rows (only q when cache is null): q and k rotated with
  *           cos/sin [n][hd/2] (if given); y = q_out [n][H*hd], k and v go to the
  *           tokens' pages of `cache`
+ * With ss_in (SWIGLU and ROPE only) x is such a y and the sums are multiplied by the row's
+ * rsqrt(sum of ss_in[row][0:ss_parts] / k + eps) before the epilogue: the RMS norm of the
+ * stream, rounded to bfloat16 before the row scale instead of after it.
  * All of a workgroup's slice of K for all rows has to fit into LDS:
  * kllm_fused_linear_lds_bytes says how much a call needs (160 KiB at most). */
 #define KLLM_FUSED_LINEAR_MAX_ROWS 32
 #define KLLM_LINEAR_OUT_PARTS 0
+#define KLLM_LINEAR_OUT_RESID 1
 #define KLLM_LINEAR_OUT_SWIGLU 2
 #define KLLM_LINEAR_OUT_ROPE 3
 typedef struct {
@@ -152,8 +161,16 @@ typedef struct {
   int nsplit;
   int max_pages, page_size, H, KV, hd;
   int act;
+  float* resid;         /* RESID */
+  const float* norm_w;  /* RESID */
+  float* ss_out;        /* RESID */
+  const float* ss_in;   /* row scale of the sums, or null; 16-byte aligned */
+  int ss_parts;
+  float eps;
 } KllmLinearOut;
 long kllm_fused_linear_lds_bytes(int n, int k, int nsplit);
+int kllm_fused_linear_resid_parts(int m, int tiles_per_wg);
+int kllm_fused_linear_max_parts(void);
 int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOut* out, const void* w, int n, int m,
                       int k, int tiles_per_wg, hipStream_t stream);
 

@@ -20,7 +20,7 @@ DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
 GEMV_MAX_ROWS = 8          # what the fused kernels take
 GEMV_BEST_ROWS = 2         # up to here they beat the MFMA kernels in bfloat16 (3 rows: 1.29 against 1.21 ms a step at 1.1B sizes)
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 
 class KernelError(RuntimeError):
@@ -91,6 +91,8 @@ def _declare(lib):
         "kllm_gemv_resid": [P, P, P, P, I, I, I, I, P],
         "kllm_gemv_resid_parts": [I],
         "kllm_fused_linear": [P, I, P, P, I, I, I, I, P],
+        "kllm_fused_linear_resid_parts": [I, I],
+        "kllm_fused_linear_max_parts": [],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
         "kllm_attn_decode_slices": [I, I, I, I, I, I],
@@ -104,14 +106,8 @@ def _declare(lib):
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = c_int
-    for name, args in OPTIONAL_SIGNATURES.items():
-        if hasattr(lib, name):
-            fn = getattr(lib, name)
-            fn.argtypes = args
-            fn.restype = c_int
-
-
-OPTIONAL_SIGNATURES = {}
+    lib.kllm_fused_linear_lds_bytes.argtypes = [I, I, I]
+    lib.kllm_fused_linear_lds_bytes.restype = L
 
 
 def _check(rc: int, what: str):
@@ -444,16 +440,19 @@ class _LinearOut(ctypes.Structure):
     _fields_ = [("y", c_void_p), ("cos_t", c_void_p), ("sin_t", c_void_p), ("cache", c_void_p),
                 ("positions", c_void_p), ("span_of_token", c_void_p), ("block_table", c_void_p),
                 ("kind", c_int), ("nsplit", c_int), ("max_pages", c_int), ("page_size", c_int),
-                ("H", c_int), ("KV", c_int), ("hd", c_int), ("act", c_int)]
+                ("H", c_int), ("KV", c_int), ("hd", c_int), ("act", c_int),
+                ("resid", c_void_p), ("norm_w", c_void_p), ("ss_out", c_void_p), ("ss_in", c_void_p),
+                ("ss_parts", c_int), ("eps", c_float)]
 
 
 FUSED_LINEAR_MAX_ROWS = 32
 FUSED_LINEAR_LDS = 160 * 1024
-LINEAR_PARTS, LINEAR_SWIGLU, LINEAR_ROPE = 0, 2, 3
+LINEAR_PARTS, LINEAR_RESID, LINEAR_SWIGLU, LINEAR_ROPE = 0, 1, 2, 3
 
 
 # Rows up to which the decode-batch kernel beats the split-K kernel plus a separate
 # elementwise launch (measured at widths 2048 -> 2560 and 2048 -> 11264).
+FUSED_NORM_BEST_ROWS = 16      # rows up to which a residual product and a consumer that scales its rows replace the norm kernel
 FUSED_ROPE_BEST_ROWS = 32      # (17 tokens at 1.1B sizes: 1.59 -> 1.55 ms a step against the tiled product and a rotation kernel)
 FUSED_SWIGLU_BEST_ROWS = 16
 
@@ -472,9 +471,30 @@ def fused_linear_fits(n, k, nsplit=1) -> bool:
     multiple of 8, and all rows of a workgroup's slice of K in LDS."""
     if n < 1 or n > FUSED_LINEAR_MAX_ROWS or k % 8:
         return False
-    kslice = -(-(-(-k // nsplit)) // 32) * 32
-    nt = -(-n // 16)
-    return n * (kslice + 136) * 2 + 2 * 4 * nt * 16 * 17 * 4 <= FUSED_LINEAR_LDS
+    return 0 < library().kllm_fused_linear_lds_bytes(int(n), int(k), int(nsplit)) <= FUSED_LINEAR_LDS
+
+
+class ScaledRows:
+    """The input of a decode batch's product as a residual product (LINEAR_RESID) left it:
+    ``xw`` [n, k] bfloat16, the residual stream's rows times the norm's weight, and ``ss``
+    [n, parts rounded up to 4] float32, partial sums of squares of the stream's rows.  The
+    consuming product multiplies its sums by rsqrt(sum of a row's ss / k + eps)."""
+
+    def __init__(self, xw, ss, parts, eps):
+        self.xw, self.ss, self.parts, self.eps = xw, ss, int(parts), float(eps)
+
+    @property
+    def shape(self):
+        return self.xw.shape
+
+
+def fused_resid_parts(n, m, k, tiles_per_wg=1) -> int:
+    """Partial sums of squares per row that a LINEAR_RESID product of these sizes leaves, or 0
+    if the decode-batch kernel does not take them."""
+    if not fused_linear_fits(n, k):
+        return 0
+    parts = library().kllm_fused_linear_resid_parts(int(m), int(tiles_per_wg))
+    return parts if 0 < parts <= library().kllm_fused_linear_max_parts() else 0
 
 
 class Rope:
@@ -487,16 +507,27 @@ class Rope:
         self.page_size, self.heads, self.kv_heads, self.head_dim = page_size, heads, kv_heads, head_dim
 
 
-def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None, act=ACT_SILU):
+def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None, act=ACT_SILU, resid=None, norm_weight=None,
+                 ss_out=None):
     """One launch for a decode batch's product of x [n, k] (bfloat16; a view
     with a row stride is taken) with w [m, k], and the step after it, by
     ``kind``: LINEAR_PARTS y float32 [nsplit, n, m]; LINEAR_SWIGLU y bfloat16
     [n, m/2]; LINEAR_ROPE y = q_out with ``rope`` describing rotation and
-    cache."""
+    cache; LINEAR_RESID adds the product to ``resid`` [n, m] float32 in place, writes
+    y bfloat16 [n, m] = the new rows times ``norm_weight`` [m] and leaves partial sums of
+    squares of the new rows in ``ss_out`` [n, fused_resid_parts rounded up to 4].  ``x`` may
+    be a ``ScaledRows`` (SWIGLU and ROPE): what a LINEAR_RESID product left, see there."""
     m, k = w.shape
     lo = _LinearOut()
     if w.dtype != torch.bfloat16:
         raise KernelError("fused_linear: bfloat16 weights only")
+    if isinstance(x, ScaledRows):
+        sr, x = x, x.xw
+        stride = -(-sr.parts // 4) * 4
+        if kind not in (LINEAR_SWIGLU, LINEAR_ROPE) or tuple(sr.ss.shape) != (x.shape[0], stride):
+            raise KernelError(f"fused_linear: row scales {tuple(sr.ss.shape)} of {sr.parts} parts do not fit "
+                              f"{x.shape[0]} rows, or the output kind {kind} takes none")
+        lo.ss_in, lo.ss_parts, lo.eps = _ptr(sr.ss, "fused_linear ss", torch.float32), sr.parts, sr.eps
     n = x.shape[0]
     lo.kind, lo.nsplit, lo.act = kind, nsplit, int(act)
     if x.dim() != 2 or x.shape[1] != k or x.dtype != torch.bfloat16 or x.stride(1) != 1 or not x.is_cuda:
@@ -504,6 +535,16 @@ def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None, act=ACT_SIL
     x_ptr, x_stride = x.data_ptr(), (x.stride(0) if n > 1 else k)
     if kind == LINEAR_PARTS:
         want, dt = (nsplit, n, m), torch.float32
+    elif kind == LINEAR_RESID:
+        want, dt = (n, m), torch.bfloat16
+        parts = library().kllm_fused_linear_resid_parts(int(m), int(tiles_per_wg))
+        if (resid is None or norm_weight is None or ss_out is None or tuple(resid.shape) != (n, m)
+                or norm_weight.numel() != m or tuple(ss_out.shape) != (n, -(-parts // 4) * 4)):
+            raise KernelError(f"fused_linear: the residual epilogue needs resid [{n}, {m}], the norm's weight [{m}] "
+                              f"and ss_out [{n}, {-(-parts // 4) * 4}]")
+        lo.resid = _ptr(resid, "fused_linear resid", torch.float32)
+        lo.norm_w = _ptr(norm_weight, "fused_linear norm weight", torch.float32)
+        lo.ss_out = _ptr(ss_out, "fused_linear ss_out", torch.float32)
     elif kind == LINEAR_SWIGLU:
         want, dt = (n, m // 2), torch.bfloat16
     elif kind == LINEAR_ROPE:

@@ -102,15 +102,19 @@ class CausalSelfAttention(Part):
                              f"(1 to {K.GENERIC_MAX_PAGE_SIZE})")
 
     def forward(self, ctx, xn, cache, sink=None):
+        dtype = self.runtime.dtype
         if isinstance(xn, Normed):
             n = xn.rows
             opts = self.runtime.options
-            gemv = (K.gemv_fits(n, self.w_in.shape[0], self.hidden, self.runtime.dtype) and n <= K.NORMED_MAX_ROWS
+            gemv = (K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype) and n <= K.NORMED_MAX_ROWS
                     and not opts.get("no_fused_gemv") and self.plain_rotation)
-            # the small-batch kernel below normalises while it stages its input
-            xn = xn.kernel_input() if gemv else xn.materialize(ctx)
+            scaled = (not gemv and xn.xw is not None and dtype == torch.bfloat16 and n <= K.FUSED_ROPE_BEST_ROWS
+                      and K.fused_linear_fits(n, self.hidden) and not opts.get("no_fused_linear")
+                      and self.plain_rotation)
+            # the small-batch kernel below normalises while it stages its input, the decode-batch
+            # kernel scales its sums by the row
+            xn = xn.kernel_input() if gemv else xn.scaled_rows() if scaled else xn.materialize(ctx)
         n = xn.shape[0]
-        dtype = self.runtime.dtype
         writes = self.own_kv
         if writes != bool(cache.write):
             raise ValueError("attention: a run must write its cache exactly when it has k/v projections")

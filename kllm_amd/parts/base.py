@@ -176,11 +176,14 @@ class Normed:
     the residual stream [n, d] (it already holds the sub-layer's output), ``ss`` [n, parts
     rounded up to 4] the partial sums of squares of its rows, ``norm`` the norm part it
     stands for (weight and eps).  A consumer whose kernel normalises while it stages its
-    input takes ``kernel_input()``; any other calls ``materialize``, which runs the norm."""
+    input takes ``kernel_input()``; one whose kernel scales its sums by the row takes
+    ``scaled_rows()`` where the producer also left ``xw``, the rows of x times the norm's
+    weight in the compute dtype; any other calls ``materialize``, which runs the norm."""
     x: torch.Tensor
     ss: torch.Tensor
     parts: int
     norm: "Part"
+    xw: Optional[torch.Tensor] = None
 
     @property
     def rows(self) -> int:
@@ -189,6 +192,10 @@ class Normed:
     def kernel_input(self):
         from .. import kernels as K
         return K.NormedInput(self.x, self.norm.weight, self.ss, self.parts, self.norm.eps)
+
+    def scaled_rows(self):
+        from .. import kernels as K
+        return K.ScaledRows(self.xw, self.ss, self.parts, self.norm.eps)
 
     def materialize(self, ctx):
         return self.norm.forward(ctx, self.x, delta=self)

@@ -61,8 +61,10 @@ class GatedFeedForward(Part):
         gemv = K.gemv_fits(n, 2 * self.intermediate, self.hidden, dtype) and not opts.get("no_fused_gemv")
         fused = (not gemv and dtype == torch.bfloat16 and n <= K.FUSED_SWIGLU_BEST_ROWS
                  and K.fused_linear_fits(n, self.hidden) and not opts.get("no_fused_linear"))
-        if isinstance(xn, Normed):     # the small-batch kernel below normalises while it stages its input
-            xn = xn.kernel_input() if gemv and n <= K.NORMED_MAX_ROWS else xn.materialize(ctx)
+        if isinstance(xn, Normed):     # the small-batch kernel below normalises while it stages its input,
+            # the decode-batch kernel scales its sums by the row
+            xn = (xn.kernel_input() if gemv and n <= K.NORMED_MAX_ROWS
+                  else xn.scaled_rows() if fused and xn.xw is not None else xn.materialize(ctx))
         h = ctx.buf("ffn.h", (n, self.intermediate), dtype)
         if gemv:
             K.gemv_swiglu(xn, self.w_gu, h, self.act)   # few tokens: both products and the gate in one launch

@@ -184,11 +184,24 @@ def linear_into(ctx, x, w, sink, tag):
     if tuple(sink.x.shape) != (n, m) or norm.weight is None or norm.weight.numel() != m:
         return None
     parts = K.resid_parts(n, m, k, x.dtype)
+    if parts:
+        ss = ctx.buf(tag + ".ss", (n, -(-parts // 4) * 4), torch.float32)
+        K.linear_resid(x, w, sink.x, ss)
+        return Normed(sink.x, ss, parts, norm)
+    if x.dtype != torch.bfloat16 or n > K.FUSED_NORM_BEST_ROWS or rt.options.get("no_fused_linear"):
+        return None
+    # a decode batch on the matrix cores: all of K in a workgroup, the addition in the epilogue, and
+    # beside the stream its rows times the norm's weight in 16 bits for a consumer that scales its sums
+    tpw = 1
+    while K.fused_resid_parts(n, m, k, tpw) == 0 and tpw < 64 and K.fused_linear_fits(n, k):
+        tpw *= 2
+    parts = K.fused_resid_parts(n, m, k, tpw)
     if parts == 0:
         return None
     ss = ctx.buf(tag + ".ss", (n, -(-parts // 4) * 4), torch.float32)
-    K.linear_resid(x, w, sink.x, ss)
-    return Normed(sink.x, ss, parts, norm)
+    xw = ctx.buf(tag + ".xw", (n, m), torch.bfloat16)
+    K.fused_linear(w, xw, K.LINEAR_RESID, x=x, tiles_per_wg=tpw, resid=sink.x, norm_weight=norm.weight, ss_out=ss)
+    return Normed(sink.x, ss, parts, norm, xw=xw)
 
 
 def linear(ctx, x, w, tag, out_dtype=torch.float32, split=True):

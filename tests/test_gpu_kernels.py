@@ -555,6 +555,78 @@ def test_fused_linear_rope_append(H, KV, hd, ps, d, tpw):
     assert (q2.cpu().double() - want2).abs().max() < 0.01 * want2.abs().max() + 1e-3
 
 
+@pytest.mark.parametrize("n,m,k,tpw", [(1, 48, 64, 1), (3, 72, 88, 1), (8, 2048, 2048, 1), (8, 2048, 5632, 1),
+                                       (13, 2048, 5632, 2), (16, 100, 264, 3), (19, 33, 3080, 1), (32, 257, 1000, 2),
+                                       (5, 4096, 14336, 1), (12, 4096, 4096, 1)])
+def test_fused_linear_resid_then_scaled_consumers(n, m, k, tpw):
+    """A decode batch's product added to the residual stream in its own epilogue, with what
+    the RMS norm behind the addition needs left beside it; then the two consumers that apply
+    the norm's row scale to their own sums (gate and rotation), against the plain functions
+    in float64: add, norm, product, epilogue."""
+    k_ = K()
+    eps = 1e-5
+    x, w = _bf(n, k, seed=1, scale=0.5), _bf(m, k, seed=2, scale=0.1)
+    resid = rnd(n, m, seed=3, scale=2.0)
+    nw = 1 + 0.2 * rnd(m, seed=4)
+    parts = k_.fused_resid_parts(n, m, k, tpw)
+    assert parts == -(-(-(-m // 16)) // tpw)
+    stride = -(-parts // 4) * 4
+    ss = torch.full((n, stride), float("nan"), device=DEV)
+    xw = torch.full((n, m), float("nan"), dtype=torch.bfloat16, device=DEV)
+    stream = resid.clone()
+    k_.fused_linear(w, xw, k_.LINEAR_RESID, x, tiles_per_wg=tpw, resid=stream, norm_weight=nw, ss_out=ss)
+    want_x = resid.cpu().double() + P.linear(x.cpu().double(), w.cpu().double())
+    bound = 1e-3 * math.sqrt(k) * 0.05 + 1e-4
+    assert (stream.cpu().double() - want_x).abs().max() < bound
+    assert (xw.cpu().double() - want_x * nw.cpu().double()).abs().max() < 0.005 * want_x.abs().max() * 1.2 + 1e-3
+    got_ss = ss[:, :parts].cpu().double().sum(1)
+    assert ((got_ss - (want_x ** 2).sum(1)).abs() / (want_x ** 2).sum(1)).max() < 1e-4
+    # the consumers: x * w in 16 bits as input, the row scale applied to the sums
+    want_n = P.rmsnorm(want_x, nw.cpu().double(), eps)
+    sr = k_.ScaledRows(xw, ss, parts, eps)
+    f = 40
+    wg = _bf(2 * f, m, seed=5, scale=0.1)
+    if k_.fused_linear_fits(n, m):
+        h = torch.full((n, f), float("nan"), dtype=torch.bfloat16, device=DEV)
+        k_.fused_linear(wg, h, k_.LINEAR_SWIGLU, sr)
+        wd = wg.cpu().double()
+        want = P.silu(P.linear(want_n, wd[:f])) * P.linear(want_n, wd[f:])
+        assert (h.cpu().double() - want).abs().max() < 0.01 * want.abs().max() + 2e-3
+        # the same numbers as the norm kernel's rows through the unscaled product, within rounding
+        xn = torch.empty(n, m, dtype=torch.bfloat16, device=DEV)
+        k_.add_rmsnorm(stream, weight=nw, out=xn, eps=eps)
+        h2 = torch.empty_like(h)
+        k_.fused_linear(wg, h2, k_.LINEAR_SWIGLU, xn)
+        assert (h.float() - h2.float()).abs().max() < 0.01 * want.abs().max() + 2e-3
+        # rotation epilogue: two heads of 16, queries only
+        H, hd = 2, 16
+        wq = _bf(H * hd, m, seed=6, scale=0.1)
+        pos = torch.arange(5, 5 + n, dtype=torch.int32, device=DEV)
+        cos = torch.empty(n, hd // 2, device=DEV)
+        sin = torch.empty(n, hd // 2, device=DEV)
+        k_.rope_tables(cos, sin, pos, hd, 10000.0)
+        q = torch.full((n, H * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        k_.fused_linear(wq, q, k_.LINEAR_ROPE, sr, rope=k_.Rope(cos, sin, None, None, None, None, 16, H, 1, hd))
+        want_q = P.rope(P.linear(want_n, wq.cpu().double()), pos.cpu().tolist(), H, hd, 10000.0)
+        assert (q.cpu().double() - want_q).abs().max() < 0.01 * want_q.abs().max() + 2e-3
+
+
+def test_fused_linear_resid_refusals():
+    k_ = K()
+    n, m, k = 4, 64, 64
+    x, w = _bf(n, k, seed=1, scale=0.5), _bf(m, k, seed=2, scale=0.1)
+    xw = torch.empty(n, m, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(k_.KernelError):       # no stream
+        k_.fused_linear(w, xw, k_.LINEAR_RESID, x)
+    with pytest.raises(k_.KernelError):       # sums of squares of the wrong width
+        k_.fused_linear(w, xw, k_.LINEAR_RESID, x, resid=torch.zeros(n, m, device=DEV),
+                        norm_weight=torch.ones(m, device=DEV), ss_out=torch.zeros(n, 8, device=DEV))
+    with pytest.raises(k_.KernelError):       # partial sums do not take a row scale
+        k_.fused_linear(w, torch.empty(1, n, m, device=DEV), k_.LINEAR_PARTS,
+                        k_.ScaledRows(x, torch.zeros(n, 4, device=DEV), 4, 1e-5))
+    assert k_.fused_resid_parts(8, 16 * 300, 64) == 0 and k_.fused_resid_parts(8, 16 * 300, 64, 2) == 150
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("n", [1, 2, 3, 4])
 @pytest.mark.parametrize("d,kin,f", [(64, 48, 88), (2048, 2048, 5632), (2048, 5632, 256), (104, 264, 72), (4096, 512, 64)])

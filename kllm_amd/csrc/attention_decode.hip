@@ -471,14 +471,24 @@ constexpr int kMaxDevices = 64;
 static float* g_scratch_ptr[kMaxDevices];        // per device, null until looked up
 static std::mutex g_scratch_mutex;
 
-// The array's address on the current device (looked up at the first call there).
-static int scratch_on_current_device(float** ptr) {
+// The array's address on the current device (looked up at the first call there).  The lookup
+// may load the module's device variables, which a thread that is recording a graph must not
+// do: a first call on a device while `stream` is being captured is refused.
+static int scratch_on_current_device(float** ptr, hipStream_t stream, bool check_capture) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) KLLM_FAIL((int)e, "attn_decode_static: hipGetDevice: %s", hipGetErrorString(e));
   KLLM_REQUIRE(dev >= 0 && dev < kMaxDevices, "attn_decode_static: device %d is outside [0, %d)", dev, kMaxDevices);
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (!g_scratch_ptr[dev]) {
+    if (check_capture) {
+      hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+      e = hipStreamIsCapturing(stream, &st);
+      if (e != hipSuccess) KLLM_FAIL((int)e, "attn_decode_static: hipStreamIsCapturing: %s", hipGetErrorString(e));
+      if (st != hipStreamCaptureStatusNone)
+        KLLM_FAIL(ERR_STATE, "attn_decode_static: the first call on device %d came while its stream is being "
+                  "captured; call kllm_attn_decode_static_init() on the device before recording", dev);
+    }
     float* p = nullptr;
     e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !p)
@@ -488,6 +498,11 @@ static int scratch_on_current_device(float** ptr) {
   }
   *ptr = g_scratch_ptr[dev];
   return 0;
+}
+
+extern "C" int kllm_attn_decode_static_init(void) {
+  float* part = nullptr;
+  return scratch_on_current_device(&part, nullptr, false);
 }
 
 extern "C" int kllm_attn_decode_static(const void* q, void* out, const void* cache, const int* positions,
@@ -504,7 +519,7 @@ extern "C" int kllm_attn_decode_static(const void* q, void* out, const void* cac
                "with a workspace",
                n, H, nslices, hd, need, (long)KLLM_ATTN_DECODE_STATIC_FLOATS);
   float* part = nullptr;
-  if (int rc = scratch_on_current_device(&part)) return rc;
+  if (int rc = scratch_on_current_device(&part, stream, true)) return rc;
   // Nothing in the scratch has to start at zero: the first kernel writes every partial result
   // (maximum, sum, output of each token, head and slice) that the second one reads.
   return attn_decode_run("attn_decode_static", q, out, part, (long)KLLM_ATTN_DECODE_STATIC_FLOATS, cache,

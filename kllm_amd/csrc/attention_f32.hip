@@ -404,6 +404,8 @@ bool attn_f32_fits(int hd, int page_size) {
   return hd >= 8 && hd <= 256 && hd % 8 == 0 && page_size > 0 && page_size % 4 == 0;
 }
 
+extern "C" int kllm_attn_f32_fits(int hd, int page_size) { return attn_f32_fits(hd, page_size) ? 1 : 0; }
+
 int attn_f32_slices(int n, int KV, int H, int max_keys) {
   // About four waves per CU across the chip (eight from one group per CU on, where partial
   // results cost little beside the keys), shared out over tokens x KV heads x blocks of 32

@@ -109,6 +109,8 @@ void set_error(const char* fmt, ...);
 
 // Compute units of the current device (cached); 256 if it cannot be asked.
 int device_cus();
+// XCDs of the current device (cached); 8 if it cannot be asked.
+int device_xcds();
 
 inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
 

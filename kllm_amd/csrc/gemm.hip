@@ -143,9 +143,9 @@ __global__ __launch_bounds__(256) void gemm_f32_tiled_kernel(const float* __rest
 // (reference: backend/model.cu:477-483, :1112-1114) -- the gated activation
 // never exists in 32-bit in memory.
 //
-// Workgroups are numbered so that the eight XCDs (which take workgroups
-// round-robin, each with an L2 of its own) each get a contiguous run of tiles
-// that share rows of X.
+// Workgroups are numbered so that the XCDs (which take workgroups round-robin,
+// each with an L2 of its own; their number is asked of the runtime) each get a
+// contiguous run of tiles that share rows of X.
 constexpr int MBN = 128;
 constexpr int MROW = 128;                     // bytes of a tile row in LDS: one stage of K
 
@@ -176,7 +176,8 @@ template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES, int WC = 2,
 __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2))) void gemm_mfma_kernel(const T* __restrict__ X,
                                                              const T* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
-                                                             int k, int tiles_x, int tiles_y, int kslice, int act) {
+                                                             int k, int tiles_x, int tiles_y, int kslice, int act,
+                                                             int xcds) {
   typedef typename MfmaOperand<T>::type op_t;   // 16 bytes of a row
   constexpr int EPC = 16 / sizeof(T);           // elements of a 16-byte chunk
   constexpr int MBK = MROW / sizeof(T);         // elements of K per stage
@@ -194,8 +195,8 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int wr = wave / WC, wc = wave % WC;
   const long total = (long)tiles_x * tiles_y;
-  const long per_xcd = (total + 7) / 8;
-  const long id = (long)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  const long per_xcd = (total + xcds - 1) / xcds;
+  const long id = (long)(blockIdx.x % xcds) * per_xcd + blockIdx.x / xcds;
   if (id >= total) return;
   // An XCD's run of tiles walks the shorter side fastest: it then reads only its share
   // of the larger operand and shares the smaller one.
@@ -362,7 +363,8 @@ static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m,
   constexpr int BM = 32 * WTM * WR, BN = 32 * WTN * WC;
   const int tx = ceil_div(m, DUAL ? BN / 2 : BN), ty = ceil_div(n, BM);
   const int kslice = ceil_div(ceil_div(k, nsplit), MBK) * MBK;
-  const dim3 grid(ceil_div((long)tx * ty, 8) * 8, nsplit);   // padded so that every XCD gets as many
+  const int xcds = device_xcds();
+  const dim3 grid(ceil_div((long)tx * ty, xcds) * xcds, nsplit);   // padded so that every XCD gets as many
   const size_t lds = (size_t)MSTAGES * (BM + BN) * MROW;
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
@@ -372,7 +374,7 @@ static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m,
     raised = 1;
   }
   hipLaunchKernelGGL((gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES, WC, WTM, WTN>), grid, dim3(64 * WR * WC), lds, stream,
-                     (const T*)x, (const T*)w, (TOUT*)y, n, m, k, tx, ty, kslice, act);
+                     (const T*)x, (const T*)w, (TOUT*)y, n, m, k, tx, ty, kslice, act, xcds);
   return 0;
 }
 
@@ -699,6 +701,10 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, float* y, int n, int 
   const dim3 grid(ceil_div(m, 64 * RT), nsplit);
   hipLaunchKernelGGL((gemm_bf16_skinny_kernel<NT, RT>), grid, dim3(256), lds, stream, x, w, y, n, m, k, kslice);
   return 0;
+}
+
+extern "C" int kllm_gemm_decode_tile_cols(int n, int m, int k) {
+  return n <= 64 && (long)m * k < kNarrowBelow ? 64 : MBN;
 }
 
 extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, int k, int dtype,

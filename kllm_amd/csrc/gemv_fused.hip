@@ -334,7 +334,8 @@ static int launch_gv_n(const void* x, const void* w, void* y, int n, int m, int 
   if (nt == 1) KLLM_GV(1);
   else if (nt == 2) KLLM_GV(2);
   else if (nt == 4) KLLM_GV(4);
-  else if (!NORMED) KLLM_GV(NORMED ? 4 : 8);     // normalising while staging is built for up to four rows
+  else if (!NORMED) KLLM_GV(8);
+  else KLLM_FAIL(ERR_ARG, "gemv: normalising while staging is built for up to %d rows, not %d", GV_NORMED_MAXN, n);
 #undef KLLM_GV
   return 0;
 }
@@ -388,13 +389,17 @@ extern "C" int kllm_gemv_resid(const void* x, const void* w, float* resid, float
   GvRope rp = {};
   rp.resid = resid;
   rp.ss_out = ss_out;
-  if (dtype == DT_F32) launch_gv<float, GV_RESID>(x, w, resid, n, m, k, 0, rp, stream);
-  else launch_gv<bf16_t, GV_RESID>(x, w, resid, n, m, k, 0, rp, stream);
+  if (int rc = dtype == DT_F32 ? launch_gv<float, GV_RESID>(x, w, resid, n, m, k, 0, rp, stream)
+                                 : launch_gv<bf16_t, GV_RESID>(x, w, resid, n, m, k, 0, rp, stream))
+    return rc;
   KLLM_CHECK_LAUNCH("gemv_resid");
   return 0;
 }
 
 extern "C" int kllm_gemv_resid_parts(int m) { return ceil_div(m / 2, GV_WAVES); }
+extern "C" int kllm_gemv_max_rows(void) { return GV_MAXN; }
+extern "C" int kllm_gemv_normed_max_rows(void) { return GV_NORMED_MAXN; }
+extern "C" int kllm_gemv_normed_max_parts(void) { return GV_SS_MAX; }
 
 extern "C" int kllm_gemv_plain(const void* x, const void* w, float* y, int n, int m, int k, int dtype,
                                const KllmNormedInput* normed, hipStream_t stream) {
@@ -402,8 +407,9 @@ extern "C" int kllm_gemv_plain(const void* x, const void* w, float* y, int n, in
   if (int rc = check_common("gemv_plain", x, w, y, n, m, k, dtype)) return rc;
   GvRope rp = {};
   if (int rc = set_norm("gemv_plain", rp, normed, n)) return rc;
-  if (dtype == DT_F32) launch_gv<float, GV_PLAIN>(x, w, y, n, m, k, 0, rp, stream);
-  else launch_gv<bf16_t, GV_PLAIN>(x, w, y, n, m, k, 0, rp, stream);
+  if (int rc = dtype == DT_F32 ? launch_gv<float, GV_PLAIN>(x, w, y, n, m, k, 0, rp, stream)
+                                 : launch_gv<bf16_t, GV_PLAIN>(x, w, y, n, m, k, 0, rp, stream))
+    return rc;
   KLLM_CHECK_LAUNCH("gemv_plain");
   return 0;
 }
@@ -416,8 +422,9 @@ extern "C" int kllm_gemv_swiglu(const void* x, const void* w_gate_up, void* h, i
   GvRope rp = {};
   rp.act = act;
   if (int rc = set_norm("gemv_swiglu", rp, normed, n)) return rc;
-  if (dtype == DT_F32) launch_gv<float, GV_SWIGLU>(x, w_gate_up, h, n, 2 * f, k, f, rp, stream);
-  else launch_gv<bf16_t, GV_SWIGLU>(x, w_gate_up, h, n, 2 * f, k, f, rp, stream);
+  if (int rc = dtype == DT_F32 ? launch_gv<float, GV_SWIGLU>(x, w_gate_up, h, n, 2 * f, k, f, rp, stream)
+                                 : launch_gv<bf16_t, GV_SWIGLU>(x, w_gate_up, h, n, 2 * f, k, f, rp, stream))
+    return rc;
   KLLM_CHECK_LAUNCH("gemv_swiglu");
   return 0;
 }
@@ -440,8 +447,9 @@ extern "C" int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_o
   rp.positions = positions; rp.span_of_token = span_of_token; rp.block_table = block_table;
   rp.max_pages = max_pages; rp.page_size = page_size; rp.H = H; rp.KV = KV; rp.hd = hd;
   if (int rc = set_norm("gemv_rope_append", rp, normed, n)) return rc;
-  if (dtype == DT_F32) launch_gv<float, GV_ROPE>(x, w_qkv, q_out, n, m, k, 0, rp, stream);
-  else launch_gv<bf16_t, GV_ROPE>(x, w_qkv, q_out, n, m, k, 0, rp, stream);
+  if (int rc = dtype == DT_F32 ? launch_gv<float, GV_ROPE>(x, w_qkv, q_out, n, m, k, 0, rp, stream)
+                                 : launch_gv<bf16_t, GV_ROPE>(x, w_qkv, q_out, n, m, k, 0, rp, stream))
+    return rc;
   KLLM_CHECK_LAUNCH("gemv_rope_append");
   return 0;
 }

@@ -34,8 +34,9 @@ int kllm_last_error(char* buf, int len);
 int kllm_device_info(int device, char* buf, int len);
 /* ABI version, bumped when a signature changes. */
 int kllm_abi_version(void);
-/* Compute units of the current device (the launch heuristics scale with it). */
+/* Compute units and XCDs of the current device (the launch heuristics scale with them). */
 int kllm_device_cus(void);
+int kllm_device_xcds(void);
 
 /* What the box reaches with nothing in the way, for quoting measured figures against: a
  * plain copy of `bytes` (a multiple of 16) and a loop of `iters` rounds of four independent
@@ -84,6 +85,9 @@ int kllm_silu_mul(const void* gu, int in_dtype, int nsplit, long split_stride, v
 int kllm_sum_splits(const float* in, int nsplit, long count, void* out, int out_dtype,
                     hipStream_t stream);
 
+/* Columns of the tiles that a decode batch of n rows (at most 64) gets against w[m][k] on the
+ * MFMA kernel: a caller that cuts K into slices counts its workgroups with it. */
+int kllm_gemm_decode_tile_cols(int n, int m, int k);
 /* y[nsplit][n][m] = x[n][k] . w[m][k]^T, 32-bit accumulation. */
 int kllm_gemm(const void* x, const void* w, void* y, int n, int m, int k, int dtype, int out_dtype,
               int algo, int nsplit, hipStream_t stream);
@@ -120,6 +124,10 @@ int kllm_gemv_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f
 int kllm_gemv_resid(const void* x, const void* w, float* resid, float* ss_out, int n, int m, int k,
                     int dtype, hipStream_t stream);
 int kllm_gemv_resid_parts(int m);
+/* Limits of the kernels above: rows of x, rows when `normed` is given, normed->parts. */
+int kllm_gemv_max_rows(void);
+int kllm_gemv_normed_max_rows(void);
+int kllm_gemv_normed_max_parts(void);
 int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_out, const float* cos_t,
                           const float* sin_t, void* cache, const int* positions,
                           const int* span_of_token, const int* block_table, int max_pages,
@@ -191,6 +199,8 @@ int kllm_attn_generic(const void* q, void* out, const void* cache, const int* po
  * of 2,048).  With token_list only the n_listed tokens it names are computed (q,
  * out and part stay indexed by token row). */
 int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, int max_keys);
+/* Whether the float32 attention on the matrix cores takes this head size and page size. */
+int kllm_attn_f32_fits(int hd, int page_size);
 int kllm_attn_decode(const void* q, void* out, float* part, long part_floats, const void* cache,
                      const int* positions, const int* span_of_token, const int* block_table,
                      int max_pages, int page_size, int n, int H, int KV, int hd, int window,
@@ -203,11 +213,15 @@ int kllm_attn_decode(const void* q, void* out, float* part, long part_floats, co
  * results go to an array that the library holds on every GPU it runs on
  * (KLLM_ATTN_DECODE_STATIC_FLOATS floats = 4 MiB, kept until the process ends); a call whose
  * n * H * nslices * (hd + 2) exceeds that is refused.  The array's address is looked up at
- * the first call on a device, which must be the current device (and the stream's).  All
- * calls on one GPU share the array and it keeps the last call's contents: calls that
- * overlap on one GPU (two streams, two threads) race; nothing in it needs clearing
- * between calls.  Same kernels, same results as kllm_attn_decode. */
+ * the first call on a device, which must be the current device (and the stream's), or by
+ * kllm_attn_decode_static_init(); a first call while the stream is being captured is refused
+ * (the lookup is not graph work): call the init function on the device before recording.
+ * All calls on one GPU share the array and it keeps the last call's contents: the caller
+ * must serialise them on one stream per GPU (calls that overlap on one GPU, from two streams
+ * or two threads, a replayed graph beside eager calls, race on it); nothing in it needs
+ * clearing between calls.  Same kernels, same results as kllm_attn_decode. */
 #define KLLM_ATTN_DECODE_STATIC_FLOATS (1 << 20)
+int kllm_attn_decode_static_init(void);
 int kllm_attn_decode_static(const void* q, void* out, const void* cache, const int* positions,
                             const int* span_of_token, const int* block_table, int max_pages,
                             int page_size, int n, int H, int KV, int hd, int window, float scale,

@@ -30,6 +30,20 @@ int device_cus() {
   return cached[dev];
 }
 
+// XCDs (dies with an L2 of their own, which take workgroups round-robin) of the current device,
+// asked once per device; 8 if it cannot be asked.
+int device_xcds() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 8;
+  if (cached[dev] == 0) {
+    int xcds = 0;
+    if (hipDeviceGetAttribute(&xcds, hipDeviceAttributeNumberOfXccs, dev) != hipSuccess || xcds <= 0) xcds = 8;
+    cached[dev] = xcds;
+  }
+  return cached[dev];
+}
+
 // ---- what the box reaches with nothing in the way (for quoting figures against) ----------
 __global__ __launch_bounds__(256) void calibrate_copy_kernel(floatx4* __restrict__ dst,
                                                              const floatx4* __restrict__ src, long n16) {
@@ -96,6 +110,7 @@ extern "C" int kllm_calibrate_mfma(int dtype, int iters, float* sink, double* fl
 }
 
 extern "C" int kllm_device_cus(void) { return kllm::device_cus(); }
+extern "C" int kllm_device_xcds(void) { return kllm::device_xcds(); }
 
 extern "C" int kllm_last_error(char* buf, int len) {
   if (!buf || len <= 0) return 0;

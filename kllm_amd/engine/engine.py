@@ -159,7 +159,6 @@ class Engine:
         ``max_requests`` requests can hold at one time."""
         o = self.options
         plan = self.model.cache_plan
-        elem = torch.empty((), dtype=self.dtype).element_size()
         if o.page_size <= 0:
             raise ValueError(f"page_size {o.page_size} must be positive")
         for part in self.model.all_parts():
@@ -175,10 +174,21 @@ class Engine:
         for g, gp in enumerate(plan.groups):
             if gp.need.kind not in ("paged", "state"):
                 raise ValueError(f"unknown cache kind {gp.need.kind!r}")
-        state_bytes = sum(gp.entries * o.max_requests * _numel(gp.need.state_shape) * 4
+        def dtype_of(need, default):
+            if need.dtype is None:
+                return default
+            dt = getattr(torch, str(need.dtype), None)
+            if not isinstance(dt, torch.dtype):
+                raise ValueError(f"cache dtype {need.dtype!r} is no torch dtype")
+            return dt
+
+        def size_of(dt):
+            return torch.empty((), dtype=dt).element_size()
+        state_bytes = sum(gp.entries * o.max_requests * _numel(gp.need.state_shape)
+                          * size_of(dtype_of(gp.need, torch.float32))
                           for gp in plan.groups if gp.need.kind == "state")
-        page_bytes = {g: gp.entries * 2 * gp.need.kv_heads * o.page_size * gp.need.head_dim * elem
-                      for g, gp in paged}
+        page_bytes = {g: gp.entries * gp.need.kv_heads * o.page_size * (gp.need.head_dim + gp.need.value_width)
+                      * size_of(dtype_of(gp.need, self.dtype)) for g, gp in paged}
         step = o.max_step_tokens or self.max_model_len or 0
         want = {}
         for g, gp in paged:
@@ -206,21 +216,25 @@ class Engine:
             if need.kind == "paged":
                 self._paged_group_of[g] = len(groups)
                 groups.append(GroupSpec(f"group{g}", o.page_size, want[g], need.window))
-                self.kv[g] = torch.zeros(
-                    gp.entries, want[g], 2, need.kv_heads, o.page_size * need.head_dim,
-                    dtype=self.dtype, device=self.device)
+                if need.value_width == need.head_dim:
+                    shape = (2, need.kv_heads, o.page_size * need.head_dim)
+                else:       # keys and values of different widths (or no values): the mixer lays a page out
+                    shape = (need.kv_heads * o.page_size * (need.head_dim + need.value_width),)
+                self.kv[g] = torch.zeros(gp.entries, want[g], *shape, dtype=dtype_of(need, self.dtype),
+                                         device=self.device)
                 self._capacity.append(
                     f"group{g}: {gp.entries} layers, {need.kv_heads} KV heads of {need.head_dim}"
+                    + (f" (values of {need.value_width})" if need.value_width != need.head_dim else "")
                     + (f", window {need.window}" if need.window else "")
                     + f": {want[g]} pages of {o.page_size} tokens = {want[g] * o.page_size} tokens, "
                     f"{want[g] * page_bytes[g] / 2**20:.1f} MiB"
                     + (f" (asked for {asked} pages)" if want[g] != asked else ""))
             else:
                 self.state[g] = torch.zeros(gp.entries, o.max_requests, *need.state_shape,
-                                            dtype=torch.float32, device=self.device)
+                                            dtype=dtype_of(need, torch.float32), device=self.device)
                 self._capacity.append(
-                    f"group{g}: {gp.entries} layers with state {tuple(need.state_shape)} in "
-                    f"{o.max_requests} slots, {self.state[g].numel() * 4 / 2**20:.1f} MiB")
+                    f"group{g}: {gp.entries} layers with state {tuple(need.state_shape)} in {o.max_requests} slots, "
+                    f"{self.state[g].numel() * self.state[g].element_size() / 2**20:.1f} MiB")
         self.cache = CacheManager(groups, o.max_requests)
 
     def capacity_report(self) -> str:
@@ -238,7 +252,8 @@ class Engine:
             ids = [p for p in per_group_pages[mg] if p >= 0]
             if ids:
                 idx = torch.tensor(ids, dtype=torch.long, device=self.device)
-                self.kv[g][:, idx] = float("nan")
+                kv = self.kv[g]
+                kv[:, idx] = float("nan") if kv.is_floating_point() else torch.iinfo(kv.dtype).min
 
     # ------------------------------------------------------------------ requests
     def open(self, request_id: Hashable):

@@ -46,13 +46,22 @@ def _bucket(pages: int) -> int:
 class SampledTokens:
     """The token ids of a sampled step, on their way to the host."""
 
-    def __init__(self, host: torch.Tensor, event: torch.cuda.Event, count: int, logits=None):
+    def __init__(self, host: torch.Tensor, event: torch.cuda.Event, count: int, logits=None, recording=None):
         self._host, self._event, self.count = host, event, count
         self._ids = None
-        # The step's float32 logits [count, vocab] on the device, in the recording's own
-        # buffer: they are what was sampled from, and hold until a step of the same batch
-        # size and table width is queued again.
-        self.logits = logits
+        self._logits, self._recording = logits, recording
+        self._use = recording.uses if recording is not None else 0
+
+    @property
+    def logits(self):
+        """The step's float32 logits [count, vocab] on the device, what was sampled from.  They
+        lie in the recording's own buffer and hold until a step of the same batch size and
+        table width is queued again; asked for after that, this raises instead of handing out
+        the later step's numbers (clone them before queuing on if they are to be kept)."""
+        if self._recording is not None and self._recording.uses != self._use:
+            raise RuntimeError("the logits of this step have been overwritten: a step of the same shape was "
+                               "queued since; read (or clone) them before queuing the next step")
+        return self._logits
 
     def ready(self) -> bool:
         return self._ids is not None or self._event.query()
@@ -84,6 +93,7 @@ class _Recording:
         self.workspace = Workspace(engine.device)
         self.graph = None
         self.replays = 0
+        self.uses = 0            # runs of the step, direct or replayed: each overwrites ``logits``
         self.logits = None
 
 
@@ -152,9 +162,10 @@ class DecodeGraphs:
             control.fill(host.numpy(), rec.layout, tokens, pos0, [rc.slot for rc in rcs], rows, tables,
                          temperatures, uniforms, token_from, lists=rec.lists)
             eng._send(host, rec.control, rec.layout.total)
+            rec.uses += 1
             if rec.graph is None:
                 self._run(rec, lens, pos0)              # the step itself, and the warm-up
-                out = self._read_back(batch, rec.logits)
+                out = self._read_back(batch, rec)
                 out.tokens()                            # before the capture's second run of the kernels
                 graph = torch.cuda.CUDAGraph()
                 # No collection of garbage while recording: it may destroy the recordings of an
@@ -173,7 +184,7 @@ class DecodeGraphs:
             else:
                 rec.graph.replay()
                 rec.replays += 1
-                out = self._read_back(batch, rec.logits)
+                out = self._read_back(batch, rec)
         except Exception:
             eng._undo(opened, reserved)
             raise
@@ -181,7 +192,7 @@ class DecodeGraphs:
         self.last = out
         return out
 
-    def _read_back(self, batch: int, logits=None) -> SampledTokens:
+    def _read_back(self, batch: int, rec: _Recording) -> SampledTokens:
         """Queue the copy of the sampled ids to the host behind the step."""
         i = self._host_next
         self._host_next = (i + 1) % len(self._host_ring)
@@ -191,5 +202,5 @@ class DecodeGraphs:
         host[:batch].copy_(self.sampled[:batch], non_blocking=True)
         event = torch.cuda.Event()
         event.record()
-        self._host_owner[i] = SampledTokens(host, event, batch, logits)
+        self._host_owner[i] = SampledTokens(host, event, batch, rec.logits, rec)
         return self._host_owner[i]

@@ -18,7 +18,6 @@ import torch
 
 DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
-GEMV_MAX_ROWS = 8          # what the fused kernels take
 GEMV_BEST_ROWS = 2         # up to here they beat the MFMA kernels in bfloat16 (3 rows: 1.29 against 1.21 ms a step at 1.1B sizes)
 ABI_VERSION = 7
 
@@ -30,6 +29,19 @@ class KernelError(RuntimeError):
 _lib = None
 _lib_path = None
 _lock = threading.Lock()
+
+
+def limit(name: str) -> int:
+    """A size limit of the kernels, asked of the library (so that the host's choice of a
+    kernel and the kernel's own checks cannot drift apart): ``gemv_max_rows``,
+    ``gemv_normed_max_rows``, ``gemv_normed_max_parts``, ``fused_linear_max_parts``."""
+    v = _limits.get(name)
+    if v is None:
+        v = _limits[name] = int(getattr(library(), "kllm_" + name)())
+    return v
+
+
+_limits = {}
 
 
 def dtype_code(dtype: torch.dtype) -> int:
@@ -97,6 +109,12 @@ def _declare(lib):
         "kllm_sample": [P, P, P, P, I, I, P],
         "kllm_attn_decode_slices": [I, I, I, I, I, I],
         "kllm_device_cus": [],
+        "kllm_device_xcds": [],
+        "kllm_gemm_decode_tile_cols": [I, I, I],
+        "kllm_gemv_max_rows": [],
+        "kllm_gemv_normed_max_rows": [],
+        "kllm_gemv_normed_max_parts": [],
+        "kllm_attn_f32_fits": [I, I],
         "kllm_calibrate_copy": [P, P, L, P],
         "kllm_calibrate_mfma": [I, I, P, P, P],
         "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, P],
@@ -294,7 +312,6 @@ class NormedInput:
     kernel while it stages X: ``x`` [n, k] float32 (the stream, already holding what was
     added), the norm's ``weight`` [k] and ``eps``, and ``ss`` [n, parts rounded up to 4]
     float32, the partial sums of squares of x's rows that a residual product left."""
-    MAX_PARTS = 512
 
     def __init__(self, x, weight, ss, parts, eps):
         self.x, self.weight, self.ss, self.parts, self.eps = x, weight, ss, int(parts), float(eps)
@@ -306,7 +323,7 @@ class NormedInput:
     def struct(self, n, k):
         stride = -(-self.parts // 4) * 4
         if (tuple(self.x.shape) != (n, k) or self.weight.numel() != k or tuple(self.ss.shape) != (n, stride)
-                or not 1 <= self.parts <= self.MAX_PARTS):
+                or not 1 <= self.parts <= limit("gemv_normed_max_parts")):
             raise KernelError(f"normed input: stream {tuple(self.x.shape)}, weight {tuple(self.weight.shape)}, sums of "
                               f"squares {tuple(self.ss.shape)} do not fit {n} x {k} with {self.parts} parts")
         return _NormedInput(_ptr(self.x, "normed x", torch.float32), _ptr(self.weight, "normed weight", torch.float32),
@@ -325,7 +342,9 @@ def _x_and_norm(x, dtype):
     return _ptr(x, "x"), None, n, k
 
 
-NORMED_MAX_ROWS = 4    # rows that the small-batch kernels normalise while they stage their input
+def normed_max_rows() -> int:
+    """Rows that the small-batch kernels normalise while they stage their input."""
+    return limit("gemv_normed_max_rows")
 
 
 def resid_parts(n, m, k, dtype, best=True):
@@ -333,10 +352,10 @@ def resid_parts(n, m, k, dtype, best=True):
     leaves (one per workgroup of eight rows of W), or 0 if the small-batch
     kernel with that epilogue does not take them (``best``: or is not the
     faster choice)."""
-    if not (gemv_fits(n, m, k, dtype, best) and n <= NORMED_MAX_ROWS):
+    if not (gemv_fits(n, m, k, dtype, best) and n <= normed_max_rows()):
         return 0
     parts = library().kllm_gemv_resid_parts(m)
-    return parts if parts <= NormedInput.MAX_PARTS else 0
+    return parts if parts <= limit("gemv_normed_max_parts") else 0
 
 
 def linear_resid(x, w, resid, ss):
@@ -382,7 +401,7 @@ def gemv_fits(n, m, k, dtype, best=True) -> bool:
     ``best``, are the faster choice: always in float32 (which has no MFMA
     kernel for decode batches), up to GEMV_BEST_ROWS rows in bfloat16."""
     v = 4 if dtype == torch.float32 else 8
-    most = GEMV_MAX_ROWS if dtype == torch.float32 or not best else GEMV_BEST_ROWS
+    most = limit("gemv_max_rows") if dtype == torch.float32 or not best else GEMV_BEST_ROWS
     return n <= most and m % 2 == 0 and k % v == 0
 
 
@@ -494,7 +513,7 @@ def fused_resid_parts(n, m, k, tiles_per_wg=1) -> int:
     if not fused_linear_fits(n, k):
         return 0
     parts = library().kllm_fused_linear_resid_parts(int(m), int(tiles_per_wg))
-    return parts if 0 < parts <= library().kllm_fused_linear_max_parts() else 0
+    return parts if 0 < parts <= limit("fused_linear_max_parts") else 0
 
 
 class Rope:
@@ -620,7 +639,12 @@ def attn_decode_slices(n, n_kv_heads, n_heads, head_dim, dtype=torch.bfloat16, m
 def attn_f32_fits(head_dim, page_size) -> bool:
     """Sizes the float32 attention on the matrix cores takes; the rest goes to
     the generic kernel."""
-    return 8 <= head_dim <= 256 and head_dim % 8 == 0 and page_size > 0 and page_size % 4 == 0
+    return bool(library().kllm_attn_f32_fits(int(head_dim), int(page_size)))
+
+
+def gemm_decode_tile_cols(n, m, k) -> int:
+    """Columns of the tiles that the MFMA kernel gives a decode batch of these sizes."""
+    return int(library().kllm_gemm_decode_tile_cols(int(n), int(m), int(k)))
 
 
 _cus = None

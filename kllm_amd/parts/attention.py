@@ -106,7 +106,7 @@ class CausalSelfAttention(Part):
         if isinstance(xn, Normed):
             n = xn.rows
             opts = self.runtime.options
-            gemv = (K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype) and n <= K.NORMED_MAX_ROWS
+            gemv = (K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype) and n <= K.normed_max_rows()
                     and not opts.get("no_fused_gemv") and self.plain_rotation)
             scaled = (not gemv and xn.xw is not None and dtype == torch.bfloat16 and n <= K.FUSED_ROPE_BEST_ROWS
                       and K.fused_linear_fits(n, self.hidden) and not opts.get("no_fused_linear")

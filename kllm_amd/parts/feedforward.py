@@ -63,7 +63,7 @@ class GatedFeedForward(Part):
                  and K.fused_linear_fits(n, self.hidden) and not opts.get("no_fused_linear"))
         if isinstance(xn, Normed):     # the small-batch kernel below normalises while it stages its input,
             # the decode-batch kernel scales its sums by the row
-            xn = (xn.kernel_input() if gemv and n <= K.NORMED_MAX_ROWS
+            xn = (xn.kernel_input() if gemv and n <= K.normed_max_rows()
                   else xn.scaled_rows() if fused and xn.xw is not None else xn.materialize(ctx))
         h = ctx.buf("ffn.h", (n, self.intermediate), dtype)
         if gemv:

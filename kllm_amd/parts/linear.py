@@ -100,9 +100,6 @@ def _mfma_f32_split(n, m, k):
     return int(nsplit)
 
 
-NARROW_BELOW = 40_000_000     # weights (elements) below which the library gives a decode batch tiles of 64 columns
-
-
 def _tiles_beat_skinny(n, m, k):
     """Decode batches of more than 16 rows (two or more of the skinny kernel's 16-row
     tiles): the tiled kernel (tiles of 64 rows, both operands through LDS in whole cache lines) takes nearly
@@ -124,9 +121,10 @@ def _decode_tile_split(n, m, k):
     has a workgroup, then further ones of at least 512, up to 16 (measured at 64 rows, in us
     by slices: 2,048 x 5,632: 14.9 with 4, 9.8 with 8; 11,264 x 2,048: 17.3 with 2, 14.3 with 4,
     17.7 with 8; 4,096 x 4,096: 12.2 with 4, 10.3 with 8, 11.2 with 16)."""
-    if m * k >= NARROW_BELOW:
+    cols = K.gemm_decode_tile_cols(n, m, k)     # the library's choice: 64 below 40 M weights
+    if cols != 64:
         return _mfma_split(n, m, k)
-    tiles, cus = -(-m // 64), K.device_cus()
+    tiles, cus = -(-m // cols), K.device_cus()
     nsplit = 1
     while nsplit < 16 and ((tiles * nsplit < cus and k // (2 * nsplit) >= 256) or k // (2 * nsplit) >= 512):
         nsplit *= 2

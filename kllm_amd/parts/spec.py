@@ -32,18 +32,31 @@ class CacheNeed:
 
     kind "paged": keys and values per token, in pages; ``window`` > 0 means
     only the last ``window`` positions are ever read, so pages behind it are
-    given back.  kind "state": one fixed-size tensor per request
-    (``state_shape``, float32), held in a slot."""
+    given back.  A token's entry is, per KV head, a key of ``head_dim`` and a
+    value of ``value_dim`` elements (default: as wide as the key; 0: no value,
+    one vector per token).  With equal widths a page is handed to the mixer as
+    [2, kv_heads, page_size * head_dim]; otherwise as a flat run of
+    kv_heads * page_size * (head_dim + value_dim) elements that the mixer lays
+    out itself.  kind "state": one fixed-size tensor per request
+    (``state_shape``), held in a slot.  ``dtype`` names the element type
+    ("float32", "bfloat16", "int32", ...); the default is the engine's compute
+    dtype for pages and float32 for state."""
     kind: str = "paged"
     kv_heads: int = 0
     head_dim: int = 0
     window: int = 0
     state_shape: Tuple[int, ...] = ()
+    value_dim: Optional[int] = None
+    dtype: Optional[str] = None
+
+    @property
+    def value_width(self) -> int:
+        return self.head_dim if self.value_dim is None else int(self.value_dim)
 
     def group_key(self):
         if self.kind == "paged":
-            return ("paged", self.kv_heads, self.head_dim, self.window)
-        return ("state",) + tuple(self.state_shape)
+            return ("paged", self.kv_heads, self.head_dim, self.window, self.value_width, self.dtype)
+        return ("state", self.dtype) + tuple(self.state_shape)
 
 
 class PartSpec:

@@ -202,6 +202,11 @@ def test_a_step_queued_ahead_takes_its_ids_from_the_device(model_dirs, dtype):
             handles.append(h)
         if ahead:
             out.append(before.tokens())
+            # a handle's logits are the recording's buffer: the last step's hold, an older step's
+            # were overwritten by a step of the same shape and are refused, not handed out
+            assert before.logits.argmax(-1).tolist() == out[-1]
+            with pytest.raises(RuntimeError, match="overwritten"):
+                handles[-2].logits
             lengths = [eng.cache.get(i).length for i in range(3)]
             with pytest.raises(ValueError, match="sampled last"):
                 eng.step_sample_ahead([StepEntry(i, [TokenRef(handles[0], i)], [0]) for i in range(3)],
@@ -319,11 +324,13 @@ def test_step_refuses_bad_input_and_leaves_the_cache_alone(model_dirs):
     eng.cache.check_invariants()
 
 
-def run_trace_program(model_dir, dtype, steps, max_tokens, out_dir):
+def run_trace_program(model_dir, dtype, steps, max_tokens, out_dir, as_module=False):
+    program = [sys.executable, "-m", "kllm_amd.replay"] if as_module else \
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run")]
+    env = dict(os.environ, PYTHONPATH=ROOT + os.pathsep + os.environ.get("PYTHONPATH", "")) if as_module else None
     proc = subprocess.Popen(
-        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
-         "--out", out_dir, "--max-tokens", str(max_tokens)],
-        stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, cwd="/")
+        program + ["--model", model_dir, "--dtype", dtype, "--out", out_dir, "--max-tokens", str(max_tokens)],
+        stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, cwd="/", env=env)
     outs = []
     for s in steps:
         proc.stdin.write(json.dumps(s) + "\n")
@@ -349,7 +356,8 @@ def test_the_trace_run_program(model_dirs, tmp_path, dtype, name):
     reqs = make_requests(cfg, [50, 21, 77, 30, 64, 12], 10)
     steps, peak = traces.mixed(reqs, seed=11)
     steps[3]["entries"][0]["want"] = []                       # a step may want nothing of a request
-    outs = run_trace_program(d, dtype, steps, peak, str(tmp_path / "out"))
+    # the program under both of its names: bin/trace_run and python -m kllm_amd.replay
+    outs = run_trace_program(d, dtype, steps, peak, str(tmp_path / "out"), as_module=dtype == "float32")
     assert outs[0].shape[1] == cfg["vocab_size"]
     rows = traces.collect(steps, outs)
     want = expected(d, cfg, reqs, dtype)

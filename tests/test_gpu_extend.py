@@ -716,3 +716,151 @@ def test_a_norm_with_a_bias_and_an_arrangement_with_the_norms_behind_the_additio
         unregister_architecture("ToyPostNormForCausalLM")
         unregister_part("block", "toy_post_norm")
         unregister_part("norm", "toy_centered")
+
+
+# ----------------------------------------------------------------------------- other cache shapes
+
+class ToyLatentMixer(Part):
+    """Caches one compressed vector per token, c_t = W_c x_t of ``width`` elements: a paged
+    cache with keys of ``width`` and no values (``value_dim=0``), so a page is a flat run that
+    this part lays out as [page_size, width].  out_t = W_o sum_j softmax_j(q_t . c_j) c_j over
+    j <= t with q_t = W_q x_t.  It also keeps the number of tokens it has seen of a request
+    in an int32 state slot and scales its output by 1 / (tokens seen so far)."""
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.hidden, self.width = self.param("hidden"), self.param("width")
+
+    def weight_specs(self):
+        return [WeightSpec(self.tensor_name("c.weight"), (self.width, self.hidden)),
+                WeightSpec(self.tensor_name("q.weight"), (self.width, self.hidden)),
+                WeightSpec(self.tensor_name("o.weight"), (self.hidden, self.width))]
+
+    def bind(self, weights):
+        self.w_c, self.w_q, self.w_o = (weights[self.tensor_name(n + ".weight")].float() for n in "cqo")
+
+    def cache_need(self):
+        return CacheNeed("paged", kv_heads=1, head_dim=self.width, value_dim=0, dtype="float32")
+
+    def forward(self, ctx, xn, cache):
+        ps = cache.page_size
+        assert cache.pages.dim() == 2 and cache.pages.shape[1] == ps * self.width and cache.pages.dtype == torch.float32
+        pages = cache.pages.view(-1, ps, self.width)
+        x = xn.float()
+        c, q = x @ self.w_c.t(), x @ self.w_q.t()
+        out = torch.empty(ctx.n, self.hidden, dtype=torch.float32, device=xn.device)
+        tables = cache.block_table.tolist()
+        for s in range(ctx.n_spans):
+            a, p0 = ctx.h_span_start[s], ctx.h_span_pos[s]
+            for i in range(ctx.h_span_len[s]):
+                p = p0 + i
+                pages[tables[s][p // ps], p % ps] = c[a + i]
+                keys = torch.stack([pages[tables[s][j // ps], j % ps] for j in range(p + 1)])
+                out[a + i] = self.w_o @ (torch.softmax(keys @ q[a + i], 0) @ keys)
+        return out
+
+
+class ToyCountMixer(Part):
+    """out_t = x_t / (tokens of the request seen so far, this one included); the count lives
+    in an int32 state slot."""
+
+    def cache_need(self):
+        return CacheNeed("state", state_shape=(1,), dtype="int32")
+
+    def forward(self, ctx, xn, cache):
+        assert cache.state.dtype == torch.int32
+        out = torch.empty(ctx.n, xn.shape[1], dtype=torch.float32, device=xn.device)
+        slots = cache.slots.tolist()
+        for s in range(ctx.n_spans):
+            a, b = ctx.h_span_start[s], ctx.h_span_start[s + 1]
+            if ctx.h_span_pos[s] == 0:
+                cache.state[slots[s]].zero_()
+            for t in range(a, b):
+                cache.state[slots[s]] += 1
+                assert int(cache.state[slots[s]]) == ctx.h_span_pos[s] + (t - a) + 1
+                out[t] = xn[t].float() / cache.state[slots[s]].float()
+        return out
+
+
+def build_latent(cfg: LlamaConfig) -> ModelSpec:
+    from kllm_amd.models.llama import build_llama
+    spec = build_llama(cfg)
+    spec.layers[0].mixer = PartSpec("toy_latent", "model.layers.0.mix", hidden=cfg.hidden_size, width=24)
+    spec.layers[1].mixer = PartSpec("toy_count", "model.layers.1.mix")
+    return spec
+
+
+def latent_reference(w, cfg, ids, dtype_round):
+    """The same model written plainly over a whole sequence on the CPU."""
+    eps = cfg["rms_norm_eps"]
+    r = (lambda t: t.to(torch.bfloat16).float()) if dtype_round else (lambda t: t)
+    T = len(ids)
+    x = P.embedding(ids, w["model.embed_tokens.weight"])
+    for i in range(cfg["num_hidden_layers"]):
+        pre = f"model.layers.{i}"
+        xn = r(P.rmsnorm(x, w[pre + ".input_layernorm.weight"], eps))
+        if i == 0:
+            c, q = xn @ w[pre + ".mix.c.weight"].t(), xn @ w[pre + ".mix.q.weight"].t()
+            mix = torch.stack([w[pre + ".mix.o.weight"] @ (torch.softmax(c[:t + 1] @ q[t], 0) @ c[:t + 1])
+                               for t in range(T)])
+        elif i == 1:
+            mix = xn / torch.arange(1, T + 1).float()[:, None]
+        else:
+            pos = torch.arange(T)
+            cc = P._cfg(cfg)
+            qq = P.rope(P.linear(xn, w[pre + ".self_attn.q_proj.weight"]), pos.tolist(), cc["H"], cc["hd"], cc["theta"])
+            kk = P.rope(P.linear(xn, w[pre + ".self_attn.k_proj.weight"]), pos.tolist(), cc["KV"], cc["hd"], cc["theta"])
+            vv = P.linear(xn, w[pre + ".self_attn.v_proj.weight"])
+            mix = P.linear(r(P.attention(r(qq), r(kk), r(vv), pos, cc["H"], cc["KV"], cc["hd"])),
+                           w[pre + ".self_attn.o_proj.weight"])
+        x = x + mix
+        xn = r(P.rmsnorm(x, w[pre + ".post_attention_layernorm.weight"], eps))
+        h = r(P.silu(P.linear(xn, w[pre + ".mlp.gate_proj.weight"])) * P.linear(xn, w[pre + ".mlp.up_proj.weight"]))
+        x = x + P.linear(h, w[pre + ".mlp.down_proj.weight"])
+    head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"]
+    return P.linear(r(P.rmsnorm(x, w["model.norm.weight"], eps)), head)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_cache_of_one_vector_per_token_and_an_integer_state(dtype):
+    """A mixer whose cache entry is one vector per token (keys of another width than the model's
+    heads, no values, float32 whatever the engine computes in) and a mixer with an int32
+    state are registered from here, get pools of their own beside attention's, and are
+    stepped in portions and mixed batches with pages used again."""
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry
+    register_part("mixer", "toy_latent", ToyLatentMixer)
+    register_part("mixer", "toy_count", ToyCountMixer)
+    register_architecture("ToyLatentForCausalLM", LlamaConfig, build_latent)
+    try:
+        cfg = dict(tiny.CONFIGS["B"], architectures=["ToyLatentForCausalLM"])
+        eng = Engine.from_random(cfg, 7, EngineOptions(dtype=dtype, num_pages=9, max_requests=3,
+                                                       poison_freed_pages=True), std=0.08, norm_std=0.2)
+        plan = eng.model.cache_plan
+        kinds = [(g.need.kind, g.need.head_dim, g.need.value_width, g.need.dtype) for g in plan.groups]
+        assert kinds == [("paged", 24, 0, "float32"), ("state", 0, 0, "int32"), ("paged", 32, 32, None)]
+        assert tuple(eng.kv[0].shape) == (1, 9, 16 * 24) and eng.kv[0].dtype == torch.float32
+        assert tuple(eng.kv[2].shape) == (1, 9, 2, 1, 16 * 32) and eng.state[1].dtype == torch.int32
+        assert "values of 0" in eng.capacity_report()
+        w = engine_weights_seed(eng, 7)
+        reqs = {"a": tiny.tokens(cfg, 45, 1), "b": tiny.tokens(cfg, 30, 2), "c": tiny.tokens(cfg, 22, 3),
+                "d": tiny.tokens(cfg, 37, 4)}
+        steps, peak = traces.mixed(reqs, seed=5, max_live=3, tail=5, max_portion=11)
+        outs = []
+        for s in steps:
+            out = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+            outs.append(out.cpu().numpy())
+            for rid in s["end"]:
+                eng.release(rid)
+        rows = traces.collect(steps, outs)
+        assert eng.cache.pools[0].total_allocs > 9                 # pages were used again
+        worst = 0.0
+        for rid, toks in reqs.items():
+            want = latent_reference(w, cfg, toks, dtype == "bfloat16")
+            for p in range(len(toks)):
+                worst = max(worst, float((torch.from_numpy(rows[(rid, p)]) - want[p]).abs().max()))
+        assert worst < (2e-4 if dtype == "float32" else 8e-2), worst
+        eng.cache.check_invariants()
+    finally:
+        unregister_architecture("ToyLatentForCausalLM")
+        unregister_part("mixer", "toy_latent")
+        unregister_part("mixer", "toy_count")

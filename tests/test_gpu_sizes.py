@@ -173,11 +173,15 @@ def test_a_whole_prompt_of_2048_tokens(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,B", [("tinyllama", 64), ("tinyllama", 24), ("tinyllama", 12), ("llama3-8b", 64),
-                                    ("llama3-8b", 12)])
+@pytest.mark.parametrize("name,B", [("tinyllama", 64), ("tinyllama", 33), ("tinyllama", 24), ("tinyllama", 12),
+                                    ("tinyllama", 8), ("tinyllama", 4), ("llama3-8b", 64), ("llama3-8b", 40),
+                                    ("llama3-8b", 17), ("llama3-8b", 12), ("llama3-8b", 8), ("llama3-8b", 3)])
 def test_decode_steps_of_many_requests_eager_and_as_graphs(name, B, dtype):
-    """64 requests decode together (and 24 and 12, which take other kernels for the
-    products: up to 16 and up to 32 rows): first through the plain step function, then queued ahead
+    """64 requests decode together (and fewer, which take other kernels for the products and for
+    attention and other hand-overs between them: up to 2, 4, 16, 32 and 64 rows, with the norm
+    folded into its neighbours or in a launch of its own, the gate in the tiled product's
+    epilogue or apart, a few more attention groups than the chip holds whole-context workgroups):
+    first through the plain step function, then queued ahead
     as HIP graphs.  Both give logits; the graphs' must equal the eager ones (the same kernels
     on the same numbers; only the width of the block table differs), for every request at
     every step, over two widths of the table, and a sample of requests is compared with the

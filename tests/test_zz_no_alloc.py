@@ -71,3 +71,12 @@ def test_a_size_beyond_the_array_is_refused_and_nothing_runs():
     assert call_static(fn, c, out, 2) == 0, last_error(lib)     # and with fewer slices it fits
     torch.cuda.synchronize()
     assert (out.cpu().double() - c["want"]).abs().max() < 2e-2
+
+
+def test_init_resolves_the_array_outside_any_recording():
+    """The address lookup has a call of its own for callers that record graphs: after it the
+    entry point does no lookup (a first call from inside a recording would be refused)."""
+    lib, fn = entry_point()
+    lib.kllm_attn_decode_static_init.restype = c_int
+    assert lib.kllm_attn_decode_static_init() == 0, last_error(lib)
+    assert lib.kllm_attn_decode_static_init() == 0

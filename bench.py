@@ -6,6 +6,10 @@ plus prefill of 2,048 tokens and decode at batch 1 and 64.
 
 Prints one JSON line.  A "step" is one decode step of the whole batch: the
 forward pass over the cache, sampling on the device, the tokens read back.
+``points`` of that line also holds, beside batch 1 and 64: the float32 path at the
+same sizes, the 2,048-token prompt in portions of 512, the decode run from 512 to
+2,048 tokens, Llama-3-8B sizes at batch 64 with contexts of 4,096, and the mixed
+serving workload at Llama-2-7B sizes (``--no-extra`` leaves those out).
 
 Other workloads, each printing one JSON line of its own (``--model`` chooses the sizes):
 
@@ -39,6 +43,7 @@ def main(argv=None):
     ap.add_argument("--context", type=int, default=2048, help="context length the timed steps end at")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    ap.add_argument("--no-extra", action="store_true", help="skip the points at other dtypes, sizes and workloads")
     ap.add_argument("--gemm", default="hip", choices=["hip", "library"])
     ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill only (for profiles)")
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page")
@@ -92,7 +97,7 @@ def main(argv=None):
         return 0
     ms, ctx = B.measure_decode(eng, args.batch, args.context, args.steps, args.warmup)
     value = args.batch * 1e3 / ms
-    need = B.decode_step_bytes(cfg, args.batch, int(ctx), elem)
+    need = eng.step_read_bytes([int(ctx)] * args.batch)      # asked of the model's parts and the cache plan
     achieved = need / (ms * 1e-3) / 1e9
     out = {
         "metric": "decode tok/s, %s sizes, random weights" % {"tinyllama-1.1b": "TinyLlama-1.1B", "llama2-7b": "Llama-2-7B",
@@ -117,10 +122,12 @@ def main(argv=None):
     cal = B.calibrate()     # the box's own copy bandwidth and MFMA rate, beside the published peaks
     out["roofline"]["measured_copy"] = cal["copy_GBs"]
     out["roofline"]["frac_of_measured_copy"] = round(achieved / cal["copy_GBs"], 4)
+    out["roofline"]["measured_read"] = cal["read_GBs"]      # a read-only stream: what a decode kernel does
+    out["roofline"]["frac_of_measured_read"] = round(achieved / cal["read_GBs"], 4)
     if not args.no_points:
         T = 2048
         pms = B.measure_prefill(eng, T)
-        flops = B.prefill_flops(cfg, T)
+        flops = eng.model.step_flops(T, T * (T + 1) / 2.0, 1)
         out["prefill"] = {"value": round(T * 1e3 / pms, 1), "tokens": T, "ms": round(pms, 3),
                           "frac": round(flops / (pms * 1e-3) / B.PEAK_FLOPS[args.dtype], 4),
                           "frac_of_measured_mfma": round(flops / (pms * 1e-3) / 1e12 / cal[f"mfma_{args.dtype}_TFLOPs"], 4)}
@@ -129,6 +136,13 @@ def main(argv=None):
             k = max(16, args.steps // 2)
             bms, _ = B.measure_decode(eng, b, args.context, k, 8)
             points[f"decode_b{b}"] = round(b * 1e3 / bms, 1)
+        if not args.no_extra and args.model == "tinyllama-1.1b" and not args.layers:
+            import gc
+            points.update(B.same_engine_points(eng))
+            del eng                               # the larger models need its memory
+            gc.collect()
+            torch.cuda.empty_cache()
+            points.update(B.other_engine_points(cfg, args.dtype, args.gemm, args.page_size))
         out["points"] = points
     print(json.dumps(out))
     return 0
@@ -145,14 +159,14 @@ def other_workload(args, cfg, full_layers, B):
                             max_model_len=args.context + 64, gemm=args.gemm, page_size=args.page_size)
         res = B.measure_decode_run(eng, args.batch, prompt_len=512, total_len=args.context)
         base.update(batch=args.batch, prompt_len=512, total_len=args.context, unit="tok/s", **res)
-        worst = B.decode_step_bytes(cfg, args.batch, args.context - 1, elem)
+        worst = eng.step_read_bytes([args.context - 1] * args.batch)
         base["frac_of_hbm_at_end"] = round(worst * res["at"][max(res["at"])] / args.batch / 1e9 / B.PEAK_HBM_GBS, 4)
     elif args.workload == "prefill-chunks":
         eng = B.make_engine(cfg, args.dtype, max_tokens=2 * 2048 + 4096, max_model_len=2048 + 64, gemm=args.gemm,
                             page_size=args.page_size)
         ms = B.measure_prefill_chunks(eng, 2048, args.chunk, reps=3, warmup=1)
         whole = B.measure_prefill(eng, 2048)
-        flops = B.prefill_flops(cfg, 2048)
+        flops = eng.model.step_flops(2048, 2048 * 2049 / 2.0, 1)
         base.update(tokens=2048, chunk=args.chunk, ms=round(ms, 3), tok_s=round(2048e3 / ms, 1),
                     frac=round(flops / (ms * 1e-3) / B.PEAK_FLOPS[args.dtype], 4),
                     whole_prompt_ms=round(whole, 3))
@@ -163,8 +177,8 @@ def other_workload(args, cfg, full_layers, B):
                             gemm=args.gemm, page_size=args.page_size, max_requests=max(64, args.requests))
         res = B.measure_mixed(eng, args.requests, 128, 2048, args.new_tokens, args.chunk)
         base.update(chunk=args.chunk, new_tokens=args.new_tokens, **res)
-        base["prefill_frac"] = round(res["prompt_tok_s"] * 2.0 * cfg["num_hidden_layers"] * B.layer_matrix_elements(cfg)
-                                     / B.PEAK_FLOPS[args.dtype], 4)
+        # the products alone (attention's share depends on the lengths drawn)
+        base["prefill_frac"] = round(res["prompt_tok_s"] * eng.model.step_flops(1, 0.0, 0) / B.PEAK_FLOPS[args.dtype], 4)
     print(json.dumps(base))
     return 0
 

@@ -53,41 +53,6 @@ def synthetic_ids(n: int, vocab: int, salt: int = 0) -> List[int]:
     return [((i + salt * 101) * 37 + 11) % vocab for i in range(n)]
 
 
-def sizes(cfg: dict) -> Dict[str, int]:
-    H, d = cfg["num_attention_heads"], cfg["hidden_size"]
-    hd = cfg.get("head_dim") or d // H
-    KV = cfg.get("num_key_value_heads") or H
-    return dict(L=cfg["num_hidden_layers"], d=d, H=H, KV=KV, hd=hd, qd=H * hd, kvd=KV * hd,
-                f=cfg["intermediate_size"], V=cfg["vocab_size"])
-
-
-def layer_matrix_elements(cfg: dict) -> int:
-    s = sizes(cfg)
-    return s["d"] * (s["qd"] + 2 * s["kvd"]) + s["qd"] * s["d"] + 3 * s["d"] * s["f"]
-
-
-def decode_step_bytes(cfg: dict, batch: int, context: int, elem: int) -> int:
-    """Bytes a decode step has to read: every weight it uses once (layer
-    matrices, output matrix, norm vectors in 32-bit, one embedding row per
-    request) and the keys and values of the live requests."""
-    s = sizes(cfg)
-    weights = (s["L"] * layer_matrix_elements(cfg) + s["V"] * s["d"] + batch * s["d"]) * elem
-    vectors = (2 * s["L"] + 1) * s["d"] * 4
-    cache = batch * context * s["L"] * 2 * s["kvd"] * elem
-    return weights + vectors + cache
-
-
-def prefill_flops(cfg: dict, tokens: int, logit_rows: int = 1) -> float:
-    """Multiply-adds times two of one whole prompt: the layer matrices for
-    every token, causal attention (scores and values), the output matrix for
-    the wanted rows."""
-    s = sizes(cfg)
-    gemm = 2.0 * tokens * s["L"] * layer_matrix_elements(cfg)
-    attn = 4.0 * s["L"] * s["H"] * s["hd"] * tokens * (tokens + 1) / 2.0
-    head = 2.0 * logit_rows * s["d"] * s["V"]
-    return gemm + attn + head
-
-
 def _sync():
     torch.cuda.synchronize()
 
@@ -264,6 +229,81 @@ def measure_mixed(engine: Engine, requests: int = 32, min_prompt: int = 128, max
             "preemptions": sched.stats["preemptions"]}
 
 
+def _attempt(pts, name, fn):
+    try:
+        fn()
+    except Exception as e:                      # the headline figures stand without this point
+        pts[name + "_error"] = f"{type(e).__name__}: {e}"[:200]
+
+
+def same_engine_points(engine: Engine) -> Dict[str, float]:
+    """Further workloads on the headline engine, as flat name -> number entries for the
+    headline line's ``points`` (the reference's bench puts everything it measures into its one
+    JSON object: cmd/bench/main.go:37-46): the 2,048-token prompt in portions of 512 and the
+    decode run from 512 to 2,048 tokens at batch 8.  A point that fails leaves
+    ``<name>_error``."""
+    pts: Dict[str, float] = {}
+
+    def run():
+        ms = measure_prefill_chunks(engine, 2048, 512, reps=3, warmup=1)
+        pts["prefill_chunks_512_ms"] = round(ms, 3)
+        res = measure_decode_run(engine, 8, prompt_len=512, total_len=2048)
+        pts["decode_run_b8_mean"] = res["mean_tok_s"]
+        for T, v in res["at"].items():
+            pts[f"decode_run_b8_T{T}"] = v
+    _attempt(pts, "same_engine", run)
+    return pts
+
+
+def other_engine_points(cfg_small: dict, dtype: str, gemm: str = "hip", page_size: int = 16) -> Dict[str, float]:
+    """The other configurations that the baseline names, each on an engine of its own (the
+    caller has released the headline engine: the larger models need its memory): the float32
+    path at the headline sizes ``cfg_small``, Llama-3-8B sizes at batch 64 with contexts of
+    4,096, and the mixed serving workload at Llama-2-7B sizes through the scheduler."""
+    import gc
+    pts: Dict[str, float] = {}
+
+    def attempt(name, fn):
+        _attempt(pts, name, fn)
+
+    def other(cfg, dt, max_tokens, max_requests, max_len, fn):
+        eng = make_engine(cfg, dt, max_tokens=max_tokens, max_requests=max_requests, max_model_len=max_len,
+                          gemm=gemm, page_size=page_size)
+        try:
+            fn(eng)
+        finally:
+            del eng
+            gc.collect()
+            torch.cuda.empty_cache()
+
+    def fp32(eng):
+        ms, ctx = measure_decode(eng, 8, 2048, 32, 8)
+        pts["fp32_decode_b8"] = round(8e3 / ms, 1)
+        pts["fp32_decode_b8_hbm_frac"] = round(eng.step_read_bytes([int(ctx)] * 8) / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)
+        pms = measure_prefill(eng, 2048)
+        pts["fp32_prefill_ms"] = round(pms, 3)
+        pts["fp32_prefill_frac"] = round(eng.model.step_flops(2048, 2048 * 2049 / 2.0, 1) / (pms * 1e-3)
+                                         / PEAK_FLOPS["float32"], 4)
+    if dtype != "float32":
+        attempt("fp32", lambda: other(cfg_small, "float32", 8 * 2048 + 4096, 8, 2048 + 64, fp32))
+
+    def llama3(eng):
+        ms, ctx = measure_decode(eng, 64, 4096, 16, 4)
+        pts["llama3_8b_b64_ctx4096_ms"] = round(ms, 3)
+        pts["llama3_8b_b64_ctx4096_tok_s"] = round(64e3 / ms, 1)
+        pts["llama3_8b_b64_ctx4096_hbm_frac"] = round(eng.step_read_bytes([int(ctx)] * 64) / (ms * 1e-3) / 1e9
+                                                      / PEAK_HBM_GBS, 4)
+    attempt("llama3_8b_b64_ctx4096", lambda: other(LLAMA3_8B, dtype, 64 * 4096 + 4096, 64, 4096 + 64, llama3))
+
+    def llama2(eng):
+        res = measure_mixed(eng, 32, 128, 2048, 64, 512)
+        pts["llama2_7b_mixed_wall_s"] = res["wall_s"]
+        pts["llama2_7b_mixed_prompt_tok_s"] = res["prompt_tok_s"]
+        pts["llama2_7b_mixed_generated_tok_s"] = res["generated_tok_s"]
+    attempt("llama2_7b_mixed", lambda: other(LLAMA2_7B, dtype, 32 * (2048 + 64 + page_size), 64, 2048 + 128, llama2))
+    return pts
+
+
 def make_engine(cfg: dict, dtype: str, max_tokens: int, seed: int = 0, **opts) -> Engine:
     options = EngineOptions(dtype=dtype, max_tokens=max_tokens, max_requests=max(64, opts.pop("max_requests", 64)),
                             **opts)
@@ -277,7 +317,8 @@ _calibration = {}
 
 def calibrate(device=None) -> Dict[str, float]:
     """What this box reaches with nothing in the way: GB/s (read + written) of a plain
-    copy kernel over 1 GiB, and TFLOP/s of a loop of independent MFMAs in registers, for
+    copy kernel over 1 GiB, GB/s of a read-only stream over the same (what a decode step's
+    kernels do), and TFLOP/s of a loop of independent MFMAs in registers, for
     bfloat16 and float32 operands.  Figures are quoted against the published peaks and
     against these."""
     if _calibration:
@@ -290,6 +331,10 @@ def calibrate(device=None) -> Dict[str, float]:
     K.calibrate_copy(dst, src)
     best = min(_event_ms(lambda: K.calibrate_copy(dst, src)) for _ in range(5))
     _calibration["copy_GBs"] = round(2 * n * 4 / (best * 1e-3) / 1e9, 1)
+    rsink = torch.zeros(K.calibrate_read_workgroups(), dtype=torch.float32, device=dev)
+    K.calibrate_read(src, rsink)
+    best = min(_event_ms(lambda: K.calibrate_read(src, rsink)) for _ in range(5))
+    _calibration["read_GBs"] = round(n * 4 / (best * 1e-3) / 1e9, 1)
     del src, dst
     sink = torch.zeros(64, dtype=torch.float32, device=dev)
     for name, code in (("bfloat16", K.DT_BF16), ("float32", K.DT_F32)):

@@ -43,6 +43,10 @@ int kllm_device_xcds(void);
  * MFMAs per wave on every CU (bfloat16 32x32x16 or float32 32x32x2); *flops receives the
  * floating-point operations of the launch.  The caller times them. */
 int kllm_calibrate_copy(void* dst, const void* src, long bytes, hipStream_t stream);
+/* A read-only stream over `bytes`: sink receives one float per workgroup
+ * (kllm_calibrate_read_workgroups() of them). */
+int kllm_calibrate_read(const void* src, long bytes, float* sink, hipStream_t stream);
+int kllm_calibrate_read_workgroups(void);
 int kllm_calibrate_mfma(int dtype, int iters, float* sink, double* flops, hipStream_t stream);
 
 /* out[t] = table[ids[t]]; with `from` (and `sampled`), token t whose from[t] >= 0 takes its id

@@ -51,6 +51,26 @@ __global__ __launch_bounds__(256) void calibrate_copy_kernel(floatx4* __restrict
     dst[i] = src[i];
 }
 
+// A read-only stream: every lane keeps eight 16-byte loads in flight and adds what it read; one
+// float per workgroup goes out, so that the loads cannot be dropped.
+__global__ __launch_bounds__(256) void calibrate_read_kernel(const floatx4* __restrict__ src, long n16,
+                                                             float* __restrict__ sink) {
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  const long stride = (long)gridDim.x * blockDim.x;
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i + 7 * stride < n16; i += 8 * stride) {
+    floatx4 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = src[i + j * stride];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc += v[j];
+  }
+  for (; i < n16; i += stride) acc += src[i];
+  __shared__ float red[16];
+  const float total = block_sum(acc[0] + acc[1] + acc[2] + acc[3], red);
+  if (threadIdx.x == 0) sink[blockIdx.x] = total;
+}
+
 // Four independent accumulator tiles per wave, `iters` rounds of one MFMA each; the result is
 // written so that the loop cannot be dropped.
 template <bool F32>
@@ -91,6 +111,17 @@ extern "C" int kllm_calibrate_copy(void* dst, const void* src, long bytes, hipSt
   hipLaunchKernelGGL(kllm::calibrate_copy_kernel, dim3(grid), dim3(256), 0, stream, (kllm::floatx4*)dst,
                      (const kllm::floatx4*)src, bytes / 16);
   KLLM_CHECK_LAUNCH("calibrate_copy");
+  return 0;
+}
+
+extern "C" int kllm_calibrate_read_workgroups(void) { return kllm::device_cus() * 16; }
+
+extern "C" int kllm_calibrate_read(const void* src, long bytes, float* sink, hipStream_t stream) {
+  KLLM_REQUIRE(src && sink && bytes > 0 && bytes % 16 == 0 && ((uintptr_t)src & 15) == 0,
+               "calibrate_read: %ld bytes must be a multiple of 16 and the buffer 16-byte aligned", bytes);
+  hipLaunchKernelGGL(kllm::calibrate_read_kernel, dim3(kllm_calibrate_read_workgroups()), dim3(256), 0, stream,
+                     (const kllm::floatx4*)src, bytes / 16, sink);
+  KLLM_CHECK_LAUNCH("calibrate_read");
   return 0;
 }
 

@@ -244,6 +244,24 @@ class Engine:
             head += f" of a budget of {self.options.memory_bytes / 2**20:.1f} MiB"
         return "\n".join([head] + ["  " + line for line in self._capacity])
 
+    def cache_read_bytes(self, contexts: Sequence[int]) -> int:
+        """Bytes of cache that a decode step of requests holding ``contexts`` tokens has to
+        read: per paged group and run, each request's keys and values (its window of them)."""
+        total = 0
+        for g, gp in enumerate(self.model.cache_plan.groups):
+            if gp.need.kind != "paged":
+                continue
+            per_token = gp.need.kv_heads * (gp.need.head_dim + gp.need.value_width) * self.kv[g].element_size()
+            readers = sum(1 for r in self.model.cache_plan.runs if r is not None and r[0] == g)
+            for c in contexts:
+                total += readers * per_token * (min(c, gp.need.window) if gp.need.window else c)
+        return total
+
+    def step_read_bytes(self, contexts: Sequence[int]) -> int:
+        """What a decode step of these requests must read at least: every weight it uses once
+        and the cache of the live requests."""
+        return self.model.step_read_bytes(len(contexts)) + self.cache_read_bytes(contexts)
+
     def cache_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in list(self.kv.values()) + list(self.state.values()))
 

@@ -140,6 +140,24 @@ class Model:
             visit(p)
         return sum(seen.values())
 
+    def step_read_bytes(self, tokens: int) -> int:
+        """Bytes of weights that a step of ``tokens`` tokens has to read: every tensor the
+        scheduled parts use, once (a tensor that two parts share counts once, at the larger
+        of what they read), as the parts themselves say."""
+        seen: Dict[int, int] = {}
+        used = [self.embedding, self.final_norm, self.head] + [self.blocks[r.layer] for r in self.schedule]
+        used += [p for _, p in self.runtime.shared.values()]
+        for part in used:
+            for ptr, nbytes in part.read_bytes(tokens).items():
+                seen[ptr] = max(seen.get(ptr, 0), nbytes)
+        return sum(seen.values())
+
+    def step_flops(self, tokens: int, keys_read: float, logit_rows: int = 1) -> float:
+        """Floating-point operations of a step of ``tokens`` tokens that read ``keys_read``
+        cached positions all together in every run, with logits at ``logit_rows`` rows."""
+        return (sum(self.blocks[r.layer].flops(tokens, keys_read) for r in self.schedule)
+                + self.head.flops(logit_rows))
+
     # ------------------------------------------------------------------ one step
     def run(self, ctx, cache_views) -> Optional[torch.Tensor]:
         """Run the step's tokens through every scheduled layer.  Returns

@@ -116,6 +116,8 @@ def _declare(lib):
         "kllm_gemv_normed_max_parts": [],
         "kllm_attn_f32_fits": [I, I],
         "kllm_calibrate_copy": [P, P, L, P],
+        "kllm_calibrate_read": [P, L, P, P],
+        "kllm_calibrate_read_workgroups": [],
         "kllm_calibrate_mfma": [I, I, P, P, P],
         "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, P],
         "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, L, I, I, P],
@@ -188,6 +190,19 @@ def calibrate_copy(dst, src):
         raise KernelError("calibrate_copy: sizes differ")
     _check(library().kllm_calibrate_copy(_ptr(dst, "copy dst"), _ptr(src, "copy src"),
                                          src.numel() * src.element_size(), _stream()), "calibrate_copy")
+
+
+def calibrate_read(src, sink):
+    """Read all of src with a plain streaming kernel (for measuring the box's read bandwidth);
+    sink: float32, one element per workgroup (calibrate_read_workgroups())."""
+    if sink.numel() < calibrate_read_workgroups():
+        raise KernelError("calibrate_read: the sink is too short")
+    _check(library().kllm_calibrate_read(_ptr(src, "read src"), src.numel() * src.element_size(),
+                                         _ptr(sink, "read sink", torch.float32), _stream()), "calibrate_read")
+
+
+def calibrate_read_workgroups() -> int:
+    return int(library().kllm_calibrate_read_workgroups())
 
 
 def calibrate_mfma(dtype_code_, iters, sink) -> float:

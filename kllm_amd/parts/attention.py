@@ -94,6 +94,10 @@ class CausalSelfAttention(Part):
     def cache_need(self):
         return CacheNeed("paged", kv_heads=self.kv_heads, head_dim=self.head_dim, window=self.window)
 
+    def flops(self, tokens, keys_read=0.0):
+        # the projections, and per key read a score and a value product for every head
+        return super().flops(tokens) + 4.0 * self.heads * self.head_dim * keys_read
+
     def check_cache(self, page_size):
         # The kernel that takes every size walks a chunk of up to 256 keys at a time, whole
         # pages of them; the faster kernels are chosen per step where the sizes fit them.

@@ -300,6 +300,22 @@ class Part:
         """Parts this part is made of (an arrangement's norms, mixer, feed-forward)."""
         return []
 
+    # ---- what a step costs at least (for rooflines; measurement code asks the model, which asks its parts)
+    def tensors(self) -> List[torch.Tensor]:
+        """The tensors this part itself holds after ``bind`` (its children's excluded)."""
+        return [v for v in vars(self).values() if isinstance(v, torch.Tensor)]
+
+    def read_bytes(self, tokens: int) -> Dict[int, int]:
+        """address -> bytes of its tensors that a step of ``tokens`` tokens has to read: all of
+        each by default (a table that is only gathered from overrides this)."""
+        return {t.data_ptr(): t.numel() * t.element_size() for t in self.tensors()}
+
+    def flops(self, tokens: int, keys_read: float = 0.0) -> float:
+        """Floating-point operations of ``tokens`` tokens through this part, the tokens reading
+        ``keys_read`` cached positions all together (a mixer adds its scores and values): two
+        per element of every matrix it holds and token, by default."""
+        return 2.0 * tokens * sum(t.numel() for t in self.tensors() if t.dim() == 2)
+
     def step_lists(self, starts: List[int], lens: List[int]) -> Dict[str, List[int]]:
         """name -> list of ints for a step whose span s covers rows
         ``starts[s] .. starts[s] + lens[s]``; only called when ``step_lists_key`` is set."""

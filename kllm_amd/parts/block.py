@@ -45,6 +45,15 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def read_bytes(self, tokens):
+        out = {}
+        for p in self.parts():
+            out.update(p.read_bytes(tokens))
+        return out
+
+    def flops(self, tokens, keys_read=0.0):
+        return sum(p.flops(tokens, keys_read) for p in self.parts())
+
     takes_next_norm = True
 
     def first_norm(self):

@@ -33,6 +33,12 @@ class TokenEmbedding(Part):
     def bind(self, weights):
         self.table = weights[self.tensor_name("weight")]
 
+    def read_bytes(self, tokens):
+        return {self.table.data_ptr(): tokens * self.hidden * self.table.element_size()}   # one row per token
+
+    def flops(self, tokens, keys_read=0.0):
+        return 0.0
+
     def forward(self, ctx, token_ids):
         x = ctx.buf("x", (ctx.n, self.hidden), torch.float32)
         if ctx.sampled is not None and ctx.token_from is not None:

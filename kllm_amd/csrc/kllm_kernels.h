@@ -12,6 +12,7 @@
  */
 #pragma once
 #include <hip/hip_runtime.h>
+#include <stdint.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -247,6 +248,19 @@ int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* qu
 /* out[r] = sampled index of logits[r][:]; temperature/uniform null: greedy. */
 int kllm_sample(int* out, const float* logits, const float* temperature, const float* uniform,
                 int rows, int vocab, hipStream_t stream);
+
+/* A step's launches in one call.  `words` is a buffer of n_words 64-bit words holding commands
+ * (executor.hpp describes the layout: entry point, argument words, structs that arguments
+ * point to); they run in order on `stream`, whatever stream argument was recorded.
+ * kllm_command_op gives the number that names an entry point of this header in a command
+ * (-1: it cannot be recorded), kllm_command_nargs its number of arguments.  Returns 0, or the
+ * code of the first command that failed with *failed = its index (-3: the buffer itself is
+ * malformed); commands before it have run, none after it.  The role of the reference's
+ * te_forward_batch (backend/shim.h:106-117): one call across the language boundary for the
+ * whole forward pass. */
+int kllm_command_op(const char* name);
+int kllm_command_nargs(int op);
+int kllm_run_commands(const uint64_t* words, long n_words, int* failed, hipStream_t stream);
 
 #ifdef __cplusplus
 }

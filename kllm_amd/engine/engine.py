@@ -12,6 +12,7 @@ passed every step (backend/shim.h:106-113).
 
 from __future__ import annotations
 
+from collections import OrderedDict
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence
 
@@ -25,7 +26,7 @@ from ..config import ModelConfig, config_from_dict, load_config, resolve_archite
 from ..parts.base import PagedCacheView, Runtime, StateCacheView, StepContext
 from ..weights import load_weights, random_weights
 from . import control
-from .graph import DecodeGraphs, SampledTokens, TokenRef
+from .graph import DecodeGraphs, SampledTokens, TokenRef, _bucket as table_bucket
 from .model import Model
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16,
@@ -80,7 +81,19 @@ class StepEntry:
     want: Sequence[int] = ()
 
 
+@dataclass
+class _StepPlan:
+    """A step's recorded launches, the logits they leave, and what must still hold for the
+    addresses in them: the scratch buffers and the control buffer not replaced since."""
+    commands: object
+    logits: Optional[torch.Tensor]
+    generation: int
+    control: int
+
+
 class Engine:
+    MAX_STEP_PLANS = 256
+
     def __init__(self, config: ModelConfig, raw_config: dict, weights_from, options: EngineOptions):
         if not torch.cuda.is_available():
             raise RuntimeError("kllm_amd runs on a GPU only; torch sees none")
@@ -111,6 +124,17 @@ class Engine:
         self._control = None
         self.steps_run = 0
         self.tokens_run = 0
+        # A step's launches go to the library as one buffer of commands, not one by one
+        # (EngineOptions.extra["launch_one_by_one"] keeps the old way, for comparison).
+        self.records_launches = not options.extra.get("launch_one_by_one")
+        # ... and a step whose shape (tokens per request, wanted rows, table widths) has been seen
+        # runs again from the commands recorded then, without going through the parts: what a
+        # part launches may depend on the shape alone and on the values it names
+        # (Part.step_values), which is also what recording a decode step as a HIP graph asks.
+        self._repeat_steps = (self.records_launches and self.model.repeatable
+                              and not options.extra.get("no_repeated_steps"))
+        self._plans: "OrderedDict[tuple, _StepPlan]" = OrderedDict()
+        self.steps_repeated = 0
         self._graphs = DecodeGraphs(self)
         # What a scheduler should know of the kernels: a step's tokens are the rows of every
         # product, and those work on tiles of this many rows.
@@ -414,7 +438,8 @@ class Engine:
         opened, reserved = self._reserve(entries)
         try:
             rcs, lens, rows, tables = self._describe(entries)
-            pages = tuple(max(1, max(len(t) for t in tg)) for tg in tables)
+            # table widths in powers of two, as recorded steps have them: few distinct layouts
+            pages = tuple(table_bucket(max(len(t) for t in tg)) for tg in tables)
             span_starts = [0]
             for l in lens:
                 span_starts.append(span_starts[-1] + l)
@@ -428,10 +453,29 @@ class Engine:
             if self._control is None or self._control.numel() < total:
                 self._control = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
             self._send(host, self._control, total)
-            ctx = control.context(self._control, layout, self.runtime, starts, pos0, lens)
-            ctx.taps = taps
-            with self.kernels.stream_scope():
-                logits = self.model.run(ctx, self._cache_views(ctx))
+            values = self.model.step_values(span_starts, lens, pos0)
+            key = (layout, tuple(lens)) if self._repeat_steps and taps is None else None
+            plan = self._plans.get(key) if key is not None else None
+            workspace = self.runtime.workspace
+            if plan is not None and plan.generation == workspace.generation and plan.control == self._control.data_ptr():
+                # a step of this shape ran before: its launches again, in one call, with this
+                # step's values in place of that step's
+                self._plans.move_to_end(key)
+                plan.commands.run(values, torch.cuda.current_stream().cuda_stream)
+                logits = plan.logits
+                self.steps_repeated += 1
+            else:
+                ctx = control.context(self._control, layout, self.runtime, starts, pos0, lens)
+                ctx.taps = taps
+                ctx.values = {k: self.kernels.StepValue(v, k) for k, v in values.items()}
+                generation = workspace.generation
+                with self.kernels.stream_scope(record=self.records_launches, keep=key is not None) as scope:
+                    logits = self.model.run(ctx, self._cache_views(ctx))
+                commands = scope.plan() if key is not None and generation == workspace.generation else None
+                if commands is not None:          # (a step that grew its scratch buffers is kept the next time)
+                    self._plans[key] = _StepPlan(commands, logits, workspace.generation, self._control.data_ptr())
+                    while len(self._plans) > self.MAX_STEP_PLANS:
+                        self._plans.popitem(last=False)
         except Exception:
             self._undo(opened, reserved)
             raise

@@ -120,7 +120,7 @@ class DecodeGraphs:
         ctx = control.context(rec.control, rec.layout, eng.runtime, starts, pos0, lens)
         ctx.workspace = rec.workspace
         ctx.sampled = self.sampled
-        with K.stream_scope():                   # the capture's stream while recording
+        with K.stream_scope(record=eng.records_launches):   # the capture's stream while recording a graph
             logits = eng.model.run(ctx, eng._cache_views(ctx))
             rec.logits = logits
             temps, uniforms = control.sampling_views(rec.control, rec.layout)

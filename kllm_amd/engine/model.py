@@ -14,7 +14,8 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from ..parts.base import Runtime, make_part
+from .. import kernels as K
+from ..parts.base import Runtime, call_part, make_part
 from ..parts.spec import CacheNeed, ModelSpec, PartSpec, WeightSpec
 
 
@@ -45,6 +46,7 @@ class Model:
         self.schedule = list(spec.schedule)
         self.cache_plan = self._plan_cache()
         self._list_providers = None
+        self._value_providers = None
 
     # ------------------------------------------------------------------ cache plan
     def _plan_cache(self) -> CachePlan:
@@ -120,6 +122,29 @@ class Model:
                 out[f"{key}.{name}"] = values
         return out
 
+    def step_values(self, starts, lens, positions) -> Dict[str, int]:
+        """The host-side numbers that the model's parts want of a step's positions:
+        "<key>.<name>" -> int."""
+        if self._value_providers is None:
+            seen = {}
+            for p in self.all_parts():
+                key = getattr(p, "step_values_key", None)
+                if key is not None and key not in seen:
+                    seen[key] = p
+            self._value_providers = seen
+        out = {}
+        for key, part in self._value_providers.items():
+            for name, value in part.step_values(list(starts), list(lens), list(positions)).items():
+                out[f"{key}.{name}"] = int(value)
+        return out
+
+    @property
+    def repeatable(self) -> bool:
+        """Whether a step of this model can be run again from its recorded commands: every part
+        records its launches, and what it launches depends on the step's shape alone (and on
+        values it names through ``step_values``)."""
+        return self.graph_safe and all(getattr(p, "records_launches", False) for p in self.all_parts())
+
     @property
     def graph_safe(self) -> bool:
         """Whether a step of this model can be recorded in a HIP graph."""
@@ -166,12 +191,13 @@ class Model:
         shared = [p for _, p in self.runtime.shared.values()]
         for p in shared:
             if hasattr(p, "prepare"):
-                p.prepare(ctx)
-        x = self.embedding.forward(ctx, ctx.token_ids)
+                call_part(p, p.prepare, ctx)
+        x = call_part(self.embedding, self.embedding.forward, ctx, ctx.token_ids)
         for p in shared:
             if hasattr(p, "on_embedding"):
-                p.on_embedding(ctx, x)
+                call_part(p, p.on_embedding, ctx, x)
         if ctx.taps is not None:
+            K.flush_recorded()                    # the copies below are torch's: behind what was recorded
             ctx.taps.append(x.clone())
         pending = None
         for i, run in enumerate(self.schedule):
@@ -180,21 +206,25 @@ class Model:
                 # the norm that will take this layer's output, if the next layer names one
                 nxt = self.blocks[self.schedule[i + 1].layer]
                 first = nxt.first_norm() if hasattr(nxt, "first_norm") else None
-                x, pending = block.forward(ctx, x, pending, cache_views[i], next_norm=first)
+                x, pending = call_part(block, block.forward, ctx, x, pending, cache_views[i], next_norm=first)
             else:
-                x, pending = block.forward(ctx, x, pending, cache_views[i])
+                x, pending = call_part(block, block.forward, ctx, x, pending, cache_views[i])
             if ctx.taps is not None:
                 if pending is not None:
-                    self.final_norm.add(ctx, x, pending)
+                    call_part(self.final_norm, self.final_norm.add, ctx, x, pending)
                     pending = None
+                K.flush_recorded()
                 ctx.taps.append(x.clone())
         if ctx.taps is not None:
-            ctx.taps.append(self.final_norm.forward(ctx, x, delta=pending, tag="xn_tap").clone())
+            tap = call_part(self.final_norm, self.final_norm.forward, ctx, x, delta=pending, tag="xn_tap")
+            K.flush_recorded()
+            ctx.taps.append(tap.clone())
             pending = None
         if ctx.logit_rows is None or ctx.logit_rows.numel() == 0:
             return None
-        xn = self.final_norm.forward(ctx, x, delta=pending, rows=ctx.logit_rows, tag="xn_rows")
-        return self.head.forward(ctx, xn)
+        xn = call_part(self.final_norm, self.final_norm.forward, ctx, x, delta=pending, rows=ctx.logit_rows,
+                       tag="xn_rows")
+        return call_part(self.head, self.head.forward, ctx, xn)
 
 
 def collect_weight_specs(spec: ModelSpec) -> List[WeightSpec]:

@@ -11,6 +11,7 @@ graph capture.
 from __future__ import annotations
 
 import ctypes
+import struct
 import threading
 from ctypes import c_char_p, c_double, c_float, c_int, c_long, c_void_p
 
@@ -104,6 +105,9 @@ def _declare(lib):
         "kllm_gemv_resid_parts": [I],
         "kllm_fused_linear": [P, I, P, P, I, I, I, I, P],
         "kllm_fused_linear_resid_parts": [I, I],
+        "kllm_command_op": [c_char_p],
+        "kllm_command_nargs": [I],
+        "kllm_run_commands": [P, L, P, P],
         "kllm_fused_linear_max_parts": [],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
@@ -130,6 +134,17 @@ def _declare(lib):
     lib.kllm_fused_linear_lds_bytes.restype = L
 
 
+# Entry points that launch work on a stream (and can be recorded into a command buffer), and
+# which of their arguments are pointers to structures that travel with the command.
+LAUNCHING = ("kllm_embed", "kllm_add_rmsnorm", "kllm_rope_tables", "kllm_rope_append", "kllm_silu_mul",
+             "kllm_sum_splits", "kllm_gemm", "kllm_gemm_swiglu", "kllm_gemv_plain", "kllm_gemv_swiglu",
+             "kllm_gemv_resid", "kllm_gemv_rope_append", "kllm_fused_linear", "kllm_attn_generic",
+             "kllm_attn_decode", "kllm_attn_prefill", "kllm_sample")
+DYNAMIC_ARGS = {"kllm_attn_prefill": (15, 16)}     # arguments that may be a StepValue
+STRUCT_ARGS = {"kllm_gemv_plain": (7,), "kllm_gemv_swiglu": (8,), "kllm_gemv_rope_append": (17,),
+               "kllm_fused_linear": (2,)}
+
+
 def _check(rc: int, what: str):
     if rc == 0:
         return
@@ -150,22 +165,251 @@ class stream_scope:
     """Within the scope every launch of this thread goes to the stream that was
     current when the scope was entered, looked up once instead of once per
     launch (a step is a few hundred launches, and the lookup costs as much as
-    a launch).  The caller must not switch streams inside the scope."""
+    a launch).  The caller must not switch streams inside the scope.
+
+    With ``record`` the launches are not made one by one: each wrapper writes its entry
+    point and arguments into a command buffer, and the library runs the buffer in one call
+    (``kllm_run_commands``) when it holds ``chunk`` commands, when ``flush_recorded`` is
+    called, and when the scope ends.  Work that reaches the stream by another way (torch
+    operations, a part that launches for itself) must come after ``flush_recorded()``, and
+    code that is not written for recording runs inside ``direct_launches()``."""
+
+    def __init__(self, record: bool = False, chunk: int = 32, keep: bool = False):
+        self._record, self._chunk, self._keep = record, chunk, keep
+        self.recorder = None
 
     def __enter__(self):
-        self._outer = getattr(_scoped, "stream", None)
+        self._outer = (getattr(_scoped, "stream", None), getattr(_scoped, "recorder", None))
         _scoped.stream = torch.cuda.current_stream().cuda_stream
+        self.recorder = _scoped.recorder = _Recorder(_scoped.stream, self._chunk, self._keep) if self._record else None
+        return self
+
+    def __exit__(self, exc_type, *exc):
+        rec = _scoped.recorder
+        _scoped.stream, _scoped.recorder = self._outer
+        if rec is not None and exc_type is None:
+            rec.flush()                      # after an error what was recorded is dropped
+        return False
+
+    def plan(self):
+        """After the scope (opened with ``keep``): everything it ran, as a ``CommandPlan`` that
+        runs the same launches again, or None if something in the scope was launched past the
+        recording (such a step cannot be repeated from its commands alone)."""
+        rec = self.recorder
+        if rec is None or not rec.keep or rec.bypassed or not rec.kept:
+            return None
+        return CommandPlan(b"".join(rec.kept), rec.patches, rec.launched)
+
+
+class StepValue(int):
+    """A number that a part worked out on the host from a step's positions (how many keys its
+    queries read, say) and hands to a kernel wrapper: it carries its name, so that a recorded
+    step can be run again with this step's value in its place."""
+
+    def __new__(cls, value, name):
+        self = super().__new__(cls, value)
+        self.name = name
+        return self
+
+
+class CommandPlan:
+    """The launches of a step as they were recorded, ready to run again with one call of the
+    library: the commands' bytes, and where the step's own values (``StepValue``) go in them."""
+
+    def __init__(self, data: bytes, patches, count: int):
+        self.size = len(data)
+        self.buf = bytearray(data)
+        self.cbuf = (ctypes.c_char * self.size).from_buffer(self.buf)
+        self.patches = list(patches)         # (byte offset, name)
+        self.count = count
+
+    def run(self, values, stream=None):
+        for off, name in self.patches:
+            _PATCH.pack_into(self.buf, off, int(values[name]))
+        failed = c_int(-1)
+        rc = library().kllm_run_commands(self.cbuf, self.size // 8, ctypes.byref(failed),
+                                         _stream() if stream is None else stream)
+        if rc:
+            buf = ctypes.create_string_buffer(512)
+            library().kllm_last_error(buf, 512)
+            raise KernelError(f"recorded step: {buf.value.decode(errors='replace')} (code {rc}; command "
+                              f"{failed.value} of {self.count}, the ones before it have run)")
+
+
+_PATCH = struct.Struct("<q")
+
+
+class _Op:
+    __slots__ = ("name", "index", "nargs", "pack", "size", "structs", "dynamic", "fn")
+
+
+_op_table = None
+
+
+def _ops():
+    """name -> how to record a call of that entry point; built once from the signatures."""
+    global _op_table
+    if _op_table is None:
+        lib = library()
+        table = {}
+        for name in LAUNCHING:
+            fn = getattr(lib, name)
+            op = _Op()
+            op.name, op.fn = name, fn
+            op.index = lib.kllm_command_op(name.encode())
+            if op.index < 0 or lib.kllm_command_nargs(op.index) != len(fn.argtypes):
+                raise KernelError(f"{name} cannot be recorded: the library knows it as command {op.index} with "
+                                  f"{lib.kllm_command_nargs(op.index)} arguments, the host has {len(fn.argtypes)}")
+            fmt, op.structs = "<Q", []
+            for i, t in enumerate(fn.argtypes):
+                if t is c_float:
+                    fmt += "f4x"
+                elif t is c_double:
+                    fmt += "d"
+                elif t is c_void_p:
+                    fmt += "Q"
+                else:
+                    fmt += "q"
+                if i in STRUCT_ARGS.get(name, ()):
+                    op.structs.append(i)
+            op.nargs = len(fn.argtypes)
+            op.dynamic = DYNAMIC_ARGS.get(name, ())
+            op.pack = struct.Struct(fmt)
+            op.size = op.pack.size
+            table[name] = op
+        _op_table = table
+    return _op_table
+
+
+class _Recorder:
+    """A step's launches as a buffer of commands (the layout is the library's, see
+    csrc/executor.hpp) and the call that runs them."""
+
+    def __init__(self, stream, chunk, keep=False):
+        self.stream, self.chunk, self.keep = stream, chunk, keep
+        self.kept, self.patches, self.kept_bytes = [], [], 0    # keep: all commands that ran, and where StepValues sit
+        self.bypassed = False                                   # something was launched past the recording
+        self.cap = 1 << 15
+        self.buf = bytearray(self.cap)
+        self.cbuf = (ctypes.c_char * self.cap).from_buffer(self.buf)
+        self.at = 0                 # bytes used
+        self.names = []             # what each command is, for error texts
+        self.ops = _ops()
+        self.run = library().kllm_run_commands
+        self.launched = 0
+
+    def _room(self, need):
+        if self.at + need > self.cap:
+            self.flush()
+            if need > self.cap:
+                del self.cbuf
+                self.cap = max(2 * self.cap, need)
+                self.buf = bytearray(self.cap)
+                self.cbuf = (ctypes.c_char * self.cap).from_buffer(self.buf)
+
+    def add(self, name, what, args):
+        op = self.ops[name]
+        if op.structs:
+            # structs travel behind the arguments; the argument is their offset in words from the
+            # command's first word
+            args = list(args)
+            payload = [(i, bytes(args[i])) for i in op.structs if args[i] is not None]
+            total = op.size + sum(-(-len(b) // 8) * 8 for _, b in payload)
+            self._room(total)
+            at = self.at + op.size
+            for i in op.structs:
+                args[i] = 0
+            for i, b in payload:
+                self.buf[at:at + len(b)] = b
+                args[i] = (at - self.at) // 8
+                at += -(-len(b) // 8) * 8
+        else:
+            total = op.size
+            self._room(total)
+        op.pack.pack_into(self.buf, self.at, op.index | (op.nargs << 16) | ((total // 8) << 32), *args)
+        if self.keep and op.dynamic:
+            for i in op.dynamic:
+                if type(args[i]) is StepValue:
+                    self.patches.append((self.kept_bytes + self.at + 8 + 8 * i, args[i].name))
+        self.at += total
+        self.names.append(what)
+        if len(self.names) >= self.chunk:
+            self.flush()
+
+    def flush(self):
+        if not self.names:
+            return
+        failed = c_int(-1)
+        rc = self.run(self.cbuf, self.at // 8, ctypes.byref(failed), self.stream)
+        if self.keep:
+            self.kept.append(bytes(self.buf[:self.at]))
+            self.kept_bytes += self.at
+        names, self.names, self.at = self.names, [], 0
+        self.launched += len(names)
+        if rc:
+            what = names[failed.value] if 0 <= failed.value < len(names) else "run_commands"
+            buf = ctypes.create_string_buffer(512)
+            library().kllm_last_error(buf, 512)
+            raise KernelError(f"{what}: {buf.value.decode(errors='replace')} (code {rc}; command {failed.value} "
+                              f"of {len(names)} recorded, the ones before it have run)")
+
+
+def flush_recorded():
+    """Run what this thread has recorded so far (nothing to do outside a recording scope):
+    call it before anything else is given to the stream."""
+    rec = getattr(_scoped, "recorder", None)
+    if rec is not None:
+        rec.flush()
+
+
+def bypass_recorded():
+    """``flush_recorded`` for work that a repeat of the recorded commands would not repeat (a
+    torch operation, a library call): the step is marked as not repeatable from its commands."""
+    rec = getattr(_scoped, "recorder", None)
+    if rec is not None:
+        rec.flush()
+        rec.bypassed = True
+
+
+def recording() -> bool:
+    return getattr(_scoped, "recorder", None) is not None
+
+
+class direct_launches:
+    """Inside, launches of this thread are made at once even in a recording scope (what was
+    recorded before runs first): for code that puts work on the stream by other ways."""
+
+    def __enter__(self):
+        self._rec = getattr(_scoped, "recorder", None)
+        if self._rec is not None:
+            self._rec.flush()
+            self._rec.bypassed = True
+            _scoped.recorder = None
         return self
 
     def __exit__(self, *exc):
-        _scoped.stream = self._outer
+        if self._rec is not None:
+            _scoped.recorder = self._rec
         return False
+
+
+def _launch(name, what, *args):
+    """Call the entry point ``name`` with ``args`` (pointers and numbers; a ctypes structure
+    stands for a pointer to it), or record the call if this thread is recording."""
+    rec = getattr(_scoped, "recorder", None)
+    if rec is not None:
+        rec.add(name, what, args)
+        return
+    fn = getattr(library(), name)
+    if name in STRUCT_ARGS:
+        args = [ctypes.byref(a) if isinstance(a, ctypes.Structure) else a for a in args]
+    _check(fn(*args), what)
 
 
 def _ptr(t, name, dtype=None, allow_none=False):
     if t is None:
         if allow_none:
-            return None
+            return 0            # a null pointer, for ctypes and in a recorded command alike
         raise KernelError(f"{name}: tensor is missing")
     if not t.is_cuda:
         raise KernelError(f"{name}: tensor is on {t.device}, the kernels run on the GPU only")
@@ -222,11 +466,10 @@ def embed(out, table, ids, from_sampled=None, sampled=None):
                           f"{ids.numel()} ids do not fit")
     if (from_sampled is None) != (sampled is None) or (from_sampled is not None and from_sampled.numel() < n):
         raise KernelError("embed: from_sampled and sampled go together, one entry per token")
-    _check(library().kllm_embed(
-        _ptr(out, "embed out", torch.float32), _ptr(table, "embed table"),
+    _launch("kllm_embed", "embed", _ptr(out, "embed out", torch.float32), _ptr(table, "embed table"),
         _ptr(ids, "embed ids", torch.int32), _ptr(from_sampled, "embed from", torch.int32, True),
         _ptr(sampled, "embed sampled", torch.int32, True), n, d, table.shape[0], dtype_code(table.dtype),
-        _stream()), "embed")
+        _stream())
 
 
 def add_rmsnorm(x, delta=None, weight=None, out=None, rows=None, eps=0.0, write_x=None):
@@ -249,23 +492,20 @@ def add_rmsnorm(x, delta=None, weight=None, out=None, rows=None, eps=0.0, write_
     if out is not None:
         if tuple(out.shape) != (n, d) or weight is None or weight.numel() != d:
             raise KernelError("add_rmsnorm: output or weight shape does not fit")
-    _check(library().kllm_add_rmsnorm(
-        _ptr(x, "add_rmsnorm x", torch.float32), _ptr(delta, "add_rmsnorm delta", None, True), ddt,
+    _launch("kllm_add_rmsnorm", "add_rmsnorm", _ptr(x, "add_rmsnorm x", torch.float32), _ptr(delta, "add_rmsnorm delta", None, True), ddt,
         nsplit, stride, _ptr(weight, "add_rmsnorm weight", torch.float32, True),
         _ptr(out, "add_rmsnorm out", None, True),
         dtype_code(out.dtype) if out is not None else DT_F32,
         _ptr(rows, "add_rmsnorm rows", torch.int32, True), n, d, float(eps), int(bool(write_x)),
-        _stream()), "add_rmsnorm")
+        _stream())
 
 
 def rope_tables(cos, sin, positions, head_dim, theta):
     n = positions.numel()
     if tuple(cos.shape) != (n, head_dim // 2) or tuple(sin.shape) != (n, head_dim // 2):
         raise KernelError("rope_tables: table shapes do not fit")
-    _check(library().kllm_rope_tables(
-        _ptr(cos, "rope cos", torch.float32), _ptr(sin, "rope sin", torch.float32),
-        _ptr(positions, "rope positions", torch.int32), n, head_dim, float(theta), _stream()),
-        "rope_tables")
+    _launch("kllm_rope_tables", "rope_tables", _ptr(cos, "rope cos", torch.float32), _ptr(sin, "rope sin", torch.float32),
+        _ptr(positions, "rope positions", torch.int32), n, head_dim, float(theta), _stream())
 
 
 def rope_append(qkv, q_out, cos, sin, cache, positions, span_of_token, block_table, page_size,
@@ -290,15 +530,13 @@ def rope_append(qkv, q_out, cos, sin, cache, positions, span_of_token, block_tab
             raise KernelError("rope_append: index arrays are too short")
     if cos is not None and (tuple(cos.shape) != (n, rot // 2) or tuple(sin.shape) != tuple(cos.shape)):
         raise KernelError("rope_append: cos/sin shapes do not fit")
-    _check(library().kllm_rope_append(
-        _ptr(qkv, "rope_append qkv"), dtype_code(qkv.dtype), nsplit, stride,
+    _launch("kllm_rope_append", "rope_append", _ptr(qkv, "rope_append qkv"), dtype_code(qkv.dtype), nsplit, stride,
         _ptr(q_out, "rope_append q_out"), _ptr(cos, "rope_append cos", torch.float32, True),
         _ptr(sin, "rope_append sin", torch.float32, True), _ptr(cache, "rope_append cache", None, True),
         _ptr(positions, "rope_append positions", torch.int32, True),
         _ptr(span_of_token, "rope_append span_of_token", torch.int32, True),
         _ptr(block_table, "rope_append block_table", torch.int32, True), max_pages, page_size, n,
-        n_heads, n_kv_heads, head_dim, rot, int(bool(interleaved)), dtype_code(q_out.dtype), _stream()),
-        "rope_append")
+        n_heads, n_kv_heads, head_dim, rot, int(bool(interleaved)), dtype_code(q_out.dtype), _stream())
 
 
 ACT_SILU, ACT_GELU_TANH = 0, 1
@@ -313,9 +551,8 @@ def silu_mul(gu, out, act=ACT_SILU):
         nsplit, stride = gu.shape[0], gu.shape[1] * gu.shape[2]
     if gu.shape[-1] != 2 * f or gu.shape[-2] != n:
         raise KernelError(f"silu_mul: input {tuple(gu.shape)} does not fit output {tuple(out.shape)}")
-    _check(library().kllm_silu_mul(
-        _ptr(gu, "silu_mul in"), dtype_code(gu.dtype), nsplit, stride, _ptr(out, "silu_mul out"),
-        dtype_code(out.dtype), n, f, int(act), _stream()), "silu_mul")
+    _launch("kllm_silu_mul", "silu_mul", _ptr(gu, "silu_mul in"), dtype_code(gu.dtype), nsplit, stride, _ptr(out, "silu_mul out"),
+        dtype_code(out.dtype), n, f, int(act), _stream())
 
 
 class _NormedInput(ctypes.Structure):
@@ -346,11 +583,11 @@ class NormedInput:
 
 
 def _x_and_norm(x, dtype):
-    """(pointer of x or None, struct or None, n, k) for an input that is a tensor or a NormedInput."""
+    """(pointer of x or 0, struct or None, n, k) for an input that is a tensor or a NormedInput."""
     if isinstance(x, NormedInput):
         n, k = x.shape
         st = x.struct(n, k)
-        return None, st, n, k
+        return 0, st, n, k
     n, k = x.shape
     if x.dtype != dtype:
         raise KernelError(f"input dtype {x.dtype}, weights {dtype}")
@@ -384,9 +621,8 @@ def linear_resid(x, w, resid, ss):
             or w.dtype != x.dtype):
         raise KernelError(f"linear_resid: x {tuple(x.shape)}, w {tuple(w.shape)}, resid {tuple(resid.shape)}, "
                           f"ss {tuple(ss.shape)} do not fit ({parts} parts)")
-    _check(library().kllm_gemv_resid(
-        _ptr(x, "resid x"), _ptr(w, "resid w"), _ptr(resid, "resid", torch.float32),
-        _ptr(ss, "resid ss", torch.float32), n, m, k, dtype_code(x.dtype), _stream()), "gemv_resid")
+    _launch("kllm_gemv_resid", "gemv_resid", _ptr(x, "resid x"), _ptr(w, "resid w"), _ptr(resid, "resid", torch.float32),
+        _ptr(ss, "resid ss", torch.float32), n, m, k, dtype_code(x.dtype), _stream())
     return parts
 
 
@@ -402,13 +638,11 @@ def gemm(x, w, y, algo, nsplit=1):
     if algo == GEMM_GEMV_LDS:
         if nsplit != 1:
             raise KernelError("gemm: the LDS gemv does not split K")
-        _check(library().kllm_gemv_plain(
-            _ptr(x, "gemv x"), _ptr(w, "gemv w"), _ptr(y, "gemv y", torch.float32), n, m, k,
-            dtype_code(x.dtype), None, _stream()), "gemv_plain")
+        _launch("kllm_gemv_plain", "gemv_plain", _ptr(x, "gemv x"), _ptr(w, "gemv w"), _ptr(y, "gemv y", torch.float32), n, m, k,
+            dtype_code(x.dtype), None, _stream())
         return
-    _check(library().kllm_gemm(
-        _ptr(x, "gemm x"), _ptr(w, "gemm w"), _ptr(y, "gemm y"), n, m, k, dtype_code(x.dtype),
-        dtype_code(y.dtype), algo, nsplit, _stream()), "gemm")
+    _launch("kllm_gemm", "gemm", _ptr(x, "gemm x"), _ptr(w, "gemm w"), _ptr(y, "gemm y"), n, m, k, dtype_code(x.dtype),
+        dtype_code(y.dtype), algo, nsplit, _stream())
 
 
 def gemv_fits(n, m, k, dtype, best=True) -> bool:
@@ -426,8 +660,8 @@ def gemm_swiglu(x, w_gate_up, h, act=ACT_SILU):
     f = h.shape[1]
     if tuple(w_gate_up.shape) != (2 * f, k) or h.shape[0] != n or x.dtype != w_gate_up.dtype or h.dtype != x.dtype:
         raise KernelError("gemm_swiglu: shapes or dtypes do not fit")
-    _check(library().kllm_gemm_swiglu(_ptr(x, "gemm x"), _ptr(w_gate_up, "gemm w"), _ptr(h, "gemm h"), n, f, k,
-                                      dtype_code(x.dtype), int(act), _stream()), "gemm_swiglu")
+    _launch("kllm_gemm_swiglu", "gemm_swiglu", _ptr(x, "gemm x"), _ptr(w_gate_up, "gemm w"), _ptr(h, "gemm h"), n, f, k,
+                                      dtype_code(x.dtype), int(act), _stream())
 
 
 def gemv_swiglu(x, w_gate_up, h, act=ACT_SILU):
@@ -437,9 +671,8 @@ def gemv_swiglu(x, w_gate_up, h, act=ACT_SILU):
     f = h.shape[1]
     if tuple(w_gate_up.shape) != (2 * f, k) or h.shape[0] != n or h.dtype != w_gate_up.dtype:
         raise KernelError("gemv_swiglu: shapes or dtypes do not fit")
-    _check(library().kllm_gemv_swiglu(xp, _ptr(w_gate_up, "gemv w"), _ptr(h, "gemv h"), n, f, k,
-                                      dtype_code(w_gate_up.dtype), int(act), ctypes.byref(st) if st else None, _stream()),
-           "gemv_swiglu")
+    _launch("kllm_gemv_swiglu", "gemv_swiglu", xp, _ptr(w_gate_up, "gemv w"), _ptr(h, "gemv h"), n, f, k,
+                                      dtype_code(w_gate_up.dtype), int(act), st, _stream())
 
 
 def gemv_rope_append(x, w_qkv, q_out, cos, sin, cache, positions, span_of_token, block_table, page_size,
@@ -460,14 +693,12 @@ def gemv_rope_append(x, w_qkv, q_out, cos, sin, cache, positions, span_of_token,
             raise KernelError("gemv_rope_append: index arrays are too short")
     if cos is not None and (tuple(cos.shape) != (n, head_dim // 2) or tuple(sin.shape) != tuple(cos.shape)):
         raise KernelError("gemv_rope_append: cos/sin shapes do not fit")
-    _check(library().kllm_gemv_rope_append(
-        xp, _ptr(w_qkv, "gemv w"), _ptr(q_out, "gemv q_out"),
+    _launch("kllm_gemv_rope_append", "gemv_rope_append", xp, _ptr(w_qkv, "gemv w"), _ptr(q_out, "gemv q_out"),
         _ptr(cos, "gemv cos", torch.float32, True), _ptr(sin, "gemv sin", torch.float32, True),
         _ptr(cache, "gemv cache", None, True), _ptr(positions, "gemv positions", torch.int32, True),
         _ptr(span_of_token, "gemv span_of_token", torch.int32, True),
         _ptr(block_table, "gemv block_table", torch.int32, True), max_pages, page_size, n, n_heads,
-        n_kv_heads, head_dim, k, dtype_code(w_qkv.dtype), ctypes.byref(st) if st else None, _stream()),
-        "gemv_rope_append")
+        n_kv_heads, head_dim, k, dtype_code(w_qkv.dtype), st, _stream())
 
 
 class _LinearOut(ctypes.Structure):
@@ -607,8 +838,8 @@ def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None, act=ACT_SIL
     if tuple(y.shape) != want or y.dtype != dt:
         raise KernelError(f"fused_linear: output {tuple(y.shape)} {y.dtype}, expected {want} {dt}")
     lo.y = _ptr(y, "fused_linear y")
-    _check(library().kllm_fused_linear(x_ptr, x_stride, ctypes.byref(lo), _ptr(w, "fused_linear w"), n, m, k,
-                                       tiles_per_wg, _stream()), "fused_linear")
+    _launch("kllm_fused_linear", "fused_linear", x_ptr, x_stride, lo, _ptr(w, "fused_linear w"), n, m, k,
+                                       tiles_per_wg, _stream())
 
 
 def sum_splits(parts, out):
@@ -616,9 +847,8 @@ def sum_splits(parts, out):
     nsplit = parts.shape[0]
     if tuple(parts.shape[1:]) != tuple(out.shape):
         raise KernelError("sum_splits: shapes do not fit")
-    _check(library().kllm_sum_splits(_ptr(parts, "sum_splits in", torch.float32), nsplit, out.numel(),
-                                     _ptr(out, "sum_splits out"), dtype_code(out.dtype), _stream()),
-           "sum_splits")
+    _launch("kllm_sum_splits", "sum_splits", _ptr(parts, "sum_splits in", torch.float32), nsplit, out.numel(),
+                                     _ptr(out, "sum_splits out"), dtype_code(out.dtype), _stream())
 
 
 def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size, n_heads,
@@ -631,13 +861,11 @@ def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size
         raise KernelError(f"attn_generic: cache {tuple(cache.shape)} does not fit")
     if positions.numel() < n or span_of_token.numel() < n:
         raise KernelError("attn_generic: index arrays are too short")
-    _check(library().kllm_attn_generic(
-        _ptr(q, "attn q"), _ptr(out, "attn out"), _ptr(cache, "attn cache"),
+    _launch("kllm_attn_generic", "attn_generic", _ptr(q, "attn q"), _ptr(out, "attn out"), _ptr(cache, "attn cache"),
         _ptr(positions, "attn positions", torch.int32),
         _ptr(span_of_token, "attn span_of_token", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size, n,
-        n_heads, n_kv_heads, head_dim, int(window), float(scale), dtype_code(q.dtype), _stream()),
-        "attn_generic")
+        n_heads, n_kv_heads, head_dim, int(window), float(scale), dtype_code(q.dtype), _stream())
 
 
 GENERIC_MAX_PAGE_SIZE = 256     # pages of the kernel that takes every size
@@ -693,14 +921,14 @@ def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, bloc
         raise KernelError(f"attn_prefill: cache {tuple(cache.shape)} does not fit")
     if query_tiles.numel() < 2 * n_tiles:
         raise KernelError("attn_prefill: tile list is too short")
-    _check(library().kllm_attn_prefill(
-        _ptr(q, "attn q"), _ptr(out, "attn out"), _ptr(cache, "attn cache"),
+    _launch("kllm_attn_prefill", "attn_prefill", _ptr(q, "attn q"), _ptr(out, "attn out"), _ptr(cache, "attn cache"),
         _ptr(query_tiles, "attn query_tiles", torch.int32), n_tiles,
         _ptr(span_start, "attn span_start", torch.int32), _ptr(span_pos, "attn span_pos", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size,
-        n_heads, n_kv_heads, head_dim, int(window), float(scale), int(keys_total), int(keys_longest),
-        dtype_code(q.dtype), _stream()),
-        "attn_prefill")
+        n_heads, n_kv_heads, head_dim, int(window), float(scale),
+        keys_total if type(keys_total) is StepValue else int(keys_total),
+        keys_longest if type(keys_longest) is StepValue else int(keys_longest),
+        dtype_code(q.dtype), _stream())
 
 
 def attn_decode(q, out, part, cache, positions, span_of_token, block_table, page_size, n_heads,
@@ -713,21 +941,18 @@ def attn_decode(q, out, part, cache, positions, span_of_token, block_table, page
         raise KernelError(f"attn_decode: cache {tuple(cache.shape)} does not fit")
     if positions.numel() < n or span_of_token.numel() < n:
         raise KernelError("attn_decode: index arrays are too short")
-    _check(library().kllm_attn_decode(
-        _ptr(q, "attn q"), _ptr(out, "attn out"), _ptr(part, "attn part", torch.float32),
+    _launch("kllm_attn_decode", "attn_decode", _ptr(q, "attn q"), _ptr(out, "attn out"), _ptr(part, "attn part", torch.float32),
         part.numel(), _ptr(cache, "attn cache"), _ptr(positions, "attn positions", torch.int32),
         _ptr(span_of_token, "attn span_of_token", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size, n,
         n_heads, n_kv_heads, head_dim, int(window), float(scale), int(nslices), dtype_code(q.dtype),
-        _ptr(token_list, "attn token_list", torch.int32, True), int(n_listed), _stream()),
-        "attn_decode")
+        _ptr(token_list, "attn token_list", torch.int32, True), int(n_listed), _stream())
 
 
 def sample(out, logits, temperature=None, uniform=None):
     rows, vocab = logits.shape
     if out.numel() < rows:
         raise KernelError("sample: output is too short")
-    _check(library().kllm_sample(
-        _ptr(out, "sample out", torch.int32), _ptr(logits, "sample logits", torch.float32),
+    _launch("kllm_sample", "sample", _ptr(out, "sample out", torch.int32), _ptr(logits, "sample logits", torch.float32),
         _ptr(temperature, "sample temperature", torch.float32, True),
-        _ptr(uniform, "sample uniform", torch.float32, True), rows, vocab, _stream()), "sample")
+        _ptr(uniform, "sample uniform", torch.float32, True), rows, vocab, _stream())

@@ -28,6 +28,7 @@ from .spec import CacheNeed, WeightSpec
 @register_part("mixer", "attention")
 class CausalSelfAttention(Part):
     graph_safe = True
+    records_launches = True
     takes_normed = True     # the q, k, v product of a decode batch applies the norm's row scale itself
     fills_sink = True       # the output projection of a decode batch adds itself to the residual stream
     # How the attention kernels want a step's spans listed: the tokens of spans of at most
@@ -48,6 +49,21 @@ class CausalSelfAttention(Part):
                     blocks += [t, s]
         return {"short": short, "blocks": blocks}
 
+    def step_values(self, starts, lens, positions):
+        """How many keys the step's query blocks read, all together and the longest block
+        alone: a whole prompt's blocks read more and more, a portion far into its context reads
+        many in every block, and the prompt kernel is chosen by that."""
+        total = longest = 0
+        for pos, n in zip(positions, lens):
+            if n <= self.SHORT_SPAN:
+                continue
+            for first in range(0, n, self.QUERY_BLOCK):
+                last = pos + min(first + self.QUERY_BLOCK, n)          # keys [0, last) are before the block's end
+                keys = min(last, self.window + self.QUERY_BLOCK) if self.window else last
+                total += keys
+                longest = max(longest, keys)
+        return {"keys_total": total, "keys_longest": longest}
+
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)
         self.hidden = int(self.param("hidden"))
@@ -55,6 +71,7 @@ class CausalSelfAttention(Part):
         self.kv_heads = int(self.param("kv_heads"))
         self.head_dim = int(self.param("head_dim"))
         self.window = int(self.param("window", 0) or 0)
+        self.step_values_key = f"attention.keys.window{self.window}"     # layers with the same window read alike
         self.own_kv = bool(self.param("own_kv", True))
         if self.heads % self.kv_heads:
             raise ValueError(f"attention: {self.heads} heads are not a multiple of {self.kv_heads} KV heads")
@@ -189,20 +206,13 @@ class CausalSelfAttention(Part):
                            self.kv_heads, self.head_dim, self.window, self.scale, total, longest)
 
     def _keys_read(self, ctx):
-        """How many keys the step's query blocks read, all together and the
-        longest block alone (from the host's copies of the spans): a whole
-        prompt's blocks read more and more, a portion far into its context
-        reads many in every block, and the prompt kernel is chosen by that."""
-        total = longest = 0
-        for pos, n in zip(ctx.h_span_pos, ctx.h_span_len):
-            if n <= self.SHORT_SPAN:
-                continue
-            for first in range(0, n, self.QUERY_BLOCK):
-                last = pos + min(first + self.QUERY_BLOCK, n)          # keys [0, last) are before the block's end
-                keys = min(last, self.window + self.QUERY_BLOCK) if self.window else last
-                total += keys
-                longest = max(longest, keys)
-        return total, longest
+        """The step's key counts (see ``step_values``), as the engine worked them out for this
+        step, or from the host's copies of the spans for a context built by hand."""
+        v, key = ctx.values, self.step_values_key
+        if key + ".keys_total" in v:
+            return v[key + ".keys_total"], v[key + ".keys_longest"]
+        own = self.step_values(ctx.h_span_start, ctx.h_span_len, ctx.h_span_pos)
+        return own["keys_total"], own["keys_longest"]
 
     def _decode(self, ctx, q, out, cache, token_list, count):
         n = q.shape[0]

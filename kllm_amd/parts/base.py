@@ -89,6 +89,7 @@ class Workspace:
 
     def __init__(self, device):
         self.device = device
+        self.generation = 0          # grows when a buffer is replaced: addresses handed out before may be gone
         self._bufs: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
         self._views: Dict[Tuple[str, tuple, torch.dtype], torch.Tensor] = {}   # handed out before
 
@@ -103,6 +104,10 @@ class Workspace:
         key = (tag, dtype)
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < numel:
+            if buf is not None:
+                from .. import kernels as K
+                K.flush_recorded()   # launches recorded with the old buffer's address run before it goes
+                self.generation += 1
             buf = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
             self._bufs[key] = buf
             for k in [k for k in self._views if k[0] == tag and k[2] == dtype]:   # views of the old buffer
@@ -231,6 +236,9 @@ class StepContext:
     # Index lists that parts asked for through ``Part.step_lists``: "<key>.<name>" -> int32
     # tensor on the device (as long as the host list was, possibly empty).
     lists: Dict[str, torch.Tensor] = field(default_factory=dict)
+    # Numbers that parts asked for through ``Part.step_values``: "<key>.<name>" -> int, worked
+    # out on the host from the step's positions.
+    values: Dict[str, int] = field(default_factory=dict)
     # Token ids that never reached the host: token t with token_from[t] >= 0 is
     # sampled[token_from[t]], what the last sampled step chose (both or neither are set).
     token_from: Optional[torch.Tensor] = None
@@ -238,6 +246,17 @@ class StepContext:
 
     def buf(self, tag, shape, dtype):
         return (self.workspace or self.runtime.workspace).get(tag, shape, dtype)
+
+
+def call_part(part, fn, *args, **kwargs):
+    """Call ``fn`` (a method of ``part``) so that its work reaches the stream in program order:
+    as it is for a part that records its launches, otherwise with the recorded launches run
+    first and recording switched off inside."""
+    from .. import kernels as K
+    if getattr(part, "records_launches", False) or not K.recording():
+        return fn(*args, **kwargs)
+    with K.direct_launches():
+        return fn(*args, **kwargs)
 
 
 class Part:
@@ -256,6 +275,7 @@ class Part:
     # ``ctx.lists["<key>.<name>"]``.  Parts with the same key share one set of lists.  The
     # lists may depend on nothing but ``starts`` and ``lens`` (a recorded step replays them).
     step_lists_key: Optional[str] = None
+    step_values_key: Optional[str] = None      # the same for ``step_values`` (see there)
     # A mixer or feed-forward whose first product can normalise its input while staging it
     # declares ``takes_normed`` and may then get a ``Normed`` as its input; one whose
     # last product can add itself to the residual stream declares ``fills_sink`` and then
@@ -264,6 +284,11 @@ class Part:
     takes_normed = False
     fills_sink = False
     fusable = False
+    # True if everything the part gives to the stream goes through the package's kernel wrappers
+    # (``kllm_amd.kernels``), which can record a step's launches and hand them to the library in
+    # one call.  A part that uses torch operations or launches by other ways leaves this False:
+    # it is then called with what was recorded already run, and its own launches made at once.
+    records_launches = False
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
         self.spec = spec
@@ -295,6 +320,17 @@ class Part:
     def check_cache(self, page_size: int) -> None:
         """Raise ValueError if this part's kernels do not take a cache with pages of
         ``page_size`` tokens; the engine asks every part before it allocates."""
+
+    def step_values(self, starts: List[int], lens: List[int], positions: List[int]) -> Dict[str, int]:
+        """name -> int for a step whose span s covers rows ``starts[s] .. starts[s] + lens[s]`` at
+        positions ``positions[s] ...``: what the part's launches need to know of the step's
+        positions on the host (a count that chooses a kernel, a bound of a loop).  The part
+        finds them as ``ctx.values["<step_values_key>.<name>"]`` and hands them to the kernel
+        wrappers as they are; a step that is run again from its recorded commands gets the new
+        step's values in their place.  Everything else of a part's launches may depend on
+        ``starts`` and ``lens`` only.  Only called when ``step_values_key`` is set; parts with
+        the same key share one set of values."""
+        return {}
 
     def children(self) -> List["Part"]:
         """Parts this part is made of (an arrangement's norms, mixer, feed-forward)."""

@@ -12,11 +12,13 @@ norm's row scale to its own sums (``Normed``).
 
 from __future__ import annotations
 
-from .base import Part, ResidualSink, make_part, register_part
+from .base import Part, ResidualSink, call_part, make_part, register_part
 
 
 @register_part("block", "pre_norm")
 class PreNormBlock(Part):
+    records_launches = True     # the arrangement itself launches nothing; its parts are called each in its own way
+
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)
         layer = self.param("layer")
@@ -74,8 +76,11 @@ class PreNormBlock(Part):
         """``next_norm``: the norm that will take this layer's pending output
         (the next layer's first norm), if the caller knows it; the feed-forward
         may then add its output to x itself."""
-        xn = self.norm_mixer.forward(ctx, x, delta=pending, **self._normed_ok(ctx, self.norm_mixer, self.mixer))
-        delta = self.mixer.forward(ctx, xn, cache, **self._sink(ctx, x, self.mixer, self.norm_ff))
-        xn = self.norm_ff.forward(ctx, x, delta=delta, **self._normed_ok(ctx, self.norm_ff, self.feed_forward))
-        pending = self.feed_forward.forward(ctx, xn, **self._sink(ctx, x, self.feed_forward, next_norm))
+        xn = call_part(self.norm_mixer, self.norm_mixer.forward, ctx, x, delta=pending,
+                       **self._normed_ok(ctx, self.norm_mixer, self.mixer))
+        delta = call_part(self.mixer, self.mixer.forward, ctx, xn, cache, **self._sink(ctx, x, self.mixer, self.norm_ff))
+        xn = call_part(self.norm_ff, self.norm_ff.forward, ctx, x, delta=delta,
+                       **self._normed_ok(ctx, self.norm_ff, self.feed_forward))
+        pending = call_part(self.feed_forward, self.feed_forward.forward, ctx, xn,
+                            **self._sink(ctx, x, self.feed_forward, next_norm))
         return x, pending

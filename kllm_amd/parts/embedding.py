@@ -20,6 +20,7 @@ from .spec import WeightSpec
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Part):
     graph_safe = True
+    records_launches = True
 
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)
@@ -51,6 +52,7 @@ class TokenEmbedding(Part):
 @register_part("head", "linear_head")
 class LinearHead(Part):
     graph_safe = True
+    records_launches = True
 
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)

@@ -20,6 +20,7 @@ from .spec import WeightSpec
 @register_part("feed_forward", "gated_mlp")
 class GatedFeedForward(Part):
     graph_safe = True
+    records_launches = True
     takes_normed = True     # the gate and up products of a decode batch apply the norm's row scale
     fills_sink = True       # the down projection of a decode batch adds itself to the residual stream
 

@@ -219,6 +219,7 @@ def linear(ctx, x, w, tag, out_dtype=torch.float32, split=True):
         K.fused_linear(w, y, K.LINEAR_PARTS, x=x, tiles_per_wg=4 if m >= 16384 else 1)
         return y[0]
     if algo == "library":
+        K.bypass_recorded()             # the library is called through torch: behind what was recorded
         if out_dtype == torch.float32:
             # float32 sums straight from the library's accumulators: a result that the caller
             # wants in 32-bit (a residual delta, logits) is never rounded to bfloat16 on the way

@@ -19,6 +19,7 @@ from .spec import WeightSpec
 @register_part("norm", "rmsnorm")
 class RMSNorm(Part):
     graph_safe = True
+    records_launches = True
     fusable = True     # a product's epilogue may do the addition, its consumer the row scale
 
     def __init__(self, spec, runtime):

@@ -20,6 +20,7 @@ from .base import Part, register_part
 @register_part("position", "rotary")
 class RotaryEncoding(Part):
     graph_safe = True
+    records_launches = True
 
 
     def __init__(self, spec, runtime):

@@ -221,6 +221,81 @@ def test_a_step_queued_ahead_takes_its_ids_from_the_device(model_dirs, dtype):
         assert [[step[i] for step in runs[1]] for i in range(3)] == want
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_steps_run_again_from_their_recorded_commands(model_dirs, dtype):
+    """A step's launches go to the library as one buffer of commands, and a step whose shape
+    was seen before runs again from the commands recorded then, with its own positions' values
+    in place.  Both give, bit for bit, what launching one by one gives: portions of equal size
+    of a long prompt (whose key counts grow), beside decode tokens of other requests."""
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry
+    cfg, d = tiny.CONFIGS["E"], model_dirs("E")
+    long_prompt, others = tiny.tokens(cfg, 900, 1), [tiny.tokens(cfg, 40 + 3 * i, 2 + i) for i in range(3)]
+    outs = {}
+
+    def run(eng):
+        got = [eng.step([StepEntry(("o", i), o[:-12], [len(o) - 13]) for i, o in enumerate(others)]).clone()]
+        fed = 0
+        for k in range(12):                    # 3 decode tokens + a portion of 64 tokens, twelve times
+            entries = [StepEntry(("o", i), [o[len(o) - 12 + k]], [0]) for i, o in enumerate(others)]
+            entries.append(StepEntry("long", long_prompt[fed:fed + 64], [0, 63]))
+            fed += 64
+            got.append(eng.step(entries).clone())
+        got.append(eng.step([StepEntry("long", long_prompt[fed:], [len(long_prompt) - fed - 1])]).clone())
+        for rid in ["long"] + [("o", i) for i in range(len(others))]:
+            eng.release(rid)
+        eng.cache.check_invariants()
+        return [g.cpu() for g in got]
+    for mode, extra in (("one by one", {"launch_one_by_one": True}), ("recorded", {"no_repeated_steps": True}),
+                        ("repeated", {})):
+        eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=2048, max_model_len=2048, extra=extra))
+        outs[mode] = run(eng)
+        if mode == "repeated":
+            # the first pass grows the scratch buffers now and then (commands recorded before that
+            # are dropped), the second records what was dropped, the third repeats every step
+            first = eng.steps_repeated
+            run(eng)
+            second = eng.steps_repeated
+            outs["repeated, third pass"] = run(eng)
+            assert eng._repeat_steps and first >= 3 and second - first >= 6, (first, second)
+            assert eng.steps_repeated - second == 14
+        else:
+            assert eng.steps_repeated == 0
+    for mode in ("recorded", "repeated", "repeated, third pass"):
+        for a, b in zip(outs["one by one"], outs[mode]):
+            assert torch.equal(a, b), mode
+    want = expected(d, cfg, {"long": long_prompt}, dtype)["long"]
+    got = outs["repeated"][-1][0].numpy()
+    assert float(np.abs(got - want[len(long_prompt) - 1]).max()) < tiny.TOL[dtype]
+
+
+def test_a_recorded_launch_that_the_library_refuses_is_named():
+    """Inside a recording scope the wrappers only write commands; the library's refusal of one
+    comes out when the commands run, with the launch's name, and the launches before it have
+    run."""
+    from kllm_amd import kernels as K
+    x = torch.ones(4, 64, device="cuda")
+    w = torch.ones(64, device="cuda")
+    out = torch.zeros(4, 64, device="cuda")
+    bad_x, bad_w, bad_y = (torch.ones(4, 12, dtype=torch.bfloat16, device="cuda"),
+                           torch.ones(8, 12, dtype=torch.bfloat16, device="cuda"), torch.zeros(1, 4, 8, device="cuda"))
+    with pytest.raises(K.KernelError, match="gemm.*command 1 of 2"):
+        with K.stream_scope(record=True):
+            K.add_rmsnorm(x, weight=w, out=out, eps=0.0)
+            K.gemm(bad_x, bad_w, bad_y, K.GEMM_MFMA_BF16, 1)          # K = 12 is no multiple of 8
+            assert float(out.abs().sum()) == 0.0                      # nothing has run yet
+    torch.cuda.synchronize()
+    assert torch.allclose(out, torch.ones_like(out), atol=1e-6)       # the norm before it did run
+    with K.stream_scope(record=True):                                 # work given to the stream by other ways
+        K.add_rmsnorm(x, weight=w, out=out, eps=3.0)                  # comes after a flush
+        K.flush_recorded()
+        assert torch.allclose(out, torch.full_like(out, 0.5), atol=1e-6)
+        with K.direct_launches():
+            assert not K.recording()
+            K.add_rmsnorm(x, weight=w, out=out, eps=0.0)
+            assert torch.allclose(out, torch.ones_like(out), atol=1e-6)
+        assert K.recording()
+
+
 def test_no_collection_of_garbage_falls_into_a_recording(model_dirs):
     """An engine that is dropped is garbage in a reference cycle, its recorded steps with
     it.  HIP refuses to destroy a graph on a thread that records one, and the error would

@@ -198,6 +198,9 @@ def test_toy_architecture_is_registered_built_and_stepped(toy_registered, dtype)
     plan = eng.model.cache_plan
     assert [g.need.kind for g in plan.groups] == ["paged", "state"] and plan.runs == [(0, 0, True), (1, 0, True)]
     assert tuple(eng.state[1].shape) == (1, 3, 40)
+    # the toy parts use torch operations: the engine calls them with its recorded launches run, and
+    # does not run such a model's steps again from recorded commands
+    assert eng.records_launches and not eng._repeat_steps
     w = engine_weights(eng)
     reqs = {"a": tiny.tokens(cfg, 45, 1), "b": tiny.tokens(cfg, 30, 2), "c": tiny.tokens(cfg, 22, 3),
             "d": tiny.tokens(cfg, 37, 4)}

@@ -11,6 +11,7 @@ graph capture.
 from __future__ import annotations
 
 import ctypes
+import functools
 import struct
 import threading
 from ctypes import c_char_p, c_double, c_float, c_int, c_long, c_void_p
@@ -731,6 +732,7 @@ def fused_tiles_per_wg(n, m, k) -> int:
     return 2 if n > 8 and m * k >= 20_000_000 else 1
 
 
+@functools.lru_cache(maxsize=4096)
 def fused_linear_fits(n, k, nsplit=1) -> bool:
     """Whether the decode-batch products take n rows of K: bfloat16 only, K a
     multiple of 8, and all rows of a workgroup's slice of K in LDS."""
@@ -753,6 +755,7 @@ class ScaledRows:
         return self.xw.shape
 
 
+@functools.lru_cache(maxsize=4096)
 def fused_resid_parts(n, m, k, tiles_per_wg=1) -> int:
     """Partial sums of squares per row that a LINEAR_RESID product of these sizes leaves, or 0
     if the decode-batch kernel does not take them."""
@@ -872,6 +875,7 @@ GENERIC_MAX_PAGE_SIZE = 256     # pages of the kernel that takes every size
 DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
 
 
+@functools.lru_cache(maxsize=4096)
 def attn_decode_slices(n, n_kv_heads, n_heads, head_dim, dtype=torch.bfloat16, max_keys=0) -> int:
     """Slices of keys for a decode batch of n tokens; ``max_keys`` bounds the keys of the
     longest request (block-table width x page size, or the window), 0 if unknown."""
@@ -885,6 +889,7 @@ def attn_f32_fits(head_dim, page_size) -> bool:
     return bool(library().kllm_attn_f32_fits(int(head_dim), int(page_size)))
 
 
+@functools.lru_cache(maxsize=4096)
 def gemm_decode_tile_cols(n, m, k) -> int:
     """Columns of the tiles that the MFMA kernel gives a decode batch of these sizes."""
     return int(library().kllm_gemm_decode_tile_cols(int(n), int(m), int(k)))

@@ -26,6 +26,8 @@ kernel.
 
 from __future__ import annotations
 
+import functools
+
 import torch
 
 from .. import kernels as K
@@ -158,6 +160,17 @@ def choose(dtype, n, m, k, options=None):
     return K.GEMM_MFMA_BF16, _mfma_split(n, m, k)
 
 
+@functools.lru_cache(maxsize=4096)
+def _resid_tiles(n, m, k):
+    """(tiles per workgroup, partial sums of squares per row) of a decode batch's residual
+    product: as few tiles to a workgroup as keep the sums of squares within what the
+    consumer reads; (1, 0) if the kernel does not take the sizes."""
+    tpw = 1
+    while K.fused_resid_parts(n, m, k, tpw) == 0 and tpw < 64 and K.fused_linear_fits(n, k):
+        tpw *= 2
+    return tpw, K.fused_resid_parts(n, m, k, tpw)
+
+
 def linear_into(ctx, x, w, sink, tag):
     """x . w^T added to the residual stream of ``sink`` in the product's own
     epilogue, for up to four tokens: returns the ``Normed`` that stands for the
@@ -190,10 +203,7 @@ def linear_into(ctx, x, w, sink, tag):
         return None
     # a decode batch on the matrix cores: all of K in a workgroup, the addition in the epilogue, and
     # beside the stream its rows times the norm's weight in 16 bits for a consumer that scales its sums
-    tpw = 1
-    while K.fused_resid_parts(n, m, k, tpw) == 0 and tpw < 64 and K.fused_linear_fits(n, k):
-        tpw *= 2
-    parts = K.fused_resid_parts(n, m, k, tpw)
+    tpw, parts = _resid_tiles(n, m, k)
     if parts == 0:
         return None
     ss = ctx.buf(tag + ".ss", (n, -(-parts // 4) * 4), torch.float32)

@@ -6,8 +6,11 @@ described but not built (docs/theory/02-autoregressive-decoding.md:122-123).
 Here both run on the device.  With temperature T > 0 the token is drawn from
 softmax(logits / T) by inverting the cumulative distribution at a uniform
 number; that number depends only on (the request's seed, how many tokens the
-request has generated), never on what else is in the batch, so a request
-samples the same tokens alone and in any batch.
+request has generated), never on what else is in the batch.  The logits
+themselves equal those of the request alone up to rounding only (which kernel
+runs, and how it cuts its sums, follows the step's size): a request samples the
+same tokens alone and in any batch except where two candidates lie within that
+rounding of each other, a last bit in float32, about a hundredth in bfloat16.
 """
 
 from __future__ import annotations

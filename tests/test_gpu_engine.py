@@ -545,6 +545,32 @@ def test_temperature_generation_matches_the_plain_sampler(model_dirs):
             ids.append(tok)
 
 
+def test_temperature_generation_in_bfloat16_alone_and_in_a_batch(model_dirs):
+    """In bfloat16 a request's logits in a batch equal those of the request alone up to
+    rounding only (the kernels follow the step's size), so the drawn tokens may part ways,
+    but only where the uniform number lies within that rounding of a boundary of the
+    cumulative distribution; up to there they are the same tokens."""
+    from kllm_amd.engine import Engine, EngineOptions
+    from kllm_amd.sampling import uniform
+    cfg, d = tiny.CONFIGS["B"], model_dirs("B", store="bfloat16")
+    eng = Engine.from_dir(d, EngineOptions(dtype="bfloat16", max_tokens=512))
+    prompts = [tiny.tokens(cfg, n, 30 + n) for n in (1, 9, 40, 70)]
+    got = eng.generate(prompts, 24, temperature=0.8, seed=100, max_batch=3, max_step_tokens=32)
+    alone = [eng.generate(p, 24, temperature=0.8, seed=100 + i) for i, p in enumerate(prompts)]
+    w = tiny.read_weights(d, as_stored_in="bfloat16")
+    same = 0
+    for i, p in enumerate(prompts):
+        agree = next((k for k, (x, y) in enumerate(zip(got[i], alone[i])) if x != y), len(alone[i]))
+        same += agree
+        if agree < len(alone[i]):
+            row = P.forward(w, cfg, list(p) + got[i][:agree])[-1]
+            cdf = torch.cumsum(P.softmax_temperature(row, 0.8), 0)
+            a, b = sorted((got[i][agree], alone[i][agree]))
+            assert b == a + 1 or float(cdf[b - 1] - cdf[a]) < 2e-2, (i, agree, a, b)    # neighbours on the CDF
+            assert abs(float(cdf[a]) - uniform(100 + i, agree)) < 2e-2, (i, agree)
+    assert same >= 60, same
+
+
 def test_command_line_generate(model_dirs):
     """The command line in the reference's manner (cmd/generate/main.go:15-50)."""
     cfg, d = tiny.CONFIGS["R"], model_dirs("R")

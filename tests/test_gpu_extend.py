@@ -328,6 +328,44 @@ def test_layers_with_a_window_have_pages_of_their_own(dtype, model_dirs, tmp_pat
         unregister_architecture("ToyWindowForCausalLM")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_of_the_windowed_model_as_graphs(dtype):
+    """Two cache groups, one of them windowed (its tables lose pages at the back while the
+    other's grow): single-token steps of two requests queued as recorded HIP graphs give, bit
+    for bit, what the eager step gives, across a change of the growing table's width."""
+    import numpy as np
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry
+    register_architecture("ToyWindowForCausalLM", LlamaConfig, build_windowed)
+    try:
+        cfg = dict(tiny.CONFIGS["B"], architectures=["ToyWindowForCausalLM"])
+        reqs = {"a": tiny.tokens(cfg, 150, 1), "b": tiny.tokens(cfg, 97, 2)}
+        prompt = {"a": 110, "b": 60}
+        outs = {}
+        for mode in ("eager", "graph"):
+            eng = Engine.from_random(cfg, 3, EngineOptions(dtype=dtype, num_pages=24, max_model_len=1 << 20,
+                                                           poison_freed_pages=True), std=0.05, norm_std=0.1)
+            eng.step([StepEntry(r, reqs[r][:prompt[r]], []) for r in reqs])
+            got = []
+            for k in range(37):
+                entries = [StepEntry(r, [reqs[r][prompt[r] + k]], [0]) for r in reqs]
+                if mode == "eager":
+                    got.append(eng.step(entries).cpu().numpy().copy())
+                else:
+                    assert eng.can_sample_ahead(entries)
+                    h = eng.step_sample_ahead(entries, [0.0, 0.0], [0.0, 0.0])
+                    h.tokens()
+                    got.append(h.logits.cpu().numpy().copy())
+            if mode == "graph":
+                assert len(eng._graphs.recordings) >= 2          # request a's table grew from 7 to 10 pages
+                assert eng.cache.pools[0].used_pages <= 2 * 3     # the window's pages only
+            eng.cache.check_invariants()
+            outs[mode] = got
+        for k, (a, b) in enumerate(zip(outs["eager"], outs["graph"])):
+            assert np.isfinite(a).all() and np.array_equal(a, b), k
+    finally:
+        unregister_architecture("ToyWindowForCausalLM")
+
+
 def test_pools_are_sized_per_group_and_from_a_byte_budget():
     """A windowed group gets no more pages than its requests can hold; a byte budget
     shrinks every pool; page sizes no kernel takes and portions larger than the engine

@@ -139,3 +139,112 @@ def test_random_configurations_match_the_plain_implementation(tmp_path, dtype):
                 assert np.isfinite(got).all(), f"{case}: {rid} position {p}"
                 err = float(np.abs(got - want[p]).max())
                 assert err < bound, f"{case}: {rid} position {p} off by {err}"
+
+
+def _all_decode(step):
+    return bool(step["entries"]) and all(len(e["tokens"]) == 1 and list(e["want"]) == [0] for e in step["entries"])
+
+
+def replay_with_graphs(engine, steps):
+    """The trace through the engine with every all-decode step queued as a recorded HIP graph
+    (``step_sample_ahead``: forward pass and greedy sampling in one replay) and every other
+    step through ``step``.  Returns (logits per step, number of graph steps)."""
+    from kllm_amd.engine import StepEntry
+    outs, queued = [], 0
+    for s in steps:
+        entries = [StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]]
+        if _all_decode(s) and engine.can_sample_ahead(entries):
+            h = engine.step_sample_ahead(entries, [0.0] * len(entries), [0.0] * len(entries))
+            ids = h.tokens()
+            logits = h.logits.cpu().numpy().copy()
+            assert all(logits[i, ids[i]] == logits[i].max() for i in range(len(ids)))   # greedy, on the device
+            outs.append(logits)
+            queued += 1
+        elif entries:
+            out = engine.step(entries)
+            outs.append(None if out is None else out.cpu().numpy().copy())
+        else:
+            outs.append(None)
+        for rid in s["end"]:
+            if rid in engine.cache:
+                engine.release(rid)
+    return outs, queued
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_all_decode_stretches_of_random_traces_as_graphs(tmp_path, dtype):
+    """The same random traces (configurations A to E, pages of 4 to 64 tokens, contexts up to
+    2,300 tokens, one to four live requests whose number and table widths change from step to
+    step) with their all-decode steps replayed as HIP graphs: logits equal the eager step's
+    bit for bit, for every request at every step."""
+    from kllm_amd.engine import Engine, EngineOptions
+    from kllm_amd.replay import Replayer
+    folders, graph_steps, recordings, cases = {}, 0, 0, 0
+    for seed in range(48):
+        name, cfg, page, requests, family, steps, peak = draw(seed)
+        if family == "whole" or not any(_all_decode(s) for s in steps):
+            continue
+        case = f"seed {seed}: {name} pages of {page}, {family}, {[len(t) for t in requests.values()]}"
+        print(case, flush=True)
+        if name not in folders:
+            folders[name] = tiny.write_model(str(tmp_path / name), cfg, seed=len(folders))
+        pool = peak + page * min(4, len(requests))
+        options = EngineOptions(dtype=dtype, max_tokens=pool, max_model_len=1 << 30,
+                                poison_freed_pages=True, page_size=page)
+        eager = Replayer(folders[name], dtype, pool, options=options)
+        want = [eager.step(s["entries"], s["end"]) for s in steps]
+        eng = Engine.from_dir(folders[name], options)
+        got, queued = replay_with_graphs(eng, steps)
+        eng.cache.check_invariants()
+        assert not eng.cache.requests, case
+        for s, a, b in zip(steps, want, got):
+            assert (a is None) == (b is None), case
+            if a is not None:
+                assert np.array_equal(a, b), f"{case}: step {s['step']} differs between the eager step and its graph"
+        graph_steps += queued
+        recordings += len(eng._graphs.recordings)
+        cases += 1
+    assert cases >= 20 and graph_steps >= 400 and recordings >= 40, (cases, graph_steps, recordings)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_token_reference_in_flight_across_a_change_of_table_width(tmp_path, dtype):
+    """Decode steps queued one ahead, each fed by a TokenRef to the one before, while the
+    requests grow past a power of two of pages (another recording, with a wider table, takes
+    over with a reference in flight), at pages of 4 and of 64 tokens and at E's long contexts:
+    the tokens are those of the eager greedy loop, the logits of every step the eager step's,
+    bit for bit."""
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry, TokenRef
+    for name, page, lens, new in (("A", 4, [29, 30, 31], 12), ("B", 64, [500, 509, 511], 10), ("E", 16, [2040, 1000], 20)):
+        cfg = tiny.CONFIGS[name]
+        folder = tiny.write_model(str(tmp_path / f"{name}{page}"), cfg, seed=1)
+        prompts = [tiny.tokens(cfg, n, 90 + i) for i, n in enumerate(lens)]
+        B = len(prompts)
+        options = EngineOptions(dtype=dtype, max_tokens=sum(lens) + B * (new + 2 * page), max_model_len=1 << 30,
+                                page_size=page)
+        runs = {}
+        for mode in ("eager", "ahead"):
+            eng = Engine.from_dir(folder, options)
+            first = eng.step([StepEntry(i, p, [len(p) - 1]) for i, p in enumerate(prompts)])
+            ids = first.argmax(-1).tolist()
+            toks, logits, before = [list(ids)], [], None
+            for k in range(new):
+                if mode == "eager":
+                    out = eng.step([StepEntry(i, [t], [0]) for i, t in enumerate(ids)])
+                    logits.append(out.cpu().numpy().copy())
+                    ids = out.argmax(-1).tolist()
+                    toks.append(list(ids))
+                    continue
+                feed = ids if before is None else [TokenRef(before, i) for i in range(B)]
+                h = eng.step_sample_ahead([StepEntry(i, [t], [0]) for i, t in enumerate(feed)], [0.0] * B, [0.0] * B)
+                logits.append(h.logits.cpu().numpy().copy())     # read before the next step is queued
+                if before is not None:
+                    toks.append(before.tokens())
+                before = h
+            if mode == "ahead":
+                toks.append(before.tokens())
+                assert len(eng._graphs.recordings) >= 2, (name, page)      # the table's width changed on the way
+            runs[mode] = (toks, logits)
+        assert runs["eager"][0] == runs["ahead"][0], (name, page)
+        for k, (a, b) in enumerate(zip(runs["eager"][1], runs["ahead"][1])):
+            assert np.array_equal(a, b), (name, page, k)

@@ -257,3 +257,38 @@ def test_prompt_portions_of_512_tokens_beside_decode_tokens():
         s["step"] = i
     eng = engine(name, dtype, max_tokens=traces.peak_tokens(steps))
     print(f"{name} {dtype} 512-token portions beside decode tokens: logits", compare_both(name, dtype, run(eng, steps), reqs))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_scheduler_with_portions_of_512_tokens_beside_decode_tokens(dtype):
+    """The scheduler itself at these sizes (the reference's end-to-end check of its scheduler:
+    engine/scheduler.go:160-189, engine/e2e/e2e_test.go:256-312): five requests, two of them
+    with prompts of more than 512 tokens, submitted together under a budget of 512 prompt
+    tokens a step, so that portions of 512 run beside the decode tokens of the requests that
+    are already generating and steps end on whole tiles of rows.  Every generated token must
+    be the plain implementation's greedy choice given the tokens before it, or lie within
+    the tolerance of it (bfloat16 may part ways at a near-tie; what follows is then judged
+    from the engine's own tokens)."""
+    from kllm_amd.engine.scheduler import Scheduler
+    name, new = "tinyllama", 12
+    cfg = SIZES[name]
+    prompts = [tiny.tokens(cfg, n, 400 + i) for i, n in enumerate([1100, 60, 700, 45, 300])]
+    eng = engine(name, dtype, max_tokens=sum(len(p) + new + 16 for p in prompts), max_requests=8)
+    sched = Scheduler(eng, max_batch=5, max_step_tokens=512 + 5, chunk_size=512)
+    ids = [sched.submit(p, new) for p in prompts]
+    results = sched.run_until_done()
+    assert sched.stats["steps"] >= 6 and sched.stats["preemptions"] == 0
+    assert not eng.cache.requests
+    eng.cache.check_invariants()
+    w = plain_weights(name, dtype)
+    tol = tiny.TOL_SIZES[dtype]
+    ties = 0
+    for i, p in zip(ids, prompts):
+        assert results[i].error is None and len(results[i].tokens) == new
+        logits = P.forward(w, cfg, list(p) + results[i].tokens[:-1])[len(p) - 1:]
+        for k, tok in enumerate(results[i].tokens):
+            best = int(logits[k].argmax())
+            if tok != best:
+                ties += 1
+                assert float(logits[k][best] - logits[k][tok]) < 2 * tol, (i, k, tok, best)
+    assert ties <= (0 if dtype == "float32" else 6), ties

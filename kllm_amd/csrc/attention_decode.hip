@@ -444,8 +444,7 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
 #undef KLLM_DEC
   KLLM_CHECK_LAUNCH(who);
   if (nslices == 1) return 0;                      // the one workgroup of a token has written the output
-  hipLaunchKernelGGL(attn_merge_kernel<bf16_t>, dim3(count, H), dim3(64), 0, stream, (bf16_t*)out, part,
-                     H, hd, nslices, token_list);
+  launch_attn_merge<bf16_t>((bf16_t*)out, part, count, H, hd, nslices, token_list, stream);
   KLLM_CHECK_LAUNCH("attn_merge");
   return 0;
 }

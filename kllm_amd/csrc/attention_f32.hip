@@ -443,8 +443,7 @@ int attn_f32_decode(const float* q, float* out, float* part, const float* cache,
   if (int rc = dispatch_f32<true>(a, items, stream)) return rc;
   KLLM_CHECK_LAUNCH("attn_decode float32");
   if (nslices > 1) {
-    hipLaunchKernelGGL(attn_merge_kernel<float>, dim3(count, H), dim3(64), 0, stream, out, part, H, hd,
-                       a.wg_merge ? nslices / kF32Waves : nslices, token_list);
+    launch_attn_merge<float>(out, part, count, H, hd, a.wg_merge ? nslices / kF32Waves : nslices, token_list, stream);
     KLLM_CHECK_LAUNCH("attn_merge float32");
   }
   return 0;

@@ -224,11 +224,33 @@ __global__ void rope_append_kernel(const TIN* __restrict__ qkv, int nsplit, long
   }
 }
 
-// The same for whole float32 sums (one split) and head sizes that are multiples of 8: a
-// thread takes four neighbouring pairs, or four values, with 16-byte loads, and its loads go
-// out before the token's page is looked up, so that the two waits overlap.
+// Four neighbouring sums of the splits at once, added in the order of sum_splits.
+__device__ __forceinline__ floatx4 sum_splits4(const float* __restrict__ p, int nsplit, long stride) {
+  floatx4 v = {0.f, 0.f, 0.f, 0.f};
+  int s = 0;
+  for (; s + 8 <= nsplit; s += 8) {
+    floatx4 t[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t[j] = *reinterpret_cast<const floatx4*>(p + (long)(s + j) * stride);
+    v += ((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]));
+  }
+  if (s + 4 <= nsplit) {
+    floatx4 t[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t[j] = *reinterpret_cast<const floatx4*>(p + (long)(s + j) * stride);
+    v += (t[0] + t[1]) + (t[2] + t[3]);
+    s += 4;
+  }
+  for (; s < nsplit; ++s) v += *reinterpret_cast<const floatx4*>(p + (long)s * stride);
+  return v;
+}
+
+// The same for float32 sums (whole, or partial sums over slices of K) and head sizes that are
+// multiples of 8: a thread takes four neighbouring pairs, or four values, with 16-byte loads,
+// and its loads go out before the token's page is looked up, so that the two waits overlap.
 template <typename T>
-__global__ void rope_append_vec_kernel(const float* __restrict__ qkv, T* __restrict__ q_out,
+__global__ void rope_append_vec_kernel(const float* __restrict__ qkv, int nsplit, long split_stride,
+                                       T* __restrict__ q_out,
                                        const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                        T* __restrict__ cache, const int* __restrict__ positions,
                                        const int* __restrict__ span_of_token,
@@ -252,8 +274,8 @@ __global__ void rope_append_vec_kernel(const float* __restrict__ qkv, T* __restr
     h = idx / half;
     j = idx % half;
     const float* src = in + (is_q ? 0 : qd) + h * hd + j;
-    a = *reinterpret_cast<const floatx4*>(src);
-    b = *reinterpret_cast<const floatx4*>(src + half);
+    a = sum_splits4(src, nsplit, split_stride);
+    b = sum_splits4(src + half, nsplit, split_stride);
     if (cos_t) {
       cc = *reinterpret_cast<const floatx4*>(cos_t + t * half + j);
       sn = *reinterpret_cast<const floatx4*>(sin_t + t * half + j);
@@ -262,7 +284,7 @@ __global__ void rope_append_vec_kernel(const float* __restrict__ qkv, T* __restr
     const int idx = (item - q_items - k_items) * 4;
     h = idx / hd;
     j = idx % hd;
-    a = *reinterpret_cast<const floatx4*>(in + qd + kvd + idx);
+    a = sum_splits4(in + qd + kvd + idx, nsplit, split_stride);
   }
   int page = 0, slot = 0;
   if (cache && !is_q) {
@@ -416,11 +438,12 @@ static int launch_rope_append(const void* qkv, int nsplit, long split_stride, vo
   const int items = H * (hd / 2) + (cache ? KV * (hd / 2) + KV * hd : 0);
   int chunks = ceil_div(items, kThreads);
   if ((long)n * chunks > 16384) chunks = ceil_div(16384, n);   // many tokens: fewer, longer workgroups
-  if (rot == hd && !interleaved && sizeof(TIN) == 4 && nsplit == 1 && hd % 8 == 0 && ((uintptr_t)qkv & 15) == 0 &&
+  if (rot == hd && !interleaved && sizeof(TIN) == 4 && hd % 8 == 0 && ((uintptr_t)qkv & 15) == 0 &&
+      (nsplit == 1 || split_stride % 4 == 0) && (H * hd + (cache ? 2 * KV * hd : 0)) % 4 == 0 &&
       ((uintptr_t)q_out & 15) == 0 && (!cache || ((uintptr_t)cache & 15) == 0) &&
       (!cos_t || (((uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0)) {
     hipLaunchKernelGGL((rope_append_vec_kernel<T>), dim3(n, ceil_div(items, 4 * kThreads)), dim3(kThreads), 0,
-                       stream, (const float*)qkv, (T*)q_out, cos_t, sin_t, (T*)cache, positions, span_of_token,
+                       stream, (const float*)qkv, nsplit, split_stride, (T*)q_out, cos_t, sin_t, (T*)cache, positions, span_of_token,
                        block_table, max_pages, page_size, H, KV, hd);
     KLLM_CHECK_LAUNCH("rope_append");
     return 0;

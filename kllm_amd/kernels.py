@@ -20,7 +20,7 @@ import torch
 
 DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
-GEMV_BEST_ROWS = 2         # up to here they beat the MFMA kernels in bfloat16 (3 rows: 1.29 against 1.21 ms a step at 1.1B sizes)
+GEMV_BEST_ROWS = 1         # up to here they beat the MFMA kernels in bfloat16 (a step at 1.1B sizes, one token: 1.047 against 1.061 ms; two: 1.123 against 1.063)
 ABI_VERSION = 7
 
 

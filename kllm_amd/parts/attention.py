@@ -128,7 +128,7 @@ class CausalSelfAttention(Part):
             n = xn.rows
             opts = self.runtime.options
             gemv = (K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype) and n <= K.normed_max_rows()
-                    and not opts.get("no_fused_gemv") and self.plain_rotation)
+                    and not opts.get("no_fused_gemv") and self.plain_rotation and xn.xw is None)
             scaled = (not gemv and xn.xw is not None and dtype == torch.bfloat16 and n <= K.FUSED_ROPE_BEST_ROWS
                       and K.fused_linear_fits(n, self.hidden) and not opts.get("no_fused_linear")
                       and self.plain_rotation)
@@ -146,7 +146,8 @@ class CausalSelfAttention(Part):
         plain_rotation = self.plain_rotation
         pages = cache.pages if writes else None
         opts = self.runtime.options
-        if K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype) and not opts.get("no_fused_gemv") and plain_rotation:
+        if (K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype) and not opts.get("no_fused_gemv") and plain_rotation
+                and not isinstance(xn, K.ScaledRows)):
             # few tokens: projections, rotation and append in one launch
             K.gemv_rope_append(xn, self.w_in, q, cos, sin, pages, ctx.positions, ctx.span_of_token,
                                cache.block_table, cache.page_size, self.heads, self.kv_heads,

@@ -60,6 +60,8 @@ class GatedFeedForward(Part):
         dtype, opts = self.runtime.dtype, self.runtime.options
         n = xn.rows if isinstance(xn, Normed) else xn.shape[0]
         gemv = K.gemv_fits(n, 2 * self.intermediate, self.hidden, dtype) and not opts.get("no_fused_gemv")
+        if gemv and isinstance(xn, Normed) and xn.xw is not None:
+            gemv = False       # the producer was the decode-batch kernel: its consumer is, too
         fused = (not gemv and dtype == torch.bfloat16 and n <= K.FUSED_SWIGLU_BEST_ROWS
                  and K.fused_linear_fits(n, self.hidden) and not opts.get("no_fused_linear"))
         if isinstance(xn, Normed):     # the small-batch kernel below normalises while it stages its input,

@@ -48,7 +48,10 @@ namespace kllm {
 // and 6.7 us for 2,048 x 2,048 weights at 8 rows; 4 ahead: 1,660 and 6.0 us; more waves to a
 // workgroup or more of X in registers measured slower for the same reason).
 constexpr int FL_AHEAD = 4;
-constexpr int XB = 8;              // 16-byte loads of X per lane that are in flight together
+// 16-byte loads of X per lane that are in flight together.  More than eight rows of K = 2,048
+// need a second batch, which waits for the first; sixteen in flight avoid that and still lose
+// to their registers (a step of 9 to 16 tokens at 1.1B sizes 1 to 4 % slower, of 8 tokens 8 %).
+constexpr int XB = 8;
 // LDS row padding (elements): zeros behind K as far as the waves' slices reach beyond it
 // (less than 32 per wave), 8 to shift banks
 constexpr int fl_pad(int nw) { return 32 * nw + 8; }
@@ -75,6 +78,7 @@ struct FlOut {
   const float* ss_in;           // SCALED: [n][ss_parts rounded up to 4], what a FL_RESID product left
   int ss_parts;
   float eps;
+  int tiled;                    // W is the copy that fl_tile_kernel made for this epilogue (see there)
 };
 
 // Row of W behind MFMA row c of a tile, or -1.  Pair epilogues: unit = pair.
@@ -224,10 +228,20 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
   // steps are padded to whole turns of both buffers.  A row, a tile or a K that does not exist
   // reads the first K of a row that does (finite numbers): the X beside it in LDS is zero, or
   // the output row is ignored.
+  // With a tiled copy of W (out.tiled) a tile's step is 1 KB in the order the lanes want it:
+  // a load instruction reads one contiguous kilobyte instead of 64 bytes of each of 16 rows
+  // (streamed alone, 2,048 x 5,632 weights: 8.5 -> 6.7 us; 11,264 x 2,048: 12.0 -> 9.9).
   const bf16_t* far_row;                                    // first K of this lane's row of W
   int far_lane_off;                                         // this lane's offset in it, or -1: no such row
+  const int far_stride = out.tiled ? 512 : 32;              // elements from a step to the next
   int far_tile = 0, far_s0 = 0;                             // the steps that are loaded next
   auto tile_ptr = [&](int t) {
+    if (out.tiled) {     // rows that do not exist hold zeros there; a tile that does not exist reads the first
+      const long tl = t < my_tiles ? tile0 + t : tile0;
+      far_row = W + ((tl * ((k + 31) / 32) + kbeg / 32) * kWave + lane) * 8;
+      far_lane_off = (wk0 / 32) * 512;
+      return;
+    }
     const long r = t < my_tiles ? fl_row<EP>((int)tile0 + t, c, m, out) : -1;
     far_row = W + (r >= 0 ? r : 0) * k + kbeg;
     far_lane_off = r >= 0 ? wk0 + 8 * g : -1;
@@ -237,7 +251,7 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
     for (int i = 0; i < FL_AHEAD; ++i) {
       const int s = far_s0 + i;
       const bool valid = far_lane_off >= 0 && s < steps && 32 * s + 8 * g < wlen;
-      buf[i] = *reinterpret_cast<const bf16x8*>(far_row + (valid ? far_lane_off + 32 * s : 0));
+      buf[i] = *reinterpret_cast<const bf16x8*>(far_row + (valid ? far_lane_off + far_stride * s : 0));
     }
     far_s0 += FL_AHEAD;
     if (far_s0 == rsteps) {
@@ -432,6 +446,22 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
   }
 }
 
+// The tiled copy of W for an epilogue: [tile][step of 32 of K][lane][8 elements], lane (g, c)
+// holding W[row of MFMA row c][32 step + 8 g ...], zeros where the row or the K is not there.
+// One workgroup of 64 lanes per (tile, step).
+template <int EP>
+__global__ __launch_bounds__(64) void fl_tile_kernel(const bf16_t* __restrict__ W, bf16_t* __restrict__ Wt, FlOut out,
+                                                     int m, int k) {
+  const int lane = threadIdx.x, g = lane / 16, c = lane % 16;
+  const int step = blockIdx.y, ksteps = gridDim.y;
+  const long tile = blockIdx.x;
+  const long r = fl_row<EP>((int)tile, c, m, out);
+  const int kk = 32 * step + 8 * g;
+  bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (r >= 0 && kk < k) v = *reinterpret_cast<const bf16x8*>(W + r * k + kk);      // k is a multiple of 8
+  *reinterpret_cast<bf16x8*>(Wt + ((tile * ksteps + step) * kWave + lane) * 8) = v;
+}
+
 static size_t fl_lds_bytes(int n, int nt, int kslice, int nw = 4) {
   return (size_t)n * (kslice + fl_pad(nw)) * sizeof(bf16_t) + (size_t)(2 * nw * nt * FL_TILE + 32) * sizeof(float);
 }
@@ -487,6 +517,40 @@ extern "C" int kllm_fused_linear_resid_parts(int m, int tiles_per_wg) {
 
 extern "C" int kllm_fused_linear_max_parts(void) { return FL_SS_MAX; }
 
+static int fl_tiles(int kind, int m) { return kind == FL_SWIGLU || kind == FL_ROPE ? ceil_div(m / 2, 8) : ceil_div(m, 16); }
+
+extern "C" long kllm_fused_linear_tiled_elements(int kind, int m, int k) {
+  if (m <= 0 || k <= 0 || k % 8) return -1;
+  return (long)fl_tiles(kind, m) * ceil_div(k, 32) * 512;
+}
+
+extern "C" int kllm_fused_linear_tile(const void* w, void* wt, int kind, int m, int k, int H, int KV, int hd,
+                                      int with_kv, hipStream_t stream) {
+  KLLM_REQUIRE(w && wt && fl_aligned16(w) && fl_aligned16(wt), "fused_linear_tile: null or unaligned pointer");
+  KLLM_REQUIRE(m > 0 && k > 0 && k % 8 == 0 && m < (1 << 30), "fused_linear_tile: bad sizes m=%d k=%d", m, k);
+  KLLM_REQUIRE(kind == FL_PARTS || kind == FL_RESID || kind == FL_SWIGLU || kind == FL_ROPE,
+               "fused_linear_tile: unknown output kind %d", kind);
+  FlOut out = {};
+  if (kind == FL_SWIGLU || kind == FL_ROPE) KLLM_REQUIRE(m % 2 == 0, "fused_linear_tile: m=%d must be even for a pair epilogue", m);
+  if (kind == FL_ROPE) {
+    KLLM_REQUIRE(H > 0 && hd > 0 && hd % 2 == 0 && (!with_kv || KV > 0) && m == H * hd + (with_kv ? 2 * KV * hd : 0),
+                 "fused_linear_tile: m=%d does not fit H=%d KV=%d hd=%d", m, H, KV, hd);
+    out.H = H;
+    out.KV = KV;
+    out.hd = hd;
+    out.cache = with_kv ? const_cast<void*>(w) : nullptr;     // only "is there a cache" is read
+  }
+  const dim3 grid(fl_tiles(kind, m), ceil_div(k, 32));
+  KLLM_REQUIRE(grid.y <= 65535u, "fused_linear_tile: K=%d is too long", k);
+  const bf16_t* wp = (const bf16_t*)w;
+  bf16_t* tp = (bf16_t*)wt;
+  if (kind == FL_SWIGLU) hipLaunchKernelGGL(fl_tile_kernel<FL_SWIGLU>, grid, dim3(64), 0, stream, wp, tp, out, m, k);
+  else if (kind == FL_ROPE) hipLaunchKernelGGL(fl_tile_kernel<FL_ROPE>, grid, dim3(64), 0, stream, wp, tp, out, m, k);
+  else hipLaunchKernelGGL(fl_tile_kernel<FL_PARTS>, grid, dim3(64), 0, stream, wp, tp, out, m, k);
+  KLLM_CHECK_LAUNCH("fused_linear_tile");
+  return 0;
+}
+
 extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOut* yout, const void* w,
                                  int n, int m, int k, int tiles_per_wg, hipStream_t stream) {
   KLLM_REQUIRE(x && yout && w && yout->y, "fused_linear: null pointer");
@@ -514,6 +578,7 @@ extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOu
   FlOut out = {};
   out.y = yout->y;
   out.act = yout->act;
+  out.tiled = yout->tiled ? 1 : 0;
   KLLM_REQUIRE(ep != FL_SWIGLU || (out.act >= 0 && out.act < ACT_COUNT), "fused_linear: unknown activation %d", out.act);
   int tiles = ceil_div(m, 16);
   const bool scaled = yout->ss_in != nullptr;

@@ -180,8 +180,17 @@ typedef struct {
   const float* ss_in;   /* row scale of the sums, or null; 16-byte aligned */
   int ss_parts;
   float eps;
+  int tiled;            /* w is the copy that kllm_fused_linear_tile made of the weights for this kind */
 } KllmLinearOut;
 long kllm_fused_linear_lds_bytes(int n, int k, int nsplit);
+/* A copy of w[m][k] in the order the kernel's lanes read it (a load instruction then reads one
+ * contiguous kilobyte instead of 64 bytes of each of 16 rows: weights stream 20-30 % faster),
+ * for one output kind (PARTS and RESID share theirs; ROPE with the heads it will be called
+ * with, with_kv: whether k and v rows follow q's): wt holds
+ * kllm_fused_linear_tiled_elements(kind, m, k) elements.  Pass it as w with out->tiled = 1. */
+long kllm_fused_linear_tiled_elements(int kind, int m, int k);
+int kllm_fused_linear_tile(const void* w, void* wt, int kind, int m, int k, int H, int KV, int hd, int with_kv,
+                           hipStream_t stream);
 int kllm_fused_linear_resid_parts(int m, int tiles_per_wg);
 int kllm_fused_linear_max_parts(void);
 int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOut* out, const void* w, int n, int m,

@@ -106,6 +106,7 @@ def _declare(lib):
         "kllm_gemv_resid_parts": [I],
         "kllm_fused_linear": [P, I, P, P, I, I, I, I, P],
         "kllm_fused_linear_resid_parts": [I, I],
+        "kllm_fused_linear_tile": [P, P, I, I, I, I, I, I, I, P],
         "kllm_command_op": [c_char_p],
         "kllm_command_nargs": [I],
         "kllm_run_commands": [P, L, P, P],
@@ -133,6 +134,8 @@ def _declare(lib):
         fn.restype = c_int
     lib.kllm_fused_linear_lds_bytes.argtypes = [I, I, I]
     lib.kllm_fused_linear_lds_bytes.restype = L
+    lib.kllm_fused_linear_tiled_elements.argtypes = [I, I, I]
+    lib.kllm_fused_linear_tiled_elements.restype = L
 
 
 # Entry points that launch work on a stream (and can be recorded into a command buffer), and
@@ -708,7 +711,7 @@ class _LinearOut(ctypes.Structure):
                 ("kind", c_int), ("nsplit", c_int), ("max_pages", c_int), ("page_size", c_int),
                 ("H", c_int), ("KV", c_int), ("hd", c_int), ("act", c_int),
                 ("resid", c_void_p), ("norm_w", c_void_p), ("ss_out", c_void_p), ("ss_in", c_void_p),
-                ("ss_parts", c_int), ("eps", c_float)]
+                ("ss_parts", c_int), ("eps", c_float), ("tiled", c_int)]
 
 
 FUSED_LINEAR_MAX_ROWS = 32
@@ -718,18 +721,26 @@ LINEAR_PARTS, LINEAR_RESID, LINEAR_SWIGLU, LINEAR_ROPE = 0, 1, 2, 3
 
 # Rows up to which the decode-batch kernel beats the split-K kernel plus a separate
 # elementwise launch (measured at widths 2048 -> 2560 and 2048 -> 11264).
+# (17 to 32 rows, where the output projection's rows still fit: 1.55 -> 1.58 ms a step at 17 tokens, 1.73 -> 1.79 at 32)
 FUSED_NORM_BEST_ROWS = 16      # rows up to which a residual product and a consumer that scales its rows replace the norm kernel
 FUSED_ROPE_BEST_ROWS = 32      # (17 tokens at 1.1B sizes: 1.59 -> 1.55 ms a step against the tiled product and a rotation kernel)
 FUSED_SWIGLU_BEST_ROWS = 16
 
 
+@functools.lru_cache(maxsize=4096)
 def fused_tiles_per_wg(n, m, k) -> int:
     """Tiles of 16 rows of W that one workgroup of the decode-batch kernel takes, one after
-    the other, with the rows of X staged once: two from 9 rows of X on against large weights
+    the other, with the rows of X staged once: from 9 rows of X on against large weights two
     (16 rows, 4,096 -> 2 x 14,336 with the gate: 58.8 us against 66.1; 4,096 -> 6,144 with the
-    rotation: 18.1 against 22.4), one otherwise (2,048 -> 2 x 5,632: 15.6 either way at 16
-    rows, 13.5 against 14.6 at 10)."""
-    return 2 if n > 8 and m * k >= 20_000_000 else 1
+    rotation: 18.1 against 22.4), or up to four if that brings the workgroups down to one
+    round of the chip (2,048 -> 2 x 5,632, 704 tiles: a step of 9 / 12 / 16 tokens at 1.1B sizes
+    1.271 / 1.297 / 1.379 ms with two, 1.254 / 1.272 / 1.353 with three), one otherwise."""
+    if n <= 8 or m * k < 20_000_000:
+        return 1
+    tiles, t = -(-m // 16), 2
+    while t < 4 and -(-tiles // t) > device_cus():
+        t += 1
+    return t
 
 
 @functools.lru_cache(maxsize=4096)
@@ -739,6 +750,37 @@ def fused_linear_fits(n, k, nsplit=1) -> bool:
     if n < 1 or n > FUSED_LINEAR_MAX_ROWS or k % 8:
         return False
     return 0 < library().kllm_fused_linear_lds_bytes(int(n), int(k), int(nsplit)) <= FUSED_LINEAR_LDS
+
+
+class TiledWeights:
+    """A copy of a weight matrix [m, k] in the order the decode-batch kernel's lanes read it, for
+    one output kind (LINEAR_PARTS serves LINEAR_RESID too; LINEAR_ROPE is made for the heads it
+    will be called with).  ``fused_linear`` takes it in place of the matrix."""
+
+    def __init__(self, data, kind, m, k, heads=None):
+        self.data, self.kind, self.shape, self.heads = data, kind, (m, k), heads
+        self.dtype = data.dtype
+
+
+def fused_linear_tile(w, kind, rope=None):
+    """The tiled copy of ``w`` [m, k] (bfloat16, k a multiple of 8) for ``kind``; ``rope`` as
+    for ``fused_linear`` (its heads and whether a cache is written decide the rows' order)."""
+    m, k = w.shape
+    if w.dtype != torch.bfloat16 or k % 8:
+        raise KernelError("fused_linear_tile: bfloat16 weights with K a multiple of 8 only")
+    base = LINEAR_PARTS if kind == LINEAR_RESID else kind
+    count = library().kllm_fused_linear_tiled_elements(base, m, k)
+    if count <= 0:
+        raise KernelError(f"fused_linear_tile: sizes {m} x {k} are not taken")
+    out = torch.empty(count, dtype=torch.bfloat16, device=w.device)
+    heads = (0, 0, 0, 0)
+    if base == LINEAR_ROPE:
+        if rope is None:
+            raise KernelError("fused_linear_tile: the rope kind needs its heads")
+        heads = (rope.heads, rope.kv_heads, rope.head_dim, int(rope.cache is not None))
+    _check(library().kllm_fused_linear_tile(_ptr(w, "tile w"), _ptr(out, "tile out"), base, m, k, *heads, _stream()),
+           "fused_linear_tile")
+    return TiledWeights(out, base, m, k, heads)
 
 
 class ScaledRows:
@@ -789,6 +831,13 @@ def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None, act=ACT_SIL
     lo = _LinearOut()
     if w.dtype != torch.bfloat16:
         raise KernelError("fused_linear: bfloat16 weights only")
+    if isinstance(w, TiledWeights):
+        if w.kind != (LINEAR_PARTS if kind == LINEAR_RESID else kind):
+            raise KernelError(f"fused_linear: the tiled weights were made for output kind {w.kind}, not {kind}")
+        if kind == LINEAR_ROPE and (rope is None or w.heads != (rope.heads, rope.kv_heads, rope.head_dim,
+                                                                 int(rope.cache is not None))):
+            raise KernelError("fused_linear: the tiled weights were made for other heads")
+        lo.tiled, w = 1, w.data
     if isinstance(x, ScaledRows):
         sr, x = x, x.xw
         stride = -(-sr.parts // 4) * 4

@@ -21,7 +21,7 @@ import torch
 
 from .. import kernels as K
 from .base import Normed, Part, register_part
-from .linear import linear, linear_into
+from .linear import linear, linear_into, tiled_copy
 from .spec import CacheNeed, WeightSpec
 
 
@@ -93,6 +93,7 @@ class CausalSelfAttention(Part):
         self.kv_dim = self.kv_heads * self.head_dim
         self.w_in = None
         self.w_o = None
+        self._tiled = {}
 
     def weight_specs(self):
         specs = [WeightSpec(self.tensor_name("q_proj.weight"), (self.q_dim, self.hidden))]
@@ -107,6 +108,14 @@ class CausalSelfAttention(Part):
         mats = [weights[self.tensor_name(n)] for n in names]
         self.w_in = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0]
         self.w_o = weights[self.tensor_name("o_proj.weight")]
+        # second copies for decode batches, in the order that kernel reads them (not tensors of
+        # the part in the sense of read_bytes: a step reads one copy or the other)
+        self._tiled = {}
+        if self.plain_rotation:
+            heads = K.Rope(None, None, True if self.own_kv else None, None, None, None, 0, self.heads, self.kv_heads,
+                           self.head_dim)
+            self._tiled["in"] = tiled_copy(self.runtime, self.w_in, K.LINEAR_ROPE, heads)
+        self._tiled["o"] = tiled_copy(self.runtime, self.w_o, K.LINEAR_PARTS)
 
     def cache_need(self):
         return CacheNeed("paged", kv_heads=self.kv_heads, head_dim=self.head_dim, window=self.window)
@@ -155,7 +164,7 @@ class CausalSelfAttention(Part):
         elif (dtype == torch.bfloat16 and n <= K.FUSED_ROPE_BEST_ROWS and K.fused_linear_fits(n, self.hidden)
               and not opts.get("no_fused_linear") and plain_rotation):
             # a decode batch: the same on the matrix cores
-            K.fused_linear(self.w_in, q, K.LINEAR_ROPE, x=xn,
+            K.fused_linear(self._tiled.get("in") or self.w_in, q, K.LINEAR_ROPE, x=xn,
                            tiles_per_wg=K.fused_tiles_per_wg(n, self.w_in.shape[0], self.hidden),
                            rope=K.Rope(cos, sin, pages, ctx.positions, ctx.span_of_token, cache.block_table,
                                        cache.page_size, self.heads, self.kv_heads, self.head_dim))
@@ -167,7 +176,7 @@ class CausalSelfAttention(Part):
         out = ctx.buf("attn.out", (n, self.q_dim), dtype)
         self.attend(ctx, q, out, cache)
         if sink is not None:
-            normed = linear_into(ctx, out, self.w_o, sink, "attn.proj")
+            normed = linear_into(ctx, out, self.w_o, sink, "attn.proj", w_tiled=self._tiled.get("o"))
             if normed is not None:
                 return normed
         return linear(ctx, out, self.w_o, "attn.proj")

@@ -13,7 +13,7 @@ import torch
 
 from .. import kernels as K
 from .base import Part, register_part
-from .linear import linear
+from .linear import linear, tiled_copy
 from .spec import WeightSpec
 
 
@@ -65,6 +65,7 @@ class LinearHead(Part):
 
     def bind(self, weights):
         self.weight = weights[self.tensor_name("weight")]
+        self._tiled = {"w": tiled_copy(self.runtime, self.weight, K.LINEAR_PARTS)}   # for decode batches
 
     def forward(self, ctx, xn_rows):
-        return linear(ctx, xn_rows, self.weight, "logits", split=False)
+        return linear(ctx, xn_rows, self.weight, "logits", split=False, w_tiled=self._tiled.get("w"))

@@ -13,7 +13,7 @@ import torch
 
 from .. import kernels as K
 from .base import Normed, Part, register_part
-from .linear import linear, linear_into
+from .linear import linear, linear_into, tiled_copy
 from .spec import WeightSpec
 
 
@@ -34,6 +34,7 @@ class GatedFeedForward(Part):
         self.act = K.ACTIVATIONS[act]
         self.w_gu = None
         self.w_down = None
+        self._tiled = {}
 
     def weight_specs(self):
         return [WeightSpec(self.tensor_name("gate_proj.weight"), (self.intermediate, self.hidden)),
@@ -44,6 +45,9 @@ class GatedFeedForward(Part):
         self.w_gu = torch.cat([weights[self.tensor_name("gate_proj.weight")],
                                weights[self.tensor_name("up_proj.weight")]], dim=0).contiguous()
         self.w_down = weights[self.tensor_name("down_proj.weight")]
+        # second copies for decode batches, in the order that kernel reads them
+        self._tiled = {"gu": tiled_copy(self.runtime, self.w_gu, K.LINEAR_SWIGLU),
+                       "down": tiled_copy(self.runtime, self.w_down, K.LINEAR_PARTS)}
 
     def _gate_in_tiles(self, n, dtype):
         """Decode batches whose gate runs in the tiled product's epilogue: more than 32 rows
@@ -73,7 +77,7 @@ class GatedFeedForward(Part):
             K.gemv_swiglu(xn, self.w_gu, h, self.act)   # few tokens: both products and the gate in one launch
         elif fused:
             # a decode batch: the same on the matrix cores
-            K.fused_linear(self.w_gu, h, K.LINEAR_SWIGLU, x=xn, act=self.act,
+            K.fused_linear(self._tiled.get("gu") or self.w_gu, h, K.LINEAR_SWIGLU, x=xn, act=self.act,
                            tiles_per_wg=K.fused_tiles_per_wg(n, 2 * self.intermediate, self.hidden))
         elif ((n > 128 or self._gate_in_tiles(n, dtype))
               and self.runtime.options.get("gemm") != "library"
@@ -86,7 +90,7 @@ class GatedFeedForward(Part):
             gu = linear(ctx, xn, self.w_gu, "ffn.gu")
             K.silu_mul(gu, h, self.act)
         if sink is not None:
-            normed = linear_into(ctx, h, self.w_down, sink, "ffn.down")
+            normed = linear_into(ctx, h, self.w_down, sink, "ffn.down", w_tiled=self._tiled.get("down"))
             if normed is not None:
                 return normed
         return linear(ctx, h, self.w_down, "ffn.down")

@@ -611,6 +611,80 @@ def test_fused_linear_resid_then_scaled_consumers(n, m, k, tpw):
         assert (q.cpu().double() - want_q).abs().max() < 0.01 * want_q.abs().max() + 2e-3
 
 
+@pytest.mark.parametrize("n,m,k,tpw", [(1, 48, 64, 1), (8, 2048, 2048, 1), (5, 100, 264, 3), (19, 34, 3080, 2),
+                                       (8, 2048, 5632, 1), (16, 520, 1000, 4)])
+def test_fused_linear_with_tiled_weights_gives_the_same_bits(n, m, k, tpw):
+    """The copy of the weights in the order the kernel's lanes read them changes addresses
+    only: every output kind gives, bit for bit, what the row-major weights give (K no
+    multiple of 32, rows no multiple of 16, several tiles to a workgroup, K in slices)."""
+    k_ = K()
+    x, w = _bf(n, k, seed=1, scale=0.5), _bf(m, k, seed=2, scale=0.1)
+    tiled = k_.fused_linear_tile(w, k_.LINEAR_PARTS)
+    for nsplit in (1, 2):
+        if not k_.fused_linear_fits(n, k, nsplit):
+            continue
+        a = torch.full((nsplit, n, m), float("nan"), device=DEV)
+        b = torch.full((nsplit, n, m), float("nan"), device=DEV)
+        k_.fused_linear(w, a, k_.LINEAR_PARTS, x, nsplit=nsplit, tiles_per_wg=tpw)
+        k_.fused_linear(tiled, b, k_.LINEAR_PARTS, x, nsplit=nsplit, tiles_per_wg=tpw)
+        assert torch.isfinite(a).all() and torch.equal(a, b), nsplit
+    if not k_.fused_linear_fits(n, k):
+        return
+    # residual epilogue: the same tiled copy
+    nw = 1 + 0.2 * rnd(m, seed=4)
+    parts = k_.fused_resid_parts(n, m, k, tpw)
+    outs = []
+    for wt in (w, tiled):
+        stream = rnd(n, m, seed=3, scale=2.0)
+        ss = torch.full((n, -(-parts // 4) * 4), float("nan"), device=DEV)
+        xw = torch.full((n, m), float("nan"), dtype=torch.bfloat16, device=DEV)
+        k_.fused_linear(wt, xw, k_.LINEAR_RESID, x, tiles_per_wg=tpw, resid=stream, norm_weight=nw, ss_out=ss)
+        outs.append((stream, xw, ss[:, :parts].clone()))
+    for a, b in zip(*outs):
+        assert torch.isfinite(a.float()).all() and torch.equal(a, b)
+    if m % 2 == 0:
+        # gate: rows (p, f + p) meet in a tile
+        f = m // 2
+        h1 = torch.full((n, f), float("nan"), dtype=torch.bfloat16, device=DEV)
+        h2 = torch.full_like(h1, float("nan"))
+        k_.fused_linear(w, h1, k_.LINEAR_SWIGLU, x, tiles_per_wg=tpw)
+        k_.fused_linear(k_.fused_linear_tile(w, k_.LINEAR_SWIGLU), h2, k_.LINEAR_SWIGLU, x, tiles_per_wg=tpw)
+        assert torch.isfinite(h1.float()).all() and torch.equal(h1, h2)
+    with pytest.raises(k_.KernelError, match="made for output kind"):
+        k_.fused_linear(tiled, torch.empty(n, m // 2, dtype=torch.bfloat16, device=DEV), k_.LINEAR_SWIGLU, x)
+
+
+@pytest.mark.parametrize("H,KV,hd,ps,d", [(4, 2, 16, 16, 64), (3, 1, 32, 16, 96), (32, 4, 64, 16, 2048), (3, 3, 80, 16, 104)])
+def test_fused_linear_rope_append_with_tiled_weights(H, KV, hd, ps, d):
+    """Projections, rotation and append from the tiled copy of [q; k; v] (rows j and j + hd/2
+    of a head meet in a tile): the same bits in q_out and in the pages as from the row-major
+    weights; a copy made for other heads is refused."""
+    k_ = K()
+    spans = [(37, 3), (0, 2), (ps - 1, 1), (5, 5)]
+    n = sum(l for _, l in spans)
+    pos = torch.tensor([p0 + i for p0, l in spans for i in range(l)], dtype=torch.int32, device=DEV)
+    sot = torch.tensor([s for s, (_, l) in enumerate(spans) for _ in range(l)], dtype=torch.int32, device=DEV)
+    bt = torch.tensor([[9, 4, 11], [2, -1, -1], [7, -1, -1], [3, -1, -1]], dtype=torch.int32, device=DEV)
+    qd, kvd = H * hd, KV * hd
+    x, w = _bf(n, d, seed=3, scale=0.5), _bf(qd + 2 * kvd, d, seed=4, scale=0.1)
+    cos = torch.empty(n, hd // 2, device=DEV)
+    sin = torch.empty(n, hd // 2, device=DEV)
+    k_.rope_tables(cos, sin, pos, hd, 10000.0)
+    got = []
+    for tile in (False, True):
+        cache = torch.zeros((12, 2, KV, ps * hd), dtype=torch.bfloat16, device=DEV)
+        q_out = torch.full((n, qd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        rope = k_.Rope(cos, sin, cache, pos, sot, bt, ps, H, KV, hd)
+        k_.fused_linear(k_.fused_linear_tile(w, k_.LINEAR_ROPE, rope) if tile else w, q_out, k_.LINEAR_ROPE, x, rope=rope)
+        got.append((q_out, cache))
+    assert torch.isfinite(got[0][0].float()).all() and float(got[0][1].float().abs().sum()) > 0
+    assert torch.equal(got[0][0], got[1][0]) and torch.equal(got[0][1], got[1][1])
+    other = k_.Rope(cos, sin, None, None, None, None, ps, H, KV, hd)
+    with pytest.raises(k_.KernelError, match="other heads"):
+        k_.fused_linear(k_.fused_linear_tile(w[:qd].contiguous(), k_.LINEAR_ROPE, other), got[0][0], k_.LINEAR_ROPE, x,
+                        rope=k_.Rope(cos, sin, got[0][1], pos, sot, bt, ps, H, KV, hd))
+
+
 def test_fused_linear_resid_refusals():
     k_ = K()
     n, m, k = 4, 64, 64
@@ -716,8 +790,9 @@ def test_fused_gemv_refuses_what_it_does_not_take():
     with pytest.raises(k_.KernelError, match="multiple of 8"):
         k_.gemv_swiglu(x, rnd(32, 60, dtype=torch.bfloat16), torch.empty(2, 16, dtype=torch.bfloat16, device=DEV))
     assert not k_.gemv_fits(2, 131, 64, torch.bfloat16) and not k_.gemv_fits(9, 64, 64, torch.float32)
-    assert k_.gemv_fits(8, 64, 100, torch.float32) and not k_.gemv_fits(2, 64, 100, torch.bfloat16)
-    assert k_.gemv_fits(2, 64, 64, torch.bfloat16) and not k_.gemv_fits(3, 64, 64, torch.bfloat16)
+    assert k_.gemv_fits(8, 64, 100, torch.float32) and not k_.gemv_fits(1, 64, 100, torch.bfloat16)
+    # in bfloat16 they are the faster choice for one row only; they take up to eight
+    assert k_.gemv_fits(1, 64, 64, torch.bfloat16) and not k_.gemv_fits(2, 64, 64, torch.bfloat16)
     assert k_.gemv_fits(8, 64, 64, torch.bfloat16, best=False) and not k_.gemv_fits(9, 64, 64, torch.bfloat16, best=False)
 
 

@@ -98,9 +98,16 @@ def tokens(cfg, n, seed):
 # logits is 1e-3 and on hidden states 1e-4 (engine/e2e/e2e_test.go:21-24);
 # ours is a hundred times tighter (measured on these configurations: at most
 # 7e-7, the same as the plain float32 implementation is from float64).
-# bfloat16: eight mantissa bits on activations of size ~1 (measured: at most
-# 3.2e-3 at logits of size 0.7 to 1.8).
-TOL = {"float32": 1e-5, "bfloat16": 1.5e-2}
+# bfloat16: eight mantissa bits on activations of size ~1.  Measured against the
+# plain implementation in float64 over the 48 random traces of
+# test_gpu_random_traces.py (30,291 positions of these configurations, every
+# way of cutting): mean 5.6e-3, 99.9 % below 1.3e-2, at most 1.76e-2 (a whole
+# prompt of configuration B), and the same figures to three digits whether the
+# RMS norm runs as a kernel of its own or is folded into the products around it
+# (rows times the norm's weight rounded to bfloat16 before the row scale instead
+# of after it: mean 5.615e-3 against 5.624e-3, 99.9 % 1.325e-2 against 1.343e-2,
+# the same maximum).  The bound is that of the random traces.
+TOL = {"float32": 1e-5, "bfloat16": 3e-2}
 
 # The same at the layer sizes of TinyLlama 1.1B, Llama-3 8B and Llama-2 7B
 # (tests/test_gpu_sizes.py; weights N(0, 0.02), logits of size 1 to 6), fixed by

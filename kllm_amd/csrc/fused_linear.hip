@@ -48,10 +48,6 @@ namespace kllm {
 // and 6.7 us for 2,048 x 2,048 weights at 8 rows; 4 ahead: 1,660 and 6.0 us; more waves to a
 // workgroup or more of X in registers measured slower for the same reason).
 constexpr int FL_AHEAD = 4;
-// 16-byte loads of X per lane that are in flight together.  More than eight rows of K = 2,048
-// need a second batch, which waits for the first; sixteen in flight avoid that and still lose
-// to their registers (a step of 9 to 16 tokens at 1.1B sizes 1 to 4 % slower, of 8 tokens 8 %).
-constexpr int XB = 8;
 // LDS row padding (elements): zeros behind K as far as the waves' slices reach beyond it
 // (less than 32 per wave), 8 to shift banks
 constexpr int fl_pad(int nw) { return 32 * nw + 8; }
@@ -152,40 +148,21 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
     }
   }
 
-  // ---- X: wave w stages rows w, w + NW, ... of the slice, eight 16-byte loads a lane at a
-  // time.  Loads return in order, so the last batch goes out before the weights: X is
-  // then in LDS and the workgroup past its barrier while the weights are still arriving.
-  // No load carries a branch (an index beyond the wave's share reads its last item again), so
-  // that the compiler can count what is in flight and wait for X alone.
-  const int chunks = klen / 8;
-  const int mine = (n - wave + NW - 1) / NW;              // rows of this wave
-  const int items = mine * chunks;
-  auto x_load = [&](int base, bf16x8 (&v)[XB]) {
-#pragma unroll
-    for (int j = 0; j < XB; ++j) {
-      const int idx = min(base + j * kWave, max(items - 1, 0));
-      const int ri = idx / chunks, ch = idx - ri * chunks;
-      const int row = min(wave + NW * ri, n - 1);         // a wave without rows reads the last row
-      v[j] = *reinterpret_cast<const bf16x8*>(X + (long)row * x_stride + kbeg + ch * 8);
+  // ---- X: wave w stages rows w, w + NW, ... of the slice straight into LDS, a kilobyte (512 of
+  // K) per instruction, without passing registers: all of them are in flight at once however
+  // many rows there are, before the weights are asked for (loads return in order).
+  {
+    const int kchunks = (klen + 511) / 512;
+    for (int r = wave; r < n; r += NW) {
+      const bf16_t* src = X + (long)r * x_stride + kbeg + lane * 8;
+      bf16_t* dst = xs + r * ld;
+      for (int ch = 0; ch < kchunks; ++ch)
+        if (ch * 512 + lane * 8 < klen)
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + ch * 512),
+                                           (__attribute__((address_space(3))) void*)(dst + ch * 512), 16, 0, 0);
     }
-  };
-  auto x_store = [&](int base, const bf16x8 (&v)[XB]) {
-#pragma unroll
-    for (int j = 0; j < XB; ++j) {
-      const int idx = base + j * kWave;
-      if (idx < items) {
-        const int ri = idx / chunks, ch = idx - ri * chunks;
-        *reinterpret_cast<bf16x8*>(&xs[(wave + NW * ri) * ld + ch * 8]) = v[j];
-      }
-    }
-  };
-  bf16x8 xv0[XB];
-  int xbase = lane;
-  for (; xbase + kWave * XB < items; xbase += kWave * XB) {   // all but the last batch (more than eight rows)
-    x_load(xbase, xv0);
-    x_store(xbase, xv0);
   }
-  x_load(xbase, xv0);
+  asm volatile("" ::: "memory");     // no later load moves in front of these: the wait below counts on it
 
   // ---- SCALED: a row's partial sums of squares, sixteen lanes to a row, asked for behind X
   // and before the weights (loads return in order)
@@ -264,8 +241,6 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
   fill(bufa);
   fill(bufb);
 
-  // ---- X into LDS: what was asked for before the weights has arrived first
-  x_store(xbase, xv0);
   {   // zeros in X's columns [klen, klen + 128): what the waves' slices of K reach beyond klen
     constexpr int per_row = 4 * NW;                         // threads to a row's 32 * NW zeros: 16 rows a pass
     const int r = tid / per_row, ch = tid % per_row;
@@ -312,6 +287,15 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
       }
     }
     rope_angles(0);
+  }
+  {
+    // X has landed in LDS when at most the loads that every wave issued behind it are still in
+    // flight: the sums of squares, the residual values and the two buffers of weights (loads of
+    // the rotation epilogue, which not every wave issues, come behind those and only make
+    // the wait a little longer).
+    constexpr int behind = (SCALED ? NT * FL_SS_LOADS : 0) + (EP == FL_RESID ? 1 + NT : 0) + 2 * FL_AHEAD;
+    static_assert(behind < 64, "vmcnt has six bits");
+    __builtin_amdgcn_s_waitcnt((behind & 0xF) | ((behind >> 4) << 14) | 0x0F70);
   }
   fl_lds_barrier();
 

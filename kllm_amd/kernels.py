@@ -20,7 +20,7 @@ import torch
 
 DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
-GEMV_BEST_ROWS = 1         # up to here they beat the MFMA kernels in bfloat16 (a step at 1.1B sizes, one token: 1.047 against 1.061 ms; two: 1.123 against 1.063)
+GEMV_BEST_ROWS = 0         # rows up to which they beat the MFMA kernels in bfloat16: none (a step at 1.1B sizes, one token: 1.036 against 0.963 ms)
 ABI_VERSION = 7
 
 
@@ -721,10 +721,9 @@ LINEAR_PARTS, LINEAR_RESID, LINEAR_SWIGLU, LINEAR_ROPE = 0, 1, 2, 3
 
 # Rows up to which the decode-batch kernel beats the split-K kernel plus a separate
 # elementwise launch (measured at widths 2048 -> 2560 and 2048 -> 11264).
-# (17 to 32 rows, where the output projection's rows still fit: 1.55 -> 1.58 ms a step at 17 tokens, 1.73 -> 1.79 at 32)
-FUSED_NORM_BEST_ROWS = 16      # rows up to which a residual product and a consumer that scales its rows replace the norm kernel
+FUSED_NORM_BEST_ROWS = 32      # rows up to which a residual product and a consumer that scales its rows replace the norm kernel
 FUSED_ROPE_BEST_ROWS = 32      # (17 tokens at 1.1B sizes: 1.59 -> 1.55 ms a step against the tiled product and a rotation kernel)
-FUSED_SWIGLU_BEST_ROWS = 16
+FUSED_SWIGLU_BEST_ROWS = 32    # (both at 32 against 16, a step at 1.1B sizes: 17 tokens 1.51 -> 1.41 ms, 32 tokens 1.70 -> 1.62; at 8B sizes 17 tokens 5.50 -> 5.19)
 
 
 @functools.lru_cache(maxsize=4096)

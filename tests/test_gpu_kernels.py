@@ -791,8 +791,8 @@ def test_fused_gemv_refuses_what_it_does_not_take():
         k_.gemv_swiglu(x, rnd(32, 60, dtype=torch.bfloat16), torch.empty(2, 16, dtype=torch.bfloat16, device=DEV))
     assert not k_.gemv_fits(2, 131, 64, torch.bfloat16) and not k_.gemv_fits(9, 64, 64, torch.float32)
     assert k_.gemv_fits(8, 64, 100, torch.float32) and not k_.gemv_fits(1, 64, 100, torch.bfloat16)
-    # in bfloat16 they are the faster choice for one row only; they take up to eight
-    assert k_.gemv_fits(1, 64, 64, torch.bfloat16) and not k_.gemv_fits(2, 64, 64, torch.bfloat16)
+    # in bfloat16 the matrix-core kernels are the faster choice at every row count; these take up to eight
+    assert not k_.gemv_fits(1, 64, 64, torch.bfloat16) and k_.gemv_fits(1, 64, 64, torch.bfloat16, best=False)
     assert k_.gemv_fits(8, 64, 64, torch.bfloat16, best=False) and not k_.gemv_fits(9, 64, 64, torch.bfloat16, best=False)
 
 

@@ -19,7 +19,9 @@
 // of the normalised row once.
 //
 // A workgroup owns tiles of 16 rows of W and one slice of K (all of K unless
-// the caller splits).  It puts its slice of X, all rows, into LDS once.  Each
+// the caller splits).  It puts its slice of X, all rows, into LDS once (where
+// they do not fit, in several passes over K, with one tile to a workgroup whose
+// sums stay in registers from pass to pass).  Each
 // of its four waves takes a quarter of the slice: it streams its part of the 16
 // rows of W straight from memory, eight 16-byte loads per lane in flight, the
 // first of them before X is staged, and multiplies with X from LDS
@@ -108,14 +110,16 @@ __device__ __forceinline__ void fl_lds_barrier() {
   asm volatile("" ::: "memory");
 }
 
-// NW waves share a tile's K; SCALED: the sums are multiplied by a row scale made from out.ss_in.
-template <int NT, int EP, int NW, bool SCALED>
+// NW waves share a tile's K; SCALED: the sums are multiplied by a row scale made from out.ss_in;
+// PASSES: the rows of X do not fit into LDS at once and go in passes of kpass of K (a kernel of
+// its own, so that the one for rows that fit carries none of it).
+template <int NT, int EP, int NW, bool SCALED, bool PASSES>
 __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __restrict__ X, FlOut out,
                                                            const bf16_t* __restrict__ W, int n, int m,
                                                            int k, int kslice, int tiles, int tiles_per_wg,
-                                                           int x_stride) {
+                                                           int x_stride, int kpass) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  const int ld = kslice + fl_pad(NW);
+  const int ld = kpass + fl_pad(NW);
   bf16_t* xs = reinterpret_cast<bf16_t*>(lds_raw);                            // [n][ld]
   float* part = reinterpret_cast<float*>(lds_raw + (size_t)n * ld * sizeof(bf16_t));   // [2][NW][NT][x row 16][17]
   float* row_scale = part + 2 * NW * NT * FL_TILE;                            // [32]
@@ -124,9 +128,12 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
   const int g = lane / 16, c = lane % 16;
   const int kbeg = blockIdx.y * kslice;
   const int klen = min(k, kbeg + kslice) - kbeg;            // a multiple of 8
-  const int kw = ((klen + NW - 1) / NW + 31) / 32 * 32;     // K of one wave
-  const int wk0 = wave * kw;                                // this wave's offset in the slice
-  const int wlen = max(0, min(klen, wk0 + kw) - wk0);
+  // The slice is staged and multiplied in passes of kpass of K (one pass where all rows of the slice
+  // fit into LDS; several only with one tile to a workgroup, whose sums then stay in registers).
+  const int npass = PASSES ? (klen + kpass - 1) / kpass : 1;
+  auto pass_len = [&](int pass) { return PASSES ? min(klen - pass * kpass, kpass) : klen; };
+  const int kw = ((pass_len(0) + NW - 1) / NW + 31) / 32 * 32;     // K of one wave in a pass
+  const int wk0 = wave * kw;                                // this wave's offset in the pass
   const int steps = kw / 32;
   const int tile0 = blockIdx.x * tiles_per_wg;
   const int my_tiles = min(tiles_per_wg, tiles - tile0);
@@ -151,17 +158,19 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
   // ---- X: wave w stages rows w, w + NW, ... of the slice straight into LDS, a kilobyte (512 of
   // K) per instruction, without passing registers: all of them are in flight at once however
   // many rows there are, before the weights are asked for (loads return in order).
-  {
-    const int kchunks = (klen + 511) / 512;
+  auto stage = [&](int pass) {
+    const int plen = pass_len(pass);
+    const int kchunks = (plen + 511) / 512;
     for (int r = wave; r < n; r += NW) {
-      const bf16_t* src = X + (long)r * x_stride + kbeg + lane * 8;
+      const bf16_t* src = X + (long)r * x_stride + kbeg + pass * kpass + lane * 8;
       bf16_t* dst = xs + r * ld;
       for (int ch = 0; ch < kchunks; ++ch)
-        if (ch * 512 + lane * 8 < klen)
+        if (ch * 512 + lane * 8 < plen)
           __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + ch * 512),
                                            (__attribute__((address_space(3))) void*)(dst + ch * 512), 16, 0, 0);
     }
-  }
+  };
+  stage(0);
   asm volatile("" ::: "memory");     // no later load moves in front of these: the wait below counts on it
 
   // ---- SCALED: a row's partial sums of squares, sixteen lanes to a row, asked for behind X
@@ -211,23 +220,27 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
   const bf16_t* far_row;                                    // first K of this lane's row of W
   int far_lane_off;                                         // this lane's offset in it, or -1: no such row
   const int far_stride = out.tiled ? 512 : 32;              // elements from a step to the next
-  int far_tile = 0, far_s0 = 0;                             // the steps that are loaded next
-  auto tile_ptr = [&](int t) {
+  int far_tile = 0, far_s0 = 0;                             // the steps that are loaded next; a tile's passes count as tiles
+  int far_wlen = 0;                                         // this wave's K in that pass
+  auto tile_ptr = [&](int u) {
+    const int t = PASSES ? u / npass : u, pass = PASSES ? u % npass : 0;
+    const int pbeg = kbeg + pass * kpass;
+    far_wlen = max(0, min(pass_len(pass), wk0 + kw) - wk0);
     if (out.tiled) {     // rows that do not exist hold zeros there; a tile that does not exist reads the first
       const long tl = t < my_tiles ? tile0 + t : tile0;
-      far_row = W + ((tl * ((k + 31) / 32) + kbeg / 32) * kWave + lane) * 8;
+      far_row = W + ((tl * ((k + 31) / 32) + pbeg / 32) * kWave + lane) * 8;
       far_lane_off = (wk0 / 32) * 512;
       return;
     }
     const long r = t < my_tiles ? fl_row<EP>((int)tile0 + t, c, m, out) : -1;
-    far_row = W + (r >= 0 ? r : 0) * k + kbeg;
+    far_row = W + (r >= 0 ? r : 0) * k + pbeg;
     far_lane_off = r >= 0 ? wk0 + 8 * g : -1;
   };
   auto fill = [&](bf16x8 (&buf)[FL_AHEAD]) {
 #pragma unroll
     for (int i = 0; i < FL_AHEAD; ++i) {
       const int s = far_s0 + i;
-      const bool valid = far_lane_off >= 0 && s < steps && 32 * s + 8 * g < wlen;
+      const bool valid = far_lane_off >= 0 && s < steps && 32 * s + 8 * g < far_wlen;
       buf[i] = *reinterpret_cast<const bf16x8*>(far_row + (valid ? far_lane_off + far_stride * s : 0));
     }
     far_s0 += FL_AHEAD;
@@ -241,13 +254,22 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
   fill(bufa);
   fill(bufb);
 
-  {   // zeros in X's columns [klen, klen + 128): what the waves' slices of K reach beyond klen
-    constexpr int per_row = 4 * NW;                         // threads to a row's 32 * NW zeros: 16 rows a pass
-    const int r = tid / per_row, ch = tid % per_row;
+  auto zero_behind = [&](int pass) {   // zeros in X's columns from the K of the pass to where the waves' slices reach
+    constexpr int per_row = 4 * NW;                         // threads to 32 * NW zeros of a row: 16 rows at a time
+    const int plen = pass_len(pass);                        // (a last pass may be shorter than the others)
+    const int r = tid / per_row;
 #pragma unroll
     for (int t = 0; t < NT; ++t)
-      if (t * 16 + r < n) *reinterpret_cast<bf16x8*>(&xs[(t * 16 + r) * ld + klen + 8 * ch]) = zero;
-  }
+      if (t * 16 + r < n) {
+        if (!PASSES) {   // all passes alike: the slices reach less than 32 NW beyond
+          *reinterpret_cast<bf16x8*>(&xs[(t * 16 + r) * ld + plen + 8 * (tid % per_row)]) = zero;
+        } else {
+          for (int at = plen + 8 * (tid % per_row); at < NW * kw; at += 8 * per_row)
+            *reinterpret_cast<bf16x8*>(&xs[(t * 16 + r) * ld + at]) = zero;
+        }
+      }
+  };
+  zero_behind(0);
   if (SCALED) {   // the rows' scales: sums in a fixed order, then across the row's sixteen lanes
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -320,11 +342,23 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
   };
 
   for (int tile = 0; tile < my_tiles; ++tile) {
-    for (int s0 = 0; s0 < rsteps; s0 += 2 * FL_AHEAD) {
-      multiply(bufa, s0);
-      fill(bufa);
-      multiply(bufb, s0 + FL_AHEAD);
-      fill(bufb);
+    for (int pass = 0; pass < npass; ++pass) {
+      if (PASSES && pass > 0) {
+        // the next columns of X take the place of the ones that every wave has multiplied; the
+        // weights asked for ahead are older loads and arrive on the way
+        fl_lds_barrier();
+        stage(pass);
+        zero_behind(pass);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0x0F70);                 // vmcnt(0)
+        fl_lds_barrier();
+      }
+      for (int s0 = 0; s0 < rsteps; s0 += 2 * FL_AHEAD) {
+        multiply(bufa, s0);
+        fill(bufa);
+        multiply(bufb, s0 + FL_AHEAD);
+        fill(bufb);
+      }
     }
     // ---- the tile is complete in this wave: meet the other waves in LDS
     float* pb = part + (tile & 1) * NW * NT * FL_TILE;
@@ -450,35 +484,45 @@ static size_t fl_lds_bytes(int n, int nt, int kslice, int nw = 4) {
   return (size_t)n * (kslice + fl_pad(nw)) * sizeof(bf16_t) + (size_t)(2 * nw * nt * FL_TILE + 32) * sizeof(float);
 }
 
-template <int NT, int EP, int NW, bool SCALED>
-static int fl_launch(const void* x, const FlOut& out, const void* w, int n, int m, int k, int kslice,
+template <int NT, int EP, int NW, bool SCALED, bool PASSES>
+static int fl_launch_passes(const void* x, const FlOut& out, const void* w, int n, int m, int k, int kslice, int kpass,
                      int nsplit, int tiles, int tiles_per_wg, int x_stride, hipStream_t stream) {
-  const size_t lds = fl_lds_bytes(n, NT, kslice, NW);
+  const size_t lds = fl_lds_bytes(n, NT, kpass, NW);
   static size_t allowed = 64 * 1024;          // one per instantiation
   if (lds > allowed) {
-    hipError_t e = hipFuncSetAttribute((const void*)fused_linear_kernel<NT, EP, NW, SCALED>,
+    hipError_t e = hipFuncSetAttribute((const void*)fused_linear_kernel<NT, EP, NW, SCALED, PASSES>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, FL_LDS_MAX);
     if (e != hipSuccess) KLLM_FAIL((int)e, "fused_linear: cannot raise the LDS limit: %s", hipGetErrorString(e));
     allowed = FL_LDS_MAX;
   }
   const dim3 grid(ceil_div(tiles, tiles_per_wg), nsplit);
-  hipLaunchKernelGGL((fused_linear_kernel<NT, EP, NW, SCALED>), grid, dim3(64 * NW), lds, stream, (const bf16_t*)x,
-                     out, (const bf16_t*)w, n, m, k, kslice, tiles, tiles_per_wg, x_stride);
+  hipLaunchKernelGGL((fused_linear_kernel<NT, EP, NW, SCALED, PASSES>), grid, dim3(64 * NW), lds, stream, (const bf16_t*)x,
+                     out, (const bf16_t*)w, n, m, k, kslice, tiles, tiles_per_wg, x_stride, kpass);
   return 0;
+}
+
+template <int NT, int EP, int NW, bool SCALED>
+static int fl_launch(const void* x, const FlOut& out, const void* w, int n, int m, int k, int kslice, int kpass,
+                     int nsplit, int tiles, int tiles_per_wg, int x_stride, hipStream_t stream) {
+  if (kpass < kslice)
+    return fl_launch_passes<NT, EP, NW, SCALED, true>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tiles_per_wg,
+                                                      x_stride, stream);
+  return fl_launch_passes<NT, EP, NW, SCALED, false>(x, out, w, n, m, k, kslice, kslice, nsplit, tiles, tiles_per_wg,
+                                                     x_stride, stream);
 }
 
 template <int NT>
 static int fl_launch_ep(int ep, bool scaled, const void* x, const FlOut& out, const void* w, int n, int m, int k,
-                        int kslice, int nsplit, int tiles, int tpw, int xs, hipStream_t st) {
+                        int kslice, int kpass, int nsplit, int tiles, int tpw, int xs, hipStream_t st) {
   switch (ep) {
-    case FL_PARTS: return fl_launch<NT, FL_PARTS, 4, false>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
-    case FL_RESID: return fl_launch<NT, FL_RESID, 4, false>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+    case FL_PARTS: return fl_launch<NT, FL_PARTS, 4, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
+    case FL_RESID: return fl_launch<NT, FL_RESID, 4, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
     case FL_SWIGLU:
-      return scaled ? fl_launch<NT, FL_SWIGLU, 4, true>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st)
-                    : fl_launch<NT, FL_SWIGLU, 4, false>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+      return scaled ? fl_launch<NT, FL_SWIGLU, 4, true>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st)
+                    : fl_launch<NT, FL_SWIGLU, 4, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
     default:
-      return scaled ? fl_launch<NT, FL_ROPE, 4, true>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st)
-                    : fl_launch<NT, FL_ROPE, 4, false>(x, out, w, n, m, k, kslice, nsplit, tiles, tpw, xs, st);
+      return scaled ? fl_launch<NT, FL_ROPE, 4, true>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st)
+                    : fl_launch<NT, FL_ROPE, 4, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
   }
 }
 
@@ -492,6 +536,25 @@ extern "C" long kllm_fused_linear_lds_bytes(int n, int k, int nsplit) {
   if (n <= 0 || k <= 0 || nsplit <= 0) return -1;
   const int kslice = ceil_div(ceil_div(k, nsplit), 32) * 32;
   return (long)fl_lds_bytes(n, ceil_div(n, 16), kslice);
+}
+
+// K of a pass for n rows of a slice of kslice: the slice itself where its rows fit into LDS, else
+// the least number of equal passes (up to FL_MAX_PASSES) whose rows do; 0 if none does.
+constexpr int FL_MAX_PASSES = 8;
+static int fl_pass_k(int n, int kslice) {
+  const int nt = ceil_div(n, 16);
+  for (int passes = 1; passes <= FL_MAX_PASSES; ++passes) {
+    const int kpass = ceil_div(ceil_div(kslice, passes), 32) * 32;
+    if (fl_lds_bytes(n, nt, kpass) <= (size_t)FL_LDS_MAX) return kpass;
+  }
+  return 0;
+}
+
+extern "C" int kllm_fused_linear_passes(int n, int k, int nsplit) {
+  if (n <= 0 || n > KLLM_FUSED_LINEAR_MAX_ROWS || k <= 0 || nsplit <= 0) return 0;
+  const int kslice = ceil_div(ceil_div(k, nsplit), 32) * 32;
+  const int kpass = fl_pass_k(n, kslice);
+  return kpass ? ceil_div(kslice < k ? kslice : k, kpass) : 0;
 }
 
 extern "C" int kllm_fused_linear_resid_parts(int m, int tiles_per_wg) {
@@ -553,9 +616,12 @@ extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOu
   const int kslice = ceil_div(ceil_div(k, nsplit), 32) * 32;
   KLLM_REQUIRE((long)kslice * (nsplit - 1) < k, "fused_linear: nsplit %d leaves an empty slice of K=%d", nsplit, k);
   const int nt = ceil_div(n, 16);
-  KLLM_REQUIRE(fl_lds_bytes(n, nt, kslice) <= (size_t)FL_LDS_MAX,
-               "fused_linear: %d rows of K=%d need %zu bytes of LDS, more than %d", n, kslice,
-               fl_lds_bytes(n, nt, kslice), FL_LDS_MAX);
+  const int kpass = fl_pass_k(n, kslice);
+  KLLM_REQUIRE(kpass > 0, "fused_linear: %d rows of K=%d need %zu bytes of LDS, more than %d even in %d passes", n,
+               kslice, fl_lds_bytes(n, nt, kslice), FL_LDS_MAX, FL_MAX_PASSES);
+  KLLM_REQUIRE(kpass >= kslice || tiles_per_wg == 1,
+               "fused_linear: %d rows of K=%d do not fit into LDS at once; in passes a workgroup takes one tile, not %d",
+               n, kslice, tiles_per_wg);
   if (x_stride <= 0) x_stride = k;
   KLLM_REQUIRE(x_stride >= k && x_stride % 8 == 0, "fused_linear: row stride %d of x does not fit K=%d", x_stride, k);
 
@@ -609,8 +675,8 @@ extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOu
     out.KV = KV;
     out.hd = hd;
   }
-  const int rc = nt == 1 ? fl_launch_ep<1>(ep, scaled, x, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream)
-                         : fl_launch_ep<2>(ep, scaled, x, out, w, n, m, k, kslice, nsplit, tiles, tiles_per_wg, x_stride, stream);
+  const int rc = nt == 1 ? fl_launch_ep<1>(ep, scaled, x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tiles_per_wg, x_stride, stream)
+                         : fl_launch_ep<2>(ep, scaled, x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tiles_per_wg, x_stride, stream);
   if (rc) return rc;
   KLLM_CHECK_LAUNCH("fused_linear");
   return 0;

@@ -155,8 +155,9 @@ int kllm_gemv_rope_append(const void* x, const void* w_qkv, void* q_out, const f
  * With ss_in (SWIGLU and ROPE only) x is such a y and the sums are multiplied by the row's
  * rsqrt(sum of ss_in[row][0:ss_parts] / k + eps) before the epilogue: the RMS norm of the
  * stream, rounded to bfloat16 before the row scale instead of after it.
- * All of a workgroup's slice of K for all rows has to fit into LDS:
- * kllm_fused_linear_lds_bytes says how much a call needs (160 KiB at most). */
+ * All of a workgroup's slice of K for all rows is staged in LDS:
+ * kllm_fused_linear_lds_bytes says how much that needs; beyond 160 KiB see
+ * kllm_fused_linear_passes. */
 #define KLLM_FUSED_LINEAR_MAX_ROWS 32
 #define KLLM_LINEAR_OUT_PARTS 0
 #define KLLM_LINEAR_OUT_RESID 1
@@ -183,6 +184,10 @@ typedef struct {
   int tiled;            /* w is the copy that kllm_fused_linear_tile made of the weights for this kind */
 } KllmLinearOut;
 long kllm_fused_linear_lds_bytes(int n, int k, int nsplit);
+/* Where that is more than LDS holds, the rows are staged and multiplied in passes over K, with
+ * one tile to a workgroup (tiles_per_wg = 1): how many passes a call needs (1: all at once; 0:
+ * the kernel does not take the sizes). */
+int kllm_fused_linear_passes(int n, int k, int nsplit);
 /* A copy of w[m][k] in the order the kernel's lanes read it (a load instruction then reads one
  * contiguous kilobyte instead of 64 bytes of each of 16 rows: weights stream 20-30 % faster),
  * for one output kind (PARTS and RESID share theirs; ROPE with the heads it will be called

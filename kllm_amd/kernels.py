@@ -106,6 +106,7 @@ def _declare(lib):
         "kllm_gemv_resid_parts": [I],
         "kllm_fused_linear": [P, I, P, P, I, I, I, I, P],
         "kllm_fused_linear_resid_parts": [I, I],
+        "kllm_fused_linear_passes": [I, I, I],
         "kllm_fused_linear_tile": [P, P, I, I, I, I, I, I, I, P],
         "kllm_command_op": [c_char_p],
         "kllm_command_nargs": [I],
@@ -751,6 +752,34 @@ def fused_linear_fits(n, k, nsplit=1) -> bool:
     return 0 < library().kllm_fused_linear_lds_bytes(int(n), int(k), int(nsplit)) <= FUSED_LINEAR_LDS
 
 
+# Passes over K up to which the decode-batch kernel is taken where the rows do not fit into LDS at
+# once, and the rows up to which that pays (a step at 1.1B sizes, 16 tokens: 1.284 -> 1.237 ms; at 8B
+# sizes 8 tokens 4.41 -> 4.08, 16 tokens 5.61 -> 4.75; from 17 rows on, two tiles of rows, the
+# tiled product and a kernel behind it are faster: 1.1B sizes, 24 tokens 1.49 against 1.62 ms).
+FUSED_LINEAR_BEST_PASSES = 4
+FUSED_LINEAR_PASSES_BEST_ROWS = 16
+
+
+@functools.lru_cache(maxsize=4096)
+def fused_linear_passes(n, k, nsplit=1) -> int:
+    """Passes over K in which the decode-batch products take n rows: 1 where all rows of a
+    workgroup's slice of K fit into LDS (``fused_linear_fits``); more, with one tile to a
+    workgroup, where they do not; 0 if the kernel does not take the sizes."""
+    if n < 1 or n > FUSED_LINEAR_MAX_ROWS or k % 8:
+        return 0
+    return int(library().kllm_fused_linear_passes(int(n), int(k), int(nsplit)))
+
+
+def fused_linear_tiles(n, m, k) -> int:
+    """Tiles per workgroup with which the decode-batch kernel is taken for n rows against
+    w [m, k] (``fused_tiles_per_wg`` where the rows fit into LDS at once, one where they go in
+    a few passes over K), or 0 where it is not taken."""
+    passes = fused_linear_passes(n, k)
+    if passes == 0 or (passes > 1 and (passes > FUSED_LINEAR_BEST_PASSES or n > FUSED_LINEAR_PASSES_BEST_ROWS)):
+        return 0
+    return fused_tiles_per_wg(n, m, k) if passes == 1 else 1
+
+
 class TiledWeights:
     """A copy of a weight matrix [m, k] in the order the decode-batch kernel's lanes read it, for
     one output kind (LINEAR_PARTS serves LINEAR_RESID too; LINEAR_ROPE is made for the heads it
@@ -800,7 +829,8 @@ class ScaledRows:
 def fused_resid_parts(n, m, k, tiles_per_wg=1) -> int:
     """Partial sums of squares per row that a LINEAR_RESID product of these sizes leaves, or 0
     if the decode-batch kernel does not take them."""
-    if not fused_linear_fits(n, k):
+    passes = fused_linear_passes(n, k)
+    if passes == 0 or (passes > 1 and tiles_per_wg != 1):
         return 0
     parts = library().kllm_fused_linear_resid_parts(int(m), int(tiles_per_wg))
     return parts if 0 < parts <= limit("fused_linear_max_parts") else 0

@@ -131,6 +131,14 @@ class CausalSelfAttention(Part):
             raise ValueError(f"attention: pages of {page_size} tokens are not built "
                              f"(1 to {K.GENERIC_MAX_PAGE_SIZE})")
 
+    def _fused_tiles(self, n):
+        """Tiles per workgroup of the decode-batch kernel for the input projections of n
+        tokens, or 0 where it is not taken."""
+        if (self.runtime.dtype != torch.bfloat16 or n > K.FUSED_ROPE_BEST_ROWS or not self.plain_rotation
+                or self.runtime.options.get("no_fused_linear")):
+            return 0
+        return K.fused_linear_tiles(n, self.w_in.shape[0], self.hidden)
+
     def forward(self, ctx, xn, cache, sink=None):
         dtype = self.runtime.dtype
         if isinstance(xn, Normed):
@@ -138,9 +146,7 @@ class CausalSelfAttention(Part):
             opts = self.runtime.options
             gemv = (K.gemv_fits(n, self.w_in.shape[0], self.hidden, dtype) and n <= K.normed_max_rows()
                     and not opts.get("no_fused_gemv") and self.plain_rotation and xn.xw is None)
-            scaled = (not gemv and xn.xw is not None and dtype == torch.bfloat16 and n <= K.FUSED_ROPE_BEST_ROWS
-                      and K.fused_linear_fits(n, self.hidden) and not opts.get("no_fused_linear")
-                      and self.plain_rotation)
+            scaled = (not gemv and xn.xw is not None and self._fused_tiles(n) > 0)
             # the small-batch kernel below normalises while it stages its input, the decode-batch
             # kernel scales its sums by the row
             xn = xn.kernel_input() if gemv else xn.scaled_rows() if scaled else xn.materialize(ctx)
@@ -161,11 +167,10 @@ class CausalSelfAttention(Part):
             K.gemv_rope_append(xn, self.w_in, q, cos, sin, pages, ctx.positions, ctx.span_of_token,
                                cache.block_table, cache.page_size, self.heads, self.kv_heads,
                                self.head_dim)
-        elif (dtype == torch.bfloat16 and n <= K.FUSED_ROPE_BEST_ROWS and K.fused_linear_fits(n, self.hidden)
-              and not opts.get("no_fused_linear") and plain_rotation):
+        elif self._fused_tiles(n) > 0:
             # a decode batch: the same on the matrix cores
             K.fused_linear(self._tiled.get("in") or self.w_in, q, K.LINEAR_ROPE, x=xn,
-                           tiles_per_wg=K.fused_tiles_per_wg(n, self.w_in.shape[0], self.hidden),
+                           tiles_per_wg=self._fused_tiles(n),
                            rope=K.Rope(cos, sin, pages, ctx.positions, ctx.span_of_token, cache.block_table,
                                        cache.page_size, self.heads, self.kv_heads, self.head_dim))
         else:

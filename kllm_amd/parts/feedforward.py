@@ -66,8 +66,9 @@ class GatedFeedForward(Part):
         gemv = K.gemv_fits(n, 2 * self.intermediate, self.hidden, dtype) and not opts.get("no_fused_gemv")
         if gemv and isinstance(xn, Normed) and xn.xw is not None:
             gemv = False       # the producer was the decode-batch kernel: its consumer is, too
-        fused = (not gemv and dtype == torch.bfloat16 and n <= K.FUSED_SWIGLU_BEST_ROWS
-                 and K.fused_linear_fits(n, self.hidden) and not opts.get("no_fused_linear"))
+        tiles = (K.fused_linear_tiles(n, 2 * self.intermediate, self.hidden)
+                 if dtype == torch.bfloat16 and n <= K.FUSED_SWIGLU_BEST_ROWS else 0)
+        fused = not gemv and tiles > 0 and not opts.get("no_fused_linear")
         if isinstance(xn, Normed):     # the small-batch kernel below normalises while it stages its input,
             # the decode-batch kernel scales its sums by the row
             xn = (xn.kernel_input() if gemv and n <= K.normed_max_rows()
@@ -78,7 +79,7 @@ class GatedFeedForward(Part):
         elif fused:
             # a decode batch: the same on the matrix cores
             K.fused_linear(self._tiled.get("gu") or self.w_gu, h, K.LINEAR_SWIGLU, x=xn, act=self.act,
-                           tiles_per_wg=K.fused_tiles_per_wg(n, 2 * self.intermediate, self.hidden))
+                           tiles_per_wg=tiles)
         elif ((n > 128 or self._gate_in_tiles(n, dtype))
               and self.runtime.options.get("gemm") != "library"
               and self.hidden % (8 if xn.dtype == torch.bfloat16 else 4) == 0):

@@ -164,9 +164,13 @@ def choose(dtype, n, m, k, options=None):
 def _resid_tiles(n, m, k):
     """(tiles per workgroup, partial sums of squares per row) of a decode batch's residual
     product: as few tiles to a workgroup as keep the sums of squares within what the
-    consumer reads; (1, 0) if the kernel does not take the sizes."""
+    consumer reads (one tile where the rows go through LDS in passes over K); (1, 0) if the
+    kernel does not take the sizes."""
+    passes = K.fused_linear_passes(n, k)
+    if passes == 0 or (passes > 1 and (passes > K.FUSED_LINEAR_BEST_PASSES or n > K.FUSED_LINEAR_PASSES_BEST_ROWS)):
+        return 1, 0
     tpw = 1
-    while K.fused_resid_parts(n, m, k, tpw) == 0 and tpw < 64 and K.fused_linear_fits(n, k):
+    while K.fused_resid_parts(n, m, k, tpw) == 0 and tpw < 64 and passes == 1:
         tpw *= 2
     return tpw, K.fused_resid_parts(n, m, k, tpw)
 

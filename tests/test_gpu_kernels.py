@@ -477,9 +477,12 @@ def _bf(*shape, seed, scale):
 
 @pytest.mark.parametrize("n,m,k,nsplit,tpw", [(1, 48, 64, 1, 1), (8, 2048, 2048, 1, 1), (5, 100, 264, 1, 3),
                                               (16, 72, 520, 2, 1), (19, 33, 4104, 3, 2), (32, 257, 1000, 1, 4),
-                                              (8, 176, 5632, 1, 1)])
+                                              (8, 176, 5632, 1, 1), (16, 48, 5632, 1, 1), (32, 257, 5000, 1, 1),
+                                              (8, 64, 14336, 1, 1), (27, 40, 9992, 2, 1)])
 def test_fused_linear_parts(n, m, k, nsplit, tpw):
-    """bfloat16 rows in, float32 sums (or partial sums over slices of K) out."""
+    """bfloat16 rows in, float32 sums (or partial sums over slices of K) out; the last sizes are
+    rows that do not fit into LDS at once and go in passes over K (two and three, the last one
+    shorter than the others)."""
     k_ = K()
     x, w = _bf(n, k, seed=1, scale=0.5), _bf(m, k, seed=2, scale=0.1)
     want = P.linear(x.cpu().double(), w.cpu().double())
@@ -557,7 +560,8 @@ def test_fused_linear_rope_append(H, KV, hd, ps, d, tpw):
 
 @pytest.mark.parametrize("n,m,k,tpw", [(1, 48, 64, 1), (3, 72, 88, 1), (8, 2048, 2048, 1), (8, 2048, 5632, 1),
                                        (13, 2048, 5632, 2), (16, 100, 264, 3), (19, 33, 3080, 1), (32, 257, 1000, 2),
-                                       (5, 4096, 14336, 1), (12, 4096, 4096, 1)])
+                                       (5, 4096, 14336, 1), (12, 4096, 4096, 1), (16, 2048, 5632, 1),
+                                       (8, 4096, 14336, 1), (24, 4088, 4096, 1)])
 def test_fused_linear_resid_then_scaled_consumers(n, m, k, tpw):
     """A decode batch's product added to the residual stream in its own epilogue, with what
     the RMS norm behind the addition needs left beside it; then the two consumers that apply
@@ -586,7 +590,7 @@ def test_fused_linear_resid_then_scaled_consumers(n, m, k, tpw):
     sr = k_.ScaledRows(xw, ss, parts, eps)
     f = 40
     wg = _bf(2 * f, m, seed=5, scale=0.1)
-    if k_.fused_linear_fits(n, m):
+    if k_.fused_linear_passes(n, m) >= 1:      # (24 rows of 4,088: in two passes)
         h = torch.full((n, f), float("nan"), dtype=torch.bfloat16, device=DEV)
         k_.fused_linear(wg, h, k_.LINEAR_SWIGLU, sr)
         wd = wg.cpu().double()
@@ -772,10 +776,16 @@ def test_fused_linear_refuses_what_it_does_not_take():
     with pytest.raises(k_.KernelError, match="multiple of 8"):
         k_.fused_linear(_bf(32, 60, seed=1, scale=0.1), torch.empty(1, 4, 32, device=DEV), k_.LINEAR_PARTS,
                         _bf(4, 60, seed=2, scale=1.0))
-    with pytest.raises(k_.KernelError, match="LDS"):
-        k_.fused_linear(_bf(16, 8192, seed=1, scale=0.1), torch.empty(1, 32, 16, device=DEV), k_.LINEAR_PARTS,
-                        _bf(32, 8192, seed=2, scale=1.0))
+    # 32 rows of 8,192 do not fit into LDS at once: they go in passes, with one tile to a workgroup only
+    with pytest.raises(k_.KernelError, match="in passes a workgroup takes one tile"):
+        k_.fused_linear(_bf(32, 8192, seed=1, scale=0.1), torch.empty(1, 32, 32, device=DEV), k_.LINEAR_PARTS,
+                        _bf(32, 8192, seed=2, scale=1.0), tiles_per_wg=2)
+    with pytest.raises(k_.KernelError, match="LDS"):        # ... and not in more than eight passes
+        k_.fused_linear(_bf(16, 32768, seed=1, scale=0.1), torch.empty(1, 32, 16, device=DEV), k_.LINEAR_PARTS,
+                        _bf(32, 32768, seed=2, scale=1.0))
     assert not k_.fused_linear_fits(32, 8192) and k_.fused_linear_fits(32, 8192, 4) and k_.fused_linear_fits(8, 5632)
+    assert k_.fused_linear_passes(32, 8192) == 4 and k_.fused_linear_passes(8, 5632) == 1
+    assert k_.fused_linear_passes(32, 32768) == 0 and k_.fused_linear_passes(16, 5632) == 2
     with pytest.raises(k_.KernelError, match="split"):
         k_.fused_linear(_bf(32, 64, seed=1, scale=0.1), torch.empty(4, 16, dtype=torch.bfloat16, device=DEV),
                         k_.LINEAR_SWIGLU, _bf(4, 64, seed=2, scale=1.0), nsplit=2)

@@ -173,13 +173,15 @@ def test_a_whole_prompt_of_2048_tokens(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,B", [("tinyllama", 64), ("tinyllama", 33), ("tinyllama", 24), ("tinyllama", 12),
-                                    ("tinyllama", 8), ("tinyllama", 4), ("llama3-8b", 64), ("llama3-8b", 40),
-                                    ("llama3-8b", 17), ("llama3-8b", 12), ("llama3-8b", 8), ("llama3-8b", 3)])
+@pytest.mark.parametrize("name,B", [("tinyllama", 64), ("tinyllama", 33), ("tinyllama", 24), ("tinyllama", 16),
+                                    ("tinyllama", 12), ("tinyllama", 8), ("tinyllama", 4), ("tinyllama", 2),
+                                    ("llama3-8b", 64), ("llama3-8b", 40), ("llama3-8b", 17), ("llama3-8b", 16),
+                                    ("llama3-8b", 12), ("llama3-8b", 8), ("llama3-8b", 3)])
 def test_decode_steps_of_many_requests_eager_and_as_graphs(name, B, dtype):
     """64 requests decode together (and fewer, which take other kernels for the products and for
     attention and other hand-overs between them: up to 2, 4, 16, 32 and 64 rows, with the norm
-    folded into its neighbours or in a launch of its own, the gate in the tiled product's
+    folded into its neighbours or in a launch of its own, the down projection's rows in one
+    pass through LDS or in two to four, the gate in the tiled product's
     epilogue or apart, a few more attention groups than the chip holds whole-context workgroups):
     first through the plain step function, then queued ahead
     as HIP graphs.  Both give logits; the graphs' must equal the eager ones (the same kernels
@@ -216,7 +218,7 @@ def test_decode_steps_of_many_requests_eager_and_as_graphs(name, B, dtype):
             eng.release(r)
     for k in range(new):
         assert np.array_equal(eager[k], graphs[k]), f"step {k}: a replayed graph and the eager step differ"
-    sample = sorted({0, B // 5, B // 2 + 1, B - 1})
+    sample = sorted({0, B // 5, min(B // 2 + 1, B - 1), B - 1})
     for stored in ([False, True] if dtype == "bfloat16" else [False]):
         want = expected(name, dtype, {rids[i]: reqs[rids[i]] for i in sample}, stored)
         worst = 0.0

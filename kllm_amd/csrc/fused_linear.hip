@@ -195,11 +195,18 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
     if (EP != FL_RESID) return;
     const long row = (long)(tile0 + tile_index) * 16 + tid % 16;
     const bool live = tid < 256 && row < m && tile_index < my_tiles;
-    res_w = out.norm_w[live ? row : 0];
+    // The indices pass through a register that the compiler cannot see into: left to itself it
+    // turns the choice of an index into a branch around two loads, and with a load inside a branch
+    // every wait of the loop becomes a wait for all loads in flight.
+    long at = live ? row : 0;
+    asm volatile("" : "+v"(at));
+    res_w = out.norm_w[at];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int xr = t * 16 + tid / 16;
-      res_old[t] = out.resid[live && xr < n ? (long)xr * m + row : 0];
+      at = live && xr < n ? (long)xr * m + row : 0;
+      asm volatile("" : "+v"(at));
+      res_old[t] = out.resid[at];
     }
   };
   if (EP == FL_RESID) {
@@ -328,16 +335,22 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
     acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
     xrow[t] = xs + min(t * 16 + c, n - 1) * ld + wk0 + 8 * g;
   }
+  // A buffer's steps: all their rows of X are asked of LDS first, without a branch between them, so
+  // that LDS answers while the wave still waits for the weights; a step beyond the wave's last
+  // multiplies with zeros (its weights are whatever the first K of the row holds).
   auto multiply = [&](const bf16x8 (&buf)[FL_AHEAD], int s0) {
+    bf16x8 b[FL_AHEAD][NT];
+#pragma unroll
+    for (int i = 0; i < FL_AHEAD; ++i)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        b[i][t] = *reinterpret_cast<const bf16x8*>(xrow[t] + 32 * min(s0 + i, steps - 1));
 #pragma unroll
     for (int i = 0; i < FL_AHEAD; ++i) {
-      if (s0 + i < steps) {
+      const bool live = s0 + i < steps;
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          const bf16x8 b = *reinterpret_cast<const bf16x8*>(xrow[t] + 32 * (s0 + i));
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf[i], b, acc[t], 0, 0, 0);
-        }
-      }
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf[i], live ? b[i][t] : zero, acc[t], 0, 0, 0);
     }
   };
 
@@ -487,7 +500,7 @@ static size_t fl_lds_bytes(int n, int nt, int kslice, int nw = 4) {
 template <int NT, int EP, int NW, bool SCALED, bool PASSES>
 static int fl_launch_passes(const void* x, const FlOut& out, const void* w, int n, int m, int k, int kslice, int kpass,
                      int nsplit, int tiles, int tiles_per_wg, int x_stride, hipStream_t stream) {
-  const size_t lds = fl_lds_bytes(n, NT, kpass, NW);
+  size_t lds = fl_lds_bytes(n, NT, kpass, NW);
   static size_t allowed = 64 * 1024;          // one per instantiation
   if (lds > allowed) {
     hipError_t e = hipFuncSetAttribute((const void*)fused_linear_kernel<NT, EP, NW, SCALED, PASSES>,

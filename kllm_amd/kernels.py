@@ -755,7 +755,8 @@ def fused_linear_fits(n, k, nsplit=1) -> bool:
 # Passes over K up to which the decode-batch kernel is taken where the rows do not fit into LDS at
 # once, and the rows up to which that pays (a step at 1.1B sizes, 16 tokens: 1.284 -> 1.237 ms; at 8B
 # sizes 8 tokens 4.41 -> 4.08, 16 tokens 5.61 -> 4.75; from 17 rows on, two tiles of rows, the
-# tiled product and a kernel behind it are faster: 1.1B sizes, 24 tokens 1.49 against 1.62 ms).
+# tiled product and a kernel behind it are as fast or faster: 1.1B sizes, 24 tokens 1.47 against
+# 1.48 ms, 32 tokens 1.59 against 1.66; 8B sizes, 24 tokens 5.71 against 6.48).
 FUSED_LINEAR_BEST_PASSES = 4
 FUSED_LINEAR_PASSES_BEST_ROWS = 16
 

@@ -22,12 +22,12 @@
 // the caller splits).  It puts its slice of X, all rows, into LDS once (where
 // they do not fit, in several passes over K, with one tile to a workgroup whose
 // sums stay in registers from pass to pass).  Each
-// of its four waves takes a quarter of the slice: it streams its part of the 16
-// rows of W straight from memory, eight 16-byte loads per lane in flight, the
-// first of them before X is staged, and multiplies with X from LDS
-// (MFMA 16x16x32: A = W tile, B = X^T, D[w row][x row]).  The four partial
-// tiles meet in LDS, are added in a fixed order, and the epilogue runs on the
-// sums; no partial sum crosses memory unless the caller splits K.
+// of its four or eight waves (see fl_waves) takes its share of the slice: it
+// streams its part of the 16 rows of W straight from memory, eight 16-byte loads
+// per lane in flight, the first of them before X is staged, and multiplies with
+// X from LDS (MFMA 16x16x32: A = W tile, B = X^T, D[w row][x row]).  The waves'
+// partial tiles meet in LDS, are added in a fixed order, and the epilogue runs on
+// the sums; no partial sum crosses memory unless the caller splits K.
 //
 // What the 16 MFMA rows of a tile are depends on the epilogue: 16 consecutive
 // rows of W, or 8 pairs (gate row p and up row p; rows j and j + hd/2 of one
@@ -385,7 +385,7 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
     const int tl = tile0 + tile;
     // Neighbouring threads take neighbouring rows of W: their stores share cache lines.
     if (EP == FL_PARTS) {
-      const int r16 = tid % 16, xc = tid / 16;
+      const int r16 = tid % 16, xc = (tid / 16) % 16;       // (with more than four waves the others repeat the stores)
       const long row = (long)tl * 16 + r16;
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
@@ -524,19 +524,40 @@ static int fl_launch(const void* x, const FlOut& out, const void* w, int n, int 
                                                      x_stride, stream);
 }
 
-template <int NT>
-static int fl_launch_ep(int ep, bool scaled, const void* x, const FlOut& out, const void* w, int n, int m, int k,
+template <int NT, int NW>
+static int fl_launch_nw(int ep, bool scaled, const void* x, const FlOut& out, const void* w, int n, int m, int k,
                         int kslice, int kpass, int nsplit, int tiles, int tpw, int xs, hipStream_t st) {
   switch (ep) {
-    case FL_PARTS: return fl_launch<NT, FL_PARTS, 4, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
-    case FL_RESID: return fl_launch<NT, FL_RESID, 4, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
+    case FL_PARTS: return fl_launch<NT, FL_PARTS, NW, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
+    case FL_RESID: return fl_launch<NT, FL_RESID, NW, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
     case FL_SWIGLU:
-      return scaled ? fl_launch<NT, FL_SWIGLU, 4, true>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st)
-                    : fl_launch<NT, FL_SWIGLU, 4, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
+      return scaled ? fl_launch<NT, FL_SWIGLU, NW, true>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st)
+                    : fl_launch<NT, FL_SWIGLU, NW, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
     default:
-      return scaled ? fl_launch<NT, FL_ROPE, 4, true>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st)
-                    : fl_launch<NT, FL_ROPE, 4, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
+      return scaled ? fl_launch<NT, FL_ROPE, NW, true>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st)
+                    : fl_launch<NT, FL_ROPE, NW, false>(x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
   }
+}
+
+template <int NT>
+static int fl_launch_ep(int ep, bool scaled, int nw, const void* x, const FlOut& out, const void* w, int n, int m, int k,
+                        int kslice, int kpass, int nsplit, int tiles, int tpw, int xs, hipStream_t st) {
+  if (nw == 8) return fl_launch_nw<NT, 8>(ep, scaled, x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
+  return fl_launch_nw<NT, 4>(ep, scaled, x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
+}
+
+// Waves of a workgroup.  Eight for the epilogues whose products run on few workgroups, on five
+// eighths of the CUs at most (the residual product: 128 for 2,048 columns; the rotation: 160 for 2,560): a wave's
+// chain of loads is half as long (8 rows of X, 2,048 x 5,632: 9.4 -> 8.2 us; 2,048 x 2,048: 5.2 ->
+// 4.9; a decode step of 8 tokens at 1.1B sizes 1.080 -> 1.042 ms).  Four for the gate, whose
+// workgroups already share their CUs (eight: 1.042 -> 1.078 ms), for the logits (no difference),
+// and wherever eight waves' partial tiles and padding leave no room for the rows of X; sixteen
+// are slower than eight everywhere.
+static int fl_waves(int ep, int n, int kslice, int kpass4, int workgroups) {
+  if (ep != FL_RESID && ep != FL_ROPE) return 4;
+  if (kpass4 < kslice) return 4;                 // rows in passes: measured with four waves only
+  if (8 * workgroups > 5 * device_cus()) return 4;   // (4,096 x 4,096 on 256 workgroups: a step of 8 tokens at 8B sizes 4.09 -> 4.12 ms with eight)
+  return fl_lds_bytes(n, ceil_div(n, 16), kslice, 8) <= (size_t)FL_LDS_MAX ? 8 : 4;
 }
 
 }  // namespace kllm
@@ -688,8 +709,9 @@ extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOu
     out.KV = KV;
     out.hd = hd;
   }
-  const int rc = nt == 1 ? fl_launch_ep<1>(ep, scaled, x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tiles_per_wg, x_stride, stream)
-                         : fl_launch_ep<2>(ep, scaled, x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tiles_per_wg, x_stride, stream);
+  const int nw = fl_waves(ep, n, kslice, kpass, ceil_div(tiles, tiles_per_wg) * nsplit);
+  const int rc = nt == 1 ? fl_launch_ep<1>(ep, scaled, nw, x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tiles_per_wg, x_stride, stream)
+                         : fl_launch_ep<2>(ep, scaled, nw, x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tiles_per_wg, x_stride, stream);
   if (rc) return rc;
   KLLM_CHECK_LAUNCH("fused_linear");
   return 0;

@@ -546,20 +546,6 @@ static int fl_launch_ep(int ep, bool scaled, int nw, const void* x, const FlOut&
   return fl_launch_nw<NT, 4>(ep, scaled, x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tpw, xs, st);
 }
 
-// Waves of a workgroup.  Eight for the epilogues whose products run on few workgroups, on five
-// eighths of the CUs at most (the residual product: 128 for 2,048 columns; the rotation: 160 for 2,560): a wave's
-// chain of loads is half as long (8 rows of X, 2,048 x 5,632: 9.4 -> 8.2 us; 2,048 x 2,048: 5.2 ->
-// 4.9; a decode step of 8 tokens at 1.1B sizes 1.080 -> 1.042 ms).  Four for the gate, whose
-// workgroups already share their CUs (eight: 1.042 -> 1.078 ms), for the logits (no difference),
-// and wherever eight waves' partial tiles and padding leave no room for the rows of X; sixteen
-// are slower than eight everywhere.
-static int fl_waves(int ep, int n, int kslice, int kpass4, int workgroups) {
-  if (ep != FL_RESID && ep != FL_ROPE) return 4;
-  if (kpass4 < kslice) return 4;                 // rows in passes: measured with four waves only
-  if (8 * workgroups > 5 * device_cus()) return 4;   // (4,096 x 4,096 on 256 workgroups: a step of 8 tokens at 8B sizes 4.09 -> 4.12 ms with eight)
-  return fl_lds_bytes(n, ceil_div(n, 16), kslice, 8) <= (size_t)FL_LDS_MAX ? 8 : 4;
-}
-
 }  // namespace kllm
 
 using namespace kllm;
@@ -575,13 +561,32 @@ extern "C" long kllm_fused_linear_lds_bytes(int n, int k, int nsplit) {
 // K of a pass for n rows of a slice of kslice: the slice itself where its rows fit into LDS, else
 // the least number of equal passes (up to FL_MAX_PASSES) whose rows do; 0 if none does.
 constexpr int FL_MAX_PASSES = 8;
-static int fl_pass_k(int n, int kslice) {
+static int fl_pass_k(int n, int kslice, int nw = 4) {
   const int nt = ceil_div(n, 16);
   for (int passes = 1; passes <= FL_MAX_PASSES; ++passes) {
     const int kpass = ceil_div(ceil_div(kslice, passes), 32) * 32;
-    if (fl_lds_bytes(n, nt, kpass) <= (size_t)FL_LDS_MAX) return kpass;
+    if (fl_lds_bytes(n, nt, kpass, nw) <= (size_t)FL_LDS_MAX) return kpass;
   }
   return 0;
+}
+
+// Waves of a workgroup.  Eight for the epilogues whose products run on few workgroups, on five
+// eighths of the CUs at most (the residual product: 128 for 2,048 columns; the rotation: 160 for 2,560): a wave's
+// chain of loads is half as long (8 rows of X, 2,048 x 5,632: 9.4 -> 8.2 us; 2,048 x 2,048: 5.2 ->
+// 4.9; a decode step of 8 tokens at 1.1B sizes 1.080 -> 1.042 ms).  Four for the gate, whose
+// workgroups already share their CUs (eight: 1.042 -> 1.078 ms), for the logits (no difference),
+// and wherever eight waves' partial tiles and padding leave no room for the rows of X; sixteen
+// are slower than eight everywhere.
+static int fl_waves(int ep, int n, int kslice, int kpass4, int workgroups, int tiles_per_wg) {
+  if (ep != FL_RESID && ep != FL_ROPE) return 4;
+  if (8 * workgroups > 5 * device_cus()) return 4;   // (4,096 x 4,096 on 256 workgroups: a step of 8 tokens at 8B sizes 4.09 -> 4.12 ms with eight)
+  // Eight waves' partial tiles and padding take room from the rows of X: they may need a pass
+  // more than four waves would, and still win (13 tokens at 1.1B sizes: 1.172 -> 1.16 ms; 16
+  // tokens, two passes either way: 1.207 -> 1.176), but passes want one tile to a workgroup.
+  // From 17 rows on a pass more loses (28 tokens: 1.59 against 1.55 ms).
+  const int kpass8 = fl_pass_k(n, kslice, 8);
+  if (!kpass8 || (kpass8 < kslice && (tiles_per_wg > 1 || (n > 16 && kpass4 >= kslice)))) return 4;
+  return 8;
 }
 
 extern "C" int kllm_fused_linear_passes(int n, int k, int nsplit) {
@@ -709,9 +714,10 @@ extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOu
     out.KV = KV;
     out.hd = hd;
   }
-  const int nw = fl_waves(ep, n, kslice, kpass, ceil_div(tiles, tiles_per_wg) * nsplit);
-  const int rc = nt == 1 ? fl_launch_ep<1>(ep, scaled, nw, x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tiles_per_wg, x_stride, stream)
-                         : fl_launch_ep<2>(ep, scaled, nw, x, out, w, n, m, k, kslice, kpass, nsplit, tiles, tiles_per_wg, x_stride, stream);
+  const int nw = fl_waves(ep, n, kslice, kpass, ceil_div(tiles, tiles_per_wg) * nsplit, tiles_per_wg);
+  const int kpass_run = nw == 4 ? kpass : fl_pass_k(n, kslice, nw);    // eight waves' partial tiles take room from the rows
+  const int rc = nt == 1 ? fl_launch_ep<1>(ep, scaled, nw, x, out, w, n, m, k, kslice, kpass_run, nsplit, tiles, tiles_per_wg, x_stride, stream)
+                         : fl_launch_ep<2>(ep, scaled, nw, x, out, w, n, m, k, kslice, kpass_run, nsplit, tiles, tiles_per_wg, x_stride, stream);
   if (rc) return rc;
   KLLM_CHECK_LAUNCH("fused_linear");
   return 0;

@@ -32,6 +32,7 @@ class ControlLayout:
     pages: tuple           # table width per cache group
     samples: int = 0       # rows of sampling parameters (temperature, uniform)
     lists: tuple = ()      # (name, count) of the index lists that parts asked for
+    refs: int = 0          # tokens that may take their id from the step sampled last (0 or n)
 
     def sections(self):
         s = [("token_ids", self.n), ("positions", self.n), ("span_of_token", self.n),
@@ -39,6 +40,7 @@ class ControlLayout:
              ("logit_rows", max(self.rows, 1))]
         s += [(f"table{g}", self.spans * m) for g, m in enumerate(self.pages)]
         s += [("temperature", self.samples), ("uniform", self.samples), ("token_from", self.samples)]
+        s += [("token_ref", self.refs)]
         s += [("list:" + name, count) for name, count in self.lists]
         return s
 
@@ -54,21 +56,25 @@ class ControlLayout:
         return self.offsets()[1]
 
 
-def layout_for(lens: Sequence[int], rows: int, pages: tuple, samples: int = 0, lists=None) -> ControlLayout:
+def layout_for(lens: Sequence[int], rows: int, pages: tuple, samples: int = 0, lists=None,
+               refs: bool = False) -> ControlLayout:
     """``lists``: name -> list of ints, the parts' index lists for these spans
-    (only their lengths enter the layout)."""
+    (only their lengths enter the layout).  ``refs``: the step has tokens whose ids are taken
+    from the step sampled last (any step, not only one of single decode tokens, whose
+    ``token_from`` has one entry per sample)."""
     sizes = tuple((name, len(v)) for name, v in (lists or {}).items())
-    return ControlLayout(sum(lens), len(lens), rows, tuple(pages), samples, sizes)
+    return ControlLayout(sum(lens), len(lens), rows, tuple(pages), samples, sizes, sum(lens) if refs else 0)
 
 
 def fill(host: np.ndarray, layout: ControlLayout, tokens: Sequence[Sequence[int]],
          pos0: Sequence[int], slots: Sequence[int], rows: Sequence[int],
          tables: Sequence[Sequence[Sequence[int]]], temperatures=None, uniforms=None,
-         token_from=None, lists=None):
+         token_from=None, lists=None, token_ref=None):
     """Write one step into ``host`` (int32).  ``tables[g][s]`` is span s's
     table in group g.  ``token_from[t] >= 0`` (sampled steps only) says that
     token t's id is not ``tokens`` but the id the last sampled step left on
-    the device at that index."""
+    the device at that index; ``token_ref`` says the same per token for a layout with
+    ``refs``."""
     offs, _ = layout.offsets()
 
     def sec(name):
@@ -104,6 +110,8 @@ def fill(host: np.ndarray, layout: ControlLayout, tokens: Sequence[Sequence[int]
         sec("temperature").view(np.float32)[:] = np.asarray(temperatures, dtype=np.float32)
         sec("uniform").view(np.float32)[:] = np.asarray(uniforms, dtype=np.float32)
         sec("token_from")[:] = -1 if token_from is None else np.asarray(token_from, dtype=np.int32)
+    if layout.refs:
+        sec("token_ref")[:] = -1 if token_ref is None else np.asarray(token_ref, dtype=np.int32)
     return starts
 
 
@@ -123,7 +131,8 @@ def context(dev: torch.Tensor, layout: ControlLayout, runtime, starts, pos0, len
         block_tables=[sec(f"table{g}").view(layout.spans, m) for g, m in enumerate(layout.pages)],
         runtime=runtime, max_span_len=max(lens), all_decode=all(l == 1 for l in lens),
         lists={name: sec("list:" + name) for name, _ in layout.lists},
-        token_from=sec("token_from") if layout.samples and layout.samples == layout.n else None)
+        token_from=(sec("token_ref") if layout.refs
+                    else sec("token_from") if layout.samples and layout.samples == layout.n else None))
 
 
 def sampling_views(dev: torch.Tensor, layout: ControlLayout):

@@ -62,6 +62,7 @@ class EngineOptions:
     attention: str = "auto"               # "auto" or "generic"
     graphs: bool = True                   # replay decode steps as HIP graphs
     max_graph_batch: int = 256            # largest decode batch that is recorded as a graph
+    graph_after_steps: int = 3            # a batch shape is recorded the n-th time it is queued ahead (before: as any step)
     poison_freed_pages: bool = False      # debugging: fill pages with NaN when they are given back
     extra: Dict[str, object] = field(default_factory=dict)
 
@@ -434,7 +435,13 @@ class Engine:
         device, in the order of the entries and of their ``want`` lists, or
         None if nothing is wanted.  Raises OutOfPages (and changes nothing) if
         the cache cannot hold the step's tokens."""
-        arrays = self._validate(entries, allow_refs=False)
+        return self._run(entries, self._validate(entries, allow_refs=False), taps, None)
+
+    def _run(self, entries, arrays, taps, sampling):
+        """The step itself.  ``sampling``: None, or (temperatures, uniforms, token_ref) for a
+        step whose wanted places are sampled on the device into the place where the next
+        step's embedding finds the ids (``token_ref[t] >= 0``: token t's id is what the step
+        sampled last left there at that index)."""
         opened, reserved = self._reserve(entries)
         try:
             rcs, lens, rows, tables = self._describe(entries)
@@ -444,12 +451,19 @@ class Engine:
             for l in lens:
                 span_starts.append(span_starts[-1] + l)
             lists = self.model.step_lists(span_starts, lens)
-            layout = control.layout_for(lens, len(rows), pages, lists=lists)
+            if sampling is None:
+                layout = control.layout_for(lens, len(rows), pages, lists=lists)
+                temps = unis = token_ref = None
+            else:
+                temps, unis, token_ref = sampling
+                layout = control.layout_for(lens, len(rows), pages, samples=len(rows), lists=lists,
+                                            refs=token_ref is not None)
             total = layout.total
             host = self._staging(total)
             pos0 = [rc.length for rc in rcs]
             starts = control.fill(host.numpy(), layout, arrays, pos0,
-                                  [rc.slot for rc in rcs], rows, tables, lists=lists)
+                                  [rc.slot for rc in rcs], rows, tables, temps, unis, lists=lists,
+                                  token_ref=token_ref)
             if self._control is None or self._control.numel() < total:
                 self._control = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
             self._send(host, self._control, total)
@@ -468,9 +482,14 @@ class Engine:
                 ctx = control.context(self._control, layout, self.runtime, starts, pos0, lens)
                 ctx.taps = taps
                 ctx.values = {k: self.kernels.StepValue(v, k) for k, v in values.items()}
+                if sampling is not None:
+                    ctx.sampled = self._graphs.sampled
                 generation = workspace.generation
                 with self.kernels.stream_scope(record=self.records_launches, keep=key is not None) as scope:
                     logits = self.model.run(ctx, self._cache_views(ctx))
+                    if sampling is not None and rows:
+                        t_dev, u_dev = control.sampling_views(self._control, layout)
+                        self.kernels.sample(self._graphs.sampled[:len(rows)], logits, t_dev, u_dev)
                 commands = scope.plan() if key is not None and generation == workspace.generation else None
                 if commands is not None:          # (a step that grew its scratch buffers is kept the next time)
                     self._plans[key] = _StepPlan(commands, logits, workspace.generation, self._control.data_ptr())
@@ -483,28 +502,62 @@ class Engine:
         return logits
 
     def can_sample_ahead(self, entries: Sequence[StepEntry]) -> bool:
-        """Whether ``step_sample_ahead`` takes these entries: single decode
-        tokens of a model whose parts can be replayed as a HIP graph."""
+        """Whether these entries are replayed as a HIP graph: single decode
+        tokens of a model whose parts can be."""
         return (self.options.graphs and self.model.graph_safe
                 and 0 < len(entries) <= self.options.max_graph_batch
                 and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
 
+    def can_queue_ahead(self, entries: Sequence[StepEntry]) -> bool:
+        """Whether ``step_sample_ahead`` takes these entries: any step whose wanted places
+        (one token sampled for each) fit the place where sampled ids are kept."""
+        return 0 < len(entries) and sum(len(e.want) for e in entries) <= self._graphs.sampled.numel()
+
     def step_sample_ahead(self, entries: Sequence[StepEntry], temperatures, uniforms) -> SampledTokens:
-        """Queue a step of single decode tokens and return without waiting for
-        it.  The sampled ids are read from the handle; the *next* step may be
-        queued before that, with ``TokenRef(handle, i)`` in place of the ids."""
-        if not self.can_sample_ahead(entries):
-            raise StepError("only batches of single decode tokens can be queued ahead")
-        return self._graphs.decode(entries, temperatures, uniforms)
+        """Queue a step whose wanted places are sampled on the device and return
+        without waiting for it.  The sampled ids are read from the handle, in the
+        order of the wanted places; the *next* step may be queued before that, with
+        ``TokenRef(handle, i)`` as the only token of an entry in place of the id.
+        Batches of single decode tokens are replayed as HIP graphs, any other step
+        (portions of prompts beside decode tokens) runs from its recorded commands."""
+        if self.can_sample_ahead(entries):
+            # (a shape that was not seen often enough yet runs as any other step does: from its
+            # recorded commands, which costs the host a little more and no recording)
+            out = self._graphs.decode(entries, temperatures, uniforms, wait_for_uses=self.can_queue_ahead(entries))
+            if out is not None:
+                return out
+        if not self.can_queue_ahead(entries):
+            raise StepError(f"a step queued ahead samples at most {self._graphs.sampled.numel()} tokens")
+        arrays = self._validate(entries, allow_refs=True)
+        token_ref = None
+        if any(isinstance(t, TokenRef) for e in entries for t in e.tokens):
+            token_ref = []
+            for e in entries:
+                if len(e.tokens) > 1 and any(isinstance(t, TokenRef) for t in e.tokens):
+                    raise StepError("a TokenRef stands alone in its entry (one decode token)")
+                for t in e.tokens:
+                    if isinstance(t, TokenRef):
+                        last = self._graphs.last
+                        if t.source is not last or not 0 <= t.index < t.source.count:
+                            raise StepError("a TokenRef must name a token of the step that was sampled last")
+                        token_ref.append(t.index)
+                    else:
+                        token_ref.append(-1)
+        count = sum(len(e.want) for e in entries)
+        if len(temperatures) != count or len(uniforms) != count:
+            raise StepError(f"{count} places are wanted, {len(temperatures)} temperatures and "
+                            f"{len(uniforms)} uniforms were given")
+        logits = self._run(entries, arrays, None, (list(temperatures), list(uniforms), token_ref))
+        return self._graphs.handle(count, logits)
 
     def step_sample(self, entries: Sequence[StepEntry], temperatures, uniforms) -> List[int]:
         """A step whose wanted places are sampled on the device: one token per
         wanted place, as host ints.  Batches of single decode tokens are
         replayed as a HIP graph (forward pass and sampling in one launch)."""
         if self.can_sample_ahead(entries):
-            return self._graphs.decode(entries, temperatures, uniforms).tokens()
+            return self.step_sample_ahead(entries, temperatures, uniforms).tokens()
         if any(isinstance(t, TokenRef) for e in entries for t in e.tokens):
-            raise StepError("a TokenRef can only stand in a batch of single decode tokens")
+            return self.step_sample_ahead(entries, temperatures, uniforms).tokens()
         logits = self.step(entries)
         if logits is None:
             return []

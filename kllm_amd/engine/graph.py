@@ -109,6 +109,7 @@ class DecodeGraphs:
         self.sampled = torch.zeros(max(engine.options.max_graph_batch, 1), dtype=torch.int32,
                                    device=engine.device)
         self.last: "SampledTokens | None" = None
+        self.seen: "OrderedDict[tuple, int]" = OrderedDict()   # times a shape was asked for before it had a recording
         self._host_ring = [torch.empty(self.sampled.numel(), dtype=torch.int32, pin_memory=True)
                            for _ in range(4)]
         self._host_owner = [None] * len(self._host_ring)   # the handle that reads from each
@@ -126,10 +127,15 @@ class DecodeGraphs:
             temps, uniforms = control.sampling_views(rec.control, rec.layout)
             K.sample(self.sampled[:rec.layout.n], logits, temps, uniforms)
 
-    def decode(self, entries, temperatures: Sequence[float], uniforms: Sequence[float]) -> SampledTokens:
+    def decode(self, entries, temperatures: Sequence[float], uniforms: Sequence[float],
+               wait_for_uses: bool = False):
         """One token for every entry (each entry is a single decode token, given
         as an id or as a TokenRef to the step sampled last).  Returns at once;
-        the ids are read from the handle."""
+        the ids are read from the handle.  ``wait_for_uses``: a shape without a recording
+        that was asked for fewer than ``EngineOptions.graph_after_steps`` times is counted and
+        left to the caller (None is returned, nothing is changed): recording costs two runs of
+        the step and the instantiation, which a shape that comes by once or twice (a batch that
+        shrinks as its requests end) never earns back."""
         eng = self.engine
         token_from, tokens = [], []
         for e in entries:
@@ -150,6 +156,16 @@ class DecodeGraphs:
             caps = tuple(_bucket(max(len(t) for t in tg)) for tg in tables)
             key = (batch, caps)
             rec = self.recordings.get(key)
+            if rec is None and wait_for_uses:
+                uses = self.seen.get(key, 0) + 1
+                if uses < eng.options.graph_after_steps:
+                    self.seen[key] = uses
+                    self.seen.move_to_end(key)
+                    while len(self.seen) > 4 * self.MAX_RECORDINGS:
+                        self.seen.popitem(last=False)
+                    eng._undo(opened, reserved)
+                    return None
+                self.seen.pop(key, None)
             if rec is None:
                 rec = _Recording(eng, batch, caps)
                 self.recordings[key] = rec
@@ -192,15 +208,25 @@ class DecodeGraphs:
         self.last = out
         return out
 
-    def _read_back(self, batch: int, rec: _Recording) -> SampledTokens:
+    def handle(self, count: int, logits) -> SampledTokens:
+        """The handle of a sampled step that was not one of this class's recordings (its
+        ``count`` ids lie in ``sampled``): the copy to the host queued behind it, and the step
+        remembered as the one sampled last."""
+        out = self._read_back(count, None, logits)
+        if count:
+            self.last = out
+        return out
+
+    def _read_back(self, batch: int, rec, logits=None) -> SampledTokens:
         """Queue the copy of the sampled ids to the host behind the step."""
         i = self._host_next
         self._host_next = (i + 1) % len(self._host_ring)
         if self._host_owner[i] is not None:
             self._host_owner[i].tokens()                # an old handle nobody has read yet: read it now
         host = self._host_ring[i]
-        host[:batch].copy_(self.sampled[:batch], non_blocking=True)
+        if batch:
+            host[:batch].copy_(self.sampled[:batch], non_blocking=True)
         event = torch.cuda.Event()
         event.record()
-        self._host_owner[i] = SampledTokens(host, event, batch, rec.logits, rec)
+        self._host_owner[i] = SampledTokens(host, event, batch, rec.logits if rec is not None else logits, rec)
         return self._host_owner[i]

@@ -31,8 +31,11 @@ Where this scheduler decides differently, and why:
   host reads ids and prepares the next batch.  The price is that an
   end-of-sequence id is seen one step late: the request has then taken one
   more step, whose token is thrown away; its pages are given back when that
-  step is over.  Anything else -- a prompt portion, an admission, a shortage
-  of pages -- first settles the step in flight and then takes the plain path.
+  step is over.  A step with prompt portions in it is queued the same way
+  where the engine takes it (``Engine.can_queue_ahead``): its decode tokens
+  name the ids of the step in flight, its portions are known.  Anything else
+  -- a shortage of pages, a preemption -- first settles the step in flight and
+  then takes the plain path.
 """
 
 from __future__ import annotations
@@ -104,8 +107,9 @@ class Scheduler:
 
     def __init__(self, engine, max_batch: Optional[int] = None,
                  max_step_tokens: Optional[int] = None, chunk_size: Optional[int] = None,
-                 row_multiple: Optional[int] = None):
+                 row_multiple: Optional[int] = None, queue_ahead: bool = True):
         self.engine = engine
+        self.queue_ahead = bool(queue_ahead)     # False: every step waits for the ids of the one before
         # The reference's default batch is 8 (engine/scheduler.go:44-46).
         self.max_batch = int(max_batch) if max_batch else 8
         self.max_step_tokens = int(max_step_tokens) if max_step_tokens else 2048
@@ -287,9 +291,12 @@ class Scheduler:
     def step(self) -> List[tuple]:
         """One iteration: plan, run, sample, finish.  Returns the
         (request id, token) pairs produced."""
-        ahead = self._decode_batch_ahead()
+        ahead = self._decode_batch_ahead() if self.queue_ahead else None
         if ahead is not None:
             return self._queue_ahead(ahead)
+        planned = self._plan_ahead() if self.queue_ahead else None
+        if planned is not None:
+            return self._queue_plan(planned)
         produced = self._settle()                # nothing is in flight below this line
         plan = self.plan()
         if not plan.entries:
@@ -360,6 +367,69 @@ class Scheduler:
             free = [b - a for a, b in zip(need, free)]
         entries = [StepEntry(self._key(r), [0], [0]) for r in self.running]
         return list(self.running) if eng.can_sample_ahead(entries) else None
+
+    def _plan_ahead(self):
+        """The next step's plan, if it can be queued behind the step in flight without
+        a decision that needs that step's ids: no request stands still for want of pages
+        (no preemption), every token is known or is the one token that the step in flight
+        is sampling, and the engine takes the step.  Admits waiting requests (as ``plan``
+        would); changes nothing else."""
+        eng = self.engine
+        if not hasattr(eng, "can_queue_ahead"):
+            return None
+        self._admit()
+        if not self.running:
+            return None
+        entries, blocked = self._try_plan()
+        if blocked is not None or not entries:
+            return None
+        in_flight = {id(r) for r, _ in self._in_flight[1]} if self._in_flight else set()
+        shaped = []
+        for pe in entries:
+            toks = pe.request.all_tokens()[pe.start:pe.start + pe.count]
+            if PENDING in toks and not (pe.count == 1 and id(pe.request) in in_flight):
+                return None
+            shaped.append(StepEntry(self._key(pe.request), [0] * pe.count, [pe.count - 1] if pe.wants_logits else []))
+        return entries if eng.can_queue_ahead(shaped) else None
+
+    def _queue_plan(self, planned: List[PlannedEntry]) -> List[tuple]:
+        """Queue a planned step (portions of prompts, decode tokens), then take in the ids
+        of the step before."""
+        from .graph import TokenRef
+        before = self._in_flight
+        place_before = {id(r): i for i, (r, _) in enumerate(before[1])} if before else {}
+        entries, temps, us, wanting = [], [], [], []
+        for pe in planned:
+            r = pe.request
+            toks = r.all_tokens()[pe.start:pe.start + pe.count]
+            if pe.count == 1 and toks[0] == PENDING:
+                toks = [TokenRef(before[0], place_before[id(r)])]
+            entries.append(StepEntry(self._key(r), toks, [pe.count - 1] if pe.wants_logits else []))
+            if pe.wants_logits:
+                wanting.append(pe)
+                temps.append(r.temperature)
+                us.append(uniform(r.seed, len(r.generated)))
+        try:
+            handle = self.engine.step_sample_ahead(entries, temps, us)
+        except Exception as exc:
+            self._fail_all([pe.request for pe in planned], exc)
+            raise
+        self.stats["steps"] += 1
+        self.stats["tokens"] += sum(pe.count for pe in planned)
+        self.stats["max_batch_seen"] = max(self.stats["max_batch_seen"], len(planned))
+        for pe in planned:
+            key = "decode_tokens" if (pe.count == 1 and pe.request.generated) else "prefill_tokens"
+            self.stats[key] += pe.count
+            pe.request.cursor += pe.count
+        places = []
+        for pe in wanting:
+            r = pe.request
+            places.append((r, len(r.generated)))
+            r.generated.append(PENDING)
+            if len(r.generated) >= r.max_new_tokens:
+                self.running.remove(r)           # its last token is on its way; it takes no further step
+        self._in_flight = (handle, places)
+        return self._take_in(before) if before else []
 
     def _queue_ahead(self, requests: List[Request]) -> List[tuple]:
         """Queue one decode token for each of ``requests``, then take in the

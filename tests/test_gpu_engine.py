@@ -221,6 +221,104 @@ def test_a_step_queued_ahead_takes_its_ids_from_the_device(model_dirs, dtype):
         assert [[step[i] for step in runs[1]] for i in range(3)] == want
 
 
+def test_a_batch_shape_is_recorded_only_when_it_comes_back(model_dirs):
+    """A decode batch is recorded as a graph the third time its shape is queued (two runs of
+    the step and the instantiation are what a recording costs); before that it runs as any
+    step does, from its recorded commands, and gives the same ids.  A scheduler whose batch
+    shrinks as requests end therefore records nothing for shapes that pass once."""
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry, TokenRef
+    cfg, d = tiny.CONFIGS["A"], model_dirs("A")
+    prompts = [tiny.tokens(cfg, n, 70 + i) for i, n in enumerate([9, 33, 4])]
+    runs = []
+    for after in (1, 3):
+        eng = Engine.from_dir(d, EngineOptions(dtype="bfloat16", max_tokens=512, graph_after_steps=after))
+        h = eng.step_sample_ahead([StepEntry(i, p, [len(p) - 1]) for i, p in enumerate(prompts)], [0.0] * 3, [0.0] * 3)
+        out, recorded = [], []
+        for _ in range(6):
+            h2 = eng.step_sample_ahead([StepEntry(i, [TokenRef(h, i)], [0]) for i in range(3)], [0.0] * 3, [0.0] * 3)
+            out.append(h.tokens())
+            recorded.append(eng._graphs.captures)
+            h = h2
+        out.append(h.tokens())
+        assert recorded == ([1] * 6 if after == 1 else [0, 0, 1, 1, 1, 1])
+        runs.append(out)
+    assert runs[0] == runs[1]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_steps_with_prompt_portions_are_queued_ahead_too(model_dirs, dtype):
+    """Any step can be queued before the ids of the step before it have reached the host:
+    a portion of a prompt beside decode tokens that name those ids (TokenRef), a prompt's last
+    portion whose first token is sampled on the device.  The ids are the ones that the same
+    steps give when every step waits for the one before and is fed from the host."""
+    from kllm_amd.engine import Engine, EngineOptions, StepEntry, TokenRef, StepError
+    cfg, d = tiny.CONFIGS["B"], model_dirs("B")
+    a, b, c = (tiny.tokens(cfg, n, 90 + n) for n in (21, 40, 7))
+    temps = {"a": 0.0, "b": 0.7, "c": 0.0}
+
+    def u(k):
+        return [0.11 * ((k * 7 + i) % 9) for i in range(3)]
+    runs = []
+    for ahead in (False, True):
+        eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=512))
+        take = eng.step_sample_ahead if ahead else (lambda e, t, w: eng.step_sample(e, t, w))
+        seen = []
+        # step 0: a whole, the first portion of b
+        h0 = take([StepEntry("a", a, [len(a) - 1]), StepEntry("b", b[:16], [])], [temps["a"]], u(0)[:1])
+        ref = (lambda h, i: TokenRef(h, i)) if ahead else (lambda h, i: h[i])
+        # step 1: a decodes the id of step 0, b's second portion, c whole
+        h1 = take([StepEntry("a", [ref(h0, 0)], [0]), StepEntry("b", b[16:32], []), StepEntry("c", c, [len(c) - 1])],
+                  [temps["a"], temps["c"]], u(1)[:2])
+        seen.append(h0.tokens() if ahead else h0)
+        # step 2: a and c decode, b's last portion gives its first token
+        h2 = take([StepEntry("a", [ref(h1, 0)], [0]), StepEntry("c", [ref(h1, 1)], [0]),
+                   StepEntry("b", b[32:], [len(b) - 33])], [temps["a"], temps["c"], temps["b"]], u(2))
+        seen.append(h1.tokens() if ahead else h1)
+        before = h2
+        for k in range(3, 9):                  # all three decode: replayed graphs from here on
+            h = take([StepEntry("a", [ref(before, 0)], [0]), StepEntry("c", [ref(before, 1)], [0]),
+                      StepEntry("b", [ref(before, 2)], [0])], [temps["a"], temps["c"], temps["b"]], u(k))
+            seen.append(before.tokens() if ahead else before)
+            before = h
+        seen.append(before.tokens() if ahead else before)
+        if ahead:
+            with pytest.raises(StepError, match="stands alone"):
+                eng.step_sample_ahead([StepEntry("a", [TokenRef(before, 0), 3], [1])], [0.0], [0.0])
+            with pytest.raises(StepError, match="sampled last"):
+                eng.step_sample_ahead([StepEntry("a", [TokenRef(h1, 0)], [0]), StepEntry("b", [5, 6], [1])],
+                                      [0.0, 0.0], [0.0, 0.0])
+        runs.append(seen)
+    assert runs[0] == runs[1]
+    if dtype == "float32":                      # the greedy request against the plain implementation
+        w = tiny.read_weights(d, as_stored_in=dtype)
+        assert [s[0] for s in runs[1]] == P.generate_greedy(w, cfg, a, len(runs[1]))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_scheduler_queues_steps_with_portions_ahead(model_dirs, dtype):
+    """Prompts in portions beside decoding requests, more requests than places: with every
+    step queued behind the one in flight the scheduler gives the tokens it gives when it waits
+    for each step, and it does queue steps with portions in them ahead."""
+    from kllm_amd.engine import Engine, EngineOptions
+    from kllm_amd.engine.scheduler import Scheduler
+    cfg, d = tiny.CONFIGS["A"], model_dirs("A")
+    prompts = [tiny.tokens(cfg, n, 30 + n) for n in (50, 9, 33, 70, 4, 21)]
+    got = []
+    for ahead in (False, True):
+        eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=1024))
+        queued = []
+        inner = eng.step_sample_ahead
+        eng.step_sample_ahead = lambda e, t, w: (queued.append(any(len(x.tokens) > 1 for x in e)), inner(e, t, w))[1]
+        sched = Scheduler(eng, max_batch=4, max_step_tokens=24, chunk_size=16, queue_ahead=ahead)
+        ids = [sched.submit(list(p), 18, temperature=0.6 if i % 2 else 0.0, seed=i) for i, p in enumerate(prompts)]
+        results = sched.run_until_done()
+        assert all(results[i].error is None and len(results[i].tokens) == 18 for i in ids)
+        assert not eng.cache.requests and all(p.free_pages == p.num_pages for p in eng.cache.pools)
+        assert (sum(queued) > 5) == ahead       # steps with portions went ahead, or none did
+        got.append([results[i].tokens for i in ids])
+    assert got[0] == got[1]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_steps_run_again_from_their_recorded_commands(model_dirs, dtype):
     """A step's launches go to the library as one buffer of commands, and a step whose shape

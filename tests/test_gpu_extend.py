@@ -343,7 +343,8 @@ def test_decode_steps_of_the_windowed_model_as_graphs(dtype):
         outs = {}
         for mode in ("eager", "graph"):
             eng = Engine.from_random(cfg, 3, EngineOptions(dtype=dtype, num_pages=24, max_model_len=1 << 20,
-                                                           poison_freed_pages=True), std=0.05, norm_std=0.1)
+                                                           poison_freed_pages=True, graph_after_steps=1),
+                                     std=0.05, norm_std=0.1)
             eng.step([StepEntry(r, reqs[r][:prompt[r]], []) for r in reqs])
             got = []
             for k in range(37):

@@ -189,7 +189,7 @@ def test_all_decode_stretches_of_random_traces_as_graphs(tmp_path, dtype):
             folders[name] = tiny.write_model(str(tmp_path / name), cfg, seed=len(folders))
         pool = peak + page * min(4, len(requests))
         options = EngineOptions(dtype=dtype, max_tokens=pool, max_model_len=1 << 30,
-                                poison_freed_pages=True, page_size=page)
+                                poison_freed_pages=True, page_size=page, graph_after_steps=1)
         eager = Replayer(folders[name], dtype, pool, options=options)
         want = [eager.step(s["entries"], s["end"]) for s in steps]
         eng = Engine.from_dir(folders[name], options)
@@ -220,7 +220,7 @@ def test_a_token_reference_in_flight_across_a_change_of_table_width(tmp_path, dt
         prompts = [tiny.tokens(cfg, n, 90 + i) for i, n in enumerate(lens)]
         B = len(prompts)
         options = EngineOptions(dtype=dtype, max_tokens=sum(lens) + B * (new + 2 * page), max_model_len=1 << 30,
-                                page_size=page)
+                                page_size=page, graph_after_steps=1)
         runs = {}
         for mode in ("eager", "ahead"):
             eng = Engine.from_dir(folder, options)

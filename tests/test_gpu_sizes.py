@@ -77,7 +77,7 @@ def engine(name, dtype, **opts):
     from kllm_amd.engine import Engine, EngineOptions
     from kllm_amd.weights.loader import target_dtype
     raw = SIZES[name]
-    options = EngineOptions(dtype=dtype, max_model_len=1 << 30, poison_freed_pages=True, **opts)
+    options = EngineOptions(dtype=dtype, max_model_len=1 << 30, poison_freed_pages=True, graph_after_steps=1, **opts)
     compute = options.torch_dtype()
     w = weights(name)
 

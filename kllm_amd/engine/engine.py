@@ -136,6 +136,9 @@ class Engine:
                               and not options.extra.get("no_repeated_steps"))
         self._plans: "OrderedDict[tuple, _StepPlan]" = OrderedDict()
         self.steps_repeated = 0
+        # ... and within a step that is walked through, layers that are alike share the walk
+        # (extra["no_repeated_layers"] switches that off, for comparison).
+        self.model.repeat_layers(self.records_launches and not options.extra.get("no_repeated_layers"))
         self._graphs = DecodeGraphs(self)
         # What a scheduler should know of the kernels: a step's tokens are the rows of every
         # product, and those work on tiles of this many rows.

@@ -47,6 +47,8 @@ class Model:
         self.cache_plan = self._plan_cache()
         self._list_providers = None
         self._value_providers = None
+        self._repeater = None          # set by ``repeat_layers``
+        self.runs_repeated = 0         # runs of the schedule that were not walked through
 
     # ------------------------------------------------------------------ cache plan
     def _plan_cache(self) -> CachePlan:
@@ -94,6 +96,7 @@ class Model:
     def bind(self, weights: Dict[str, torch.Tensor]) -> None:
         for p in self.parts():
             p.bind(weights)
+        self.runtime.tensors_changed()
 
     def all_parts(self):
         """Every part of the model, those inside arrangements and the shared ones included."""
@@ -137,6 +140,12 @@ class Model:
             for name, value in part.step_values(list(starts), list(lens), list(positions)).items():
                 out[f"{key}.{name}"] = int(value)
         return out
+
+    def repeat_layers(self, on: bool = True) -> None:
+        """Whether runs of layers that are alike share the host's work within a step (see
+        ``repeat.LayerRepeater``); only a model whose steps are ``repeatable`` takes it."""
+        from .repeat import LayerRepeater
+        self._repeater = LayerRepeater(self) if on and self.repeatable else None
 
     @property
     def repeatable(self) -> bool:
@@ -199,16 +208,27 @@ class Model:
         if ctx.taps is not None:
             K.flush_recorded()                    # the copies below are torch's: behind what was recorded
             ctx.taps.append(x.clone())
-        pending = None
-        for i, run in enumerate(self.schedule):
-            block = self.blocks[run.layer]
+        def walk_through(i, x, pending):
+            block = self.blocks[self.schedule[i].layer]
             if getattr(block, "takes_next_norm", False) and i + 1 < len(self.schedule):
                 # the norm that will take this layer's output, if the next layer names one
                 nxt = self.blocks[self.schedule[i + 1].layer]
                 first = nxt.first_norm() if hasattr(nxt, "first_norm") else None
-                x, pending = call_part(block, block.forward, ctx, x, pending, cache_views[i], next_norm=first)
-            else:
-                x, pending = call_part(block, block.forward, ctx, x, pending, cache_views[i])
+                return call_part(block, block.forward, ctx, x, pending, cache_views[i], next_norm=first)
+            return call_part(block, block.forward, ctx, x, pending, cache_views[i])
+
+        pending = None
+        # runs whose layers are alike are walked through twice a step, the others' commands
+        # are those of the first with their own tensors' addresses
+        repeater = self._repeater.step(ctx, cache_views) if self._repeater is not None else None
+        for i in range(len(self.schedule)):
+            if repeater is not None:
+                x, pending = repeater.run(i, x, pending, walk_through)
+                if i + 1 == len(self.schedule):
+                    x, pending = repeater.current(x, pending)
+                    self.runs_repeated += repeater.repeated
+                continue
+            x, pending = walk_through(i, x, pending)
             if ctx.taps is not None:
                 if pending is not None:
                     call_part(self.final_norm, self.final_norm.add, ctx, x, pending)

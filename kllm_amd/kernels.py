@@ -302,6 +302,7 @@ class _Recorder:
         self.ops = _ops()
         self.run = library().kllm_run_commands
         self.launched = 0
+        self.copy = None            # a RecordedRun that takes a copy of every command added, or None
 
     def _room(self, need):
         if self.at + need > self.cap:
@@ -332,12 +333,31 @@ class _Recorder:
             total = op.size
             self._room(total)
         op.pack.pack_into(self.buf, self.at, op.index | (op.nargs << 16) | ((total // 8) << 32), *args)
+        copy = self.copy
         if self.keep and op.dynamic:
             for i in op.dynamic:
                 if type(args[i]) is StepValue:
                     self.patches.append((self.kept_bytes + self.at + 8 + 8 * i, args[i].name))
+                    if copy is not None:
+                        copy.patches.append((len(copy.data) + 8 + 8 * i, args[i].name))
+        if copy is not None:
+            copy.data += self.buf[self.at:self.at + total]
+            copy.names.append(what)
         self.at += total
         self.names.append(what)
+        if len(self.names) >= self.chunk:
+            self.flush()
+
+    def add_commands(self, data, names, patches=()):
+        """Commands that are written already (``data``: their bytes in the buffer's layout,
+        ``names``: what each is, ``patches``: (byte offset in data, name) of the step's values
+        in them), behind what was recorded so far."""
+        self._room(len(data))
+        self.buf[self.at:self.at + len(data)] = data
+        if self.keep:
+            self.patches.extend((self.kept_bytes + self.at + off, name) for off, name in patches)
+        self.at += len(data)
+        self.names.extend(names)
         if len(self.names) >= self.chunk:
             self.flush()
 
@@ -357,6 +377,42 @@ class _Recorder:
             library().kllm_last_error(buf, 512)
             raise KernelError(f"{what}: {buf.value.decode(errors='replace')} (code {rc}; command {failed.value} "
                               f"of {len(names)} recorded, the ones before it have run)")
+
+
+class RecordedRun:
+    """A copy of the commands that a stretch of a recording scope added (see ``copy_recorded``):
+    their bytes, what each is, and where the step's values (``StepValue``) sit in them."""
+
+    def __init__(self):
+        self.data, self.names, self.patches = bytearray(), [], []
+
+
+class copy_recorded:
+    """Inside, every command that this thread records is also copied into ``self.run`` (a
+    ``RecordedRun``); ``self.run`` is None outside a recording scope, and ``whole`` is False
+    afterwards if something inside was launched past the recording."""
+
+    def __enter__(self):
+        self._rec = getattr(_scoped, "recorder", None)
+        self.run, self.whole = None, False
+        if self._rec is not None and self._rec.copy is None:
+            self.run = self._rec.copy = RecordedRun()
+            self._bypassed = self._rec.bypassed
+            self._rec.bypassed = False
+        return self
+
+    def __exit__(self, *exc):
+        if self.run is not None:
+            self._rec.copy = None
+            self.whole = not self._rec.bypassed and getattr(_scoped, "recorder", None) is self._rec
+            self._rec.bypassed = self._rec.bypassed or self._bypassed
+        return False
+
+
+def add_recorded(data, names, patches=()):
+    """Add commands that are written already to this thread's recording (``RecordedRun``'s
+    fields, possibly changed)."""
+    _scoped.recorder.add_commands(data, names, patches)
 
 
 def flush_recorded():

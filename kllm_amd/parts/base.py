@@ -129,10 +129,16 @@ class Runtime:
     workspace: Workspace = None
     options: Dict[str, Any] = field(default_factory=dict)
     shared: Dict[int, Any] = field(default_factory=dict)   # parts used by several layers
+    tensor_epoch: int = 0                   # grows when parts may hold other tensors than before
 
     def __post_init__(self):
         if self.workspace is None:
             self.workspace = Workspace(self.device)
+
+    def tensors_changed(self):
+        """A part that puts another tensor in the place of one it holds, other than in
+        ``bind``, says so here: addresses that were looked up before are looked up again."""
+        self.tensor_epoch += 1
 
     def shared_part(self, category: str, spec: PartSpec):
         """The one instance of a part that several layers name with the same

@@ -211,6 +211,7 @@ class LayerRepeater:
         self.worthwhile = any(k is not None for k in self.keys)
         self._names: Dict[int, _Names] = {}
         self._epoch = None
+        self.last = None
 
     def names(self, i) -> _Names:
         epoch = self.model.runtime.tensor_epoch
@@ -235,7 +236,8 @@ class LayerRepeater:
         the residual stream is tapped layer by layer)."""
         if not self.worthwhile or ctx.taps is not None or not K.recording():
             return None
-        return _StepRepeater(self, ctx, cache_views)
+        self.last = _StepRepeater(self, ctx, cache_views)      # (kept for whoever asks why a step was walked through)
+        return self.last
 
 
 class _StepRepeater:
@@ -247,6 +249,7 @@ class _StepRepeater:
         self.off = False
         self.stale = None        # (template, index): x and pending are the template's, standing for that run's
         self.repeated = 0
+        self.why: List[str] = []  # what ended the repeating, of the step or of a kind of run
 
     # -- what the model's loop calls
     def run(self, i, x, pending, call):
@@ -279,12 +282,15 @@ class _StepRepeater:
             out = call(i, x, pending)
         if copied.run is None or not copied.whole or self.workspace.generation != self.generation:
             self.off = True              # launches past the recording, or buffers that moved: no more of this
+            self.why.append(f"run {i}: " + ("a scratch buffer grew" if self.workspace.generation != self.generation
+                                            else "something was launched past the recording"))
             return out
         try:
             gave_shape = _shape(out, names)
         except _Unnamed:
             self.templates[key] = t = t or _Template(i, copied.run, None, None, None, None)
             t.dead = True
+            self.why.append(f"run {i}: it gave something that holds a part of another layer, or an object without attributes")
             return out
         if t is None:
             self.templates[key] = _Template(i, copied.run, (x, pending), out, given_shape, gave_shape)
@@ -307,6 +313,9 @@ class _StepRepeater:
         if (given_shape != t.given_shape or gave_shape != t.gave_shape or len(a.data) != len(b.data)
                 or a.names != b.names or a.patches != b.patches or len(a.data) % 8):
             t.dead = True
+            self.why.append(f"runs {t.index} and {j}: " + (
+                "they were given other buffers" if given_shape != t.given_shape else
+                "they gave other buffers" if gave_shape != t.gave_shape else "they launched other kernels"))
             return
         wa = np.frombuffer(bytes(a.data), dtype=np.uint64)
         wb = np.frombuffer(bytes(b.data), dtype=np.uint64)
@@ -320,6 +329,7 @@ class _StepRepeater:
                 self.owner.forget(j)
         if found is None:
             t.dead = True
+            self.why.append(f"runs {t.index} and {j}: their commands differ in a word that no tensor of the layers explains")
             return
         t.words = wa
         t.at = np.array([f[0] for f in found], dtype=np.int64)

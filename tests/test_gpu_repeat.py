@@ -230,6 +230,8 @@ def test_scratch_buffers_that_alternate_between_layers_end_the_repeating(dtype, 
         outs = replay_both(engs, steps)
         assert check_rows(steps, outs, want, tiny.TOL[dtype]) == 87
         assert engs[0].model.runs_repeated == 0
+        why = engs[0].model._repeater.last.why
+        assert why and all("buffers" in w or "no tensor" in w for w in why), why
     finally:
         unregister_architecture("ToyTurningForCausalLM")
         unregister_part("feed_forward", "toy_turning")

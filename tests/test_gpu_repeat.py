@@ -101,6 +101,31 @@ def test_repeated_layers_in_steps_that_run_again_from_their_commands(dtype):
     assert engs[0].steps_repeated - before >= 30 and engs[0].model.runs_repeated >= 3
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_repeated_layers_in_a_recorded_graph(dtype):
+    """A batch of decode tokens recorded as a HIP graph: the recording walks through two
+    layers of a kind as any step does; its replays sample what the walked engine samples."""
+    from kllm_amd.engine import StepEntry, TokenRef
+    cfg = DEEP["M"]
+    engs = engines(cfg, dtype, max_tokens=1024, max_model_len=256, graph_after_steps=1)
+    prompts = {rid: tiny.tokens(cfg, n, seed) for seed, (rid, n) in enumerate([("a", 40), ("b", 9), ("c", 75)])}
+    for rid, toks in prompts.items():
+        for e in engs:
+            e.step([StepEntry(rid, toks, [])])
+    before = engs[0].model.runs_repeated
+    last, ids = [None, None], [[3, 4, 5], [3, 4, 5]]
+    for step in range(24):
+        for k, e in enumerate(engs):
+            entries = [StepEntry(rid, [ids[k][j] if last[k] is None else TokenRef(last[k], j)], [0])
+                       for j, rid in enumerate(prompts)]
+            last[k] = e.step_sample_ahead(entries, [0.0, 0.7, 1.3], [0.0, 0.31 + 0.01 * step, 0.77])
+        got = [h.tokens() for h in last]
+        assert got[0] == got[1], step
+        assert torch.equal(last[0].logits, last[1].logits), step
+    assert engs[0]._graphs.captures >= 1 and sum(r.replays for r in engs[0]._graphs.recordings.values()) >= 20
+    assert engs[0].model.runs_repeated > before            # (both runs of a recording: 2 x 6 of 10 layers)
+
+
 def build_windows_in_turn(cfg: LlamaConfig) -> ModelSpec:
     from kllm_amd.models.llama import build_llama
     spec = build_llama(cfg)

@@ -368,6 +368,10 @@ class _StepRepeater:
 
     # -- every further run
     def _repeat(self, t: _Template, i, x, pending, chained) -> bool:
+        if self.workspace.generation != self.generation:
+            self.off = True              # a run of another kind made a scratch buffer grow: the first run's addresses are gone
+            self.why.append(f"run {i}: a scratch buffer grew")
+            return False
         names = self.owner.names(i)
         if names.parts.keys() != self.owner.names(t.index).parts.keys():
             return False
@@ -387,7 +391,8 @@ class _StepRepeater:
                 values.append(tensor.data_ptr())
             else:
                 address = names.address.get(path)
-                if address is None:
+                if address is None:              # a tensor that this layer makes when it is first walked through:
+                    self.owner.forget(i)         # walked through now, looked up again the next time
                     return False
                 values.append(address)
         words = t.words.copy()

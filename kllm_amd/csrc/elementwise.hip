@@ -245,9 +245,17 @@ __device__ __forceinline__ floatx4 sum_splits4(const float* __restrict__ p, int 
   return v;
 }
 
+constexpr int kRopeRun = 16;   // neighbouring tokens whose workgroups share an XCD in the kernel below
+
 // The same for float32 sums (whole, or partial sums over slices of K) and head sizes that are
 // multiples of 8: a thread takes four neighbouring pairs, or four values, with 16-byte loads,
 // and its loads go out before the token's page is looked up, so that the two waits overlap.
+// Workgroups are numbered so that a run of kRopeRun neighbouring tokens stays on one XCD (the
+// XCDs take workgroups round-robin).  Of a run, `chunks` workgroups per token rotate queries
+// and keys (a token's row of each is contiguous in q_out and in its page); `vblocks` more take
+// the values of all its tokens, 64 elements of every token each, lanes of neighbouring tokens
+// side by side: a value's place in its page is two bytes beside its neighbour token's, so
+// sixteen lanes fill a 32-byte sector where a workgroup per token would write two bytes of it.
 template <typename T>
 __global__ void rope_append_vec_kernel(const float* __restrict__ qkv, int nsplit, long split_stride,
                                        T* __restrict__ q_out,
@@ -255,59 +263,62 @@ __global__ void rope_append_vec_kernel(const float* __restrict__ qkv, int nsplit
                                        T* __restrict__ cache, const int* __restrict__ positions,
                                        const int* __restrict__ span_of_token,
                                        const int* __restrict__ block_table, int max_pages,
-                                       int page_size, int H, int KV, int hd) {
+                                       int page_size, int H, int KV, int hd, int n, int chunks,
+                                       int vblocks, int xcds) {
   typedef T tx4 __attribute__((ext_vector_type(4)));
-  const long t = blockIdx.x;
+  const int xcd = blockIdx.x % xcds, seq = blockIdx.x / xcds;
+  const int per_run = kRopeRun * chunks + vblocks;
+  const int at = seq % per_run;
+  const long t0 = ((long)(seq / per_run) * xcds + xcd) * kRopeRun;
   const int half = hd / 2;
   const int qd = H * hd, kvd = cache ? KV * hd : 0;
+  const long block = (long)page_size * hd;
+  if (at >= kRopeRun * chunks) {
+    // values: thread = (token of the run, four neighbouring elements)
+    const long t = t0 + threadIdx.x % kRopeRun;
+    const int idx = (at - kRopeRun * chunks) * (4 * kThreads / kRopeRun) + (threadIdx.x / kRopeRun) * 4;
+    if (t >= n || idx >= kvd) return;
+    const floatx4 a = sum_splits4(qkv + t * (qd + 2 * kvd) + qd + kvd + idx, nsplit, split_stride);
+    const int pos = positions[t];
+    const int page = block_table[(long)span_of_token[t] * max_pages + pos / page_size];
+    const int h = idx / hd, j = idx % hd;
+    T* v = cache + (((long)page * 2 + 1) * KV + h) * block + pos % page_size;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[(long)(j + e) * page_size] = from_f32<T>(a[e]);
+    return;
+  }
+  const long t = t0 + at % kRopeRun;
+  if (t >= n) return;
   const float* in = qkv + t * (qd + 2 * kvd);
   const int q_items = H * half / 4, k_items = cache ? KV * half / 4 : 0;
-  const int items = q_items + k_items + kvd / 4;
-  const int item = blockIdx.y * blockDim.x + threadIdx.x;
-  if (item >= items) return;
-  const bool rotated = item < q_items + k_items;
+  const int item = (at / kRopeRun) * blockDim.x + threadIdx.x;
+  if (item >= q_items + k_items) return;
   const bool is_q = item < q_items;
-  int h, j;
-  floatx4 a, b = {0, 0, 0, 0}, cc = {1, 1, 1, 1}, sn = {0, 0, 0, 0};
-  if (rotated) {
-    const int idx = (is_q ? item : item - q_items) * 4;
-    h = idx / half;
-    j = idx % half;
-    const float* src = in + (is_q ? 0 : qd) + h * hd + j;
-    a = sum_splits4(src, nsplit, split_stride);
-    b = sum_splits4(src + half, nsplit, split_stride);
-    if (cos_t) {
-      cc = *reinterpret_cast<const floatx4*>(cos_t + t * half + j);
-      sn = *reinterpret_cast<const floatx4*>(sin_t + t * half + j);
-    }
-  } else {
-    const int idx = (item - q_items - k_items) * 4;
-    h = idx / hd;
-    j = idx % hd;
-    a = sum_splits4(in + qd + kvd + idx, nsplit, split_stride);
+  const int idx = (is_q ? item : item - q_items) * 4;
+  const int h = idx / half, j = idx % half;
+  const float* src = in + (is_q ? 0 : qd) + h * hd + j;
+  const floatx4 a = sum_splits4(src, nsplit, split_stride);
+  const floatx4 b = sum_splits4(src + half, nsplit, split_stride);
+  floatx4 cc = {1, 1, 1, 1}, sn = {0, 0, 0, 0};
+  if (cos_t) {
+    cc = *reinterpret_cast<const floatx4*>(cos_t + t * half + j);
+    sn = *reinterpret_cast<const floatx4*>(sin_t + t * half + j);
   }
   int page = 0, slot = 0;
-  if (cache && !is_q) {
+  if (!is_q) {
     const int pos = positions[t];
     page = block_table[(long)span_of_token[t] * max_pages + pos / page_size];
     slot = pos % page_size;
   }
-  const long block = (long)page_size * hd;
-  if (rotated) {
-    tx4 lo, hi;
+  tx4 lo, hi;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      lo[e] = from_f32<T>(a[e] * cc[e] - b[e] * sn[e]);
-      hi[e] = from_f32<T>(b[e] * cc[e] + a[e] * sn[e]);
-    }
-    T* o = is_q ? q_out + t * qd + h * hd : cache + (((long)page * 2 + 0) * KV + h) * block + (long)slot * hd;
-    *reinterpret_cast<tx4*>(o + j) = lo;
-    *reinterpret_cast<tx4*>(o + j + half) = hi;
-  } else {
-    T* v = cache + (((long)page * 2 + 1) * KV + h) * block + slot;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) v[(long)(j + e) * page_size] = from_f32<T>(a[e]);
+  for (int e = 0; e < 4; ++e) {
+    lo[e] = from_f32<T>(a[e] * cc[e] - b[e] * sn[e]);
+    hi[e] = from_f32<T>(b[e] * cc[e] + a[e] * sn[e]);
   }
+  T* o = is_q ? q_out + t * qd + h * hd : cache + (((long)page * 2 + 0) * KV + h) * block + (long)slot * hd;
+  *reinterpret_cast<tx4*>(o + j) = lo;
+  *reinterpret_cast<tx4*>(o + j + half) = hi;
 }
 
 // out[t, i] = act(gate[t, i]) * up[t, i], gate = cols [0, f), up = cols [f, 2f)
@@ -442,9 +453,13 @@ static int launch_rope_append(const void* qkv, int nsplit, long split_stride, vo
       (nsplit == 1 || split_stride % 4 == 0) && (H * hd + (cache ? 2 * KV * hd : 0)) % 4 == 0 &&
       ((uintptr_t)q_out & 15) == 0 && (!cache || ((uintptr_t)cache & 15) == 0) &&
       (!cos_t || (((uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0)) {
-    hipLaunchKernelGGL((rope_append_vec_kernel<T>), dim3(n, ceil_div(items, 4 * kThreads)), dim3(kThreads), 0,
+    const int pairs = H * (hd / 2) + (cache ? KV * (hd / 2) : 0);
+    const int vchunks = ceil_div(pairs, 4 * kThreads), xcds = device_xcds();
+    const int vblocks = cache ? ceil_div((long)KV * hd, 4 * kThreads / kRopeRun) : 0;
+    const long runs = ceil_div(ceil_div(n, kRopeRun), xcds) * xcds;     // padded: every XCD gets as many
+    hipLaunchKernelGGL((rope_append_vec_kernel<T>), dim3(runs * (kRopeRun * vchunks + vblocks)), dim3(kThreads), 0,
                        stream, (const float*)qkv, nsplit, split_stride, (T*)q_out, cos_t, sin_t, (T*)cache, positions, span_of_token,
-                       block_table, max_pages, page_size, H, KV, hd);
+                       block_table, max_pages, page_size, H, KV, hd, n, vchunks, vblocks, xcds);
     KLLM_CHECK_LAUNCH("rope_append");
     return 0;
   }

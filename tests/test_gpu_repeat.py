@@ -14,7 +14,7 @@ import plain_llama as P
 import tiny
 import traces
 from kllm_amd.config import LlamaConfig, register_architecture, unregister_architecture
-from kllm_amd.parts import LayerSpec, ModelSpec, Part, PartSpec, Run, register_part, unregister_part
+from kllm_amd.parts import ModelSpec, Part, PartSpec, Run, register_part, unregister_part
 
 pytestmark = pytest.mark.gpu
 

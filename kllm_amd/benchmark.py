@@ -94,6 +94,8 @@ class DecodeLoop:
 
     def __init__(self, engine: Engine, rids, first_tokens):
         self.engine, self.rids, self.toks = engine, list(rids), list(first_tokens)
+        # steady decoding is what is timed: the batch's graph is recorded in the warm-up
+        self._graph_after, engine.options.graph_after_steps = engine.options.graph_after_steps, 1
         self.zeros = [0.0] * len(self.rids)
         self.ahead = engine.can_sample_ahead([StepEntry(r, [t], [0]) for r, t in zip(self.rids, self.toks)])
 
@@ -123,6 +125,7 @@ class DecodeLoop:
     def release(self):
         for r in self.rids:
             self.engine.release(r)
+        self.engine.options.graph_after_steps = self._graph_after
 
 
 def measure_decode(engine: Engine, batch: int, context_end: int, steps: int, warmup: int):

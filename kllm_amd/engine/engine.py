@@ -62,7 +62,7 @@ class EngineOptions:
     attention: str = "auto"               # "auto" or "generic"
     graphs: bool = True                   # replay decode steps as HIP graphs
     max_graph_batch: int = 256            # largest decode batch that is recorded as a graph
-    graph_after_steps: int = 3            # a batch shape is recorded the n-th time it is queued ahead (before: as any step)
+    graph_after_steps: int = 8            # a batch shape is recorded the n-th time it is queued ahead (before: as any step)
     poison_freed_pages: bool = False      # debugging: fill pages with NaN when they are given back
     extra: Dict[str, object] = field(default_factory=dict)
 

@@ -222,8 +222,8 @@ def test_a_step_queued_ahead_takes_its_ids_from_the_device(model_dirs, dtype):
 
 
 def test_a_batch_shape_is_recorded_only_when_it_comes_back(model_dirs):
-    """A decode batch is recorded as a graph the third time its shape is queued (two runs of
-    the step and the instantiation are what a recording costs); before that it runs as any
+    """A decode batch is recorded as a graph the n-th time its shape is queued (here the third;
+    two runs of the step and the instantiation are what a recording costs); before that it runs as any
     step does, from its recorded commands, and gives the same ids.  A scheduler whose batch
     shrinks as requests end therefore records nothing for shapes that pass once."""
     from kllm_amd.engine import Engine, EngineOptions, StepEntry, TokenRef
@@ -305,7 +305,7 @@ def test_the_scheduler_queues_steps_with_portions_ahead(model_dirs, dtype):
     prompts = [tiny.tokens(cfg, n, 30 + n) for n in (50, 9, 33, 70, 4, 21)]
     got = []
     for ahead in (False, True):
-        eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=1024))
+        eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=1024, graph_after_steps=2))
         queued = []
         inner = eng.step_sample_ahead
         eng.step_sample_ahead = lambda e, t, w: (queued.append(any(len(x.tokens) > 1 for x in e)), inner(e, t, w))[1]
@@ -414,7 +414,7 @@ def test_no_collection_of_garbage_falls_into_a_recording(model_dirs):
     gc.callbacks.append(watch)
     try:
         for _ in range(2):
-            eng = Engine.from_dir(d, EngineOptions(dtype="float32", max_tokens=128))
+            eng = Engine.from_dir(d, EngineOptions(dtype="float32", max_tokens=128, graph_after_steps=1))
             gc.set_threshold(1, 1, 1)
             outs.append(eng.generate(prompt, 6))
             gc.set_threshold(*before)
@@ -600,7 +600,7 @@ def test_generation_when_pages_run_out(model_dirs, dtype):
     cfg, d = tiny.CONFIGS["A"], model_dirs("A")
     prompts = [tiny.tokens(cfg, n, 50 + n) for n in (40, 33, 50, 20)]
     new = 30
-    eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=176, poison_freed_pages=True))
+    eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=176, poison_freed_pages=True, graph_after_steps=2))
     sched = Scheduler(eng, max_batch=4, max_step_tokens=64)
     ids = [sched.submit(list(p), new, seed=i) for i, p in enumerate(prompts)]
     results = sched.run_until_done()

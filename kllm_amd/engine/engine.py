@@ -440,14 +440,15 @@ class Engine:
         the cache cannot hold the step's tokens."""
         return self._run(entries, self._validate(entries, allow_refs=False), taps, None)
 
-    def _run(self, entries, arrays, taps, sampling):
+    def _run(self, entries, arrays, taps, sampling, reserved=None):
         """The step itself.  ``sampling``: None, or (temperatures, uniforms, token_ref) for a
         step whose wanted places are sampled on the device into the place where the next
         step's embedding finds the ids (``token_ref[t] >= 0``: token t's id is what the step
-        sampled last left there at that index)."""
-        opened, reserved = self._reserve(entries)
+        sampled last left there at that index).  ``reserved``: a ``ReservedStep`` whose pages
+        are reserved already."""
+        opened, reserved_ids = (reserved.opened, reserved.reserved) if reserved is not None else self._reserve(entries)
         try:
-            rcs, lens, rows, tables = self._describe(entries)
+            rcs, lens, rows, tables = reserved.described if reserved is not None else self._describe(entries)
             # table widths in powers of two, as recorded steps have them: few distinct layouts
             pages = tuple(table_bucket(max(len(t) for t in tg)) for tg in tables)
             span_starts = [0]
@@ -499,7 +500,7 @@ class Engine:
                     while len(self._plans) > self.MAX_STEP_PLANS:
                         self._plans.popitem(last=False)
         except Exception:
-            self._undo(opened, reserved)
+            self._undo(opened, reserved_ids)
             raise
         self._commit(entries)
         return logits
@@ -523,12 +524,19 @@ class Engine:
         ``TokenRef(handle, i)`` as the only token of an entry in place of the id.
         Batches of single decode tokens are replayed as HIP graphs, any other step
         (portions of prompts beside decode tokens) runs from its recorded commands."""
+        count = sum(len(e.want) for e in entries)
+        if len(temperatures) != count or len(uniforms) != count:
+            raise StepError(f"{count} places are wanted, {len(temperatures)} temperatures and "
+                            f"{len(uniforms)} uniforms were given")
         if self.can_sample_ahead(entries):
             # (a shape that was not seen often enough yet runs as any other step does: from its
             # recorded commands, which costs the host a little more and no recording)
             out = self._graphs.decode(entries, temperatures, uniforms, wait_for_uses=self.can_queue_ahead(entries))
-            if out is not None:
+            if isinstance(out, SampledTokens):
                 return out
+            logits = self._run(entries, out.arrays, None, (list(temperatures), list(uniforms), out.token_ref),
+                               reserved=out)
+            return self._graphs.handle(count, logits)
         if not self.can_queue_ahead(entries):
             raise StepError(f"a step queued ahead samples at most {self._graphs.sampled.numel()} tokens")
         arrays = self._validate(entries, allow_refs=True)
@@ -546,10 +554,6 @@ class Engine:
                         token_ref.append(t.index)
                     else:
                         token_ref.append(-1)
-        count = sum(len(e.want) for e in entries)
-        if len(temperatures) != count or len(uniforms) != count:
-            raise StepError(f"{count} places are wanted, {len(temperatures)} temperatures and "
-                            f"{len(uniforms)} uniforms were given")
         logits = self._run(entries, arrays, None, (list(temperatures), list(uniforms), token_ref))
         return self._graphs.handle(count, logits)
 

@@ -75,6 +75,17 @@ class SampledTokens:
         return self._ids
 
 
+class ReservedStep:
+    """A step whose entries are checked and whose pages are reserved, on its way to
+    ``Engine._run``: the entries' ids as arrays, where their ids come from on the device
+    (or None), and what ``Engine._reserve`` and ``Engine._describe`` returned."""
+    __slots__ = ("arrays", "token_ref", "opened", "reserved", "described")
+
+    def __init__(self, arrays, token_ref, opened, reserved, described):
+        self.arrays, self.token_ref = arrays, token_ref
+        self.opened, self.reserved, self.described = opened, reserved, described
+
+
 class TokenRef:
     """In place of a token id in a step's entry: "what ``source`` chose at
     ``index``", for a source that is the step sampled last."""
@@ -133,8 +144,9 @@ class DecodeGraphs:
         as an id or as a TokenRef to the step sampled last).  Returns at once;
         the ids are read from the handle.  ``wait_for_uses``: a shape without a recording
         that was asked for fewer than ``EngineOptions.graph_after_steps`` times is counted and
-        left to the caller (None is returned, nothing is changed): recording costs two runs of
-        the step and the instantiation, which a shape that comes by once or twice (a batch that
+        left to the caller: a ``ReservedStep`` is returned, the entries checked and their pages
+        reserved, which the caller runs (``Engine._run``) or undoes.  Recording costs two runs of
+        the step and the instantiation, which a shape that comes by a few times (a batch that
         shrinks as its requests end) never earns back."""
         eng = self.engine
         token_from, tokens = [], []
@@ -148,10 +160,10 @@ class DecodeGraphs:
             else:
                 token_from.append(-1)
                 tokens.append([int(t)])
-        eng._validate(entries)
+        arrays = eng._validate(entries)
         opened, reserved = eng._reserve(entries)
         try:
-            rcs, lens, rows, tables = eng._describe(entries)
+            described = rcs, lens, rows, tables = eng._describe(entries)
             batch = len(entries)
             caps = tuple(_bucket(max(len(t) for t in tg)) for tg in tables)
             key = (batch, caps)
@@ -163,8 +175,8 @@ class DecodeGraphs:
                     self.seen.move_to_end(key)
                     while len(self.seen) > 4 * self.MAX_RECORDINGS:
                         self.seen.popitem(last=False)
-                    eng._undo(opened, reserved)
-                    return None
+                    # (what was checked and reserved goes with the step, not back)
+                    return ReservedStep(arrays, token_from if max(token_from) >= 0 else None, opened, reserved, described)
                 self.seen.pop(key, None)
             if rec is None:
                 rec = _Recording(eng, batch, caps)

@@ -167,6 +167,45 @@ def test_rope_append(dtype, H, KV, hd, ps, nsplit):
     assert (q2.cpu().double() - qkv[0, :, :qd].cpu().double()).abs().max() < tol(dtype) * 4
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,KV,hd,ps,nsplit", [(8, 8, 128, 16, 1), (32, 4, 64, 16, 3), (5, 5, 48, 32, 2), (2, 2, 256, 8, 1)])
+def test_rope_append_many_tokens(dtype, H, KV, hd, ps, nsplit):
+    """Hundreds of tokens in three spans that begin inside a page and cross many: the kernel
+    takes runs of 16 neighbouring tokens, which here begin and end anywhere in spans and pages,
+    and the values of a run are written by lanes side by side; the last run is not full."""
+    theta = 10000.0
+    spans = [(21, 150), (0, 37), (100, 118)]
+    n = sum(l for _, l in spans)
+    pos = torch.tensor([p0 + i for p0, l in spans for i in range(l)], dtype=torch.int32, device=DEV)
+    sot = torch.tensor([s for s, (_, l) in enumerate(spans) for _ in range(l)], dtype=torch.int32, device=DEV)
+    width = max(-(-(p0 + l) // ps) for p0, l in spans)
+    order = torch.randperm(3 * width, generator=torch.Generator().manual_seed(3)).tolist()
+    tables = [order[s * width:(s + 1) * width] for s in range(3)]
+    bt = torch.tensor(tables, dtype=torch.int32, device=DEV)
+    qd, kvd = H * hd, KV * hd
+    qkv = rnd(nsplit, n, qd + 2 * kvd, seed=6)
+    cos = torch.empty(n, hd // 2, device=DEV)
+    sin = torch.empty(n, hd // 2, device=DEV)
+    K().rope_tables(cos, sin, pos, hd, theta)
+    cache = torch.full((3 * width, 2, KV, ps * hd), float("nan"), dtype=dtype, device=DEV)
+    q_out = torch.empty(n, qd, dtype=dtype, device=DEV)
+    K().rope_append(qkv, q_out, cos, sin, cache, pos, sot, bt, ps, H, KV, hd)
+    full = qkv.cpu().double().sum(0)
+    want_q = P.rope(full[:, :qd], pos.cpu().tolist(), H, hd, theta)
+    want_k = P.rope(full[:, qd:qd + kvd], pos.cpu().tolist(), KV, hd, theta)
+    want_v = full[:, qd + kvd:]
+    assert (q_out.cpu().double() - want_q).abs().max() < tol(dtype) * 4
+    off, written = 0, 0
+    for s, (p0, l) in enumerate(spans):
+        k, v = read_cache(cache, tables[s], p0 + l, KV, hd, ps)
+        assert (k[p0:].double() - want_k[off:off + l]).abs().max() < tol(dtype) * 4
+        assert (v[p0:].double() - want_v[off:off + l]).abs().max() < tol(dtype) * 4
+        assert torch.isnan(k[:p0]).all() and torch.isnan(v[:p0]).all()
+        off += l
+        written += l
+    assert int((~torch.isnan(cache)).sum()) == 2 * written * kvd          # nothing else was written
+
+
 # ------------------------------------------------------------------ silu gate
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -88,15 +88,18 @@ def test_a_second_run_is_explained_by_its_own_tensors():
     (na, _, _), (nb, _, _), (nc, _, _) = names_of(1, rt), names_of(2, rt), names_of(3, rt)
     table = torch.zeros(4, dtype=torch.int32)
     va, vb = (PagedCacheView(torch.zeros(1024), table, 16) for _ in range(2))
-    scratch = torch.zeros(8).data_ptr()
+    held = torch.zeros(8)
+    scratch = held.data_ptr()
     wa, wb = words_of(na, va, scratch), words_of(nb, vb, scratch)
     found = R._StepRepeater._explain(wa, wb, na, nb, va, vb)
     assert [(i, p) for i, p, _ in found if p[0] != "c"] == [(1, ("b", "w")), (5, ("n", "more", "'gu'", "data"))]
-    assert sorted((i, p, o) for i, p, o in found if p[0] == "c") == [(6, ("c", "pages"), 256), (7, ("c", "block_table"), 0)]
+    # (the table both views share is the same word in both runs: it may be named or left as it is)
+    in_views = sorted((i, p, o) for i, p, o in found if p[0] == "c")
+    assert in_views[0] == (6, ("c", "pages"), 256) and in_views[1:] in ([], [(7, ("c", "block_table"), 0)])
     assert [o for i, p, o in found if i == 1] == [64]
     # a word that differs and is no tensor's address (a scratch buffer that alternates): no
     other = wb.copy()
-    other[2] = torch.zeros(8).data_ptr() or 1
+    other[2] = wb[2] + np.uint64(1 << 20)
     assert R._StepRepeater._explain(wa, other, na, nb, va, vb) is None
     # a word that names a tensor of the first run's layer, where the second names another tensor of its own: no
     other = wb.copy()
@@ -143,3 +146,55 @@ def test_what_a_block_gave_is_handed_on_in_another_runs_name():
         raise AssertionError
     except R._Unnamed:
         pass
+
+
+def test_recorded_commands_are_copied_and_added_with_their_step_values():
+    """The recording side of repeated layers: commands written inside ``copy_recorded`` are also
+    kept apart, with the places of the step's values in them, and ``add_recorded`` puts such
+    commands behind what was recorded, the places moved along.  Nothing is launched here: the
+    recording is dropped, not run (the library is only asked for its table of entry points)."""
+    import pytest
+    from kllm_amd import kernels as K
+    try:
+        K._ops()
+    except Exception as exc:                       # no built library where this runs
+        pytest.skip(f"the kernel library is not there: {exc}")
+    rec = K._Recorder(stream=0, chunk=10 ** 9, keep=True)
+    K._scoped.recorder = rec
+    try:
+        n_args = K._ops()["kllm_attn_prefill"].nargs
+        dynamic = K._ops()["kllm_attn_prefill"].dynamic
+        args = [1000 + i for i in range(n_args)]
+        args[14] = 0.125                                              # the scale, a float
+        args[dynamic[0]], args[dynamic[1]] = K.StepValue(777, "keys.total"), K.StepValue(55, "keys.longest")
+        K._launch("kllm_attn_prefill", "before", *args)
+        first = rec.at
+        with K.copy_recorded() as copied:
+            K._launch("kllm_attn_prefill", "attention", *args)
+            K._launch("kllm_silu_mul", "gate", 1, 2, 3, 4, 5, 6, 7, 8, 9, 0)
+        assert copied.whole and copied.run.names == ["attention", "gate"]
+        assert bytes(copied.run.data) == bytes(rec.buf[first:rec.at])
+        assert copied.run.patches == [(8 + 8 * dynamic[0], "keys.total"), (8 + 8 * dynamic[1], "keys.longest")]
+        assert rec.patches[2:] == [(first + off, name) for off, name in copied.run.patches]
+        # the same commands again, as a layer that is alike would add them
+        words = np.frombuffer(bytes(copied.run.data), dtype=np.uint64).copy()
+        words[1] = 424242                                              # the first argument of the first command
+        second = rec.at
+        K.add_recorded(words.tobytes(), copied.run.names, copied.run.patches)
+        assert rec.names == ["before", "attention", "gate", "attention", "gate"]
+        assert int(np.frombuffer(bytes(rec.buf[second:second + 16]), dtype=np.uint64)[1]) == 424242
+        assert bytes(rec.buf[second + 16:rec.at]) == bytes(copied.run.data[16:])
+        assert rec.patches[4:] == [(second + off, name) for off, name in copied.run.patches]
+        # something launched past the recording inside: the copy is not whole
+        with K.copy_recorded() as broken:
+            K._launch("kllm_silu_mul", "gate", 1, 2, 3, 4, 5, 6, 7, 8, 9, 0)
+            rec.bypassed = True                                        # (what bypass_recorded and direct_launches leave)
+        assert not broken.whole and rec.bypassed
+        # outside a recording there is nothing to copy
+        K._scoped.recorder = None
+        with K.copy_recorded() as nothing:
+            pass
+        assert nothing.run is None and not nothing.whole
+    finally:
+        rec.names = []                                                 # dropped, not run
+        K._scoped.recorder = None

@@ -33,6 +33,9 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 
   const int r = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const float* row = logits + (long)r * vocab;
+  // (asked for here, so that the trip to memory runs beside the logits')
+  const float temp = temperature ? temperature[r] : 0.f;
+  const float u = uniform ? uniform[r] : 0.f;
   // Each thread owns one contiguous segment, so thread order is index order.
   // Segments are multiples of four logits, so that a row whose length is one too is read
   // in 16-byte pieces, eight of them in flight per thread.
@@ -78,7 +81,6 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   int arg = wave_idx[0];
   for (int w = 1; w < kSampleWaves; ++w)
     if (wave_idx[w] < vocab && (arg == vocab || wave_val[w] > mx)) { mx = wave_val[w]; arg = wave_idx[w]; }
-  const float temp = temperature ? temperature[r] : 0.f;
   if (!(temp > 0.f)) {
     if (tid == 0) out[r] = arg;
     return;
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   const float prev = __shfl_up(incl, 1, kWave);
   const float excl = before + (lane == 0 ? 0.f : prev);
   incl += before;
-  const float target = uniform[r] * total;
+  const float target = u * total;
   if (sum > 0.f && target >= excl && target < incl) {
     float c = excl;
     int idx = hi - 1;

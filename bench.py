@@ -15,7 +15,7 @@ Other workloads, each printing one JSON line of its own (``--model`` chooses the
 
     --workload decode-run      prompts of 512 tokens decoded to 2,048: mean tok/s over the run
                                and at context lengths 512, 1280 and 2047 (--batch)
-    --workload prefill-chunks  a 2,048-token prompt in portions of --chunk tokens
+    --workload prefill-chunks  a prompt of --context tokens (2,048) in portions of --chunk tokens
     --workload mixed           --requests prompts of 128 to 2,048 tokens through the scheduler,
                                prefilled in portions of --chunk tokens beside decode tokens
     --kernel NAME --shape a,b,..   one kernel alone (gemm n,m,k; gemm_swiglu n,f,k; attn_prefill
@@ -81,13 +81,13 @@ def main(argv=None):
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     elem = 2 if args.dtype == "bfloat16" else 4
-    if args.workload != "headline":
-        return other_workload(args, cfg, full_layers, B)
-    max_batch = args.batch if args.no_points else max(args.batch, 64)
     extra = {}
     for item in filter(None, args.extra.split(",")):
         key, _, val = item.partition("=")
         extra[key] = int(val) if val.lstrip("-").isdigit() else (val or True)
+    if args.workload != "headline":
+        return other_workload(args, cfg, full_layers, B, extra)
+    max_batch = args.batch if args.no_points else max(args.batch, 64)
     eng = B.make_engine(cfg, args.dtype, max_tokens=max_batch * args.context + 4096, max_requests=max_batch,
                         max_model_len=args.context + 64, gemm=args.gemm, page_size=args.page_size, extra=extra)
 
@@ -148,7 +148,7 @@ def main(argv=None):
     return 0
 
 
-def other_workload(args, cfg, full_layers, B):
+def other_workload(args, cfg, full_layers, B, extra):
     import torch
     elem = 2 if args.dtype == "bfloat16" else 4
     base = {"workload": args.workload, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
@@ -162,14 +162,15 @@ def other_workload(args, cfg, full_layers, B):
         worst = eng.step_read_bytes([args.context - 1] * args.batch)
         base["frac_of_hbm_at_end"] = round(worst * res["at"][max(res["at"])] / args.batch / 1e9 / B.PEAK_HBM_GBS, 4)
     elif args.workload == "prefill-chunks":
-        eng = B.make_engine(cfg, args.dtype, max_tokens=2 * 2048 + 4096, max_model_len=2048 + 64, gemm=args.gemm,
-                            page_size=args.page_size)
-        ms = B.measure_prefill_chunks(eng, 2048, args.chunk, reps=3, warmup=1)
-        whole = B.measure_prefill(eng, 2048)
-        flops = eng.model.step_flops(2048, 2048 * 2049 / 2.0, 1)
-        base.update(tokens=2048, chunk=args.chunk, ms=round(ms, 3), tok_s=round(2048e3 / ms, 1),
-                    frac=round(flops / (ms * 1e-3) / B.PEAK_FLOPS[args.dtype], 4),
-                    whole_prompt_ms=round(whole, 3))
+        tokens = args.context                      # the prompt's length (2,048 unless --context says otherwise)
+        eng = B.make_engine(cfg, args.dtype, max_tokens=2 * tokens + 4096, max_model_len=tokens + 64, gemm=args.gemm,
+                            page_size=args.page_size, extra=extra)
+        ms = B.measure_prefill_chunks(eng, tokens, args.chunk, reps=3 if tokens <= 8192 else 2, warmup=1)
+        flops = eng.model.step_flops(tokens, tokens * (tokens + 1) / 2.0, 1)
+        base.update(tokens=tokens, chunk=args.chunk, ms=round(ms, 3), tok_s=round(tokens * 1e3 / ms, 1),
+                    frac=round(flops / (ms * 1e-3) / B.PEAK_FLOPS[args.dtype], 4))
+        if tokens <= 8192:                         # (a longer prompt in one step wants scratch buffers of its own size)
+            base["whole_prompt_ms"] = round(B.measure_prefill(eng, tokens), 3)
     else:
         # room for every request's prompt and new tokens at once (no preemption in the timed run)
         tokens = args.requests * (2048 + args.new_tokens + args.page_size)

@@ -12,22 +12,20 @@ namespace kllm {
 // every read is a trip to memory: all reads of sixteen slices (maxima, sums and this lane's
 // DV elements of each output) go out together, and every lane works out the weights for
 // itself, so that sixteen slices cost one trip and no exchange between lanes.  Further
-// rounds of sixteen (long contexts) are merged with a running maximum.
-template <typename T, int DV>   // DV: elements of a head per lane (head size up to 64 DV)
-__global__ __launch_bounds__(64) void attn_merge_kernel(T* __restrict__ out,
-                                                        const float* __restrict__ part, int H, int hd,
-                                                        int nslices, const int* __restrict__ token_list) {
-  const int t = token_list ? token_list[blockIdx.x] : blockIdx.x;
-  const int h = blockIdx.y, lane = threadIdx.x;
+// rounds of sixteen (long contexts) are merged with a running maximum.  (R: the slices of a
+// round, for callers with few.)
+template <typename T, int DV, int R = 16>   // DV: elements of a head per lane (head size up to 64 DV); R: slices a round
+__device__ __forceinline__ void attn_merge_one(T* __restrict__ out, const float* __restrict__ part, int t, int h, int H,
+                                               int hd, int nslices, int lane) {
   const int stride = hd + 2;
   const float* p = part + ((long)t * H + h) * nslices * stride;
   float M = -INFINITY, denom = 0.f, o[DV];
 #pragma unroll
   for (int v = 0; v < DV; ++v) o[v] = 0.f;
-  for (int s0 = 0; s0 < nslices; s0 += 16) {
-    float ms[16], ls[16], os[DV][16];
+  for (int s0 = 0; s0 < nslices; s0 += R) {
+    float ms[R], ls[R], os[DV][R];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
+    for (int j = 0; j < R; ++j) {
       const float* q = p + (long)(s0 + j < nslices ? s0 + j : 0) * stride;   // beyond the last slice: a valid address
       ms[j] = q[hd];
       ls[j] = q[hd + 1];
@@ -36,7 +34,7 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(T* __restrict__ out,
     }
     float m = M;
 #pragma unroll
-    for (int j = 0; j < 16; ++j)
+    for (int j = 0; j < R; ++j)
       if (s0 + j < nslices) m = fmaxf(m, ms[j]);
     if (m == -INFINITY) continue;                      // nothing but empty slices so far
     const float keep = expf(M - m);                    // 0 in the first round that holds a key
@@ -44,7 +42,7 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(T* __restrict__ out,
 #pragma unroll
     for (int v = 0; v < DV; ++v) o[v] *= keep;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
+    for (int j = 0; j < R; ++j) {
       if (s0 + j < nslices && ms[j] != -INFINITY) {
         const float w = expf(ms[j] - m);
         denom += w * ls[j];
@@ -57,6 +55,14 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(T* __restrict__ out,
 #pragma unroll
   for (int v = 0; v < DV; ++v)
     if (lane + 64 * v < hd) out[((long)t * H + h) * hd + lane + 64 * v] = from_f32<T>(o[v] / denom);
+}
+
+template <typename T, int DV>
+__global__ __launch_bounds__(64) void attn_merge_kernel(T* __restrict__ out,
+                                                        const float* __restrict__ part, int H, int hd,
+                                                        int nslices, const int* __restrict__ token_list) {
+  const int t = token_list ? token_list[blockIdx.x] : blockIdx.x;
+  attn_merge_one<T, DV>(out, part, t, blockIdx.y, H, hd, nslices, threadIdx.x);
 }
 
 // Launches the merge for `count` tokens (all, or those that token_list names).

@@ -42,6 +42,7 @@
 #include <type_traits>
 
 #include "attention_f32.hpp"
+#include "attention_merge.hpp"
 #include "common.hpp"
 #include "kllm_kernels.h"
 
@@ -52,6 +53,8 @@ constexpr int kQueryBlock = 32 * kPrefillWaves;   // queries of a workgroup
 // Limits of the division-free page arithmetic (page_magic in the first kernel).
 constexpr int kPrefillMaxPage = 2048;
 constexpr int kPrefillMaxKeys = 1 << 24;
+constexpr int kPrefillMaxSlices = 4;              // workgroups that may share out the keys of one block and head
+constexpr int kPrefillSliceFromKeys = 1280;       // ... when the longest block reads at least this many
 
 template <int HDT>
 struct PrefillShape {
@@ -72,7 +75,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ query_tiles, int n_tiles, const int* __restrict__ span_start,
     const int* __restrict__ span_pos, const int* __restrict__ block_table, int max_pages,
-    int page_size, unsigned page_magic, int H, int KV, int window, float scale) {
+    int page_size, unsigned page_magic, int H, int KV, int window, float scale, float* __restrict__ part) {
   typedef PrefillShape<HDT> S;
   constexpr int hd = S::hd, KS = S::KS, NB = S::NB, KT = S::KT, KLD = S::KLD, VLD = S::VLD, CPT = S::CPT;
   extern __shared__ __attribute__((aligned(16))) bf16_t tiles_lds[];   // [PAR][2][kBuf]
@@ -129,8 +132,12 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
 
   const int kb0 = lowest / 32 * 32;
   const int ntiles_all = (blk_qmax - kb0) / KT + 1;
-  const int ntiles = (ntiles_all + PAR - 1) / PAR;          // steps of the loop: the same for both groups
-  auto tile_key = [&](int t) { return kb0 + KT * (PAR * t + par); };   // first key of this group's t-th tile
+  // The tiles go in turn to the slices (workgroups of the same block and head, blockIdx.y: where
+  // the blocks alone leave CUs idle) and, within a slice, to the groups of waves.
+  const int nslices = gridDim.y, slice = blockIdx.y;
+  const int ntiles = (ntiles_all + PAR * nslices - 1) / (PAR * nslices);   // steps of the loop: the same for all
+  auto tile_no = [&](int t) { return nslices * (PAR * t + par) + slice; };
+  auto tile_key = [&](int t) { return kb0 + KT * tile_no(t); };   // first key of this group's t-th tile
   // page and slot of a key: a shift and a mask when the page size is a power of two
   // Page of a key without a division: page_magic = ceil(2^35 / page_size) from the host, exact
   // for keys below 2^24 and pages of up to 2,048 tokens (kPrefillMaxKeys, checked at the launch).
@@ -169,7 +176,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
 #pragma unroll
     for (int j = 0; j < CPT; ++j) {
       const int key0 = tile_key(t) + 16 * half_of[j];
-      const bool ok = PAR * t + par < ntiles_all && key_ok(key0);
+      const bool ok = tile_no(t) < ntiles_all && key_ok(key0);
       // A vector load although the address is the same in every lane: a scalar load would be
       // counted together with the LDS operations, and every wait for LDS would wait for it.
       int index = ok ? page_index(key0) : 0;
@@ -201,7 +208,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     return T;
   };
   auto stash = [&](const Stage& T, int t, bf16_t* buf) {
-    if (PAR * t + par >= ntiles_all) return;
+    if (tile_no(t) >= ntiles_all) return;
     const int kb = tile_key(t);
     const bool v_edge = kb < first_page_key || kb + KT > kv_len;   // slots that may hold anything
 #pragma unroll
@@ -395,7 +402,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     if (par == 1) return;
     const float m1 = mine[(HDT * 16) * kWave], l1 = mine[(HDT * 16 + 1) * kWave];
     const float M = fmaxf(m, m1);
-    // M is finite for a lane with a query: one of the groups holds the query's own key
+    // (M is -inf where neither group had a key for the lane's query: a slice of the keys that ends before it)
     const float w0 = (M == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m - M) * c2);   // exp2(-inf) = 0
     const float w1 = (M == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m1 - M) * c2);
     l = l * w0 + l1 * w1;
@@ -403,8 +410,25 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     for (int r = 0; r < HDT; ++r)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[r][i] = acc[r][i] * w0 + mine[(16 * r + i) * kWave] * w1;
+    m = M;
   }
   if (!active || c >= nq) return;
+  if (nslices > 1) {
+    // Keys in slices: the slice's sums as they are, with its maximum (in units of the scaled
+    // scores, as the merge takes it) and its sum of probabilities; a slice without a key for
+    // this query leaves a maximum of -inf.  Rows of hd + 2 floats are 8-byte aligned.
+    float* prow = part + (((long)tq * H + h) * nslices + slice) * (hd + 2);
+#pragma unroll
+    for (int r = 0; r < HDT; ++r)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        float* dst = prow + 32 * r + 8 * b + 4 * g;
+        *reinterpret_cast<floatx2*>(dst) = floatx2{acc[r][4 * b], acc[r][4 * b + 1]};
+        *reinterpret_cast<floatx2*>(dst + 2) = floatx2{acc[r][4 * b + 2], acc[r][4 * b + 3]};
+      }
+    if (g == 0) *reinterpret_cast<floatx2*>(prow + hd) = floatx2{m * scale, l};
+    return;
+  }
   const float inv = 1.f / l;                                  // finite: a query reads its own key
   bf16_t* orow = out + ((long)tq * H + h) * hd;
 #pragma unroll
@@ -416,6 +440,22 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
       for (int j = 0; j < 4; ++j) v[j] = (bf16_t)(acc[r][4 * b + j] * inv);
       *reinterpret_cast<bf16x4*>(orow + 32 * r + 8 * b + 4 * g) = v;
     }
+}
+
+// The merge of the slices' results, one wave per (query, head); a block's queries are the
+// rows from its first to the end of its span, at most kQueryBlock.
+constexpr int kMergeWaves = 8;   // (query, head) pairs of a workgroup of the merge below
+
+template <int DV>
+__global__ __launch_bounds__(64 * kMergeWaves) void attn_prefill_merge_kernel(
+    bf16_t* __restrict__ out, const float* __restrict__ part, const int* __restrict__ query_tiles,
+    const int* __restrict__ span_start, int H, int hd, int nslices) {
+  const int tile = blockIdx.x / kQueryBlock;
+  const int t = query_tiles[2 * tile] + blockIdx.x % kQueryBlock;
+  if (t >= span_start[query_tiles[2 * tile + 1] + 1]) return;
+  const int h = blockIdx.y * kMergeWaves + threadIdx.x / kWave;
+  if (h >= H) return;
+  attn_merge_one<bf16_t, DV, 4>(out, part, t, h, H, hd, nslices, threadIdx.x % kWave);
 }
 
 // ---------------------------------------------------------------------------
@@ -688,7 +728,7 @@ template <int HDT, int PAR>
 static void launch_prefill_par(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
                                const int* query_tiles, int n_tiles, const int* span_start,
                                const int* span_pos, const int* block_table, int max_pages, int page_size,
-                               int H, int KV, int window, float scale) {
+                               int H, int KV, int window, float scale, float* part = nullptr, int nslices = 1) {
   typedef PrefillShape<HDT> S;
   const size_t lds = (size_t)PAR * 2 * S::kBuf * sizeof(bf16_t);   // also holds the groups' merge
   static int raised = 0;
@@ -698,9 +738,14 @@ static void launch_prefill_par(int grid, hipStream_t stream, const void* q, void
     raised = 1;
   }
   const unsigned page_magic = (unsigned)(((1UL << 35) + page_size - 1) / page_size);   // ceil(2^35 / page_size)
-  hipLaunchKernelGGL((attn_prefill_mfma_kernel<HDT, PAR>), dim3(grid), dim3(64 * kPrefillWaves * PAR), lds, stream,
+  hipLaunchKernelGGL((attn_prefill_mfma_kernel<HDT, PAR>), dim3(grid, nslices), dim3(64 * kPrefillWaves * PAR), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, query_tiles, n_tiles,
-                     span_start, span_pos, block_table, max_pages, page_size, page_magic, H, KV, window, scale);
+                     span_start, span_pos, block_table, max_pages, page_size, page_magic, H, KV, window, scale, part);
+  if (nslices > 1) {
+    const dim3 mgrid(n_tiles * kQueryBlock, ceil_div(H, kMergeWaves));
+    hipLaunchKernelGGL((attn_prefill_merge_kernel<(HDT + 1) / 2>), mgrid, dim3(64 * kMergeWaves), 0, stream,
+                       (bf16_t*)out, part, query_tiles, span_start, H, 32 * HDT, nslices);
+  }
 }
 
 template <int HDT>
@@ -742,8 +787,18 @@ template <int HDT>
 static void launch_prefill(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
                            const int* query_tiles, int n_tiles, const int* span_start,
                            const int* span_pos, const int* block_table, int max_pages, int page_size,
-                           int H, int KV, int window, float scale, long keys_total, int keys_longest) {
+                           int H, int KV, int window, float scale, long keys_total, int keys_longest,
+                           float* part, int nslices) {
   const int cus = device_cus();
+  // (the caller asked kllm_attn_prefill_slices: few blocks of a large head.  The slices' results
+  // pass through memory and a second kernel, about 10 us for 512 queries of 32 heads; they pay
+  // from about 1,280 keys to the longest block on, see there.)
+  if (nslices > 1 && keys_longest >= kPrefillSliceFromKeys) {
+    launch_prefill_par<HDT, PrefillShape<HDT>::kMaxPar>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start,
+                                                        span_pos, block_table, max_pages, page_size, H, KV, window,
+                                                        scale, part, nslices);
+    return;
+  }
   bool chain_bound = true;
   if (keys_total > 0 && keys_longest > 0)   // tiles of a CU's share of all blocks against the longest block's
     chain_bound = 5 * (keys_total * H / cus) < 6 * (long)keys_longest;
@@ -763,11 +818,27 @@ static void launch_prefill(int grid, hipStream_t stream, const void* q, void* ou
 
 using namespace kllm;
 
+// Slices of the keys over workgroups (with a merge behind them) for a step of n_tiles blocks:
+// for heads of 128 and more, whose blocks have no kernel that shares out the keys more finely,
+// as many (2 or 4) as still leave no more workgroups than CUs.  512 queries of 32 heads of 128
+// behind 1,536 cached keys: 52 us in one slice, 44 in two (34 for the slices, the rest for their
+// results' way through memory and the merge); behind 3,584: 92 and 65; behind 512: 30 and 33,
+// from the first token 20 and 28; 256 queries behind 1,024: 33 and 28 in four.  1,024 queries
+// (one block per CU): no gain.  The launch takes the slices when the longest block reads at
+// least kPrefillSliceFromKeys keys (keys_longest; not when the caller does not say).
+extern "C" int kllm_attn_prefill_slices(int n_tiles, int H, int hd) {
+  if (hd < 128 || n_tiles <= 0 || H <= 0) return 1;
+  const long blocks = (long)n_tiles * H;
+  int slices = 1;
+  while (slices < kPrefillMaxSlices && blocks * slices * 2 <= device_cus()) slices *= 2;
+  return slices;
+}
+
 extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                                  int n_tiles, const int* span_start, const int* span_pos,
                                  const int* block_table, int max_pages, int page_size, int H, int KV,
-                                 int hd, int window, float scale, long keys_total, int keys_longest, int dtype,
-                                 hipStream_t stream) {
+                                 int hd, int window, float scale, long keys_total, int keys_longest, float* part,
+                                 long part_floats, int nslices, int n_rows, int dtype, hipStream_t stream) {
   KLLM_REQUIRE(q && out && cache && query_tiles && span_start && span_pos && block_table,
                "attn_prefill: null pointer");
   KLLM_REQUIRE(keys_total >= 0 && keys_longest >= 0, "attn_prefill: negative numbers of keys");
@@ -789,12 +860,18 @@ extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, co
                max_pages, kPrefillMaxPage, kPrefillMaxKeys);
   const long items = (long)n_tiles * H;
   KLLM_REQUIRE(items < (1L << 31), "attn_prefill: too many tiles");
+  KLLM_REQUIRE(nslices >= 1 && nslices <= kPrefillMaxSlices && (nslices == 1 || kllm_attn_prefill_slices(n_tiles, H, hd) > 1),
+               "attn_prefill: %d slices of the keys for %d blocks of %d heads of %d (kllm_attn_prefill_slices says how many)",
+               nslices, n_tiles, H, hd);
+  KLLM_REQUIRE(nslices == 1 || (part && n_rows > 0 && part_floats >= (long)n_rows * H * nslices * (hd + 2)),
+               "attn_prefill: %d slices need room for %d rows x %d heads x %d slices x (%d + 2) floats", nslices, n_rows,
+               H, nslices, hd);
   const int grid = (int)items;
 #define KLLM_PF(HDT)                                                                              \
   case HDT:                                                                                       \
     launch_prefill<HDT>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,  \
                         block_table, max_pages, page_size, H, KV, window, scale, keys_total,      \
-                        keys_longest);                                                            \
+                        keys_longest, part, nslices);                                             \
     break
   switch (hd / 32) {
     KLLM_PF(1); KLLM_PF(2); KLLM_PF(3); KLLM_PF(4); KLLM_PF(6); KLLM_PF(8);

@@ -256,8 +256,14 @@ int kllm_attn_decode_static(const void* q, void* out, const void* cache, const i
 int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                       int n_tiles, const int* span_start, const int* span_pos,
                       const int* block_table, int max_pages, int page_size, int H, int KV, int hd,
-                      int window, float scale, long keys_total, int keys_longest, int dtype,
-                      hipStream_t stream);
+                      int window, float scale, long keys_total, int keys_longest, float* part,
+                      long part_floats, int nslices, int n_rows, int dtype, hipStream_t stream);
+/* nslices of kllm_attn_prefill: how many workgroups share out the keys of a block and head
+ * (1: none; more where few blocks of a large head would leave CUs idle; taken only when
+ * keys_longest says that the longest block reads 1,280 keys or more).  With more than one,
+ * `part` is room for n_rows (the rows of q) x H x nslices x (hd + 2) floats, and the results
+ * are merged by a second kernel of the same call. */
+int kllm_attn_prefill_slices(int n_tiles, int H, int hd);
 
 /* out[r] = sampled index of logits[r][:]; temperature/uniform null: greedy. */
 int kllm_sample(int* out, const float* logits, const float* temperature, const float* uniform,

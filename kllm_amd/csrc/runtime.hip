@@ -150,7 +150,7 @@ extern "C" int kllm_last_error(char* buf, int len) {
   return (int)strlen(buf);
 }
 
-extern "C" int kllm_abi_version(void) { return 7; }
+extern "C" int kllm_abi_version(void) { return 8; }
 
 // Reference: te_device_info, backend/shim.cu:25-34.
 extern "C" int kllm_device_info(int device, char* buf, int len) {

@@ -21,7 +21,7 @@ import torch
 DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
 GEMV_BEST_ROWS = 0         # rows up to which they beat the MFMA kernels in bfloat16: none (a step at 1.1B sizes, one token: 1.036 against 0.963 ms)
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 class KernelError(RuntimeError):
@@ -127,7 +127,8 @@ def _declare(lib):
         "kllm_calibrate_read_workgroups": [],
         "kllm_calibrate_mfma": [I, I, P, P, P],
         "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, P],
-        "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, L, I, I, P],
+        "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, L, I, P, L, I, I, I, P],
+        "kllm_attn_prefill_slices": [I, I, I],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -1047,13 +1048,32 @@ PREFILL_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
 PREFILL_QUERY_BLOCK = 128      # tokens of one request that a workgroup of the prompt kernel takes
 
 
+def attn_prefill_slices(n_tiles, n_heads, head_dim, dtype=torch.bfloat16) -> int:
+    """Workgroups that share out the keys of a block and head in ``attn_prefill`` (1: none):
+    more where few blocks of a large head would leave CUs idle; the library says."""
+    if dtype != torch.bfloat16:
+        return 1
+    return int(library().kllm_attn_prefill_slices(int(n_tiles), int(n_heads), int(head_dim)))
+
+
 def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, block_table, page_size,
-                 n_heads, n_kv_heads, head_dim, window, scale, keys_total=0, keys_longest=0):
+                 n_heads, n_kv_heads, head_dim, window, scale, keys_total=0, keys_longest=0, part=None,
+                 nslices=None):
     """query_tiles [n_tiles, 2] int32: (first token row, span) of each block of up to
     PREFILL_QUERY_BLOCK consecutive tokens of one span.  ``keys_total`` and
     ``keys_longest``: how many keys the blocks read, all together and the longest block
-    alone, if the caller knows (the kernel is chosen by them)."""
+    alone, if the caller knows (the kernel is chosen by them).  ``part``: float32 room for the
+    slices' partial results where ``attn_prefill_slices`` says more than one (rows of q x heads
+    x slices x (head_dim + 2)); made here if the caller brings none.  ``nslices``: 1 to do
+    without slices, or what ``attn_prefill_slices`` says (the default)."""
     n = q.shape[0]
+    if nslices is None:
+        nslices = attn_prefill_slices(n_tiles, n_heads, head_dim, q.dtype)
+    need = n * n_heads * nslices * (head_dim + 2) if nslices > 1 else 0
+    if nslices > 1 and part is None:
+        part = torch.empty(need, dtype=torch.float32, device=q.device)
+    if nslices > 1 and (part.dtype != torch.float32 or part.numel() < need):
+        raise KernelError(f"attn_prefill: {nslices} slices need {need} floats of room, {part.numel()} {part.dtype} given")
     if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape)
             or q.dtype != cache.dtype or out.dtype != q.dtype):
         raise KernelError("attn_prefill: q/out shapes or dtypes do not fit")
@@ -1068,6 +1088,7 @@ def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, bloc
         n_heads, n_kv_heads, head_dim, int(window), float(scale),
         keys_total if type(keys_total) is StepValue else int(keys_total),
         keys_longest if type(keys_longest) is StepValue else int(keys_longest),
+        _ptr(part, "attn part", torch.float32, True) if nslices > 1 else 0, need, nslices, n,
         dtype_code(q.dtype), _stream())
 
 

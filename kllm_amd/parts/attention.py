@@ -216,9 +216,15 @@ class CausalSelfAttention(Part):
             self._decode(ctx, q, out, cache, None if n_short == n else short, n_short)
         if n_blocks:
             total, longest = self._keys_read(ctx)
+            part = None
+            slices = (1 if self.runtime.options.get("no_attention_slices")
+                      else K.attn_prefill_slices(n_blocks, self.heads, self.head_dim, q.dtype))
+            if slices > 1:     # few blocks of a large head: their keys in slices over workgroups, merged in the same call
+                part = ctx.buf("attn.block_part", (n * self.heads * slices * (self.head_dim + 2),), torch.float32)
             K.attn_prefill(q, out, cache.pages, blocks, n_blocks, ctx.span_start,
                            ctx.span_pos, cache.block_table, cache.page_size, self.heads,
-                           self.kv_heads, self.head_dim, self.window, self.scale, total, longest)
+                           self.kv_heads, self.head_dim, self.window, self.scale, total, longest, part=part,
+                           nslices=slices)
 
     def _keys_read(self, ctx):
         """The step's key counts (see ``step_values``), as the engine worked them out for this

@@ -81,6 +81,26 @@ def test_a_long_prompt_with_more_query_blocks_than_cus(model_dirs):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_portions_far_into_a_long_context_with_few_large_heads(model_dirs, dtype):
+    """1,900 tokens of a model with three heads of 128 in portions of 300 and less: from 1,280
+    keys on, the keys of a portion's blocks go in slices over several workgroups whose results
+    a second kernel merges (bfloat16); every position's logits against the plain model's, and
+    the same prompt beside a second request in portions that end inside blocks."""
+    from kllm_amd import kernels as K
+    cfg, d = tiny.CONFIGS["F"], model_dirs("F")
+    assert K.attn_prefill_slices(3, cfg["num_attention_heads"], cfg["head_dim"]) == 4
+    reqs = make_requests(cfg, [1900, 1500], 6)
+    want = expected(d, cfg, reqs, dtype)
+    steps = traces.portions(reqs, seed=2, sizes=(300, 257, 31, 300, 128, 2, 300, 129))
+    rows, rep = replay(d, dtype, steps, traces.peak_tokens(steps))
+    compare(rows, want, dtype, reqs)
+    assert (("attn.block_part", torch.float32) in rep.engine.runtime.workspace._bufs) == (dtype == "bfloat16")
+    steps, peak = traces.mixed(reqs, seed=3, max_live=2, tail=8, max_portion=290)
+    rows, _ = replay(d, dtype, steps, peak)
+    compare(rows, want, dtype, reqs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name,lengths", [("A", [33, 100]), ("B", [40, 129]), ("C", [50]), ("D", [45])])
 def test_bulk_then_last_32_one_by_one(model_dirs, name, lengths, dtype):
     cfg, d = tiny.CONFIGS[name], model_dirs(name)

@@ -946,10 +946,11 @@ def attention_case(H, KV, hd, ps, dtype, window, spans, seed=0):
                 span_pos=torch.tensor([a for a, _ in spans], dtype=torch.int32, device=DEV))
 
 
-def run_prefill(c, min_len=1, keys=(0, 0)):
+def run_prefill(c, min_len=1, keys=(0, 0), part=None):
     """The prompt kernel over the spans of at least min_len tokens; returns
     (output, mask of the rows it computed).  ``keys``: what the caller says
-    about the keys that the blocks read (all together, the longest block)."""
+    about the keys that the blocks read (all together, the longest block).  ``part``:
+    room for the partial results of slices of the keys."""
     tiles, rows = [], torch.zeros(c["q"].shape[0], dtype=torch.bool)
     start = 0
     for s, (_, b) in enumerate(c["spans"]):
@@ -960,7 +961,7 @@ def run_prefill(c, min_len=1, keys=(0, 0)):
     qt = torch.tensor(tiles, dtype=torch.int32, device=DEV)
     out = torch.full_like(c["q"], float("nan"))
     K().attn_prefill(c["q"], out, c["cache"], qt, len(tiles), c["span_start"], c["span_pos"], c["bt"],
-                     c["ps"], c["H"], c["KV"], c["hd"], c["window"], c["scale"], *keys)
+                     c["ps"], c["H"], c["KV"], c["hd"], c["window"], c["scale"], *keys, part=part)
     return out, rows
 
 
@@ -1006,22 +1007,37 @@ def test_attention_generic(H, KV, hd, ps, dtype, window):
 
 @pytest.mark.parametrize("H,KV,hd,ps", [(4, 2, 32, 16), (3, 1, 64, 16), (8, 2, 64, 32), (5, 5, 96, 16),
                                         (2, 1, 128, 16), (2, 2, 192, 16), (2, 1, 256, 16), (32, 4, 64, 16),
-                                        (4, 2, 64, 48), (2, 1, 128, 48), (2, 2, 192, 80)])
+                                        (4, 2, 64, 48), (2, 1, 128, 48), (2, 2, 192, 80), (12, 4, 128, 16),
+                                        (16, 2, 128, 32), (6, 6, 256, 16)])
 @pytest.mark.parametrize("window", [0, 37, 200])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_attention_prefill(H, KV, hd, ps, window, dtype):
     """Whole prompts of ragged lengths, portions behind cached keys that start
-    and end inside pages and query tiles, and a one-token span, in one launch."""
+    and end inside pages and query tiles, and a one-token span, in one launch.  With heads of
+    128 and more and so few blocks, the blocks' keys go in four or two slices over workgroups
+    (a slice may hold no key of a query) and a second kernel merges them."""
     c = attention_case(H, KV, hd, ps, dtype, window,
                        [(0, 45), (300, 9), (0, 100), (37, 70), (5, 1), (16, 32), (31, 33)], seed=5)
     out, rows = run_prefill(c)
     assert rows.all() and torch.isfinite(out).all()
     err = (out.cpu().double() - c["want"]).abs().max()
     assert err < attn_tol(dtype), float(err)
+    if dtype == torch.bfloat16:
+        want_slices = {(2, 128): 4, (2, 192): 4, (2, 256): 4, (12, 128): 2, (16, 128): 2, (6, 256): 4}.get((H, hd), 1)
+        assert K().attn_prefill_slices(7, H, hd) == want_slices       # (the seven spans are seven blocks)
+    # told that the longest block reads many keys, the launch takes the slices (where there are any)
+    slices = K().attn_prefill_slices(7, H, hd, dtype)
+    part = torch.full((c["q"].shape[0] * H * slices * (hd + 2),), float("nan"), device=DEV)
+    out3, _ = run_prefill(c, keys=(20000, 4000), part=part)
+    assert torch.isfinite(out3).all() and (out3.cpu().double() - c["want"]).abs().max() < attn_tol(dtype)
+    assert bool(torch.isfinite(part).any()) == (slices > 1)      # the slices' results went through it
+    _, _ = run_prefill(c, part=part.fill_(float("nan")))
+    assert not torch.isfinite(part).any()                         # ... and not when nothing is said about the keys
     # only the listed spans are touched (fewer query blocks: possibly another of the kernels)
-    out2, rows2 = run_prefill(c, min_len=33)
-    assert torch.isnan(out2.cpu()[~rows2]).all() and torch.isfinite(out2.cpu()[rows2]).all()
-    assert (out2.cpu().double() - c["want"])[rows2].abs().max() < attn_tol(dtype)
+    for keys in ((0, 0), (20000, 4000)):
+        out2, rows2 = run_prefill(c, min_len=33, keys=keys)
+        assert torch.isnan(out2.cpu()[~rows2]).all() and torch.isfinite(out2.cpu()[rows2]).all()
+        assert (out2.cpu().double() - c["want"])[rows2].abs().max() < attn_tol(dtype)
 
 
 def test_attention_prefill_refuses_tables_beyond_its_page_arithmetic():

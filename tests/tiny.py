@@ -6,7 +6,7 @@ width, vocabulary, rotary base, context, eps, tying.  C is multi-head
 (KV = H) with a head size that is not hidden/heads, a width and a vocabulary
 that are not powers of two.  D has sizes the fast kernels refuse (they must
 fall back, never give a wrong result).  E has many heads and room for long
-prompts.  R is the reference's own tiny model
+prompts.  F has few heads of 128 and room for long prompts.  R is the reference's own tiny model
 (tools/make_test_model.py:47-100).
 """
 
@@ -43,6 +43,11 @@ CONFIGS = {
     "E": _cfg(num_hidden_layers=1, hidden_size=64, num_attention_heads=16, num_key_value_heads=4,
               head_dim=32, intermediate_size=96, vocab_size=96, rope_theta=10000.0,
               max_position_embeddings=4096, rms_norm_eps=1e-5, tie_word_embeddings=False),
+    # few heads of 128 and a long context: portions of a prompt far into it share out a block's
+    # keys over several workgroups
+    "F": _cfg(num_hidden_layers=2, hidden_size=72, num_attention_heads=3, num_key_value_heads=1,
+              head_dim=128, intermediate_size=80, vocab_size=101, rope_theta=100000.0,
+              max_position_embeddings=4096, rms_norm_eps=1e-5, tie_word_embeddings=True),
     "R": _cfg(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2,
               head_dim=16, intermediate_size=128, vocab_size=512, rope_theta=10000.0,
               max_position_embeddings=256, rms_norm_eps=1e-6, tie_word_embeddings=False,

@@ -347,11 +347,13 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, 
   // 12.6 us with 13), but no more than the chip holds at a time (10 tokens x 8 KV heads of
   // 128 at 4,096 keys, two workgroups a CU: 35.5 us with 6, 41.1 us with 8, which is 640
   // workgroups).  A wave should have two tiles of 16 keys at least: 16 workgroups to a group
-  // at contexts of 2,048, more where the caller says that requests may be longer, up to 32
-  // and, beyond 16,384 keys, 64: every workgroup more is a partial result more to merge (one
-  // token, 4 KV heads of 64, attention and merge in us with 16 / 32 / 64 / 128 workgroups to
-  // a group: 8,192 keys 14.3 / 12.5 / 13.4 / 19.4, 16,384 keys 22.7 / 15.9 / 15.9 / 21.0,
-  // 32,768 keys 37.0 / 25.3 / 20.0 / 26.0, 131,072 keys 129 / 70.6 / 44.7 / 47.1).
+  // at contexts of 2,048, 32 at 4,096 and 64 from 8,192 keys on: every workgroup more is a
+  // partial result more to merge, but the merge asks for all of them at once (one token, 4 KV
+  // heads of 64, attention and merge in us with 16 / 32 / 64 workgroups to a group: 2,048 keys
+  // 7.2 / 7.4 / 8.2, 4,096 keys 9.5 / 7.9 / 8.5, 8,192 keys 13.5 / 10.4 / 9.3, 16,384 keys
+  // 21.5 / 14.2 / 12.8, 32,768 keys 37.4 / 22.9 / 16.7, 131,072 keys 143 / 76.4 / 45.9; four
+  // tokens: 2,048 keys 8.2 / 8.7 / 9.8, 8,192 keys 15.7 / 13.1 / 15.5; when the merge took
+  // sixteen at a time, 64 workgroups at 32,768 keys took 23.2 us and 16 at 2,048 keys 8.6).
   const int head_tiles = (H / KV + 15) / 16;
   long groups = (long)n * KV * head_tiles;
   const int hdt = (hd + 15) / 16;
@@ -378,7 +380,7 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, 
   const long fit = (long)decode_resident(hdt, heads, false) * device_cus() / groups;   // what the chip holds at a time
   if (wg > fit) wg = (int)fit;
   int most = max_keys > 2048 ? max_keys / (32 * kDecodeWavesShared) : 16;
-  const int cap = max_keys > 16384 ? 64 : 32;
+  const int cap = max_keys >= 8192 ? 64 : 32;
   if (most > cap) most = cap;
   if (wg > most) wg = most;
   if (wg < 1) wg = 1;

@@ -1174,11 +1174,12 @@ def test_attention_decode_takes_more_slices_for_longer_contexts():
     H, KV, hd, ps, dtype = 8, 2, 64, 16, torch.bfloat16
     few = k_.attn_decode_slices(1, KV, H, hd, dtype, 2048)
     assert few == k_.attn_decode_slices(1, KV, H, hd, dtype) == 16
+    assert k_.attn_decode_slices(1, KV, H, hd, dtype, 4096) == 32 and k_.attn_decode_slices(1, KV, H, hd, dtype, 8192) == 64
     assert k_.attn_decode_slices(k_.device_cus(), 1, 8, hd, dtype) == 1     # a workgroup to a token
     c = attention_case(H, KV, hd, ps, dtype, 0, [(20000, 1), (37, 1)], seed=9)
     many = k_.attn_decode_slices(2, KV, H, hd, dtype, c["bt"].shape[1] * ps)
     assert few < many <= 64
-    for ns in (1, few, many, 256):
+    for ns in (1, 2, 7, few, 17, 32, 33, many, 65, 100, 256):      # (up to 64 slices: the merge that asks for all at once)
         out = run_attention("decode", c["q"], c["cache"], c["pos"], c["sot"], c["bt"], ps, H, KV, hd, 0, c["scale"], ns)
         assert (out.cpu().double() - c["want"]).abs().max() < attn_tol(dtype), ns
 

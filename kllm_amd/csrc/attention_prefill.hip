@@ -455,7 +455,7 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attn_prefill_merge_kernel(
   if (t >= span_start[query_tiles[2 * tile + 1] + 1]) return;
   const int h = blockIdx.y * kMergeWaves + threadIdx.x / kWave;
   if (h >= H) return;
-  attn_merge_one<bf16_t, DV, 4>(out, part, t, h, H, hd, nslices, threadIdx.x % kWave);
+  attn_merge_wide<bf16_t, DV, kPrefillMaxSlices>(out, part, t, h, H, hd, nslices, threadIdx.x % kWave);
 }
 
 // ---------------------------------------------------------------------------

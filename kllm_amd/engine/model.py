@@ -210,10 +210,14 @@ class Model:
             ctx.taps.append(x.clone())
         def walk_through(i, x, pending):
             block = self.blocks[self.schedule[i].layer]
-            if getattr(block, "takes_next_norm", False) and i + 1 < len(self.schedule):
-                # the norm that will take this layer's output, if the next layer names one
-                nxt = self.blocks[self.schedule[i + 1].layer]
-                first = nxt.first_norm() if hasattr(nxt, "first_norm") else None
+            if getattr(block, "takes_next_norm", False):
+                # the norm that will take this layer's output: the next layer's first, if it names
+                # one, and the final norm behind the last layer
+                if i + 1 < len(self.schedule):
+                    nxt = self.blocks[self.schedule[i + 1].layer]
+                    first = nxt.first_norm() if hasattr(nxt, "first_norm") else None
+                else:
+                    first = self.final_norm
                 return call_part(block, block.forward, ctx, x, pending, cache_views[i], next_norm=first)
             return call_part(block, block.forward, ctx, x, pending, cache_views[i])
 
